@@ -1,0 +1,266 @@
+/*
+ * fusor_hip.h -- C ABI of libfusor_hip.so, an AMD Instinct MI355X (gfx950) backend for
+ * the quantized-inference hot path of Fusor (floneum/kalosm).
+ *
+ * The reference has no C ABI: its backend seam is the Rust enum facade of the
+ * `fusor` crate (`Tensor::{Cpu,Gpu}`, `QMatrix::{Cpu*,Gpu}`, `Device::{Cpu,Gpu}`).
+ * Each entry point below names the reference method it stands in for
+ * (paths relative to the reference tree).  A Rust `Hip` arm of those enums binds
+ * these symbols one to one.
+ *
+ * Conventions
+ *   - Every function returns fh_status (0 = ok, negative = error); the message of
+ *     the last error on the calling thread is fh_last_error().  Nothing aborts or
+ *     throws across the boundary.  The reference panics on programmer errors
+ *     (shape mismatch: fusor-ml/cpu/src/quantized.rs:270-274); here they are
+ *     FH_ERR_INVALID.
+ *   - All device pointers (`*_dev`) come from fh_malloc on the same fh_device.
+ *     Work is enqueued on the device's single HIP stream and is asynchronous;
+ *     fh_device_sync and the blocking copies are the only synchronisation points
+ *     (the reference executes at `materialize()/as_slice()`,
+ *     fusor-ml/core/src/tensor/mod.rs:197-274).
+ *   - Calls on one fh_device must be serialised by the caller; handles may move
+ *     between threads.
+ *   - Tensors are row-major contiguous f32 unless a stride argument says otherwise.
+ */
+#ifndef FUSOR_HIP_H
+#define FUSOR_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
+
+typedef int32_t fh_status;
+enum {
+    FH_OK = 0,
+    FH_ERR_INVALID = -1,     /* bad argument / shape mismatch */
+    FH_ERR_HIP = -2,         /* a HIP runtime call failed */
+    FH_ERR_UNSUPPORTED = -3, /* GgufReadError::UnsupportedDType (fusor-ml/core/src/quantized/mod.rs:485) */
+    FH_ERR_OOM = -4,
+    FH_ERR_NO_DEVICE = -5    /* Device::gpu() failed (fusor-ml/fusor/src/device.rs:29-39) */
+};
+
+/* GgmlType ids, fusor-ml/gguf/src/lib.rs:35-50 */
+enum { FH_Q4_0 = 2, FH_Q8_0 = 8, FH_Q4_K = 12, FH_Q6_K = 14 };
+
+/* MaskKind, fusor-ml/fusor/src/composite/flash_attention.rs:12-24 */
+enum { FH_MASK_NONE = 0, FH_MASK_CAUSAL = 1, FH_MASK_ADDITIVE = 2 };
+
+/* element types of attention operands */
+enum { FH_F32 = 0, FH_F16 = 1 };
+
+typedef struct fh_device fh_device;
+typedef struct fh_qmatrix fh_qmatrix;
+typedef struct fh_kvcache fh_kvcache;
+typedef struct fh_llama fh_llama;
+
+const char *fh_last_error(void);
+/* Version string of the library, and the gfx target it was built for. */
+const char *fh_version(void);
+
+/* ------------------------------------------------------------------ device
+ * Device::gpu() / Device::auto(), fusor-ml/fusor/src/device.rs:29-39, :60-78. */
+fh_status fh_device_count(int32_t *count);
+fh_status fh_device_create(int32_t ordinal, fh_device **out);
+fh_status fh_device_destroy(fh_device *dev);
+fh_status fh_device_sync(fh_device *dev);
+/* Name, compute-unit count and memory of the device (for reports). */
+fh_status fh_device_info(fh_device *dev, char *name, size_t name_cap, int32_t *compute_units,
+                         uint64_t *total_mem_bytes);
+
+/* Tensor::from_slice / new / zeros / as_slice, fusor-ml/fusor/src/lib.rs:356-368. */
+fh_status fh_malloc(fh_device *dev, size_t bytes, void **out_dev);
+fh_status fh_free(fh_device *dev, void *ptr_dev);
+fh_status fh_memset(fh_device *dev, void *ptr_dev, int32_t byte, size_t bytes);
+fh_status fh_upload(fh_device *dev, void *dst_dev, const void *src_host, size_t bytes);   /* blocking */
+fh_status fh_download(fh_device *dev, void *dst_host, const void *src_dev, size_t bytes); /* blocking */
+fh_status fh_copy(fh_device *dev, void *dst_dev, const void *src_dev, size_t bytes);      /* async */
+
+/* Event timing on the device's stream (the reference's FUSOR_TRACE_GPU_KERNELS timestamp
+ * queries, fusor-ml/core/src/compute_graph/resolve/run.rs:483-497). */
+fh_status fh_timer_start(fh_device *dev);
+fh_status fh_timer_stop(fh_device *dev, float *elapsed_ms); /* blocks until the stream reaches it */
+
+/* ----------------------------------------------------------------- weights
+ * QMatrix::from_raw_bytes(&Device, shape, &[u8], GgmlType), fusor-ml/fusor/src/quantized.rs:183-225.
+ * `bytes` is the raw GGUF block stream of an [n, k] weight (blocks contiguous along k);
+ * it is re-laid-out on the device, the host buffer is not referenced after return. */
+fh_status fh_qmatrix_from_gguf_bytes(fh_device *dev, uint32_t ggml_type, int64_t n, int64_t k,
+                                     const void *bytes, size_t len, fh_qmatrix **out);
+/* QMatrix::concat_rows, fusor-ml/fusor/src/quantized.rs:102-112 (same type and k). */
+fh_status fh_qmatrix_concat_rows(fh_device *dev, const fh_qmatrix *const *parts, int32_t count,
+                                 fh_qmatrix **out);
+fh_status fh_qmatrix_free(fh_qmatrix *q);
+/* QMatrix::shape / ggml_type, fusor-ml/fusor/src/quantized.rs:114-180. */
+fh_status fh_qmatrix_info(const fh_qmatrix *q, uint32_t *ggml_type, int64_t *n, int64_t *k,
+                          uint64_t *device_bytes);
+/* QMatrix::dequantize::<R>() -> Tensor<R,f32>, fusor-ml/fusor/src/quantized.rs:233-279.
+ * out_dev is [n, k] f32; values are bit-identical to GgufBlock::dequantize
+ * (fusor-ml/gguf/src/lib.rs:828-846, :1284-1288, :1526-1556, :2034-2085). */
+fh_status fh_qmatrix_dequantize(const fh_qmatrix *q, float *out_dev);
+/* Embedding::forward, fusor-ml/fusor/src/layers/embedding.rs:43-89: out[t,:] = dequantize(W)[ids[t],:].
+ * ids_dev is u32 [count] on the device; ids >= n give FH_ERR_INVALID only when checked on the host
+ * (pass ids_host != NULL to have them validated before launch). */
+fh_status fh_embed_rows(const fh_qmatrix *q, const uint32_t *ids_dev, const uint32_t *ids_host,
+                        int32_t count, float *out_dev);
+
+/* ------------------------------------------------------------------ matmul
+ * Tensor<R,f32>::q_mat_mul(&QMatrix), fusor-ml/fusor/src/lib.rs:1132-1223 ->
+ * fusor-ml/cpu/src/quantized.rs:246-365: y[m, n] = sum_k x[m, k] * dequantize(W)[n, k].
+ * x_dev [m, k] f32, y_dev [m, n] f32.  Any m >= 1; m <= 16 takes the bandwidth-tuned
+ * decode kernels, larger m the MFMA tile kernel. */
+fh_status fh_qmatmul(const fh_qmatrix *q, const float *x_dev, int32_t m, float *y_dev);
+/* Epilogue forms the reference folds into the same dispatch:
+ *   fh_qmatmul_add2:  y = (x.W^T + a) + b       raw/attention_layer.rs:168-173
+ *   fh_qmatmul_swiglu: W = concat_rows(gate, up); y[m, i] = silu(g[m,i]) * u[m,i], y is [m, n/2]
+ *                                               raw/attention_layer.rs:186-196 */
+fh_status fh_qmatmul_add2(const fh_qmatrix *q, const float *x_dev, int32_t m, const float *a_dev,
+                          const float *b_dev, float *y_dev);
+fh_status fh_qmatmul_swiglu(const fh_qmatrix *q, const float *x_dev, int32_t m, float *y_dev);
+/* Prefill activations given as bf16 (raw u16 bit patterns): same product, x_dev is [m, k] bf16. */
+fh_status fh_qmatmul_bf16(const fh_qmatrix *q, const uint16_t *x_bf16_dev, int32_t m, float *y_dev);
+/* The Q8_0 x Q8 variant: activations quantised per 32 along k exactly as BlockQ8_0::quantize
+ * (fusor-ml/gguf/src/lib.rs:1150-1230, round half to even as on an AVX2 host) and each block
+ * combined as GgufBlock::vec_dot (fusor-ml/gguf/src/lib.rs:1315-1358): integer dot, then
+ * (sum as f32) * (d_w * d_a), summed over blocks in k order.  Q8_0 and Q4_0 weights only.
+ * isums_dev (optional, int32 [m, n, k/32]) receives the exact integer block sums. */
+fh_status fh_qmatmul_q8(const fh_qmatrix *q, const float *x_dev, int32_t m, float *y_dev,
+                        int32_t *isums_dev);
+/* BlockQ8_0::quantize over a flat f32 array (count % 32 == 0): out_dev is count/32 blocks of 34 bytes. */
+fh_status fh_q8_0_quantize(fh_device *dev, const float *x_dev, int64_t count, void *out_dev);
+
+/* Kernel selection override for measurement (the reference's FUSOR_* tile overrides,
+ * fusor-ml/tile-ir-kernels/src/dispatch.rs:15-20).  key/value pairs documented in the README of
+ * the csrc directory; unknown keys give FH_ERR_INVALID. */
+fh_status fh_set_option(fh_device *dev, const char *key, int64_t value);
+
+/* -------------------------------------------------------------------- norm
+ * rms_norm_fused / rms_norm_residual_fused, fusor-ml/fusor/src/composite/normalization.rs:287-401:
+ * y = ((x [+ residual]) / sqrt(mean((x [+ residual])^2) + eps)) * w [+ bias].  residual_dev and
+ * bias_dev may be NULL.  x, residual, y are [rows, cols]; w, bias are [cols]. */
+fh_status fh_rms_norm(fh_device *dev, const float *x_dev, const float *residual_dev,
+                      const float *w_dev, const float *bias_dev, float eps, int32_t rows,
+                      int32_t cols, float *y_dev);
+
+/* -------------------------------------------------------------------- rope
+ * RopeCache::new, fusor-ml/fusor/src/composite/rope.rs:241-275 and
+ * models/kalosm-llama/src/raw/rope.rs:63-85: cos/sin tables [ctx, head_dim/2] built on the
+ * host in f32 (powf, mul, cosf/sinf) and uploaded. */
+fh_status fh_rope_tables(fh_device *dev, int32_t head_dim, int32_t ctx, float theta, float *cos_dev,
+                         float *sin_dev);
+/* RopeCache::forward{,_interleaved}(&q, &k, start_pos), rope.rs:284-329.  q is [b, hq, s, d] and
+ * k is [b, hk, s, d] as VIEWS: element (b, h, t, c) of q lives at q_dev[b*q_sb + h*q_sh + t*q_st + c]
+ * (strides in elements), likewise k.  Outputs are contiguous [b, h, s, d].  One launch rotates both. */
+fh_status fh_rope_pair(fh_device *dev, const float *q_dev, int64_t q_sb, int64_t q_sh, int64_t q_st,
+                       const float *k_dev, int64_t k_sb, int64_t k_sh, int64_t k_st, int32_t b,
+                       int32_t hq, int32_t hk, int32_t s, int32_t d, const float *cos_dev,
+                       const float *sin_dev, int32_t table_rows, int32_t start_pos,
+                       int32_t interleaved, float *q_out_dev, float *k_out_dev);
+
+/* ---------------------------------------------------------------- KV cache
+ * KvCache::new / append / reset, fusor-ml/fusor/src/cache/kv_cache.rs:24-63 and
+ * tensor_cache.rs:70-114, :304-312.  One object holds all layers.  Storage is
+ * [layer][kv_head][capacity][head_dim] per K and V, f32 (the reference's cache type,
+ * models/kalosm-llama/src/raw/cache.rs:18) or f16.  Capacity grows to the next power of two
+ * (minimum 256, capped at max_len) preserving contents; exceeding max_len is FH_ERR_INVALID
+ * (sliding-window eviction is outside this library's scope). */
+fh_status fh_kvcache_create(fh_device *dev, int32_t layers, int32_t kv_heads, int32_t head_dim,
+                            int32_t max_len, int32_t dtype, fh_kvcache **out);
+fh_status fh_kvcache_destroy(fh_kvcache *c);
+fh_status fh_kvcache_reset(fh_kvcache *c);
+/* Append s positions to `layer`.  k and v are [kv_heads, s, head_dim] f32 views with head stride
+ * `sh` and position stride `st` (elements).  The cache length advances when the LAST layer is
+ * appended (all layers receive the same s per step). */
+fh_status fh_kvcache_append(fh_kvcache *c, int32_t layer, const float *k_dev, const float *v_dev,
+                            int64_t sh, int64_t st, int32_t s);
+/* Current length, capacity, and the device pointers of one layer's K and V planes
+ * ([kv_heads, capacity, head_dim]). */
+fh_status fh_kvcache_view(const fh_kvcache *c, int32_t layer, int32_t *len, int32_t *capacity,
+                          const void **k_dev, const void **v_dev);
+
+/* --------------------------------------------------------------- attention
+ * Tensor<4>::flash_attention(&k, &v, scale, Option<(&mask, MaskKind)>),
+ * fusor-ml/fusor/src/composite/flash_attention.rs:58-109 (GQA: kv head = h / (hq / hkv)).
+ * q [b, hq, sq, d] view with strides (elements) q_sb, q_sh, q_st; k, v [b, hkv, skv, d] views
+ * with strides kv_sb, kv_sh, kv_st; out contiguous [b, hq, sq, d].  dtype is FH_F32 or FH_F16 for
+ * q/k/v/out alike (kv may be f16 with f32 q via fh_flash_attention_ex).  mask_dev is
+ * [sq, skv] f32 for FH_MASK_ADDITIVE, ignored otherwise.  FH_MASK_CAUSAL lets query i see keys
+ * j <= i + (skv - sq) (attention_mask.rs:46-66 with the offset padding of mask_cache.rs:73-88).
+ * d <= 256; d of 64 or 128 takes the tuned kernels. */
+fh_status fh_flash_attention(fh_device *dev, int32_t dtype, const void *q_dev, int64_t q_sb,
+                             int64_t q_sh, int64_t q_st, const void *k_dev, const void *v_dev,
+                             int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int32_t b, int32_t hq,
+                             int32_t hkv, int32_t sq, int32_t skv, int32_t d, float scale,
+                             int32_t mask_kind, const float *mask_dev, void *out_dev);
+/* As above with separate element types: q/out of q_dtype, k/v of kv_dtype. */
+fh_status fh_flash_attention_ex(fh_device *dev, int32_t q_dtype, int32_t kv_dtype, const void *q_dev,
+                                int64_t q_sb, int64_t q_sh, int64_t q_st, const void *k_dev,
+                                const void *v_dev, int64_t kv_sb, int64_t kv_sh, int64_t kv_st,
+                                int32_t b, int32_t hq, int32_t hkv, int32_t sq, int32_t skv,
+                                int32_t d, float scale, int32_t mask_kind, const float *mask_dev,
+                                void *out_dev);
+
+/* -------------------------------------------------------------------- glue
+ * silu(g) * u, fusor-ml/fusor/src/composite/activations.rs:47-65 + raw/attention_layer.rs:195 */
+fh_status fh_swiglu(fh_device *dev, const float *gate_dev, const float *up_dev, float *y_dev,
+                    int64_t count);
+/* (a + b) + c, models/kalosm-llama/src/raw/mod.rs:1036; c_dev may be NULL for a + b. */
+fh_status fh_add3(fh_device *dev, const float *a_dev, const float *b_dev, const float *c_dev,
+                  float *y_dev, int64_t count);
+/* [s, h, d] -> [h, s, d] (reshape + transpose(1,2) + to_concrete) and back; f32. */
+fh_status fh_transpose_shd(fh_device *dev, const float *x_dev, int32_t s, int32_t h, int32_t d,
+                           float *y_dev);
+fh_status fh_cast_f32_f16(fh_device *dev, const float *x_dev, void *y_f16_dev, int64_t count);
+fh_status fh_cast_f16_f32(fh_device *dev, const void *x_f16_dev, float *y_dev, int64_t count);
+fh_status fh_cast_f32_bf16(fh_device *dev, const float *x_dev, void *y_bf16_dev, int64_t count);
+/* Tensor::top_k_pairs(1), fusor-ml/fusor/src/lib.rs:416-447: largest finite value, ties to the
+ * larger index, non-finite skipped; *id_dev = 0xFFFFFFFF when nothing is finite. */
+fh_status fh_argmax(fh_device *dev, const float *x_dev, int64_t count, uint32_t *id_dev);
+
+/* ----------------------------------------------------------------- decoder
+ * Model::forward for the Llama architecture, models/kalosm-llama/src/raw/mod.rs:851-865,
+ * :925-1049 (Separate attention variant + Llama feed-forward, interleaved RoPE), with the
+ * greedy decode loop of model/inference.rs:11-396 reduced to argmax. */
+typedef struct {
+    int32_t n_layers, d_model, n_heads, n_kv_heads, head_dim, ffn, vocab, ctx;
+    float eps, theta;
+    int32_t kv_dtype;       /* FH_F32 (reference) or FH_F16 */
+    int32_t fuse_qkv;       /* concat_rows(q, k, v) as raw/mod.rs:511 */
+    int32_t fuse_gate_up;   /* concat_rows(gate, up) as raw/attention_layer.rs:96-107 */
+    int32_t use_graph;      /* capture one decode step in a hipGraph and replay it */
+} fh_llama_config;
+
+fh_status fh_llama_create(fh_device *dev, const fh_llama_config *cfg, fh_llama **out);
+fh_status fh_llama_destroy(fh_llama *m);
+/* Load one GGUF tensor by its GGUF name (`token_embd.weight`, `blk.N.attn_q.weight`, ...,
+ * models/kalosm-llama/src/raw/mod.rs:473-604).  ggml_type 0 (F32) for norm vectors. */
+fh_status fh_llama_load_tensor(fh_llama *m, const char *name, uint32_t ggml_type, int64_t n,
+                               int64_t k, const void *bytes, size_t len);
+/* Fuse/concatenate what the config asks for and allocate the step buffers; call once after loading. */
+fh_status fh_llama_finalize(fh_llama *m);
+fh_status fh_llama_reset(fh_llama *m);
+/* Run `count` new tokens at the current position; logits_host (optional, [vocab]) and
+ * hidden_host (optional, [d_model], the final-norm hidden state) are of the LAST token. */
+fh_status fh_llama_forward(fh_llama *m, const uint32_t *tokens_host, int32_t count,
+                           float *logits_host, float *hidden_host);
+/* Greedy decode: feeds `first_token`, then each argmax, for `steps` steps entirely on the device
+ * (the sampled id stays resident, as the reference's run-ahead path, model/inference.rs:38-173);
+ * out_tokens_host receives the `steps` sampled ids.  elapsed_ms (optional) is the device time. */
+fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, int32_t steps,
+                                 uint32_t *out_tokens_host, float *elapsed_ms);
+/* Bytes of weights read per decoded token (for roofline reports). */
+fh_status fh_llama_weight_bytes(const fh_llama *m, uint64_t *bytes);
+
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
+#ifdef __cplusplus
+}
+#endif
+#endif /* FUSOR_HIP_H */

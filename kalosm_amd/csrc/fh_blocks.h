@@ -1,0 +1,122 @@
+// Device-side accessors of the tiled weight layouts (see fh_internal.h) and the bit-exact
+// block decode of the four GGUF formats.  The arithmetic follows GgufBlock::dequantize
+// (fusor-ml/gguf/src/lib.rs:828-846, :1284-1288, :1526-1556, :2034-2085) operation for
+// operation; the library is built with -ffp-contract=off so `a*b - c` is never fused.
+#pragma once
+#include "fh_internal.h"
+
+typedef _Float16 fh_half;
+
+__device__ __forceinline__ float fh_h2f(uint16_t bits) {
+    fh_half h;
+    __builtin_memcpy(&h, &bits, 2);
+    return (float)h;
+}
+
+// ---- byte addresses inside a tile record -------------------------------------------------
+// Q4_K: record 2304 B
+__device__ __host__ __forceinline__ int q4k_hdr_off(int j) { return 16 * j; }
+__device__ __host__ __forceinline__ int q4k_qs_off(int j, int i) { // i: byte 0..127 of the block's qs
+    int p = i >> 6, w = i & 63, c2 = w >> 5, o = w & 31, g = o >> 3, r = o & 7;
+    return 256 + p * 1024 + (g * 16 + j) * 16 + c2 * 8 + r;
+}
+// Q6_K: record 3360 B
+__device__ __host__ __forceinline__ int q6k_ql_off(int j, int i) { // i: 0..127
+    int p = i >> 6, o = i & 63, g = o >> 4, r = o & 15;
+    return p * 1024 + (g * 16 + j) * 16 + r;
+}
+__device__ __host__ __forceinline__ int q6k_qh_off(int j, int i) { // i: 0..63
+    int p = i >> 5, o = i & 31, g = o >> 3, r = o & 7;
+    return 2048 + p * 512 + (g * 16 + j) * 8 + r;
+}
+__device__ __host__ __forceinline__ int q6k_sc_off(int j, int i) { return 3072 + 16 * j + i; }
+__device__ __host__ __forceinline__ int q6k_d_off(int j) { return 3328 + 2 * j; }
+// Q8_0: record 1088 B = two blocks
+__device__ __host__ __forceinline__ int q80_q_off(int j, int u, int i) { // u: block in record, i: 0..31
+    int g = i >> 3, r = i & 7;
+    return (g * 16 + j) * 16 + u * 8 + r;
+}
+__device__ __host__ __forceinline__ int q80_d_off(int j, int u) { return 1024 + 4 * j + 2 * u; }
+// Q4_0: record 1152 B = four blocks
+__device__ __host__ __forceinline__ int q40_q_off(int j, int u, int i) { // i: byte 0..15
+    int g = i >> 2, r = i & 3;
+    return (g * 16 + j) * 16 + u * 4 + r;
+}
+__device__ __host__ __forceinline__ int q40_d_off(int j, int u) { return 1024 + 8 * j + 2 * u; }
+
+__device__ __forceinline__ uint16_t fh_ld16(const uint8_t *p) { return *(const uint16_t *)p; }
+
+// ---- one dequantised element -------------------------------------------------------------
+__device__ __forceinline__ float deq_elem_q4_0(const QView &q, int64_t row, int64_t k) {
+    int64_t b = k >> 5;
+    int e = (int)(k & 31);
+    const uint8_t *rec = q.data + ((row >> 4) * q.recs + (b >> 2)) * (int64_t)q.rec_bytes;
+    int j = (int)(row & 15), u = (int)(b & 3);
+    float d = fh_h2f(fh_ld16(rec + q40_d_off(j, u)));
+    uint8_t byte = rec[q40_q_off(j, u, e & 15)];
+    int v = (e < 16 ? (byte & 0x0F) : (byte >> 4)) - 8;
+    return (float)v * d;
+}
+
+__device__ __forceinline__ float deq_elem_q8_0(const QView &q, int64_t row, int64_t k) {
+    int64_t b = k >> 5;
+    int e = (int)(k & 31);
+    const uint8_t *rec = q.data + ((row >> 4) * q.recs + (b >> 1)) * (int64_t)q.rec_bytes;
+    int j = (int)(row & 15), u = (int)(b & 1);
+    float d = fh_h2f(fh_ld16(rec + q80_d_off(j, u)));
+    int v = (int)(int8_t)rec[q80_q_off(j, u, e)];
+    return (float)v * d;
+}
+
+__device__ __forceinline__ void q4k_scale_min(const uint8_t *p, int s, int &sc, int &mn) {
+    if (s < 4) {
+        sc = p[s] & 63;
+        mn = p[4 + s] & 63;
+    } else {
+        sc = (p[4 + s] & 0x0F) | ((p[s - 4] >> 6) << 4);
+        mn = (p[4 + s] >> 4) | ((p[s] >> 6) << 4);
+    }
+}
+
+__device__ __forceinline__ float deq_elem_q4_k(const QView &q, int64_t row, int64_t k) {
+    int64_t b = k >> 8;
+    int e = (int)(k & 255);
+    const uint8_t *rec = q.data + ((row >> 4) * q.recs + b) * (int64_t)q.rec_bytes;
+    int j = (int)(row & 15);
+    const uint8_t *h = rec + q4k_hdr_off(j);
+    float d = fh_h2f(fh_ld16(h)), dmin = fh_h2f(fh_ld16(h + 2));
+    int s = e >> 5; // sub-block 0..7
+    int sc, mn;
+    q4k_scale_min(h + 4, s, sc, mn);
+    int c = e >> 6, l = e & 31;
+    uint8_t byte = rec[q4k_qs_off(j, 32 * c + l)];
+    int v = (s & 1) ? (byte >> 4) : (byte & 0x0F);
+    float scale = (float)sc * d;
+    float off = (float)mn * dmin;
+    float prod = scale * (float)v;
+    return prod - off;
+}
+
+__device__ __forceinline__ float deq_elem_q6_k(const QView &q, int64_t row, int64_t k) {
+    int64_t b = k >> 8;
+    int e = (int)(k & 255);
+    const uint8_t *rec = q.data + ((row >> 4) * q.recs + b) * (int64_t)q.rec_bytes;
+    int j = (int)(row & 15);
+    int n = e >> 7, jj = (e >> 5) & 3, l = e & 31;
+    uint8_t lo = rec[q6k_ql_off(j, 64 * n + l + ((jj & 1) ? 32 : 0))];
+    uint8_t hi = rec[q6k_qh_off(j, 32 * n + l)];
+    int nib = (jj & 2) ? (lo >> 4) : (lo & 0x0F);
+    int v = (int)(int8_t)((((hi >> (2 * jj)) & 3) << 4) | nib) - 32;
+    int sc = (int)(int8_t)rec[q6k_sc_off(j, 8 * n + 2 * jj + (l >> 4))];
+    float d = fh_h2f(fh_ld16(rec + q6k_d_off(j)));
+    float ds = d * (float)sc;
+    return ds * (float)v;
+}
+
+template <int T>
+__device__ __forceinline__ float deq_elem(const QView &q, int64_t row, int64_t k) {
+    if (T == FH_Q4_0) return deq_elem_q4_0(q, row, k);
+    if (T == FH_Q8_0) return deq_elem_q8_0(q, row, k);
+    if (T == FH_Q4_K) return deq_elem_q4_k(q, row, k);
+    return deq_elem_q6_k(q, row, k);
+}

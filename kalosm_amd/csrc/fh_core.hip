@@ -1,0 +1,171 @@
+// Device, memory, error and timing entry points of libfusor_hip.so.
+#include "fh_internal.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+static thread_local char g_err[512] = "";
+
+void fh_set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" const char *fh_last_error(void) { return g_err; }
+extern "C" const char *fh_version(void) { return "fusor-hip 0.1 (gfx950)"; }
+
+extern "C" fh_status fh_device_count(int32_t *count) {
+    FH_REQUIRE(count, "count is NULL");
+    int c = 0;
+    hipError_t e = hipGetDeviceCount(&c);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        c = 0;
+    }
+    *count = c;
+    return FH_OK;
+}
+
+extern "C" fh_status fh_device_create(int32_t ordinal, fh_device **out) {
+    FH_REQUIRE(out, "out is NULL");
+    *out = nullptr;
+    int c = 0;
+    if (hipGetDeviceCount(&c) != hipSuccess || c <= 0) {
+        (void)hipGetLastError();
+        FH_FAIL(FH_ERR_NO_DEVICE, "no HIP device available");
+    }
+    FH_REQUIRE(ordinal >= 0 && ordinal < c, "device ordinal %d out of range (have %d)", ordinal, c);
+    FH_HIP(hipSetDevice(ordinal));
+    hipDeviceProp_t p;
+    FH_HIP(hipGetDeviceProperties(&p, ordinal));
+    if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
+        FH_FAIL(FH_ERR_NO_DEVICE, "device %d is %s; this library holds gfx950 code only", ordinal, p.gcnArchName);
+    fh_device *d = new fh_device();
+    d->ordinal = ordinal;
+    d->compute_units = p.multiProcessorCount;
+    FH_HIP(hipStreamCreate(&d->stream));
+    FH_HIP(hipEventCreate(&d->ev_start));
+    FH_HIP(hipEventCreate(&d->ev_stop));
+    *out = d;
+    return FH_OK;
+}
+
+extern "C" fh_status fh_device_destroy(fh_device *dev) {
+    if (!dev) return FH_OK;
+    (void)hipSetDevice(dev->ordinal);
+    (void)hipStreamSynchronize(dev->stream);
+    if (dev->act_buf) (void)hipFree(dev->act_buf);
+    if (dev->part_buf) (void)hipFree(dev->part_buf);
+    (void)hipEventDestroy(dev->ev_start);
+    (void)hipEventDestroy(dev->ev_stop);
+    (void)hipStreamDestroy(dev->stream);
+    delete dev;
+    return FH_OK;
+}
+
+extern "C" fh_status fh_device_sync(fh_device *dev) {
+    FH_REQUIRE(dev, "dev is NULL");
+    FH_HIP(hipStreamSynchronize(dev->stream));
+    return FH_OK;
+}
+
+extern "C" fh_status fh_device_info(fh_device *dev, char *name, size_t name_cap, int32_t *compute_units,
+                                    uint64_t *total_mem_bytes) {
+    FH_REQUIRE(dev, "dev is NULL");
+    hipDeviceProp_t p;
+    FH_HIP(hipGetDeviceProperties(&p, dev->ordinal));
+    if (name && name_cap) snprintf(name, name_cap, "%s (%s)", p.name, p.gcnArchName);
+    if (compute_units) *compute_units = p.multiProcessorCount;
+    if (total_mem_bytes) *total_mem_bytes = (uint64_t)p.totalGlobalMem;
+    return FH_OK;
+}
+
+extern "C" fh_status fh_malloc(fh_device *dev, size_t bytes, void **out_dev) {
+    FH_REQUIRE(dev && out_dev, "NULL argument");
+    *out_dev = nullptr;
+    if (bytes == 0) bytes = 16;
+    FH_HIP(hipSetDevice(dev->ordinal));
+    FH_HIP(hipMalloc(out_dev, bytes));
+    return FH_OK;
+}
+
+extern "C" fh_status fh_free(fh_device *dev, void *ptr_dev) {
+    FH_REQUIRE(dev, "dev is NULL");
+    if (!ptr_dev) return FH_OK;
+    FH_HIP(hipStreamSynchronize(dev->stream));
+    FH_HIP(hipFree(ptr_dev));
+    return FH_OK;
+}
+
+extern "C" fh_status fh_memset(fh_device *dev, void *ptr_dev, int32_t byte, size_t bytes) {
+    FH_REQUIRE(dev && ptr_dev, "NULL argument");
+    FH_HIP(hipMemsetAsync(ptr_dev, byte, bytes, dev->stream));
+    return FH_OK;
+}
+
+extern "C" fh_status fh_upload(fh_device *dev, void *dst_dev, const void *src_host, size_t bytes) {
+    FH_REQUIRE(dev && dst_dev && (src_host || bytes == 0), "NULL argument");
+    if (!bytes) return FH_OK;
+    FH_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, dev->stream));
+    FH_HIP(hipStreamSynchronize(dev->stream));
+    return FH_OK;
+}
+
+extern "C" fh_status fh_download(fh_device *dev, void *dst_host, const void *src_dev, size_t bytes) {
+    FH_REQUIRE(dev && src_dev && (dst_host || bytes == 0), "NULL argument");
+    if (!bytes) return FH_OK;
+    FH_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, dev->stream));
+    FH_HIP(hipStreamSynchronize(dev->stream));
+    return FH_OK;
+}
+
+extern "C" fh_status fh_copy(fh_device *dev, void *dst_dev, const void *src_dev, size_t bytes) {
+    FH_REQUIRE(dev && dst_dev && src_dev, "NULL argument");
+    if (!bytes) return FH_OK;
+    FH_HIP(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, dev->stream));
+    return FH_OK;
+}
+
+extern "C" fh_status fh_timer_start(fh_device *dev) {
+    FH_REQUIRE(dev, "dev is NULL");
+    FH_HIP(hipEventRecord(dev->ev_start, dev->stream));
+    return FH_OK;
+}
+
+extern "C" fh_status fh_timer_stop(fh_device *dev, float *elapsed_ms) {
+    FH_REQUIRE(dev && elapsed_ms, "NULL argument");
+    FH_HIP(hipEventRecord(dev->ev_stop, dev->stream));
+    FH_HIP(hipEventSynchronize(dev->ev_stop));
+    FH_HIP(hipEventElapsedTime(elapsed_ms, dev->ev_start, dev->ev_stop));
+    return FH_OK;
+}
+
+fh_status fh_dev_scratch(fh_device *dev, void **buf, size_t *cap, size_t need) {
+    if (*cap >= need) return FH_OK;
+    if (*buf) {
+        FH_HIP(hipStreamSynchronize(dev->stream));
+        FH_HIP(hipFree(*buf));
+        *buf = nullptr;
+        *cap = 0;
+    }
+    size_t want = need < (1u << 20) ? (1u << 20) : need;
+    FH_HIP(hipMalloc(buf, want));
+    *cap = want;
+    return FH_OK;
+}
+
+extern "C" fh_status fh_set_option(fh_device *dev, const char *key, int64_t value) {
+    FH_REQUIRE(dev && key, "NULL argument");
+    if (!strcmp(key, "matvec_kernel")) dev->opt_matvec_kernel = value;
+    else if (!strcmp(key, "matvec_splitk")) dev->opt_matvec_splitk = value;
+    else if (!strcmp(key, "matvec_waves")) dev->opt_matvec_waves = value;
+    else if (!strcmp(key, "attn_splits")) dev->opt_attn_splits = value;
+    else if (!strcmp(key, "matmul_kernel")) dev->opt_matmul_kernel = value;
+    else FH_FAIL(FH_ERR_INVALID, "unknown option '%s'", key);
+    return FH_OK;
+}
+
+size_t fh_dtype_size(int dtype) { return dtype == FH_F16 ? 2 : 4; }

@@ -1,0 +1,477 @@
+// Row and pointwise kernels of the decoder: rms_norm (+residual), RoPE pair, SwiGLU, residual adds,
+// head transposes, casts, greedy argmax, KV-cache append.
+#include "fh_internal.h"
+
+#include <cmath>
+#include <vector>
+
+typedef _Float16 fh_half;
+
+__device__ __forceinline__ float block_sum(float v, float *sh) { // blockDim multiple of 64, <= 1024
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) sh[w] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nw; i++) t += sh[i];
+    return t;
+}
+
+// ------------------------------------------------------------------------------ rms_norm
+// fusor-ml/fusor/src/composite/normalization.rs:404-460 (x^2, sum/len, +eps, sqrt, x/rms, *w, +b),
+// residual form :394-397.  One workgroup per row.
+__global__ __launch_bounds__(1024) void k_rms_norm(const float *__restrict__ x, const float *__restrict__ res,
+                                                    const float *__restrict__ w, const float *__restrict__ bias,
+                                                    float eps, int cols, float *__restrict__ y) {
+    __shared__ float sh[16];
+    const int64_t off = (int64_t)blockIdx.x * cols;
+    float acc = 0.f;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+        float t = x[off + c];
+        if (res) t = t + res[off + c];
+        acc = fmaf(t, t, acc);
+    }
+    float total = block_sum(acc, sh);
+    float mean = total / (float)cols;
+    float rms = sqrtf(mean + eps);
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+        float t = x[off + c];
+        if (res) t = t + res[off + c];
+        float o = (t / rms) * w[c];
+        if (bias) o = o + bias[c];
+        y[off + c] = o;
+    }
+}
+
+extern "C" fh_status fh_rms_norm(fh_device *dev, const float *x_dev, const float *residual_dev, const float *w_dev,
+                                 const float *bias_dev, float eps, int32_t rows, int32_t cols, float *y_dev) {
+    FH_REQUIRE(dev && x_dev && w_dev && y_dev, "NULL argument");
+    FH_REQUIRE(rows > 0 && cols > 0, "empty input [%d, %d]", rows, cols);
+    int threads = cols >= 4096 ? 1024 : (cols >= 1024 ? 256 : 64);
+    k_rms_norm<<<dim3((unsigned)rows), dim3(threads), 0, dev->stream>>>(x_dev, residual_dev, w_dev, bias_dev, eps, cols,
+                                                                       y_dev);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+// ------------------------------------------------------------------------------ rope
+// Tables: fusor-ml/fusor/src/composite/rope.rs:241-246 + models/kalosm-llama/src/raw/rope.rs:63-85.
+// Built on the host in f32 with the C library (the reference builds them with Rust's f32
+// powf/sin/cos, i.e. the platform libm).
+extern "C" fh_status fh_rope_tables(fh_device *dev, int32_t head_dim, int32_t ctx, float theta, float *cos_dev,
+                                    float *sin_dev) {
+    FH_REQUIRE(dev && cos_dev && sin_dev, "NULL argument");
+    FH_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && ctx > 0, "bad head_dim %d / ctx %d", head_dim, ctx);
+    int half = head_dim / 2;
+    std::vector<float> inv(half), c((size_t)ctx * half), s((size_t)ctx * half);
+    for (int i = 0; i < head_dim; i += 2) inv[i / 2] = 1.0f / powf(theta, (float)i / (float)head_dim);
+    for (int p = 0; p < ctx; p++)
+        for (int i = 0; i < half; i++) {
+            float a = (float)p * inv[i];
+            c[(size_t)p * half + i] = cosf(a);
+            s[(size_t)p * half + i] = sinf(a);
+        }
+    FH_TRY(fh_upload(dev, cos_dev, c.data(), c.size() * 4));
+    FH_TRY(fh_upload(dev, sin_dev, s.data(), s.size() * 4));
+    return FH_OK;
+}
+
+// rope.rs:77-108 (interleaved) and :46-68 (half split).  Each product is rounded on its own.
+// One thread per rotated pair; q and k share the launch (the reference's fused pair kernel,
+// fusor-ml/core/src/composite/rope_fused.rs:31-75).  pos_dev, when not NULL, overrides start_pos.
+__global__ __launch_bounds__(256) void k_rope_pair(const float *__restrict__ q, int64_t q_sb, int64_t q_sh, int64_t q_st,
+                                                    const float *__restrict__ k, int64_t k_sb, int64_t k_sh, int64_t k_st,
+                                                    int b, int hq, int hk, int s, int d, const float *__restrict__ cs,
+                                                    const float *__restrict__ sn, int table_rows, int start_pos,
+                                                    const int *__restrict__ pos_dev, int interleaved,
+                                                    float *__restrict__ qo, float *__restrict__ ko) {
+    const int half = d >> 1;
+    const int64_t nq = (int64_t)b * hq * s * half, nk = (int64_t)b * hk * s * half;
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= nq + nk) return;
+    const bool isk = idx >= nq;
+    if (isk) idx -= nq;
+    const int h = isk ? hk : hq;
+    int i = (int)(idx % half);
+    int64_t r = idx / half;
+    int t = (int)(r % s);
+    r /= s;
+    int hh = (int)(r % h), bb = (int)(r / h);
+    const float *src = isk ? k + bb * k_sb + hh * k_sh + t * k_st : q + bb * q_sb + hh * q_sh + t * q_st;
+    float *dst = (isk ? ko : qo) + (((int64_t)bb * h + hh) * s + t) * d;
+    int pos = (pos_dev ? *pos_dev : start_pos) + t;
+    if (pos >= table_rows) pos = table_rows - 1; // host validates; never read outside the table
+    const float c = cs[(int64_t)pos * half + i], sv = sn[(int64_t)pos * half + i];
+    if (interleaved) {
+        float x0 = src[2 * i], x1 = src[2 * i + 1];
+        float ac = x0 * c, bs = x1 * sv, as = x0 * sv, bc = x1 * c;
+        dst[2 * i] = ac - bs;
+        dst[2 * i + 1] = as + bc;
+    } else {
+        float x0 = src[i], x1 = src[i + half];
+        float a0 = x0 * c, r0 = (-x1) * sv, a1 = x1 * c, r1 = x0 * sv;
+        dst[i] = a0 + r0;
+        dst[i + half] = a1 + r1;
+    }
+}
+
+extern "C" fh_status fh_rope_pair(fh_device *dev, const float *q_dev, int64_t q_sb, int64_t q_sh, int64_t q_st,
+                                  const float *k_dev, int64_t k_sb, int64_t k_sh, int64_t k_st, int32_t b, int32_t hq,
+                                  int32_t hk, int32_t s, int32_t d, const float *cos_dev, const float *sin_dev,
+                                  int32_t table_rows, int32_t start_pos, int32_t interleaved, float *q_out_dev,
+                                  float *k_out_dev) {
+    FH_REQUIRE(dev && q_dev && k_dev && cos_dev && sin_dev && q_out_dev && k_out_dev, "NULL argument");
+    FH_REQUIRE(b > 0 && hq > 0 && hk > 0 && s > 0 && d > 0 && d % 2 == 0, "bad shape");
+    FH_REQUIRE(start_pos >= 0 && start_pos + s <= table_rows, "positions [%d, %d) exceed the %d table rows", start_pos,
+               start_pos + s, table_rows);
+    int64_t total = ((int64_t)b * hq * s + (int64_t)b * hk * s) * (d / 2);
+    k_rope_pair<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream>>>(
+        q_dev, q_sb, q_sh, q_st, k_dev, k_sb, k_sh, k_st, b, hq, hk, s, d, cos_dev, sin_dev, table_rows, start_pos,
+        nullptr, interleaved, q_out_dev, k_out_dev);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_rope_pair_devpos(fh_device *dev, const float *q, const float *k, int hq, int hk, int d, const float *cos_t,
+                              const float *sin_t, int table_rows, const int *pos_dev, float *q_out, float *k_out) {
+    int64_t total = (int64_t)(hq + hk) * (d / 2);
+    k_rope_pair<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream>>>(
+        q, 0, d, 0, k, 0, d, 0, 1, hq, hk, 1, d, cos_t, sin_t, table_rows, 0, pos_dev, 1, q_out, k_out);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+// ------------------------------------------------------------------------------ pointwise
+// silu(x) = x / (exp(-x) + 1), fusor-ml/fusor/src/composite/activations.rs:47-65
+__global__ void k_swiglu(const float *__restrict__ g, const float *__restrict__ u, float *__restrict__ y, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        float x = g[i];
+        y[i] = (x / (expf(-x) + 1.0f)) * u[i];
+    }
+}
+// gu is [rows, 2f]: gate | up per row; y is [rows, f]
+__global__ void k_swiglu_rows(const float *__restrict__ gu, int rows, int f, float *__restrict__ y) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)rows * f) return;
+    int64_t r = i / f, c = i % f;
+    float x = gu[r * 2 * f + c];
+    y[i] = (x / (expf(-x) + 1.0f)) * gu[r * 2 * f + f + c];
+}
+__global__ void k_add3(const float *__restrict__ a, const float *__restrict__ b, const float *__restrict__ c,
+                       float *__restrict__ y, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        float t = a[i] + b[i];
+        y[i] = c ? t + c[i] : t;
+    }
+}
+__global__ void k_transpose_shd(const float *__restrict__ x, int s, int h, int d, float *__restrict__ y) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t n = (int64_t)s * h * d;
+    if (i >= n) return;
+    int c = (int)(i % d);
+    int64_t r = i / d;
+    int hh = (int)(r % h), t = (int)(r / h); // input index (t, hh, c)
+    y[((int64_t)hh * s + t) * d + c] = x[i];
+}
+__global__ void k_f32_f16(const float *__restrict__ x, fh_half *__restrict__ y, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = (fh_half)x[i];
+}
+__global__ void k_f16_f32(const fh_half *__restrict__ x, float *__restrict__ y, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = (float)x[i];
+}
+__global__ void k_f32_bf16(const float *__restrict__ x, uint16_t *__restrict__ y, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        uint32_t u = __float_as_uint(x[i]);
+        if ((u & 0x7FFFFFFFu) > 0x7F800000u) y[i] = (uint16_t)((u >> 16) | 0x40); // quiet NaN
+        else y[i] = (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);            // round to nearest even
+    }
+}
+
+#define FH_GRID1D(n) dim3((unsigned)(((n) + 255) / 256)), dim3(256), 0, dev->stream
+#define FH_CHECK_COUNT(n) FH_REQUIRE((n) > 0 && ((n) + 255) / 256 < (1ll << 31), "count %lld out of range", (long long)(n))
+
+extern "C" fh_status fh_swiglu(fh_device *dev, const float *gate_dev, const float *up_dev, float *y_dev, int64_t count) {
+    FH_REQUIRE(dev && gate_dev && up_dev && y_dev, "NULL argument");
+    FH_CHECK_COUNT(count);
+    k_swiglu<<<FH_GRID1D(count)>>>(gate_dev, up_dev, y_dev, count);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+fh_status fh_swiglu_rows(fh_device *dev, const float *gu, int rows, int f, float *y) {
+    int64_t count = (int64_t)rows * f;
+    k_swiglu_rows<<<FH_GRID1D(count)>>>(gu, rows, f, y);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+extern "C" fh_status fh_add3(fh_device *dev, const float *a_dev, const float *b_dev, const float *c_dev, float *y_dev,
+                             int64_t count) {
+    FH_REQUIRE(dev && a_dev && b_dev && y_dev, "NULL argument");
+    FH_CHECK_COUNT(count);
+    k_add3<<<FH_GRID1D(count)>>>(a_dev, b_dev, c_dev, y_dev, count);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+extern "C" fh_status fh_transpose_shd(fh_device *dev, const float *x_dev, int32_t s, int32_t h, int32_t d, float *y_dev) {
+    FH_REQUIRE(dev && x_dev && y_dev, "NULL argument");
+    int64_t count = (int64_t)s * h * d;
+    FH_CHECK_COUNT(count);
+    k_transpose_shd<<<FH_GRID1D(count)>>>(x_dev, s, h, d, y_dev);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+extern "C" fh_status fh_cast_f32_f16(fh_device *dev, const float *x_dev, void *y_f16_dev, int64_t count) {
+    FH_REQUIRE(dev && x_dev && y_f16_dev, "NULL argument");
+    FH_CHECK_COUNT(count);
+    k_f32_f16<<<FH_GRID1D(count)>>>(x_dev, (fh_half *)y_f16_dev, count);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+extern "C" fh_status fh_cast_f16_f32(fh_device *dev, const void *x_f16_dev, float *y_dev, int64_t count) {
+    FH_REQUIRE(dev && x_f16_dev && y_dev, "NULL argument");
+    FH_CHECK_COUNT(count);
+    k_f16_f32<<<FH_GRID1D(count)>>>((const fh_half *)x_f16_dev, y_dev, count);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+extern "C" fh_status fh_cast_f32_bf16(fh_device *dev, const float *x_dev, void *y_bf16_dev, int64_t count) {
+    FH_REQUIRE(dev && x_dev && y_bf16_dev, "NULL argument");
+    FH_CHECK_COUNT(count);
+    k_f32_bf16<<<FH_GRID1D(count)>>>(x_dev, (uint16_t *)y_bf16_dev, count);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+// ------------------------------------------------------------------------------ argmax
+// fusor-ml/fusor/src/lib.rs:416-447 with k = 1: largest finite value, ties to the larger index.
+// Single workgroup; the logits row (vocab x 4 B) is small next to the lm-head weights.
+__device__ __forceinline__ void amax_merge(float &v, uint32_t &id, float ov, uint32_t oid) {
+    if (oid == 0xFFFFFFFFu) return;
+    if (id == 0xFFFFFFFFu || ov > v || (ov == v && oid > id)) {
+        v = ov;
+        id = oid;
+    }
+}
+__global__ __launch_bounds__(1024) void k_argmax(const float *__restrict__ x, int64_t n, uint32_t *__restrict__ out) {
+    __shared__ float sv[16];
+    __shared__ uint32_t si[16];
+    float v = 0.f;
+    uint32_t id = 0xFFFFFFFFu;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        float t = x[i];
+        if (isfinite(t)) amax_merge(v, id, t, (uint32_t)i);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        float ov = __shfl_xor(v, o, 64);
+        uint32_t oid = (uint32_t)__shfl_xor((int)id, o, 64);
+        amax_merge(v, id, ov, oid);
+    }
+    int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) {
+        sv[w] = v;
+        si[w] = id;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < (int)(blockDim.x >> 6); i++) amax_merge(v, id, sv[i], si[i]);
+        *out = id;
+    }
+}
+extern "C" fh_status fh_argmax(fh_device *dev, const float *x_dev, int64_t count, uint32_t *id_dev) {
+    FH_REQUIRE(dev && x_dev && id_dev, "NULL argument");
+    FH_REQUIRE(count > 0 && count < 0xFFFFFFFFll, "count %lld out of range", (long long)count);
+    k_argmax<<<dim3(1), dim3(1024), 0, dev->stream>>>(x_dev, count, id_dev);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+// ------------------------------------------------------------------------------ KV cache
+// fusor-ml/fusor/src/cache/tensor_cache.rs:70-114 (in-place slice write into a grown backing buffer),
+// :304-312 (power-of-two growth, minimum 256, capped at max_len).
+static int kv_alloc_len(int required, int max_len) {
+    int min_alloc = 256 < max_len ? 256 : max_len;
+    int p = 1;
+    while (p < required) p <<= 1;
+    if (p < min_alloc) p = min_alloc;
+    if (p > max_len) p = max_len;
+    return p;
+}
+
+extern "C" fh_status fh_kvcache_create(fh_device *dev, int32_t layers, int32_t kv_heads, int32_t head_dim,
+                                       int32_t max_len, int32_t dtype, fh_kvcache **out) {
+    FH_REQUIRE(dev && out, "NULL argument");
+    FH_REQUIRE(layers > 0 && kv_heads > 0 && head_dim > 0 && max_len > 0, "bad cache shape");
+    FH_REQUIRE(dtype == FH_F32 || dtype == FH_F16, "cache dtype must be FH_F32 or FH_F16");
+    fh_kvcache *c = new fh_kvcache();
+    c->dev = dev;
+    c->layers = layers;
+    c->kv_heads = kv_heads;
+    c->head_dim = head_dim;
+    c->max_len = max_len;
+    c->dtype = dtype;
+    hipError_t e = hipMalloc((void **)&c->len_dev, 256);
+    if (e != hipSuccess) {
+        delete c;
+        FH_FAIL(FH_ERR_OOM, "hipMalloc failed: %s", hipGetErrorString(e));
+    }
+    int zero = 0;
+    (void)hipMemcpy(c->len_dev, &zero, 4, hipMemcpyHostToDevice);
+    *out = c;
+    return FH_OK;
+}
+
+extern "C" fh_status fh_kvcache_destroy(fh_kvcache *c) {
+    if (!c) return FH_OK;
+    (void)hipStreamSynchronize(c->dev->stream);
+    if (c->k) (void)hipFree(c->k);
+    if (c->v) (void)hipFree(c->v);
+    if (c->len_dev) (void)hipFree(c->len_dev);
+    delete c;
+    return FH_OK;
+}
+
+__global__ void k_set_int(int *p, int v) { *p = v; }
+__global__ void k_inc_int(int *p) { *p = *p + 1; }
+
+extern "C" fh_status fh_kvcache_reset(fh_kvcache *c) {
+    FH_REQUIRE(c, "NULL argument");
+    c->len = 0; // the reference drops its buffers (tensor_cache.rs:60-65); capacity is kept here
+    k_set_int<<<1, 1, 0, c->dev->stream>>>(c->len_dev, 0);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+// copy [layers][heads][old_cap][d] -> [layers][heads][new_cap][d] for the first `len` positions
+__global__ void k_kv_regrow(const uint32_t *__restrict__ src, uint32_t *__restrict__ dst, int64_t rows, int len,
+                            int old_cap, int new_cap, int words_per_pos) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t per_row = (int64_t)len * words_per_pos;
+    if (i >= rows * per_row) return;
+    int64_t r = i / per_row, o = i % per_row;
+    dst[r * new_cap * words_per_pos + o] = src[r * old_cap * words_per_pos + o];
+}
+
+fh_status fh_kvcache_reserve(fh_kvcache *c, int required) {
+    FH_REQUIRE(required <= c->max_len, "KV cache overflow: %d positions needed, max_len %d", required, c->max_len);
+    if (required <= c->capacity) return FH_OK;
+    int cap = kv_alloc_len(required, c->max_len);
+    size_t es = fh_dtype_size(c->dtype);
+    size_t bytes = (size_t)c->layers * c->kv_heads * cap * c->head_dim * es;
+    void *nk = nullptr, *nv = nullptr;
+    FH_HIP(hipMalloc(&nk, bytes));
+    hipError_t e = hipMalloc(&nv, bytes);
+    if (e != hipSuccess) {
+        (void)hipFree(nk);
+        FH_FAIL(FH_ERR_OOM, "hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+    }
+    hipStream_t s = c->dev->stream;
+    if (c->len > 0 && c->k) {
+        int wpp = (int)(c->head_dim * es / 4);
+        int64_t rows = (int64_t)c->layers * c->kv_heads, total = rows * c->len * wpp;
+        dim3 grid((unsigned)((total + 255) / 256));
+        k_kv_regrow<<<grid, 256, 0, s>>>((const uint32_t *)c->k, (uint32_t *)nk, rows, c->len, c->capacity, cap, wpp);
+        k_kv_regrow<<<grid, 256, 0, s>>>((const uint32_t *)c->v, (uint32_t *)nv, rows, c->len, c->capacity, cap, wpp);
+    }
+    FH_HIP(hipStreamSynchronize(s));
+    if (c->k) (void)hipFree(c->k);
+    if (c->v) (void)hipFree(c->v);
+    c->k = nk;
+    c->v = nv;
+    c->capacity = cap;
+    return FH_OK;
+}
+
+// k_src / v_src: [heads, s, d] f32 views, each with its own head and position stride (elements).
+// The write position comes from pos_dev when given (graph replay), else from p0.
+template <typename TO>
+__global__ void k_kv_append(const float *__restrict__ ks, int64_t k_sh, int64_t k_st, const float *__restrict__ vs,
+                            int64_t v_sh, int64_t v_st, int heads, int s, int d, TO *__restrict__ kc,
+                            TO *__restrict__ vc, int cap, int p0, const int *__restrict__ pos_dev) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t n = (int64_t)heads * s * d;
+    if (i >= n) return;
+    int c = (int)(i % d);
+    int64_t r = i / d;
+    int t = (int)(r % s), h = (int)(r / s);
+    int pos = (pos_dev ? *pos_dev : p0) + t;
+    if (pos >= cap) return; // the host guarantees capacity; never write outside the plane
+    int64_t dofs = ((int64_t)h * cap + pos) * d + c;
+    kc[dofs] = (TO)ks[h * k_sh + t * k_st + c];
+    vc[dofs] = (TO)vs[h * v_sh + t * v_st + c];
+}
+
+static fh_status kv_append_launch(fh_kvcache *c, int layer, const float *k, int64_t k_sh, int64_t k_st, const float *v,
+                                  int64_t v_sh, int64_t v_st, int s, int p0, const int *pos_dev) {
+    size_t plane = (size_t)c->kv_heads * c->capacity * c->head_dim;
+    int64_t n = (int64_t)c->kv_heads * s * c->head_dim;
+    dim3 grid((unsigned)((n + 255) / 256));
+    hipStream_t stream = c->dev->stream;
+    if (c->dtype == FH_F32)
+        k_kv_append<float><<<grid, 256, 0, stream>>>(k, k_sh, k_st, v, v_sh, v_st, c->kv_heads, s, c->head_dim,
+                                                     (float *)c->k + layer * plane, (float *)c->v + layer * plane,
+                                                     c->capacity, p0, pos_dev);
+    else
+        k_kv_append<fh_half><<<grid, 256, 0, stream>>>(k, k_sh, k_st, v, v_sh, v_st, c->kv_heads, s, c->head_dim,
+                                                       (fh_half *)c->k + layer * plane, (fh_half *)c->v + layer * plane,
+                                                       c->capacity, p0, pos_dev);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+// Append with separate K / V strides at an explicit position; capacity must already be reserved.
+fh_status fh_kvcache_append_kv(fh_kvcache *c, int layer, const float *k, int64_t k_sh, int64_t k_st, const float *v,
+                               int64_t v_sh, int64_t v_st, int s, int pos) {
+    FH_REQUIRE(pos + s <= c->capacity, "KV append [%d, %d) beyond the reserved capacity %d", pos, pos + s, c->capacity);
+    return kv_append_launch(c, layer, k, k_sh, k_st, v, v_sh, v_st, s, pos, nullptr);
+}
+
+fh_status fh_kvcache_set_len_dev(fh_kvcache *c, int len) {
+    k_set_int<<<1, 1, 0, c->dev->stream>>>(c->len_dev, len);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+extern "C" fh_status fh_kvcache_append(fh_kvcache *c, int32_t layer, const float *k_dev, const float *v_dev, int64_t sh,
+                                       int64_t st, int32_t s) {
+    FH_REQUIRE(c && k_dev && v_dev, "NULL argument");
+    FH_REQUIRE(layer >= 0 && layer < c->layers && s > 0, "bad layer %d / s %d", layer, s);
+    FH_TRY(fh_kvcache_reserve(c, c->len + s));
+    FH_TRY(kv_append_launch(c, layer, k_dev, sh, st, v_dev, sh, st, s, c->len, nullptr));
+    if (layer == c->layers - 1) {
+        c->len += s;
+        k_set_int<<<1, 1, 0, c->dev->stream>>>(c->len_dev, c->len);
+        FH_HIP(hipGetLastError());
+    }
+    return FH_OK;
+}
+
+// Graph-replayed decode step: position read from len_dev; the host mirrors the length afterwards.
+fh_status fh_kvcache_append_devpos(fh_kvcache *c, int layer, const float *k, const float *v, int64_t sh) {
+    return kv_append_launch(c, layer, k, sh, 0, v, sh, 0, 1, 0, c->len_dev);
+}
+
+// End of a graph-replayed decode step: advance the device-side length.
+fh_status fh_kvcache_advance_dev(fh_kvcache *c) {
+    k_inc_int<<<1, 1, 0, c->dev->stream>>>(c->len_dev);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+extern "C" fh_status fh_kvcache_view(const fh_kvcache *c, int32_t layer, int32_t *len, int32_t *capacity,
+                                     const void **k_dev, const void **v_dev) {
+    FH_REQUIRE(c, "NULL argument");
+    FH_REQUIRE(layer >= 0 && layer < c->layers, "bad layer %d", layer);
+    size_t plane = (size_t)c->kv_heads * c->capacity * c->head_dim * fh_dtype_size(c->dtype);
+    if (len) *len = c->len;
+    if (capacity) *capacity = c->capacity;
+    if (k_dev) *k_dev = c->k ? (const uint8_t *)c->k + layer * plane : nullptr;
+    if (v_dev) *v_dev = c->v ? (const uint8_t *)c->v + layer * plane : nullptr;
+    return FH_OK;
+}

@@ -1,0 +1,158 @@
+// Internal declarations shared by the translation units of libfusor_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include <string>
+#include <vector>
+
+#include "../../include/fusor_hip.h"
+
+// ---------------------------------------------------------------- errors
+void fh_set_error(const char *fmt, ...);
+#define FH_FAIL(code, ...)            \
+    do {                              \
+        fh_set_error(__VA_ARGS__);    \
+        return (code);                \
+    } while (0)
+#define FH_REQUIRE(cond, ...)                         \
+    do {                                              \
+        if (!(cond)) FH_FAIL(FH_ERR_INVALID, __VA_ARGS__); \
+    } while (0)
+#define FH_HIP(call)                                                                          \
+    do {                                                                                      \
+        hipError_t e_ = (call);                                                               \
+        if (e_ != hipSuccess) {                                                               \
+            fh_set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), __FILE__, __LINE__); \
+            return e_ == hipErrorOutOfMemory ? FH_ERR_OOM : FH_ERR_HIP;                       \
+        }                                                                                     \
+    } while (0)
+#define FH_TRY(call)                  \
+    do {                              \
+        fh_status s_ = (call);        \
+        if (s_ != FH_OK) return s_;   \
+    } while (0)
+
+// ---------------------------------------------------------------- device
+struct fh_device {
+    int ordinal = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    int compute_units = 0;
+    // activation staging for the MFMA decode kernels (grown on demand)
+    void *act_buf = nullptr;
+    size_t act_cap = 0;
+    // split-K partial sums
+    float *part_buf = nullptr;
+    size_t part_cap = 0;
+    // options (fh_set_option)
+    int64_t opt_matvec_kernel = 0;   // 0 auto, 1 generic VALU, 2 MFMA
+    int64_t opt_matvec_splitk = 0;   // 0 auto, else forced split count
+    int64_t opt_matvec_waves = 0;    // 0 auto
+    int64_t opt_attn_splits = 0;     // 0 auto
+    int64_t opt_matmul_kernel = 0;   // 0 auto, 1 generic
+};
+
+fh_status fh_dev_scratch(fh_device *dev, void **buf, size_t *cap, size_t need);
+
+// ---------------------------------------------------------------- weights
+// Device layouts.  All of them hold exactly the bits of the GGUF block stream,
+// re-ordered so that a 64-lane wavefront reads them with 16-byte loads.
+//
+// Rows are grouped in tiles of 16 (the N extent of one MFMA); a matrix whose row
+// count is not a multiple of 16 is padded with all-zero blocks.  kb = k / block
+// elements.  For tile t and record r the record lives at
+//   base + (t * records_per_tile + r) * record_bytes.
+//
+// FH_Q4_K (record = one 256-block of 16 rows, 2304 B)
+//   [0,256)      header: row j at 16*j: d f16, dmin f16, 12 packed scale bytes (as in GGUF)
+//   [256,2304)   quants: for p in {0,1}, lane l = g*16 + j (g in 0..3):
+//                16 B at 256 + p*1024 + l*16 = qs_j[64p + 8g .. +8] ++ qs_j[64p + 32 + 8g .. +8]
+// FH_Q6_K (record = one 256-block of 16 rows, 3360 B)
+//   [0,2048)     ql: for p in {0,1}, lane l = g*16 + j: 16 B at p*1024 + l*16 = ql_j[64p + 16g .. +16]
+//   [2048,3072)  qh: for p in {0,1}, lane l: 8 B at 2048 + p*512 + l*8 = qh_j[32p + 8g .. +8]
+//   [3072,3328)  scales: row j at 3072 + 16*j (16 x i8)
+//   [3328,3360)  d: row j at 3328 + 2*j (f16)
+// FH_Q8_0 (record = two 32-blocks of 16 rows, 1088 B; kb padded to even with zero blocks)
+//   [0,1024)     quants: lane l = g*16 + j: 16 B at l*16 = q_j[blk 2r][8g .. +8] ++ q_j[blk 2r+1][8g .. +8]
+//   [1024,1088)  d: row j at 1024 + 4*j: d[blk 2r], d[blk 2r+1] (f16 x2)
+// FH_Q4_0 (record = four 32-blocks of 16 rows, 1152 B; kb padded to a multiple of 4)
+//   [0,1024)     quants: lane l = g*16 + j: 16 B at l*16 = for u in 0..3: qs_j[blk 4r+u][4g .. +4]
+//   [1024,1152)  d: row j at 1024 + 8*j: d[blk 4r .. 4r+3] (f16 x4)
+struct fh_qmatrix {
+    fh_device *dev = nullptr;
+    uint32_t type = 0;
+    int64_t n = 0, k = 0;
+    int64_t n_pad = 0;       // rows padded to a multiple of 16
+    int64_t kb = 0;          // blocks per row (unpadded)
+    int64_t recs = 0;        // records per tile
+    int rec_bytes = 0;
+    uint8_t *data = nullptr; // device
+    size_t bytes = 0;
+};
+
+static inline int fh_block_elems(uint32_t t) {
+    switch (t) {
+    case FH_Q4_0: case FH_Q8_0: return 32;
+    case FH_Q4_K: case FH_Q6_K: return 256;
+    default: return 0;
+    }
+}
+static inline int fh_block_bytes(uint32_t t) {
+    switch (t) {
+    case FH_Q4_0: return 18;
+    case FH_Q8_0: return 34;
+    case FH_Q4_K: return 144;
+    case FH_Q6_K: return 210;
+    default: return 0;
+    }
+}
+static inline int fh_rec_blocks(uint32_t t) {   // blocks per record (per row)
+    switch (t) {
+    case FH_Q4_0: return 4;
+    case FH_Q8_0: return 2;
+    default: return 1;
+    }
+}
+static inline int fh_rec_bytes(uint32_t t) { return 16 * fh_rec_blocks(t) * fh_block_bytes(t); }
+
+// A plain-data view passed to kernels by value.
+struct QView {
+    const uint8_t *data;
+    int64_t n, k, kb, recs;
+    int rec_bytes;
+};
+static inline QView fh_view(const fh_qmatrix *q) {
+    QView v{q->data, q->n, q->k, q->kb, q->recs, q->rec_bytes};
+    return v;
+}
+
+// ---------------------------------------------------------------- launches implemented per file
+fh_status fh_launch_qmatvec(const fh_qmatrix *q, const float *x, int m, float *y, int epilogue,
+                            const float *a, const float *b);
+fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y);
+enum { FH_EPI_NONE = 0, FH_EPI_ADD2 = 1, FH_EPI_SWIGLU = 2 };
+
+struct fh_kvcache {
+    fh_device *dev = nullptr;
+    int layers = 0, kv_heads = 0, head_dim = 0, max_len = 0, dtype = FH_F32;
+    int len = 0, capacity = 0;
+    void *k = nullptr, *v = nullptr; // [layers][kv_heads][capacity][head_dim]
+    int *len_dev = nullptr;          // device copy of len (for graph-replayed decode steps)
+};
+size_t fh_dtype_size(int dtype);
+fh_status fh_kvcache_reserve(fh_kvcache *c, int required);
+// append reading the write position from c->len_dev (graph friendly), s == 1
+fh_status fh_kvcache_append_devpos(fh_kvcache *c, int layer, const float *k, const float *v, int64_t sh);
+fh_status fh_kvcache_advance_dev(fh_kvcache *c);
+fh_status fh_kvcache_append_kv(fh_kvcache *c, int layer, const float *k, int64_t k_sh, int64_t k_st, const float *v,
+                               int64_t v_sh, int64_t v_st, int s, int pos);
+fh_status fh_kvcache_set_len_dev(fh_kvcache *c, int len);
+fh_status fh_swiglu_rows(fh_device *dev, const float *gu, int rows, int f, float *y);
+// decode attention reading the KV length from a device int (graph friendly)
+fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *q, const void *k,
+                                     const void *v, int64_t kv_sh, int64_t kv_st, int hq, int hkv,
+                                     int d, float scale, const int *len_dev, int max_len, float *out);
+fh_status fh_rope_pair_devpos(fh_device *dev, const float *q, const float *k, int hq, int hk, int d,
+                              const float *cos_t, const float *sin_t, int table_rows,
+                              const int *pos_dev, float *q_out, float *k_out);

@@ -1,0 +1,390 @@
+// Llama-architecture decoder built from the C-ABI operators of this library.
+// Reference: models/kalosm-llama/src/raw/mod.rs:851-865, :925-1049 (Model::forward),
+// raw/attention_layer.rs:130-237 (feed-forward), :281-426 / :514-694 (attention),
+// raw/rope.rs:87-112 (interleaved RoPE for the llama architecture), model/inference.rs:11-396
+// (decode loop, here greedy).
+#include "fh_internal.h"
+
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <string>
+
+struct fh_llama_layer {
+    fh_qmatrix *wq = nullptr, *wk = nullptr, *wv = nullptr, *wo = nullptr;
+    fh_qmatrix *gate = nullptr, *up = nullptr, *down = nullptr;
+    fh_qmatrix *qkv = nullptr, *gate_up = nullptr;
+    float *attn_norm = nullptr, *ffn_norm = nullptr;
+};
+
+struct fh_llama {
+    fh_device *dev = nullptr;
+    fh_llama_config c{};
+    std::vector<fh_llama_layer> layers;
+    fh_qmatrix *embd = nullptr, *output = nullptr;
+    bool output_is_embd = false;
+    float *out_norm = nullptr;
+    float *cos_t = nullptr, *sin_t = nullptr;
+    fh_kvcache *cache = nullptr;
+    bool finalized = false;
+    int pos = 0;
+    // step buffers (sized for `cap_s` tokens)
+    int cap_s = 0;
+    uint32_t *ids = nullptr;
+    float *x = nullptr, *xn = nullptr, *qkv = nullptr, *qrot = nullptr, *krot = nullptr, *att = nullptr, *att_t = nullptr,
+          *attn_out = nullptr, *gu = nullptr, *act = nullptr, *ff = nullptr, *logits = nullptr;
+    // greedy decode state
+    uint32_t *tok_dev = nullptr, *out_tok_dev = nullptr;
+    int *step_dev = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    hipGraph_t graph = nullptr;
+    int captured_capacity = -1;
+};
+
+static void free_dev(void *p) {
+    if (p) (void)hipFree(p);
+}
+
+extern "C" fh_status fh_llama_create(fh_device *dev, const fh_llama_config *cfg, fh_llama **out) {
+    FH_REQUIRE(dev && cfg && out, "NULL argument");
+    *out = nullptr;
+    FH_REQUIRE(cfg->n_layers > 0 && cfg->d_model > 0 && cfg->n_heads > 0 && cfg->n_kv_heads > 0 && cfg->head_dim > 0 &&
+                   cfg->ffn > 0 && cfg->vocab > 0 && cfg->ctx > 0,
+               "bad decoder configuration");
+    FH_REQUIRE(cfg->n_heads % cfg->n_kv_heads == 0, "n_heads %d not divisible by n_kv_heads %d", cfg->n_heads, cfg->n_kv_heads);
+    FH_REQUIRE(cfg->head_dim == 64 || cfg->head_dim == 128, "head_dim %d unsupported (64 or 128)", cfg->head_dim);
+    fh_llama *m = new fh_llama();
+    m->dev = dev;
+    m->c = *cfg;
+    m->layers.resize(cfg->n_layers);
+    *out = m;
+    return FH_OK;
+}
+
+static void free_steps(fh_llama *m) {
+    free_dev(m->ids); free_dev(m->x); free_dev(m->xn); free_dev(m->qkv); free_dev(m->qrot); free_dev(m->krot);
+    free_dev(m->att); free_dev(m->att_t); free_dev(m->attn_out); free_dev(m->gu); free_dev(m->act); free_dev(m->ff);
+    m->ids = nullptr;
+    m->x = m->xn = m->qkv = m->qrot = m->krot = m->att = m->att_t = m->attn_out = m->gu = m->act = m->ff = nullptr;
+    m->cap_s = 0;
+    m->captured_capacity = -1; // a captured decode step holds these pointers
+}
+
+extern "C" fh_status fh_llama_destroy(fh_llama *m) {
+    if (!m) return FH_OK;
+    (void)hipStreamSynchronize(m->dev->stream);
+    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
+    if (m->graph) (void)hipGraphDestroy(m->graph);
+    for (auto &l : m->layers) {
+        fh_qmatrix_free(l.wq); fh_qmatrix_free(l.wk); fh_qmatrix_free(l.wv); fh_qmatrix_free(l.wo);
+        fh_qmatrix_free(l.gate); fh_qmatrix_free(l.up); fh_qmatrix_free(l.down);
+        fh_qmatrix_free(l.qkv); fh_qmatrix_free(l.gate_up);
+        free_dev(l.attn_norm); free_dev(l.ffn_norm);
+    }
+    fh_qmatrix_free(m->embd);
+    if (!m->output_is_embd) fh_qmatrix_free(m->output);
+    free_dev(m->out_norm); free_dev(m->cos_t); free_dev(m->sin_t);
+    free_dev(m->logits); free_dev(m->tok_dev); free_dev(m->out_tok_dev); free_dev(m->step_dev);
+    free_steps(m);
+    fh_kvcache_destroy(m->cache);
+    delete m;
+    return FH_OK;
+}
+
+static fh_status load_f32(fh_llama *m, float **dst, int64_t want, int64_t n, int64_t k, const void *bytes, size_t len,
+                          const char *name) {
+    int64_t count = n * (k > 0 ? k : 1);
+    FH_REQUIRE(count == want && len == (size_t)want * 4, "%s: expected %lld f32 values, got [%lld, %lld] / %zu bytes", name,
+               (long long)want, (long long)n, (long long)k, len);
+    free_dev(*dst);
+    *dst = nullptr;
+    FH_TRY(fh_malloc(m->dev, len, (void **)dst));
+    return fh_upload(m->dev, *dst, bytes, len);
+}
+
+extern "C" fh_status fh_llama_load_tensor(fh_llama *m, const char *name, uint32_t ggml_type, int64_t n, int64_t k,
+                                          const void *bytes, size_t len) {
+    FH_REQUIRE(m && name && bytes, "NULL argument");
+    FH_REQUIRE(!m->finalized, "decoder already finalized");
+    const fh_llama_config &c = m->c;
+    const int64_t D = c.d_model, QD = (int64_t)c.n_heads * c.head_dim, KD = (int64_t)c.n_kv_heads * c.head_dim;
+    auto loadq = [&](fh_qmatrix **dst, int64_t wn, int64_t wk) -> fh_status {
+        FH_REQUIRE(n == wn && k == wk, "%s: expected [%lld, %lld], got [%lld, %lld]", name, (long long)wn, (long long)wk,
+                   (long long)n, (long long)k);
+        fh_qmatrix_free(*dst);
+        *dst = nullptr;
+        return fh_qmatrix_from_gguf_bytes(m->dev, ggml_type, n, k, bytes, len, dst);
+    };
+    if (!strcmp(name, "token_embd.weight")) return loadq(&m->embd, c.vocab, D);
+    if (!strcmp(name, "output.weight")) return loadq(&m->output, c.vocab, D);
+    if (!strcmp(name, "output_norm.weight")) return load_f32(m, &m->out_norm, D, n, k, bytes, len, name);
+    int li = -1;
+    char field[64] = "";
+    if (sscanf(name, "blk.%d.%63s", &li, field) == 2 && li >= 0 && li < c.n_layers) {
+        fh_llama_layer &l = m->layers[li];
+        if (!strcmp(field, "attn_q.weight")) return loadq(&l.wq, QD, D);
+        if (!strcmp(field, "attn_k.weight")) return loadq(&l.wk, KD, D);
+        if (!strcmp(field, "attn_v.weight")) return loadq(&l.wv, KD, D);
+        if (!strcmp(field, "attn_output.weight")) return loadq(&l.wo, D, QD);
+        if (!strcmp(field, "ffn_gate.weight")) return loadq(&l.gate, c.ffn, D);
+        if (!strcmp(field, "ffn_up.weight")) return loadq(&l.up, c.ffn, D);
+        if (!strcmp(field, "ffn_down.weight")) return loadq(&l.down, D, c.ffn);
+        if (!strcmp(field, "attn_norm.weight")) return load_f32(m, &l.attn_norm, D, n, k, bytes, len, name);
+        if (!strcmp(field, "ffn_norm.weight")) return load_f32(m, &l.ffn_norm, D, n, k, bytes, len, name);
+    }
+    FH_FAIL(FH_ERR_INVALID, "unknown tensor name '%s'", name);
+}
+
+static fh_status ensure_steps(fh_llama *m, int s) {
+    if (s <= m->cap_s) return FH_OK;
+    (void)hipStreamSynchronize(m->dev->stream);
+    free_steps(m);
+    const fh_llama_config &c = m->c;
+    const size_t D = c.d_model, QD = (size_t)c.n_heads * c.head_dim, KD = (size_t)c.n_kv_heads * c.head_dim, F = c.ffn;
+    size_t S = (size_t)s;
+    FH_TRY(fh_malloc(m->dev, S * 4, (void **)&m->ids));
+    FH_TRY(fh_malloc(m->dev, S * D * 4, (void **)&m->x));
+    FH_TRY(fh_malloc(m->dev, S * D * 4, (void **)&m->xn));
+    FH_TRY(fh_malloc(m->dev, S * (QD + 2 * KD) * 4, (void **)&m->qkv));
+    FH_TRY(fh_malloc(m->dev, S * QD * 4, (void **)&m->qrot));
+    FH_TRY(fh_malloc(m->dev, S * KD * 4, (void **)&m->krot));
+    FH_TRY(fh_malloc(m->dev, S * QD * 4, (void **)&m->att));
+    FH_TRY(fh_malloc(m->dev, S * QD * 4, (void **)&m->att_t));
+    FH_TRY(fh_malloc(m->dev, S * D * 4, (void **)&m->attn_out));
+    FH_TRY(fh_malloc(m->dev, S * 2 * F * 4, (void **)&m->gu));
+    FH_TRY(fh_malloc(m->dev, S * F * 4, (void **)&m->act));
+    FH_TRY(fh_malloc(m->dev, S * D * 4, (void **)&m->ff));
+    m->cap_s = s;
+    return FH_OK;
+}
+
+extern "C" fh_status fh_llama_finalize(fh_llama *m) {
+    FH_REQUIRE(m, "NULL argument");
+    FH_REQUIRE(!m->finalized, "decoder already finalized");
+    const fh_llama_config &c = m->c;
+    FH_REQUIRE(m->embd && m->out_norm, "token_embd.weight / output_norm.weight missing");
+    if (!m->output) { // falls back to the embedding table, raw/mod.rs:480-486
+        m->output = m->embd;
+        m->output_is_embd = true;
+    }
+    for (int i = 0; i < c.n_layers; i++) {
+        fh_llama_layer &l = m->layers[i];
+        FH_REQUIRE(l.wq && l.wk && l.wv && l.wo && l.gate && l.up && l.down && l.attn_norm && l.ffn_norm,
+                   "layer %d is missing tensors", i);
+        if (c.fuse_qkv) {
+            const fh_qmatrix *parts[3] = {l.wq, l.wk, l.wv};
+            fh_status st = fh_qmatrix_concat_rows(m->dev, parts, 3, &l.qkv);
+            if (st == FH_OK) {
+                FH_HIP(hipStreamSynchronize(m->dev->stream));
+                fh_qmatrix_free(l.wq); fh_qmatrix_free(l.wk); fh_qmatrix_free(l.wv);
+                l.wq = l.wk = l.wv = nullptr;
+            } else if (st != FH_ERR_UNSUPPORTED) return st;
+        }
+        if (c.fuse_gate_up) {
+            const fh_qmatrix *parts[2] = {l.gate, l.up};
+            fh_status st = fh_qmatrix_concat_rows(m->dev, parts, 2, &l.gate_up);
+            if (st == FH_OK) {
+                FH_HIP(hipStreamSynchronize(m->dev->stream));
+                fh_qmatrix_free(l.gate); fh_qmatrix_free(l.up);
+                l.gate = l.up = nullptr;
+            } else if (st != FH_ERR_UNSUPPORTED) return st;
+        }
+    }
+    size_t tbl = (size_t)c.ctx * (c.head_dim / 2) * 4;
+    FH_TRY(fh_malloc(m->dev, tbl, (void **)&m->cos_t));
+    FH_TRY(fh_malloc(m->dev, tbl, (void **)&m->sin_t));
+    FH_TRY(fh_rope_tables(m->dev, c.head_dim, c.ctx, c.theta, m->cos_t, m->sin_t));
+    FH_TRY(fh_kvcache_create(m->dev, c.n_layers, c.n_kv_heads, c.head_dim, c.ctx, c.kv_dtype, &m->cache));
+    FH_TRY(fh_malloc(m->dev, (size_t)c.vocab * 4, (void **)&m->logits));
+    FH_TRY(fh_malloc(m->dev, 256, (void **)&m->tok_dev));
+    FH_TRY(fh_malloc(m->dev, (size_t)c.ctx * 4 + 256, (void **)&m->out_tok_dev));
+    FH_TRY(fh_malloc(m->dev, 256, (void **)&m->step_dev));
+    FH_TRY(ensure_steps(m, 1));
+    m->finalized = true;
+    return FH_OK;
+}
+
+extern "C" fh_status fh_llama_reset(fh_llama *m) {
+    FH_REQUIRE(m && m->finalized, "decoder not finalized");
+    m->pos = 0;
+    return fh_kvcache_reset(m->cache);
+}
+
+extern "C" fh_status fh_llama_weight_bytes(const fh_llama *m, uint64_t *bytes) {
+    FH_REQUIRE(m && bytes, "NULL argument");
+    uint64_t t = 0;
+    auto add = [&](const fh_qmatrix *q) {
+        if (q) t += (uint64_t)q->n * q->kb * fh_block_bytes(q->type);
+    };
+    for (auto &l : m->layers) {
+        add(l.wq); add(l.wk); add(l.wv); add(l.wo); add(l.gate); add(l.up); add(l.down); add(l.qkv); add(l.gate_up);
+    }
+    add(m->output); // the lm-head; the embedding table contributes one row per token
+    *bytes = t;
+    return FH_OK;
+}
+
+// One decoder pass over `s` tokens whose ids are already in m->ids.  dev_pos: read the position
+// from the cache's device-side length (graph replay, s == 1) instead of m->pos.
+static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
+    const fh_llama_config &c = m->c;
+    fh_device *dev = m->dev;
+    const int D = c.d_model, H = c.n_heads, HK = c.n_kv_heads, hd = c.head_dim, F = c.ffn;
+    const int QD = H * hd, KD = HK * hd;
+    const int pos = m->pos;
+    const float scale = (float)(1.0 / sqrt((double)hd)); // attention_layer.rs:674
+    FH_TRY(fh_embed_rows(m->embd, m->ids, nullptr, s, m->x));
+    for (int li = 0; li < c.n_layers; li++) {
+        fh_llama_layer &l = m->layers[li];
+        FH_TRY(fh_rms_norm(dev, m->x, nullptr, l.attn_norm, nullptr, c.eps, s, D, m->xn));
+        const float *qp, *kp, *vp;
+        int64_t row;
+        if (l.qkv) {
+            FH_TRY(fh_qmatmul(l.qkv, m->xn, s, m->qkv));
+            row = QD + 2 * KD;
+            qp = m->qkv;
+            kp = m->qkv + QD;
+            vp = m->qkv + QD + KD;
+        } else {
+            float *qb = m->qkv, *kb2 = m->qkv + (size_t)s * QD, *vb = kb2 + (size_t)s * KD;
+            FH_TRY(fh_qmatmul(l.wq, m->xn, s, qb));
+            FH_TRY(fh_qmatmul(l.wk, m->xn, s, kb2));
+            FH_TRY(fh_qmatmul(l.wv, m->xn, s, vb));
+            row = 0; // per-tensor strides below
+            qp = qb; kp = kb2; vp = vb;
+        }
+        const int64_t q_st = row ? row : QD, k_st = row ? row : KD;
+        if (dev_pos) {
+            FH_TRY(fh_rope_pair_devpos(dev, qp, kp, H, HK, hd, m->cos_t, m->sin_t, c.ctx, m->cache->len_dev, m->qrot, m->krot));
+            FH_TRY(fh_kvcache_append_devpos(m->cache, li, m->krot, vp, hd));
+            size_t plane = (size_t)HK * m->cache->capacity * hd * fh_dtype_size(c.kv_dtype);
+            const uint8_t *kc = (const uint8_t *)m->cache->k + li * plane, *vc = (const uint8_t *)m->cache->v + li * plane;
+            FH_TRY(fh_attention_decode_devlen(dev, c.kv_dtype, m->qrot, kc, vc, (int64_t)m->cache->capacity * hd, hd, H, HK,
+                                              hd, scale, m->cache->len_dev, m->cache->capacity, m->att));
+        } else {
+            FH_TRY(fh_rope_pair(dev, qp, 0, hd, q_st, kp, 0, hd, k_st, 1, H, HK, s, hd, m->cos_t, m->sin_t, c.ctx, pos, 1,
+                                m->qrot, m->krot));
+            FH_TRY(fh_kvcache_reserve(m->cache, pos + s));
+            // K (rotated) is [HK, s, hd] contiguous; V is a view of the projection output
+            FH_TRY(fh_kvcache_append_kv(m->cache, li, m->krot, (int64_t)s * hd, hd, vp, hd, k_st, s, pos));
+            size_t plane = (size_t)HK * m->cache->capacity * hd * fh_dtype_size(c.kv_dtype);
+            const uint8_t *kc = (const uint8_t *)m->cache->k + li * plane, *vc = (const uint8_t *)m->cache->v + li * plane;
+            FH_TRY(fh_flash_attention_ex(dev, FH_F32, c.kv_dtype, m->qrot, 0, (int64_t)s * hd, hd, kc, vc, 0,
+                                         (int64_t)m->cache->capacity * hd, hd, 1, H, HK, s, pos + s, hd, scale,
+                                         s > 1 ? FH_MASK_CAUSAL : FH_MASK_NONE, nullptr, m->att));
+        }
+        const float *att_in = m->att; // [H, s, hd]; for s == 1 this already is [s, H*hd]
+        if (s > 1) {
+            FH_TRY(fh_transpose_shd(dev, m->att, H, s, hd, m->att_t));
+            att_in = m->att_t;
+        }
+        FH_TRY(fh_qmatmul(l.wo, att_in, s, m->attn_out));
+        FH_TRY(fh_rms_norm(dev, m->attn_out, m->x, l.ffn_norm, nullptr, c.eps, s, D, m->xn));
+        if (l.gate_up && s <= 2) {
+            FH_TRY(fh_qmatmul_swiglu(l.gate_up, m->xn, s, m->act));
+        } else if (l.gate_up) {
+            FH_TRY(fh_qmatmul(l.gate_up, m->xn, s, m->gu)); // [s, 2F]: gate | up per row
+            // split the halves: silu(gate) * up with row stride 2F
+            FH_TRY(fh_swiglu_rows(dev, m->gu, s, F, m->act));
+        } else {
+            FH_TRY(fh_qmatmul(l.gate, m->xn, s, m->gu));
+            FH_TRY(fh_qmatmul(l.up, m->xn, s, m->gu + (size_t)s * F));
+            FH_TRY(fh_swiglu(dev, m->gu, m->gu + (size_t)s * F, m->act, (int64_t)s * F));
+        }
+        if (s == 1) { // forward_add_residuals, attention_layer.rs:147-174: (down(act) + attn) + residual
+            FH_TRY(fh_qmatmul_add2(l.down, m->act, 1, m->attn_out, m->x, m->x));
+        } else {      // raw/mod.rs:1036
+            FH_TRY(fh_qmatmul(l.down, m->act, s, m->ff));
+            FH_TRY(fh_add3(dev, m->ff, m->attn_out, m->x, m->x, (int64_t)s * D));
+        }
+    }
+    FH_TRY(fh_rms_norm(dev, m->x + (size_t)(s - 1) * D, nullptr, m->out_norm, nullptr, c.eps, 1, D, m->xn));
+    FH_TRY(fh_qmatmul(m->output, m->xn, 1, m->logits));
+    return FH_OK;
+}
+
+extern "C" fh_status fh_llama_forward(fh_llama *m, const uint32_t *tokens_host, int32_t count, float *logits_host,
+                                      float *hidden_host) {
+    FH_REQUIRE(m && m->finalized && tokens_host, "decoder not finalized or NULL tokens");
+    FH_REQUIRE(count > 0 && count <= 65535, "count %d out of range", count);
+    FH_REQUIRE(m->pos + count <= m->c.ctx, "context overflow: %d + %d > %d", m->pos, count, m->c.ctx);
+    for (int i = 0; i < count; i++)
+        FH_REQUIRE(tokens_host[i] < (uint32_t)m->c.vocab, "token id %u at %d outside the vocabulary of %d", tokens_host[i], i,
+                   m->c.vocab);
+    FH_TRY(ensure_steps(m, count));
+    FH_TRY(fh_upload(m->dev, m->ids, tokens_host, (size_t)count * 4));
+    FH_TRY(run_layers(m, count, false));
+    // all layers appended: advance the cache
+    m->pos += count;
+    m->cache->len = m->pos;
+    FH_TRY(fh_kvcache_set_len_dev(m->cache, m->pos));
+    if (hidden_host) FH_TRY(fh_download(m->dev, hidden_host, m->xn, (size_t)m->c.d_model * 4));
+    if (logits_host) FH_TRY(fh_download(m->dev, logits_host, m->logits, (size_t)m->c.vocab * 4));
+    FH_TRY(fh_device_sync(m->dev));
+    return FH_OK;
+}
+
+__global__ void k_store_token(const uint32_t *tok, uint32_t *ids, uint32_t *out, int *step) {
+    uint32_t t = *tok;
+    ids[0] = t == 0xFFFFFFFFu ? 0u : t; // next step's input (a non-finite logits row yields id 0)
+    out[*step] = t;
+    *step = *step + 1;
+}
+__global__ void k_set_u32(uint32_t *p, uint32_t v) { *p = v; }
+
+static fh_status decode_step_enqueue(fh_llama *m) {
+    FH_TRY(run_layers(m, 1, true));
+    FH_TRY(fh_kvcache_advance_dev(m->cache));
+    FH_TRY(fh_argmax(m->dev, m->logits, m->c.vocab, m->tok_dev));
+    k_store_token<<<1, 1, 0, m->dev->stream>>>(m->tok_dev, m->ids, m->out_tok_dev, m->step_dev);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+extern "C" fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, int32_t steps, uint32_t *out_tokens_host,
+                                            float *elapsed_ms) {
+    FH_REQUIRE(m && m->finalized && out_tokens_host, "decoder not finalized or NULL output");
+    FH_REQUIRE(steps > 0 && m->pos + steps <= m->c.ctx, "context overflow: %d + %d > %d", m->pos, steps, m->c.ctx);
+    FH_REQUIRE(first_token < (uint32_t)m->c.vocab, "token id %u outside the vocabulary", first_token);
+    fh_device *dev = m->dev;
+    hipStream_t s = dev->stream;
+    // capacity is fixed for the whole run so that no reallocation happens between steps
+    FH_TRY(fh_kvcache_reserve(m->cache, m->pos + steps));
+    k_set_u32<<<1, 1, 0, s>>>(m->ids, first_token);
+    k_set_u32<<<1, 1, 0, s>>>((uint32_t *)m->step_dev, 0u);
+    FH_HIP(hipGetLastError());
+    int done = 0;
+    if (m->c.use_graph) {
+        // One eager step sizes every scratch buffer and sets kernel attributes; the capture then
+        // records launches only.  The graph depends on the cache capacity (strides), so it is
+        // rebuilt when the capacity changed since the last capture.
+        if (!m->graph_exec || m->captured_capacity != m->cache->capacity) {
+            FH_TRY(fh_timer_start(dev));
+            FH_TRY(decode_step_enqueue(m));
+            done = 1;
+            FH_HIP(hipStreamSynchronize(s));
+            if (m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
+            if (m->graph) { (void)hipGraphDestroy(m->graph); m->graph = nullptr; }
+            FH_HIP(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+            fh_status st = decode_step_enqueue(m);
+            hipError_t e = hipStreamEndCapture(s, &m->graph);
+            if (st != FH_OK) return st;
+            FH_HIP(e);
+            FH_HIP(hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
+            m->captured_capacity = m->cache->capacity;
+        } else {
+            FH_TRY(fh_timer_start(dev));
+        }
+        for (; done < steps; done++) FH_HIP(hipGraphLaunch(m->graph_exec, s));
+    } else {
+        FH_TRY(fh_timer_start(dev));
+        for (; done < steps; done++) FH_TRY(decode_step_enqueue(m));
+    }
+    float ms = 0.f;
+    FH_TRY(fh_timer_stop(dev, &ms));
+    if (elapsed_ms) *elapsed_ms = ms;
+    m->pos += steps;
+    m->cache->len = m->pos;
+    FH_TRY(fh_download(dev, out_tokens_host, m->out_tok_dev, (size_t)steps * 4));
+    return FH_OK;
+}

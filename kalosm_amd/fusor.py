@@ -1,0 +1,408 @@
+"""Host-side mirror of the `fusor` crate's operator surface for the quantized-inference path,
+bound to libfusor_hip.so.  Names and argument meaning follow the reference facade
+(fusor-ml/fusor/src: device.rs, quantized.rs, lib.rs, composite/*.rs, cache/*.rs, layers/*.rs) so
+tests read like the reference's own.  Every operator runs on the HIP library; nothing here computes
+on the host except shape bookkeeping and host<->device copies.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence
+
+import numpy as np
+
+from . import _lib
+from ._lib import (F16, F32, MASK_ADDITIVE, MASK_CAUSAL, MASK_NONE, Q4_0, Q4_K, Q6_K, Q8_0, FusorHipError, check)
+
+__all__ = ["Device", "Tensor", "QMatrix", "RopeCache", "KvCache", "MaskKind", "GgmlType", "FusorHipError"]
+
+
+class GgmlType:
+    """fusor-ml/gguf/src/lib.rs:35-50"""
+    Q4_0, Q8_0, Q4K, Q6K = Q4_0, Q8_0, Q4_K, Q6_K
+    BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256}
+    BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210}
+
+
+class MaskKind:
+    """fusor-ml/fusor/src/composite/flash_attention.rs:12-24"""
+    QKMask, Causal = MASK_ADDITIVE, MASK_CAUSAL
+
+
+_NP = {"f32": np.float32, "f16": np.float16, "bf16": np.uint16, "u32": np.uint32, "i32": np.int32, "u8": np.uint8}
+
+
+class Device:
+    """fusor::Device::Gpu (fusor-ml/fusor/src/device.rs:7-78) on HIP."""
+
+    def __init__(self, ordinal: int = 0):
+        self._lib = _lib.load()
+        h = C.c_void_p()
+        check(self._lib.fh_device_create(ordinal, C.byref(h)))
+        self._h = h
+
+    @staticmethod
+    def gpu(ordinal: int = 0) -> "Device":
+        return Device(ordinal)
+
+    @staticmethod
+    def count() -> int:
+        n = C.c_int32()
+        check(_lib.load().fh_device_count(C.byref(n)))
+        return n.value
+
+    def info(self) -> dict:
+        name = C.create_string_buffer(256)
+        cu, mem = C.c_int32(), C.c_uint64()
+        check(self._lib.fh_device_info(self._h, name, 256, C.byref(cu), C.byref(mem)))
+        return {"name": name.value.decode(), "compute_units": cu.value, "total_mem": mem.value}
+
+    def sync(self) -> None:
+        check(self._lib.fh_device_sync(self._h))
+
+    def set_option(self, key: str, value: int) -> None:
+        check(self._lib.fh_set_option(self._h, key.encode(), value))
+
+    def timer_start(self) -> None:
+        check(self._lib.fh_timer_start(self._h))
+
+    def timer_stop(self) -> float:
+        ms = C.c_float()
+        check(self._lib.fh_timer_stop(self._h, C.byref(ms)))
+        return ms.value
+
+    # -- memory
+    def alloc(self, nbytes: int) -> int:
+        p = C.c_void_p()
+        check(self._lib.fh_malloc(self._h, nbytes, C.byref(p)))
+        return p.value
+
+    def free(self, ptr: int) -> None:
+        check(self._lib.fh_free(self._h, C.c_void_p(ptr)))
+
+    def close(self) -> None:
+        if self._h is not None:
+            self._lib.fh_device_destroy(self._h)
+            self._h = None
+
+
+class Tensor:
+    """A contiguous row-major device tensor (fusor::Tensor::Gpu).  dtype in f32/f16/bf16/u32/i32/u8."""
+
+    def __init__(self, device: Device, shape: Sequence[int], dtype: str = "f32", ptr: Optional[int] = None):
+        self.device, self.shape, self.dtype = device, tuple(int(s) for s in shape), dtype
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * np.dtype(_NP[dtype]).itemsize
+        self._own = ptr is None
+        self.ptr = device.alloc(max(self.nbytes, 16)) if ptr is None else ptr
+
+    # Tensor::from_slice / Tensor::new (fusor-ml/fusor/src/lib.rs:356-368)
+    @staticmethod
+    def from_slice(device: Device, data, dtype: str = "f32") -> "Tensor":
+        a = np.ascontiguousarray(data, dtype=_NP[dtype])
+        t = Tensor(device, a.shape, dtype)
+        if a.nbytes:
+            check(device._lib.fh_upload(device._h, C.c_void_p(t.ptr), a.ctypes.data_as(C.c_void_p), a.nbytes))
+        return t
+
+    @staticmethod
+    def zeros(device: Device, shape, dtype: str = "f32") -> "Tensor":
+        t = Tensor(device, shape, dtype)
+        check(device._lib.fh_memset(device._h, C.c_void_p(t.ptr), 0, max(t.nbytes, 1)))
+        return t
+
+    @staticmethod
+    def filled_bytes(device: Device, shape, byte: int, dtype: str = "f32") -> "Tensor":
+        """A buffer pre-filled with a byte pattern ("poisoned" outputs, as the reference's dirty buffer pool)."""
+        t = Tensor(device, shape, dtype)
+        check(device._lib.fh_memset(device._h, C.c_void_p(t.ptr), byte, max(t.nbytes, 1)))
+        return t
+
+    def as_slice(self) -> np.ndarray:
+        """Blocking read-back (Tensor::as_slice)."""
+        out = np.empty(self.shape, _NP[self.dtype])
+        if out.nbytes:
+            check(self.device._lib.fh_download(self.device._h, out.ctypes.data_as(C.c_void_p), C.c_void_p(self.ptr),
+                                               out.nbytes))
+        return out
+
+    def reshape(self, shape) -> "Tensor":
+        shape = tuple(shape)
+        assert int(np.prod(shape)) == int(np.prod(self.shape)), "reshape changes the element count"
+        t = Tensor(self.device, shape, self.dtype, ptr=self.ptr)
+        t._keep = self
+        return t
+
+    def cast(self, dtype: str) -> "Tensor":
+        if dtype == self.dtype:
+            return self
+        out = Tensor(self.device, self.shape, dtype)
+        n = int(np.prod(self.shape))
+        L, d = self.device._lib, self.device._h
+        if (self.dtype, dtype) == ("f32", "f16"):
+            check(L.fh_cast_f32_f16(d, C.c_void_p(self.ptr), C.c_void_p(out.ptr), n))
+        elif (self.dtype, dtype) == ("f16", "f32"):
+            check(L.fh_cast_f16_f32(d, C.c_void_p(self.ptr), C.c_void_p(out.ptr), n))
+        elif (self.dtype, dtype) == ("f32", "bf16"):
+            check(L.fh_cast_f32_bf16(d, C.c_void_p(self.ptr), C.c_void_p(out.ptr), n))
+        else:
+            raise FusorHipError(_lib.FH_ERR_UNSUPPORTED, f"cast {self.dtype}->{dtype}")
+        return out
+
+    # ---- operators -------------------------------------------------------------------------
+    def q_mat_mul(self, w: "QMatrix", out: Optional["Tensor"] = None) -> "Tensor":
+        """Tensor::q_mat_mul (fusor-ml/fusor/src/lib.rs:1132-1223); rank 1, 2 or 3 (rank 1 is viewed as [1, k])."""
+        k = self.shape[-1]
+        if k != w.k:
+            raise FusorHipError(_lib.FH_ERR_INVALID,
+                                f"Matrix dimension mismatch: lhs columns ({k}) != weight in_features ({w.k})")
+        m = int(np.prod(self.shape[:-1])) if len(self.shape) > 1 else 1
+        oshape = (*self.shape[:-1], w.n) if len(self.shape) > 1 else (w.n,)
+        out = out or Tensor(self.device, oshape, "f32")
+        L = self.device._lib
+        if self.dtype == "bf16":
+            check(L.fh_qmatmul_bf16(w._h, C.c_void_p(self.ptr), m, C.c_void_p(out.ptr)))
+        else:
+            assert self.dtype == "f32"
+            check(L.fh_qmatmul(w._h, C.c_void_p(self.ptr), m, C.c_void_p(out.ptr)))
+        return out
+
+    def q_mat_mul_add2(self, w: "QMatrix", first: "Tensor", second: "Tensor") -> "Tensor":
+        """(x.W^T + first) + second, the decode epilogue of raw/attention_layer.rs:147-174."""
+        m = int(np.prod(self.shape[:-1]))
+        out = Tensor(self.device, (*self.shape[:-1], w.n), "f32")
+        check(self.device._lib.fh_qmatmul_add2(w._h, C.c_void_p(self.ptr), m, C.c_void_p(first.ptr),
+                                               C.c_void_p(second.ptr), C.c_void_p(out.ptr)))
+        return out
+
+    def q_mat_mul_swiglu(self, gate_up: "QMatrix") -> "Tensor":
+        """silu(x.Wg^T) * (x.Wu^T) with gate_up = concat_rows(gate, up), raw/attention_layer.rs:186-196."""
+        m = int(np.prod(self.shape[:-1]))
+        out = Tensor(self.device, (*self.shape[:-1], gate_up.n // 2), "f32")
+        check(self.device._lib.fh_qmatmul_swiglu(gate_up._h, C.c_void_p(self.ptr), m, C.c_void_p(out.ptr)))
+        return out
+
+    def q_mat_mul_q8(self, w: "QMatrix", want_isums: bool = False):
+        """The Q8_0 x Q8 integer variant (per-32 activation quantisation + vec_dot)."""
+        m = int(np.prod(self.shape[:-1]))
+        out = Tensor(self.device, (*self.shape[:-1], w.n), "f32")
+        isums = Tensor(self.device, (m, w.n, w.k // 32), "i32") if want_isums else None
+        check(self.device._lib.fh_qmatmul_q8(w._h, C.c_void_p(self.ptr), m, C.c_void_p(out.ptr),
+                                             C.c_void_p(isums.ptr) if isums else None))
+        return (out, isums) if want_isums else out
+
+    def quantize_q8_0(self) -> "Tensor":
+        n = int(np.prod(self.shape))
+        out = Tensor(self.device, (n // 32, 34), "u8")
+        check(self.device._lib.fh_q8_0_quantize(self.device._h, C.c_void_p(self.ptr), n, C.c_void_p(out.ptr)))
+        return out
+
+    def rms_norm_fused(self, weight: "Tensor", bias: Optional["Tensor"], eps: float) -> "Tensor":
+        """fusor-ml/fusor/src/composite/normalization.rs:287-326"""
+        return self._rms(None, weight, bias, eps)
+
+    def rms_norm_residual_fused(self, residual: "Tensor", weight: "Tensor", bias: Optional["Tensor"],
+                                eps: float) -> "Tensor":
+        """normalization.rs:356-401"""
+        return self._rms(residual, weight, bias, eps)
+
+    def _rms(self, residual, weight, bias, eps):
+        cols = self.shape[-1]
+        rows = int(np.prod(self.shape[:-1])) if len(self.shape) > 1 else 1
+        assert weight.shape == (cols,)
+        out = Tensor(self.device, self.shape, "f32")
+        check(self.device._lib.fh_rms_norm(self.device._h, C.c_void_p(self.ptr),
+                                           C.c_void_p(residual.ptr) if residual else None, C.c_void_p(weight.ptr),
+                                           C.c_void_p(bias.ptr) if bias else None, eps, rows, cols,
+                                           C.c_void_p(out.ptr)))
+        return out
+
+    def flash_attention(self, k: "Tensor", v: "Tensor", scale: float, mask=None,
+                        q_strides: Optional[Sequence[int]] = None) -> "Tensor":
+        """Tensor<4>::flash_attention(&k, &v, scale, Option<(&mask, MaskKind)>)
+        (fusor-ml/fusor/src/composite/flash_attention.rs:58-109).  `mask` is None, MaskKind.Causal, or a
+        ([sq, skv] f32 Tensor, MaskKind.QKMask) pair.  q_strides = (batch, head, position) element strides of a
+        transposed query view whose logical shape is self.shape (the [b,s,h,d] -> [b,h,s,d] case)."""
+        b, hq, sq, d = self.shape
+        b2, hkv, skv, d2 = k.shape
+        if hq % hkv:
+            raise FusorHipError(_lib.FH_ERR_INVALID,
+                                f"Number of Q heads ({hq}) must be divisible by number of K/V heads ({hkv})")
+        assert (b2, d2) == (b, d) and v.shape == k.shape
+        kind, mptr = MASK_NONE, None
+        if mask is not None:
+            if mask == MaskKind.Causal:
+                kind = MASK_CAUSAL
+            else:
+                mt, kind = mask
+                if kind == MASK_ADDITIVE:
+                    assert mt.shape == (sq, skv), f"QKMask shape {mt.shape} does not match expected [{sq}, {skv}]"
+                    mptr = C.c_void_p(mt.ptr)
+        qs = q_strides or (hq * sq * d, sq * d, d)
+        qdt = F16 if self.dtype == "f16" else F32
+        kdt = F16 if k.dtype == "f16" else F32
+        out = Tensor(self.device, (b, hq, sq, d), self.dtype)
+        check(self.device._lib.fh_flash_attention_ex(self.device._h, qdt, kdt, C.c_void_p(self.ptr), qs[0], qs[1], qs[2],
+                                                     C.c_void_p(k.ptr), C.c_void_p(v.ptr), hkv * skv * d, skv * d, d, b,
+                                                     hq, hkv, sq, skv, d, scale, kind, mptr, C.c_void_p(out.ptr)))
+        return out
+
+    def silu_mul(self, up: "Tensor") -> "Tensor":
+        """silu(self) * up (activations.rs:47-65, raw/attention_layer.rs:195)"""
+        out = Tensor(self.device, self.shape, "f32")
+        check(self.device._lib.fh_swiglu(self.device._h, C.c_void_p(self.ptr), C.c_void_p(up.ptr), C.c_void_p(out.ptr),
+                                         int(np.prod(self.shape))))
+        return out
+
+    def add(self, b: "Tensor", c: Optional["Tensor"] = None) -> "Tensor":
+        """(self + b) [+ c]"""
+        out = Tensor(self.device, self.shape, "f32")
+        check(self.device._lib.fh_add3(self.device._h, C.c_void_p(self.ptr), C.c_void_p(b.ptr),
+                                       C.c_void_p(c.ptr) if c else None, C.c_void_p(out.ptr), int(np.prod(self.shape))))
+        return out
+
+    def transpose_shd(self) -> "Tensor":
+        """[s, h, d] -> [h, s, d] materialised (reshape + transpose(1, 2) + to_concrete)."""
+        s, h, d = self.shape
+        out = Tensor(self.device, (h, s, d), "f32")
+        check(self.device._lib.fh_transpose_shd(self.device._h, C.c_void_p(self.ptr), s, h, d, C.c_void_p(out.ptr)))
+        return out
+
+    def top_k_pairs_1(self) -> int:
+        """Tensor::top_k_pairs(1) (fusor-ml/fusor/src/lib.rs:416-447): the greedy token id, or -1."""
+        out = Tensor(self.device, (1,), "u32")
+        check(self.device._lib.fh_argmax(self.device._h, C.c_void_p(self.ptr), int(np.prod(self.shape)),
+                                         C.c_void_p(out.ptr)))
+        v = int(out.as_slice()[0])
+        return -1 if v == 0xFFFFFFFF else v
+
+    def __del__(self):
+        try:
+            if self._own and self.ptr and self.device._h is not None:
+                self.device.free(self.ptr)
+        except Exception:
+            pass
+
+
+class QMatrix:
+    """fusor::QMatrix::Gpu (fusor-ml/fusor/src/quantized.rs:80-279)."""
+
+    def __init__(self, device: Device, handle):
+        self.device, self._h = device, handle
+        t, n, k, b = C.c_uint32(), C.c_int64(), C.c_int64(), C.c_uint64()
+        check(device._lib.fh_qmatrix_info(handle, C.byref(t), C.byref(n), C.byref(k), C.byref(b)))
+        self.ggml_type, self.n, self.k, self.device_bytes = t.value, n.value, k.value, b.value
+
+    @staticmethod
+    def from_raw_bytes(device: Device, shape: Sequence[int], raw, ty: int) -> "QMatrix":
+        n, k = int(shape[0]), int(shape[1])
+        a = np.ascontiguousarray(raw).view(np.uint8).reshape(-1)
+        h = C.c_void_p()
+        check(device._lib.fh_qmatrix_from_gguf_bytes(device._h, ty, n, k, a.ctypes.data_as(C.c_void_p), a.nbytes,
+                                                     C.byref(h)))
+        return QMatrix(device, h)
+
+    @staticmethod
+    def concat_rows(matrices: Sequence["QMatrix"]) -> Optional["QMatrix"]:
+        dev = matrices[0].device
+        arr = (C.c_void_p * len(matrices))(*[m._h for m in matrices])
+        h = C.c_void_p()
+        st = dev._lib.fh_qmatrix_concat_rows(dev._h, arr, len(matrices), C.byref(h))
+        if st == _lib.FH_ERR_UNSUPPORTED:
+            return None  # the reference returns Option::None when it cannot concatenate
+        check(st)
+        return QMatrix(dev, h)
+
+    def shape(self):
+        return (self.n, self.k)
+
+    def dequantize(self) -> Tensor:
+        out = Tensor(self.device, (self.n, self.k), "f32")
+        check(self.device._lib.fh_qmatrix_dequantize(self._h, C.c_void_p(out.ptr)))
+        return out
+
+    def embed(self, ids) -> Tensor:
+        """Embedding::forward (fusor-ml/fusor/src/layers/embedding.rs:43-89)"""
+        idh = np.ascontiguousarray(ids, dtype=np.uint32).reshape(-1)
+        idt = Tensor.from_slice(self.device, idh, "u32")
+        out = Tensor(self.device, (idh.size, self.k), "f32")
+        check(self.device._lib.fh_embed_rows(self._h, C.c_void_p(idt.ptr), idh.ctypes.data_as(C.c_void_p), idh.size,
+                                             C.c_void_p(out.ptr)))
+        return out
+
+    def __del__(self):
+        try:
+            if self._h and self.device._h is not None:
+                self.device._lib.fh_qmatrix_free(self._h)
+        except Exception:
+            pass
+
+
+class RopeCache:
+    """fusor::RopeCache (fusor-ml/fusor/src/composite/rope.rs:248-329)."""
+
+    def __init__(self, device: Device, cos: Tensor, sin: Tensor):
+        self.device, self.cos, self.sin = device, cos, sin
+
+    @staticmethod
+    def new(head_dim: int, context_length: int, rope_theta: float, device: Device) -> "RopeCache":
+        cos = Tensor(device, (context_length, head_dim // 2), "f32")
+        sin = Tensor(device, (context_length, head_dim // 2), "f32")
+        check(device._lib.fh_rope_tables(device._h, head_dim, context_length, rope_theta, C.c_void_p(cos.ptr),
+                                         C.c_void_p(sin.ptr)))
+        return RopeCache(device, cos, sin)
+
+    @staticmethod
+    def from_parts(cos: Tensor, sin: Tensor) -> "RopeCache":
+        return RopeCache(cos.device, cos, sin)
+
+    def _fwd(self, q: Tensor, k: Tensor, start_pos: int, interleaved: bool, q_strides=None, k_strides=None):
+        b, hq, s, d = q.shape
+        _, hk, _, _ = k.shape
+        qs = q_strides or (hq * s * d, s * d, d)
+        ks = k_strides or (hk * s * d, s * d, d)
+        qo, ko = Tensor(self.device, q.shape, "f32"), Tensor(self.device, k.shape, "f32")
+        check(self.device._lib.fh_rope_pair(self.device._h, C.c_void_p(q.ptr), qs[0], qs[1], qs[2], C.c_void_p(k.ptr),
+                                            ks[0], ks[1], ks[2], b, hq, hk, s, d, C.c_void_p(self.cos.ptr),
+                                            C.c_void_p(self.sin.ptr), self.cos.shape[0], start_pos, int(interleaved),
+                                            C.c_void_p(qo.ptr), C.c_void_p(ko.ptr)))
+        return qo, ko
+
+    def forward(self, q, k, start_pos, **kw):
+        return self._fwd(q, k, start_pos, False, **kw)
+
+    def forward_interleaved(self, q, k, start_pos, **kw):
+        return self._fwd(q, k, start_pos, True, **kw)
+
+
+class KvCache:
+    """fusor::KvCache (fusor-ml/fusor/src/cache/kv_cache.rs:24-63) for `layers` layers at once."""
+
+    def __init__(self, device: Device, layers: int, kv_heads: int, head_dim: int, max_len: int, dtype: str = "f32"):
+        self.device, self.layers, self.kv_heads, self.head_dim, self.dtype = device, layers, kv_heads, head_dim, dtype
+        h = C.c_void_p()
+        check(device._lib.fh_kvcache_create(device._h, layers, kv_heads, head_dim, max_len, F16 if dtype == "f16" else F32,
+                                            C.byref(h)))
+        self._h = h
+
+    def append(self, layer: int, k: Tensor, v: Tensor) -> None:
+        """k, v: [kv_heads, s, head_dim] f32 contiguous."""
+        hk, s, d = k.shape
+        check(self.device._lib.fh_kvcache_append(self._h, layer, C.c_void_p(k.ptr), C.c_void_p(v.ptr), s * d, d, s))
+
+    def view(self, layer: int):
+        ln, cap, kp, vp = C.c_int32(), C.c_int32(), C.c_void_p(), C.c_void_p()
+        check(self.device._lib.fh_kvcache_view(self._h, layer, C.byref(ln), C.byref(cap), C.byref(kp), C.byref(vp)))
+        shape = (self.kv_heads, cap.value, self.head_dim)
+        kt = Tensor(self.device, shape, self.dtype, ptr=kp.value) if kp.value else None
+        vt = Tensor(self.device, shape, self.dtype, ptr=vp.value) if vp.value else None
+        return ln.value, cap.value, kt, vt
+
+    def reset(self) -> None:
+        check(self.device._lib.fh_kvcache_reset(self._h))
+
+    def __del__(self):
+        try:
+            if self._h and self.device._h is not None:
+                self.device._lib.fh_kvcache_destroy(self._h)
+        except Exception:
+            pass

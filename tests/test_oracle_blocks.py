@@ -1,0 +1,283 @@
+"""Pins the CPU checker's block decode, f16 conversion and quantized matmul against the reference's own
+known answers, an independent numpy restatement, and what the mathematics fixes."""
+import numpy as np
+import pytest
+
+import refgen
+from refgen import Q4_0, Q4_K, Q6_K, Q8_0
+
+ALL = [Q4_0, Q8_0, Q4_K, Q6_K]
+
+
+def h16(v):
+    return np.frombuffer(np.float32(v).astype(np.float16).tobytes(), np.uint8)
+
+
+def test_f16_exhaustive_round_trip(oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    f = oracle.f16_to_f32(bits)
+    want = bits.view(np.float16).astype(np.float32)
+    assert np.array_equal(f.view(np.uint32), want.view(np.uint32))
+    back = oracle.f32_to_f16(f)
+    nan = np.isnan(want)
+    assert np.array_equal(back[~nan], bits[~nan])
+
+
+def test_f32_to_f16_rounding_matches_numpy(oracle):
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(200000).astype(np.float32) * s for s in (1e-8, 1e-5, 1e-3, 1, 100, 70000)])
+    # exact ties and the subnormal boundary
+    x = np.concatenate([x, np.float32([65504, 65519.99, 65520, 6.1e-5, 5.96e-8, 2.98e-8, 2.9802322e-8, 0.0, -0.0])])
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(oracle.f32_to_f16(x), want)
+
+
+def test_block_sizes(oracle):
+    # gguf/src/lib.rs:764-769, :1122-1127, :1425-1432, :1933-1944
+    assert [oracle.lib().fo_block_bytes(t) for t in ALL] == [18, 34, 144, 210]
+    assert [oracle.lib().fo_block_elems(t) for t in ALL] == [32, 32, 256, 256]
+
+
+def test_known_answers_528(oracle):
+    """core/src/quantized/matmul/tests.rs:1337-1397: scale 1, packed 0x99 / 0x77 (Q4_0), q = +1 / -1 (Q8_0),
+    x = 1..32  ->  +528 / -528."""
+    x = np.arange(1, 33, dtype=np.float32)[None, :]
+    raw = np.concatenate([h16(1.0), np.full(16, 0x99, np.uint8), h16(1.0), np.full(16, 0x77, np.uint8)])
+    y = oracle.q_mat_mul(Q4_0, x, raw, 2)
+    assert y.shape == (1, 2) and y[0, 0] == 528.0 and y[0, 1] == -528.0
+    raw = np.concatenate([h16(1.0), np.full(32, 1, np.uint8), h16(1.0), np.full(32, 0xFF, np.uint8)])
+    y = oracle.q_mat_mul(Q8_0, x, raw, 2)
+    assert y[0, 0] == 528.0 and y[0, 1] == -528.0
+
+
+def test_q4k_unit_scales_32896(oracle):
+    """The Q4_K analogue of tests.rs:1399-1423 / gguf lib.rs:2378-2408: d = 1, dmin = 0,
+    scales [1,1,1,1,0,0,0,0,1,1,1,1] make every sub-scale 1 and every min 0, nibbles 0x11 -> weights 1,
+    x = 1..256 -> 32896."""
+    raw = np.concatenate([h16(1.0), h16(0.0), np.uint8([1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1]), np.full(128, 0x11, np.uint8)])
+    sc, mn = oracle.unpack_k4_scales(raw[4:16])
+    assert sc.tolist() == [1] * 8 and mn.tolist() == [0] * 8
+    assert np.array_equal(oracle.dequantize(Q4_K, raw), np.ones(256, np.float32))
+    x = np.arange(1, 257, dtype=np.float32)[None, :]
+    assert oracle.q_mat_mul(Q4_K, x, raw, 1)[0, 0] == 32896.0
+
+
+def test_q4k_nibble_identity(oracle):
+    """d = 1, dmin = 0, unit sub-scales: dequantize returns the nibbles in the order low(chunk c), high(chunk c)."""
+    rng = np.random.default_rng(1)
+    qs = rng.integers(0, 256, 128, dtype=np.uint8)
+    raw = np.concatenate([h16(1.0), h16(0.0), np.uint8([1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1]), qs])
+    out = oracle.dequantize(Q4_K, raw).reshape(4, 2, 32)
+    c = qs.reshape(4, 32)
+    assert np.array_equal(out[:, 0, :], (c & 15).astype(np.float32))
+    assert np.array_equal(out[:, 1, :], (c >> 4).astype(np.float32))
+
+
+def test_k4_scale_unpack_brute_force(oracle):
+    """Every 6-bit (scale, min) assignment survives pack -> unpack, and the unpack matches the bit diagram of
+    gguf/src/lib.rs:2143-2173 on random 12-byte patterns."""
+    from kalosm_amd import synth
+
+    rng = np.random.default_rng(2)
+    for _ in range(300):
+        sc = rng.integers(0, 64, 8, dtype=np.uint8)
+        mn = rng.integers(0, 64, 8, dtype=np.uint8)
+        s2, m2 = oracle.unpack_k4_scales(synth.pack_k4_scales(sc, mn))
+        assert np.array_equal(s2, sc) and np.array_equal(m2, mn)
+    for v in range(64):  # each field on its own, all values
+        for j in range(8):
+            sc = np.zeros(8, np.uint8); mn = np.zeros(8, np.uint8)
+            sc[j] = v
+            s2, m2 = oracle.unpack_k4_scales(synth.pack_k4_scales(sc, mn))
+            assert s2[j] == v and s2.sum() == v and m2.sum() == 0
+            s2, m2 = oracle.unpack_k4_scales(synth.pack_k4_scales(mn, sc))
+            assert m2[j] == v and m2.sum() == v and s2.sum() == 0
+    for _ in range(300):  # the diagram, read bit by bit
+        p = rng.integers(0, 256, 12, dtype=np.uint8)
+        s2, m2 = oracle.unpack_k4_scales(p)
+        for j in range(4):
+            assert s2[j] == (p[j] & 0x3F) and m2[j] == (p[4 + j] & 0x3F)
+            assert s2[4 + j] == ((p[8 + j] & 0x0F) | ((p[j] >> 6) << 4))
+            assert m2[4 + j] == ((p[8 + j] >> 4) | ((p[4 + j] >> 6) << 4))
+
+
+def test_q6k_special_cases(oracle):
+    """d = 1, all sub-scales 1: output = 6-bit code - 32 with ql supplying the low and qh the high bits."""
+    rng = np.random.default_rng(3)
+    ql = rng.integers(0, 256, 128, dtype=np.uint8)
+    qh = rng.integers(0, 256, 64, dtype=np.uint8)
+    raw = np.concatenate([ql, qh, np.ones(16, np.uint8), h16(1.0)])
+    out = oracle.dequantize(Q6_K, raw)
+    for n in range(2):
+        for l in range(32):
+            h = int(qh[32 * n + l])
+            a, c = int(ql[64 * n + l]), int(ql[64 * n + l + 32])
+            want = [((h & 3) << 4 | (a & 15)) - 32, (((h >> 2) & 3) << 4 | (c & 15)) - 32,
+                    (((h >> 4) & 3) << 4 | (a >> 4)) - 32, (((h >> 6) & 3) << 4 | (c >> 4)) - 32]
+            got = [out[128 * n + l + 32 * j] for j in range(4)]
+            assert got == [float(w) for w in want]
+    # one sub-scale at a time selects its 16 outputs
+    for g in range(16):
+        sc = np.zeros(16, np.uint8); sc[g] = 0xFE  # -2 as i8
+        raw = np.concatenate([np.full(128, 0xFF, np.uint8), np.full(64, 0xFF, np.uint8), sc, h16(0.5)])
+        out = oracle.dequantize(Q6_K, raw)
+        want = np.zeros(256, np.float32)
+        want[16 * g:16 * g + 16] = 0.5 * -2 * 31
+        assert np.array_equal(out, want)
+
+
+@pytest.mark.parametrize("ty", ALL)
+def test_dequantize_matches_independent_numpy(oracle, ty):
+    """Random blocks incl. negative / subnormal f16 scales, sub-scales 0 and 63, all-zero and all-0xFF quants:
+    the C checker and the numpy restatement agree bit for bit."""
+    from kalosm_amd import synth
+
+    rng = np.random.default_rng(10 + ty)
+    raw = synth.random_blocks(ty, 512, rng).reshape(512, -1).copy()
+    raw[0, :] = 0
+    raw[1, :] = 0xFF  # scale field 0xFFFF is a NaN f16: both sides must propagate it
+    if ty == Q4_K:
+        raw[2, 0:2] = h16(3e-6); raw[2, 2:4] = h16(-2e-6)           # subnormal d / dmin
+        raw[3, 4:16] = synth.pack_k4_scales(np.full(8, 63, np.uint8), np.zeros(8, np.uint8))
+        raw[4, 4:16] = synth.pack_k4_scales(np.zeros(8, np.uint8), np.full(8, 63, np.uint8))
+    if ty == Q6_K:
+        raw[2, 208:210] = h16(-4e-6)
+        raw[3, 192:208] = 0x80  # -128
+    if ty in (Q4_0, Q8_0):
+        raw[2, 0:2] = h16(-5e-7)
+    a = oracle.dequantize(ty, raw)
+    b = refgen.np_dequantize(ty, raw)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+@pytest.mark.parametrize("ty", ALL)
+def test_dequantize_reference_generators(oracle, ty):
+    """The reference's deterministic fixture bytes (conformance common/quantized.rs:175-272)."""
+    raw = refgen.REF_GENERATORS[ty](40)
+    a = oracle.dequantize(ty, raw)
+    b = refgen.np_dequantize(ty, raw)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert np.isfinite(a).all()
+
+
+def test_q4k_reference_fixture_block(oracle):
+    """gguf/src/lib.rs:2322-2331: BlockQ4K{d = 0.1, dmin = 0.05, scales = [8,16,...,96], data[i] = (3i) % 256};
+    spot-check elements against the formula evaluated by hand in float32."""
+    scales = np.arange(8, 104, 8, dtype=np.uint8)
+    data = ((3 * np.arange(128)) % 256).astype(np.uint8)
+    raw = np.concatenate([h16(0.1), h16(0.05), scales, data])
+    out = oracle.dequantize(Q4_K, raw)
+    d = np.float32(np.float16(0.1)); dm = np.float32(np.float16(0.05))
+    sc, mn = oracle.unpack_k4_scales(scales)
+    # element 0: sub-block 0, low nibble of data[0] = 0;  element 37: sub-block 1, high nibble of data[5] = 15
+    assert out[0] == np.float32(np.float32(sc[0]) * d) * np.float32(0) - np.float32(np.float32(mn[0]) * dm)
+    assert out[37] == np.float32(np.float32(np.float32(sc[1]) * d) * np.float32(data[5] >> 4)) - np.float32(np.float32(mn[1]) * dm)
+    # element 200: chunk 3 (bytes 96..127), low nibbles -> sub-block 6, l = 8 -> data[104]
+    assert out[200] == np.float32(np.float32(np.float32(sc[6]) * d) * np.float32(data[104] & 15)) - np.float32(np.float32(mn[6]) * dm)
+
+
+@pytest.mark.parametrize("ty", ALL)
+def test_qmatmul_invariants(oracle, ty):
+    """one-hot picks a single dequantised weight exactly (tests.rs:951-995); zeros give exact zeros
+    (:450-476, :997-1020); float64 dense product within rounding; thread count and the fast form do not
+    change a bit; batched == unbatched."""
+    from kalosm_amd import synth
+
+    n, k = 96, 1024
+    raw = synth.random_weight(ty, n, k, seed=5)
+    w = oracle.dequantize(ty, raw).reshape(n, k)
+    x = np.zeros((1, k), np.float32)
+    x[0, 777] = 0.125
+    y = oracle.q_mat_mul(ty, x, raw, n)
+    assert np.array_equal(y[0], np.float32(0.125) * w[:, 777])
+    assert np.array_equal(oracle.q_mat_mul(ty, np.zeros((3, k), np.float32), raw, n), np.zeros((3, n), np.float32))
+    zraw = np.zeros_like(raw)
+    assert np.array_equal(oracle.q_mat_mul(ty, np.ones((1, k), np.float32), zraw, n), np.zeros((1, n), np.float32))
+    xs = synth.random_activation(5, k, seed=6)
+    y = oracle.q_mat_mul(ty, xs, raw, n, threads=1)
+    want = refgen.np_matmul_f64(ty, xs, raw, n)
+    scale = np.abs(xs.astype(np.float64)) @ np.abs(w.astype(np.float64)).T
+    assert (np.abs(y - want) <= 2e-6 * scale + 1e-30).all()
+    for th in (2, 3, 8):
+        assert np.array_equal(oracle.q_mat_mul(ty, xs, raw, n, threads=th), y)
+    assert np.array_equal(oracle.q_mat_mul(ty, xs, raw, n, fast=True), y)
+    assert np.array_equal(oracle.q_mat_mul(ty, xs[:1], raw, n, threads=4), y[:1])      # m == 1 column split
+    for r in range(5):                                                                # batched == unbatched
+        assert np.array_equal(oracle.q_mat_mul(ty, xs[r:r + 1], raw, n), y[r:r + 1])
+    # linearity in x (exact for power-of-two scaling)
+    assert np.array_equal(oracle.q_mat_mul(ty, xs * 4, raw, n), y * 4)
+
+
+def test_qmatmul_lane_order_is_the_reference_fold(oracle):
+    """cpu/src/quantized.rs:641-675 + cpu/src/reduce.rs:166-172: 8 lane accumulators over k (lane = k mod 8, fused
+    multiply-add), then a left fold from 0.0.  Replayed here in numpy with exact FMA emulation in float64."""
+    from kalosm_amd import synth
+
+    n, k = 4, 512
+    raw = synth.random_weight(Q4_K, n, k, seed=7)
+    w = oracle.dequantize(Q4_K, raw).reshape(n, k)
+    x = synth.random_activation(1, k, seed=8)[0]
+    y = oracle.q_mat_mul(Q4_K, x[None, :], raw, n)[0]
+    for r in range(n):
+        acc = np.zeros(8, np.float32)
+        for i in range(0, k, 8):
+            # fma in float64 then one rounding: exact because the product of two f32 fits in f64 and the
+            # sum with an f32 is rounded once to f64 (53 bits) before the f32 rounding; double rounding can only
+            # differ on ties at 2^-29 relative, which random data does not hit
+            acc = (x[i:i + 8].astype(np.float64) * w[r, i:i + 8].astype(np.float64) + acc.astype(np.float64)).astype(np.float32)
+        s = np.float32(0.0)
+        for l in range(8):
+            s = np.float32(s + acc[l])
+        assert y[r] == s
+
+
+def test_q8_0_quantize_closed_form(oracle):
+    """gguf/src/lib.rs:1150-1164: amax, scale = amax/127 as f16, q = round(x * 127/amax); round trip < 0.02
+    (:2264-2276); ties: half-even on the AVX2 path (:1198), half-away on the scalar path (:1157)."""
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal(32 * 50).astype(np.float32)
+    blk = oracle.q8_0_quantize(x).reshape(50, 34)
+    xb = x.reshape(50, 32)
+    amax = np.abs(xb).max(1)
+    assert np.array_equal(blk[:, 0:2].copy().view(np.float16)[:, 0], (amax / np.float32(127)).astype(np.float16))
+    inv = np.float32(127) / amax
+    q = np.rint(xb * inv[:, None]).astype(np.int8)
+    assert np.array_equal(blk[:, 2:].view(np.int8), q)
+    deq = oracle.dequantize(Q8_0, blk.reshape(-1)).reshape(50, 32)
+    assert np.abs(deq - xb).max() < 0.02
+    # ties
+    t = np.zeros(32, np.float32); t[0] = 127.0; t[1] = 0.5; t[2] = 1.5; t[3] = -2.5; t[4] = 2.5
+    he = oracle.q8_0_quantize(t)[2:].view(np.int8)
+    ha = oracle.q8_0_quantize(t, round_half_away=True)[2:].view(np.int8)
+    assert he[:5].tolist() == [127, 0, 2, -2, 2] and ha[:5].tolist() == [127, 1, 2, -3, 3]
+    z = oracle.q8_0_quantize(np.zeros(32, np.float32))
+    assert not z.any()
+
+
+def test_vec_dot_exact(oracle):
+    """gguf/src/lib.rs:1315-1358, :927-938: integer dot, then (sum as f32) * (d_w * d_a)."""
+    rng = np.random.default_rng(11)
+    for _ in range(50):
+        w = np.concatenate([h16(rng.normal(0, 0.02)), rng.integers(-127, 128, 32, dtype=np.int8).view(np.uint8)])
+        a = np.concatenate([h16(abs(rng.normal(0, 0.02))), rng.integers(-127, 128, 32, dtype=np.int8).view(np.uint8)])
+        s = int(w[2:].view(np.int8).astype(np.int32) @ a[2:].view(np.int8).astype(np.int32))
+        dw = np.float32(w[:2].copy().view(np.float16)[0]); da = np.float32(a[:2].copy().view(np.float16)[0])
+        assert oracle.vec_dot_q8_0_q8_0(w, a) == float(np.float32(s) * np.float32(dw * da))
+        w4 = np.concatenate([h16(rng.normal(0, 0.02)), rng.integers(0, 256, 16, dtype=np.uint8)])
+        lo = (w4[2:] & 15).astype(np.int32) - 8; hi = (w4[2:] >> 4).astype(np.int32) - 8
+        av = a[2:].view(np.int8).astype(np.int32)
+        s4 = int(lo @ av[:16] + hi @ av[16:])
+        d4 = np.float32(w4[:2].copy().view(np.float16)[0])
+        assert oracle.vec_dot_q4_0_q8_0(w4, a) == float(np.float32(s4) * np.float32(d4 * da))
+    # vec_dot agrees with dequantize . activations within the reference's own 5-10 % bound (gguf lib.rs:2210-2260)
+    from kalosm_amd import synth
+    raw = synth.random_weight(Q8_0, 8, 256, seed=12)
+    x = synth.random_activation(2, 256, seed=13)
+    y, isums = oracle.q8_0_matmul_q8(x, raw, 8, want_isums=True)
+    want = refgen.np_matmul_f64(Q8_0, x, raw, 8)
+    assert np.abs(y - want).max() <= 0.05 * np.abs(want).max() + 1e-3
+    aq = oracle.q8_0_quantize(x).reshape(2, 8, 34)
+    wq = raw.reshape(8, 8, 34)
+    ref = np.einsum("rbi,cbi->rcb", aq[:, :, 2:].view(np.int8).astype(np.int64), wq[:, :, 2:].view(np.int8).astype(np.int64))
+    assert np.array_equal(isums, ref.astype(np.int32))
