@@ -1,0 +1,166 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized decode hot path on one MI355X.
+
+A step is one pass of the Q4_K decode matvec (batch 1) over the four Llama-3-8B layer shapes
+(4096x4096 q/o, 1024x4096 k/v, 14336x4096 gate/up, 4096x14336 down), activations f32 N(0,1), weights
+random Q4_K super-blocks (f16 d/dmin ~ N(0, 0.02), 6-bit scales/mins, uniform nibbles), all resident in
+HBM before the timed region.  Each shape rotates over enough distinct weight buffers to exceed the
+256 MB last-level cache, so the bytes really come from HBM.
+
+Prints ONE JSON line: whole-path GB/s (algorithmic bytes / device time), the roofline of the dominant
+kernel and the CPU checker timed on the host cores beside it.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]  # (n, k)
+HBM_PEAK_GBS = 8000.0
+ROTATE_BYTES = 640 << 20  # > 2x the 256 MB Infinity Cache
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--m", type=int, default=1, help="activation rows (decode batch)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--e2e", action="store_true", help="also run the 8B-architecture decoder (tok/s) and report it")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (nothing in it uses a second); run with --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    from kalosm_amd import synth
+    from kalosm_amd.fusor import Device, QMatrix, Tensor
+
+    dev = Device.gpu(0)
+    info = dev.info()
+    m = args.m
+    ty = synth.Q4_K
+
+    # ---- resident inputs
+    sets = []
+    for si, (n, k) in enumerate(SHAPES):
+        wbytes = n * (k // 256) * 144
+        copies = max(2, -(-ROTATE_BYTES // wbytes))
+        raw = synth.random_weight(ty, n, k, seed=1000 + si)
+        qs = [QMatrix.from_raw_bytes(dev, (n, k), raw, ty) for _ in range(copies)]
+        x = Tensor.from_slice(dev, synth.random_activation(m, k, seed=2000 + si))
+        y = Tensor(dev, (m, n), "f32")
+        sets.append(dict(n=n, k=k, qs=qs, x=x, y=y, raw=raw, bytes=synth.matvec_bytes(ty, n, k, m)))
+
+    def run_shape(s, launches, offset=0):
+        qs, x, y = s["qs"], s["x"], s["y"]
+        for i in range(launches):
+            x.q_mat_mul(qs[(offset + i) % len(qs)], out=y)
+
+    # ---- warmup, then the timed steps (per shape trains inside one bracketed region)
+    # The K launches of a shape are recorded once and replayed as one submission (the reference submits one
+    # command buffer per resolve); host launch overhead of the Python/ctypes loop stays out of the device time.
+    for s in sets:
+        run_shape(s, args.warmup)
+    dev.sync()
+    graphs = []
+    for s in sets:
+        dev.graph_begin()
+        run_shape(s, args.steps, offset=args.warmup)
+        graphs.append(dev.graph_end())
+    per_shape_ms = []
+    t_wall0 = time.perf_counter()
+    for g in graphs:
+        dev.timer_start()
+        g.launch()
+        per_shape_ms.append(dev.timer_stop())
+    dev.sync()
+    wall_ms = (time.perf_counter() - t_wall0) * 1e3
+    total_ms = float(sum(per_shape_ms))
+    step_bytes = sum(s["bytes"] for s in sets)
+    value = step_bytes * args.steps / (total_ms * 1e-3) / 1e9
+    shapes_out = []
+    for s, ms in zip(sets, per_shape_ms):
+        us = ms * 1e3 / args.steps
+        shapes_out.append({"n": s["n"], "k": s["k"], "us_per_launch": round(us, 3),
+                           "GBps": round(s["bytes"] / (us * 1e-6) / 1e9, 1),
+                           "frac_hbm_peak": round(s["bytes"] / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
+    # dominant kernel: the Q4_K MFMA matvec; its launches are the step's four, so the per-launch average is
+    # (bytes of the four shapes / 4) over (device time / launches).  The device time also contains the small
+    # activation-staging kernel that precedes every matvec, so this understates the kernel itself.
+    launches = args.steps * len(sets)
+    avg_us = total_ms * 1e3 / launches
+    achieved = (step_bytes / len(sets)) / (avg_us * 1e-6) / 1e9
+    out = {
+        "metric": "Q4_K matvec GB/s (% HBM peak); Q4_K_M 8B-arch decode tok/s, batch 1, 1 GPU",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(total_ms / args.steps, 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: Q4_K decode matvec at Llama-3-8B layer shapes "
+                               "(4096x4096, 1024x4096, 14336x4096, 4096x14336), batch %d, one launch each per step" % m,
+                   "batch": m, "weights_rotated_bytes_per_shape": ROTATE_BYTES, "device": info["name"],
+                   "compute_units": info["compute_units"]},
+        "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "shapes": shapes_out,
+        "wall_ms_timed_region": round(wall_ms, 2),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "k_qmv_q4k_mfma", "avg_launch_us": round(avg_us, 3),
+                     "algorithmic_bytes_per_launch": step_bytes // len(sets)},
+    }
+
+    # ---- CPU baseline: the checker's q_mat_mul (a C restatement of fusor-ml/cpu, not the Rust binary),
+    # same shapes and inputs, all host cores, bounded repetitions
+    if not args.no_cpu:
+        from oracle import oracle
+
+        oracle.build()
+        threads = oracle.default_threads()
+        t_budget, reps_done, cpu_s, cpu_bytes = 12.0, 0, 0.0, 0
+        xs = [s["x"].as_slice() for s in sets]
+        for s, x in zip(sets, xs):  # warm
+            oracle.q_mat_mul(ty, x, s["raw"], s["n"], threads=threads)
+        while cpu_s < t_budget and reps_done < 20:
+            t0 = time.perf_counter()
+            for s, x in zip(sets, xs):
+                oracle.q_mat_mul(ty, x, s["raw"], s["n"], threads=threads)
+            cpu_s += time.perf_counter() - t0
+            cpu_bytes += step_bytes
+            reps_done += 1
+        out["cpu_baseline"] = {"value": round(cpu_bytes / cpu_s / 1e9, 3), "unit": "GB/s", "cores": threads,
+                               "kind": "port",
+                               "sample": "%d repetitions of the same four matvecs (same weights and activations), "
+                                         "%d threads with the reference's static column split" % (reps_done, threads)}
+        # parity of the timed configuration against the checker
+        worst = 0.0
+        for s, x in zip(sets, xs):
+            s["x"].q_mat_mul(s["qs"][0], out=s["y"])
+            got = s["y"].as_slice()
+            want = oracle.q_mat_mul(ty, x, s["raw"], s["n"], threads=threads)
+            diff = np.abs(got - want)
+            ok = (diff <= 1e-2) | (diff <= 1e-3 * np.maximum(np.abs(got), np.abs(want)))
+            if not ok.all():
+                print("bench.py: PARITY FAILURE at shape", s["n"], s["k"], "max abs", diff.max(), file=sys.stderr)
+                return 1
+            worst = max(worst, float(diff.max()))
+        out["parity_max_abs_err"] = worst
+
+    if args.e2e:
+        from kalosm_amd import e2e
+        out["e2e"] = e2e.run(dev)
+
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

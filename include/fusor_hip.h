@@ -59,6 +59,7 @@ typedef struct fh_device fh_device;
 typedef struct fh_qmatrix fh_qmatrix;
 typedef struct fh_kvcache fh_kvcache;
 typedef struct fh_llama fh_llama;
+typedef struct fh_graph fh_graph;
 
 const char *fh_last_error(void);
 /* Version string of the library, and the gfx target it was built for. */
@@ -86,6 +87,18 @@ fh_status fh_copy(fh_device *dev, void *dst_dev, const void *src_dev, size_t byt
  * queries, fusor-ml/core/src/compute_graph/resolve/run.rs:483-497). */
 fh_status fh_timer_start(fh_device *dev);
 fh_status fh_timer_stop(fh_device *dev, float *elapsed_ms); /* blocks until the stream reaches it */
+
+/* Record-and-replay of a sequence of operator calls (the reference records a lazy graph and submits one
+ * command buffer per resolve, fusor-ml/core/src/compute_graph/resolve/run.rs).  Between begin and end the
+ * operator calls on `dev` are captured into a hipGraph instead of running; fh_graph_launch replays them.
+ * Every buffer the captured calls touch must stay alive and unchanged in address; run the same calls once
+ * eagerly first so that the library's internal scratch buffers are already sized (a capture that would
+ * have to allocate fails with FH_ERR_INVALID).  Blocking calls (upload, download, sync, free) are not
+ * allowed while capturing. */
+fh_status fh_graph_begin(fh_device *dev);
+fh_status fh_graph_end(fh_device *dev, fh_graph **out);
+fh_status fh_graph_launch(fh_graph *g);
+fh_status fh_graph_free(fh_graph *g);
 
 /* ----------------------------------------------------------------- weights
  * QMatrix::from_raw_bytes(&Device, shape, &[u8], GgmlType), fusor-ml/fusor/src/quantized.rs:183-225.

@@ -47,6 +47,10 @@ SIGNATURES = {
     "fh_copy": [_p, _p, _p, _sz],
     "fh_timer_start": [_p],
     "fh_timer_stop": [_p, C.POINTER(_f32)],
+    "fh_graph_begin": [_p],
+    "fh_graph_end": [_p, _pp],
+    "fh_graph_launch": [_p],
+    "fh_graph_free": [_p],
     "fh_qmatrix_from_gguf_bytes": [_p, _u32, _i64, _i64, _p, _sz, _pp],
     "fh_qmatrix_concat_rows": [_p, _pp, _i32, _pp],
     "fh_qmatrix_free": [_p],

@@ -100,9 +100,20 @@ extern "C" fh_status fh_free(fh_device *dev, void *ptr_dev) {
     return FH_OK;
 }
 
+// A fill kernel rather than hipMemsetAsync, so the call can be recorded into a graph.
+__global__ void k_fill_bytes(uint8_t *p, uint8_t v, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) p[i] = v;
+}
+
 extern "C" fh_status fh_memset(fh_device *dev, void *ptr_dev, int32_t byte, size_t bytes) {
     FH_REQUIRE(dev && ptr_dev, "NULL argument");
-    FH_HIP(hipMemsetAsync(ptr_dev, byte, bytes, dev->stream));
+    if (!bytes) return FH_OK;
+    size_t blocks = (bytes + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    k_fill_bytes<<<dim3((unsigned)blocks), dim3(256), 0, dev->stream>>>((uint8_t *)ptr_dev, (uint8_t)byte, bytes);
+    FH_HIP(hipGetLastError());
     return FH_OK;
 }
 
@@ -145,6 +156,9 @@ extern "C" fh_status fh_timer_stop(fh_device *dev, float *elapsed_ms) {
 
 fh_status fh_dev_scratch(fh_device *dev, void **buf, size_t *cap, size_t need) {
     if (*cap >= need) return FH_OK;
+    if (dev->capturing)
+        FH_FAIL(FH_ERR_INVALID, "a captured call needs %zu bytes of scratch but only %zu are allocated: run the "
+                                "sequence once eagerly before capturing it", need, *cap);
     if (*buf) {
         FH_HIP(hipStreamSynchronize(dev->stream));
         FH_HIP(hipFree(*buf));
@@ -162,9 +176,62 @@ extern "C" fh_status fh_set_option(fh_device *dev, const char *key, int64_t valu
     if (!strcmp(key, "matvec_kernel")) dev->opt_matvec_kernel = value;
     else if (!strcmp(key, "matvec_splitk")) dev->opt_matvec_splitk = value;
     else if (!strcmp(key, "matvec_waves")) dev->opt_matvec_waves = value;
+    else if (!strcmp(key, "matvec_tiles")) dev->opt_matvec_tiles = value;
+    else if (!strcmp(key, "matvec_per")) dev->opt_matvec_per = value;
     else if (!strcmp(key, "attn_splits")) dev->opt_attn_splits = value;
     else if (!strcmp(key, "matmul_kernel")) dev->opt_matmul_kernel = value;
     else FH_FAIL(FH_ERR_INVALID, "unknown option '%s'", key);
+    return FH_OK;
+}
+
+struct fh_graph {
+    fh_device *dev = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+extern "C" fh_status fh_graph_begin(fh_device *dev) {
+    FH_REQUIRE(dev, "dev is NULL");
+    FH_REQUIRE(!dev->capturing, "a capture is already in progress");
+    FH_HIP(hipStreamSynchronize(dev->stream));
+    FH_HIP(hipStreamBeginCapture(dev->stream, hipStreamCaptureModeThreadLocal));
+    dev->capturing = true;
+    return FH_OK;
+}
+
+extern "C" fh_status fh_graph_end(fh_device *dev, fh_graph **out) {
+    FH_REQUIRE(dev && out, "NULL argument");
+    FH_REQUIRE(dev->capturing, "no capture in progress");
+    *out = nullptr;
+    dev->capturing = false;
+    hipGraph_t g = nullptr;
+    FH_HIP(hipStreamEndCapture(dev->stream, &g));
+    hipGraphExec_t ex = nullptr;
+    hipError_t e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(g);
+        FH_FAIL(FH_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    }
+    fh_graph *r = new fh_graph();
+    r->dev = dev;
+    r->graph = g;
+    r->exec = ex;
+    *out = r;
+    return FH_OK;
+}
+
+extern "C" fh_status fh_graph_launch(fh_graph *g) {
+    FH_REQUIRE(g && g->exec, "NULL graph");
+    FH_HIP(hipGraphLaunch(g->exec, g->dev->stream));
+    return FH_OK;
+}
+
+extern "C" fh_status fh_graph_free(fh_graph *g) {
+    if (!g) return FH_OK;
+    (void)hipStreamSynchronize(g->dev->stream);
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    delete g;
     return FH_OK;
 }
 

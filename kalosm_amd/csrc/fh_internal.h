@@ -39,6 +39,7 @@ struct fh_device {
     hipStream_t stream = nullptr;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     int compute_units = 0;
+    bool capturing = false;          // between fh_graph_begin and fh_graph_end
     // activation staging for the MFMA decode kernels (grown on demand)
     void *act_buf = nullptr;
     size_t act_cap = 0;
@@ -49,6 +50,8 @@ struct fh_device {
     int64_t opt_matvec_kernel = 0;   // 0 auto, 1 generic VALU, 2 MFMA
     int64_t opt_matvec_splitk = 0;   // 0 auto, else forced split count
     int64_t opt_matvec_waves = 0;    // 0 auto
+    int64_t opt_matvec_tiles = 0;    // 0 auto, else 1 / 2 / 4 row tiles per workgroup
+    int64_t opt_matvec_per = 0;      // 0 auto, else 1 / 2 / 4 blocks per wavefront
     int64_t opt_attn_splits = 0;     // 0 auto
     int64_t opt_matmul_kernel = 0;   // 0 auto, 1 generic
 };
@@ -132,6 +135,7 @@ fh_status fh_launch_qmatvec(const fh_qmatrix *q, const float *x, int m, float *y
                             const float *a, const float *b);
 fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y);
 enum { FH_EPI_NONE = 0, FH_EPI_ADD2 = 1, FH_EPI_SWIGLU = 2 };
+fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b);
 
 struct fh_kvcache {
     fh_device *dev = nullptr;

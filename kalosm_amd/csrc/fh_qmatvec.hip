@@ -73,254 +73,280 @@ static fh_status launch_generic(const fh_qmatrix *q, const float *x, int m, floa
     return FH_OK;
 }
 
-// ------------------------------------------------------------------------------ activation staging
-// x [m, k] f32 -> operand image for the MFMA kernels whose step covers 32 consecutive k:
-//   xp   halfs, index (((s*4 + g)*nc + col)*8 + h): step s = k/32, g = (k%32)/8, col = 2*row + part
-//        (part 0 = hi, 1 = lo), h = slot of k%8 under the byte order [0,2,1,3,4,6,5,7] that the
-//        nibble masks 0x000F000F / (>>8) produce.
-//   sx   f32 [m, k/32]: sum of the ORIGINAL x over each 32 (the min / centre terms)
-//   fs   f32 [m, ceil(k/256)]: 2^(24 - e) where 2^e is the power of two that normalised the
-//        256-group to [2^14, 2^15) before the split (undoes both it and the 2^-24 of the codes)
-// One wavefront per (row, 256-group); lane owns 4 consecutive k.
-__global__ __launch_bounds__(256) void k_act_prep32(const float *__restrict__ x, int m, int k, int nc,
-                                                     _Float16 *__restrict__ xp, float *__restrict__ sx,
-                                                     float *__restrict__ fs) {
-    int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    int k256 = (k + 255) >> 8;
-    int64_t gid = (int64_t)blockIdx.x * 4 + wave;
-    if (gid >= (int64_t)m * k256) return;
-    int row = (int)(gid / k256), b = (int)(gid % k256);
-    int k0 = b * 256 + lane * 4;
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (k0 < k) v = *(const float4 *)(x + (int64_t)row * k + k0); // k % 32 == 0, so a lane is all in or all out
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
-    int e = 0;
-    if (amax > 0.f && amax < INFINITY) {
-        int ex;
-        (void)frexpf(amax, &ex); // amax = f * 2^ex, f in [0.5, 1)  ->  floor(log2) = ex - 1
-        e = 14 - (ex - 1);
-        e = e > 100 ? 100 : (e < -100 ? -100 : e);
-    }
-    float sc = ldexpf(1.0f, e);
-    float xs[4] = {v.x * sc, v.y * sc, v.z * sc, v.w * sc};
-    _Float16 hi[4], lo[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        hi[i] = (_Float16)xs[i];
-        lo[i] = (_Float16)(xs[i] - (float)hi[i]);
-    }
-    if (k0 < k) {
-        int s = k0 >> 5, g = (k0 & 31) >> 3, half = (k0 & 7) >> 2; // half: slots 0..3 or 4..7
-        int64_t base = (((int64_t)s * 4 + g) * nc + 2 * row) * 8 + half * 4;
-        _Float16 oh[4] = {hi[0], hi[2], hi[1], hi[3]};
-        _Float16 ol[4] = {lo[0], lo[2], lo[1], lo[3]};
-        uint2 ph, pl;
-        __builtin_memcpy(&ph, oh, 8);
-        __builtin_memcpy(&pl, ol, 8);
-        *(uint2 *)(xp + base) = ph;     // column 2*row     (hi)
-        *(uint2 *)(xp + base + 8) = pl; // column 2*row + 1 (lo)
-    }
-    float s4 = (v.x + v.y) + (v.z + v.w);
-    s4 += __shfl_xor(s4, 1, 64);
-    s4 += __shfl_xor(s4, 2, 64);
-    s4 += __shfl_xor(s4, 4, 64);
-    if ((lane & 7) == 0 && k0 < k) sx[(int64_t)row * (k >> 5) + (k0 >> 5)] = s4;
-    if (lane == 0) fs[(int64_t)row * k256 + b] = ldexpf(1.0f, 24 - e);
-}
-
 // ------------------------------------------------------------------------------ Q4_K MFMA
-// Workgroup = S wavefronts on one 16-row tile (two tiles with the SwiGLU epilogue); wavefront w
-// takes blocks [w*per, (w+1)*per).  Lane l: j = l & 15 is its weight row inside the tile (B operand
-// column, and the accumulator column), g = l >> 4 its k-group inside a 32-step.
-// NC = staged activation columns = 2 * rows (hi, lo per row), NC in {2, 4}.
-template <int NC, int EPI>
-__global__ __launch_bounds__(1024) void k_qmv_q4k_mfma(QView q, const uint4 *__restrict__ xp,
-                                                        const float *__restrict__ sx, const float *__restrict__ fs,
-                                                        float *__restrict__ y, const float *__restrict__ ea,
-                                                        const float *__restrict__ eb, int S) {
-    constexpr int M = NC / 2;
-    extern __shared__ uint4 lds[];
-    const int kb = (int)q.kb, k32 = kb * 8;
-    uint4 *l_xp = lds;                              // k32 * 4 * NC
-    float *l_sx = (float *)(lds + k32 * 4 * NC);    // M * k32
-    float *l_fs = l_sx + M * k32;                   // M * kb
-    float *l_red = l_fs + M * kb;                   // S * 2 * M * 16
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, g = lane >> 4;
-    for (int i = tid; i < k32 * 4 * NC; i += blockDim.x) l_xp[i] = xp[i];
-    for (int i = tid; i < M * k32; i += blockDim.x) l_sx[i] = sx[i];
-    for (int i = tid; i < M * kb; i += blockDim.x) l_fs[i] = fs[i];
-    __syncthreads();
+// Work split: a workgroup owns T tiles of 16 weight rows (2T with the SwiGLU epilogue: T gate tiles and
+// the T matching up tiles); its S wavefronts split k, wavefront w taking blocks [w*per, (w+1)*per) one
+// 256-block per round.  Lane l: j = l & 15 is its weight row inside a tile (B operand column and
+// accumulator column), g = l >> 4 its k-group inside a 32-wide MFMA step.
+//
+// Per round a wavefront
+//   1. has the T x 2304 B of the NEXT round already in flight (register double buffer),
+//   2. stages its 256 activations per row: each 32-group is normalised by a power of two to
+//      [2^14, 2^15), split exactly into f16 hi + lo, and written to wavefront-private LDS in operand
+//      order (step s = k/32, g = (k%32)/8, slots in the byte order [0,2,1,3,4,6,5,7] that the nibble
+//      masks produce); the group sums of the original x and the factors 2^(24-e) go beside them,
+//   3. runs 8 MFMA steps per tile (one per sub-block) and applies d * sc_j * 2^(24-e_j) in f32.
+// M = activation rows (1 or 2); operand columns are (hi, lo) per row.
+struct Q4KRegs {
+    uint4 h, qa, qb;
+};
 
-    const int per = (kb + S - 1) / S;
-    const int b0 = wave * per, b1 = min(kb, b0 + per);
+template <int M, int T, int EPI>
+__global__ __launch_bounds__((T * (EPI == FH_EPI_SWIGLU ? 2 : 1)) >= 2 ? 512 : 1024) void k_qmv_q4k_mfma(QView q, const float *__restrict__ x, float *__restrict__ y,
+                                                        const float *__restrict__ ea, const float *__restrict__ eb,
+                                                        int S, int per) {
+    constexpr int NC = 2 * M;
     constexpr int NT = EPI == FH_EPI_SWIGLU ? 2 : 1;
-    const int64_t tiles_out = (EPI == FH_EPI_SWIGLU ? q.n / 2 : q.n + 15) / 16; // exact /16 for SwiGLU (host checks)
+    constexpr int TT = T * NT;
+    constexpr int WLDS = 32 * NC + 4 * M; // uint4 per wavefront: operand image + (sums, factors)
+    extern __shared__ uint4 lds[];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, g = lane >> 4;
+    uint4 *w_xp = lds + wave * WLDS;
+    float *w_sf = (float *)(w_xp + 32 * NC); // [m][0..7] group sums, [m][8..15] factors
+    float *l_red = (float *)(lds + S * WLDS); // [S][TT][M][16]
+    const int kb = (int)q.kb, K = (int)q.k;
+    const int b0 = wave * per;
+    const int nb = min(per, kb - b0); // <= 0 for surplus wavefronts
+    const int64_t nout = EPI == FH_EPI_SWIGLU ? q.n / 2 : q.n;
+    const int64_t tiles_out = (nout + 15) / 16;
+
+    const uint8_t *tb[TT];
+    bool tv[TT];
+#pragma unroll
+    for (int t = 0; t < TT; t++) {
+        const int64_t to = (int64_t)blockIdx.x * T + (t % T);
+        tv[t] = to < tiles_out;
+        const int64_t tile = to + (int64_t)(t / T) * (nout / 16); // up tiles follow the gate tiles (n % 32 == 0)
+        tb[t] = q.data + (tile * q.recs + b0) * 2304;
+    }
+    Q4KRegs cur[TT], nxt[TT];
+    float4 xc[M], xn[M];
+    auto loadw = [&](Q4KRegs *w, int r) {
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            if (tv[t]) {
+                const uint8_t *rec = tb[t] + (int64_t)r * 2304;
+                w[t].h = *(const uint4 *)(rec + 16 * j);
+                w[t].qa = *(const uint4 *)(rec + 256 + lane * 16);
+                w[t].qb = *(const uint4 *)(rec + 1280 + lane * 16);
+            } else {
+                w[t].h = w[t].qa = w[t].qb = make_uint4(0, 0, 0, 0);
+            }
+        }
+    };
+    auto loadx = [&](float4 *xv, int r) {
+#pragma unroll
+        for (int i = 0; i < M; i++) xv[i] = *(const float4 *)(x + (int64_t)i * K + (int64_t)(b0 + r) * 256 + lane * 4);
+    };
+    float acc[TT][NC], mins[TT][M];
+#pragma unroll
+    for (int t = 0; t < TT; t++) {
+#pragma unroll
+        for (int i = 0; i < NC; i++) acc[t][i] = 0.f;
+#pragma unroll
+        for (int i = 0; i < M; i++) mins[t][i] = 0.f;
+    }
+    if (nb > 0) {
+        loadw(cur, 0);
+        loadx(xc, 0);
+    }
     const uint32_t LO = 0x000F000Fu, HI = 0x00F000F0u;
-    float outv[NT][M];
+    for (int r = 0; r < nb; r++) {
+        if (r + 1 < nb) {
+            loadw(nxt, r + 1);
+            loadx(xn, r + 1);
+        }
+        // ---- stage the activations of this block (lane owns k = 4*lane .. 4*lane+3)
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-        const int64_t tile = (int64_t)blockIdx.x + (int64_t)t * tiles_out;
-        const uint8_t *rec = q.data + (tile * q.recs + b0) * 2304;
-        floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-        float mins[M];
+        for (int i = 0; i < M; i++) {
+            const float4 v = xc[i];
+            float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+            amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+            amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+            amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+            int e = 0;
+            if (amax > 0.f && amax < INFINITY) {
+                int ex;
+                (void)frexpf(amax, &ex); // amax = f * 2^ex, f in [0.5, 1)
+                e = 15 - ex;
+                e = e > 100 ? 100 : (e < -100 ? -100 : e);
+            }
+            const float sc = ldexpf(1.0f, e);
+            const float xs[4] = {v.x * sc, v.y * sc, v.z * sc, v.w * sc};
+            _Float16 hi[4], lo[4];
 #pragma unroll
-        for (int i = 0; i < M; i++) mins[i] = 0.f;
-        for (int b = b0; b < b1; b++, rec += 2304) {
-            const uint4 h = *(const uint4 *)(rec + 16 * j);
-            const uint4 qa = *(const uint4 *)(rec + 256 + lane * 16);
-            const uint4 qb = *(const uint4 *)(rec + 1280 + lane * 16);
+            for (int c = 0; c < 4; c++) {
+                hi[c] = (_Float16)xs[c];
+                lo[c] = (_Float16)(xs[c] - (float)hi[c]);
+            }
+            const _Float16 oh[4] = {hi[0], hi[2], hi[1], hi[3]}, ol[4] = {lo[0], lo[2], lo[1], lo[3]};
+            uint2 ph, pl;
+            __builtin_memcpy(&ph, oh, 8);
+            __builtin_memcpy(&pl, ol, 8);
+            const int s = lane >> 3, gg = (lane >> 1) & 3, half = lane & 1;
+            uint2 *dst = (uint2 *)(w_xp + (s * 4 + gg) * NC + 2 * i);
+            dst[half] = ph;     // column 2i   (hi)
+            dst[2 + half] = pl; // column 2i+1 (lo)
+            float s4 = (v.x + v.y) + (v.z + v.w);
+            s4 += __shfl_xor(s4, 1, 64);
+            s4 += __shfl_xor(s4, 2, 64);
+            s4 += __shfl_xor(s4, 4, 64);
+            if ((lane & 7) == 0) {
+                w_sf[i * 16 + s] = s4;
+                w_sf[i * 16 + 8 + s] = ldexpf(1.0f, 24 - e);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        // ---- operands shared by the T tiles
+        half8 av[8];
+#pragma unroll
+        for (int st = 0; st < 8; st++) {
+            uint4 ao = make_uint4(0, 0, 0, 0);
+            if (j < NC) ao = w_xp[(st * 4 + g) * NC + j];
+            __builtin_memcpy(&av[st], &ao, 16);
+        }
+        float fac[M][8], sxa[M], sxb[M];
+#pragma unroll
+        for (int i = 0; i < M; i++) {
+            const float4 f0 = *(const float4 *)(w_sf + i * 16 + 8), f1 = *(const float4 *)(w_sf + i * 16 + 12);
+            fac[i][0] = f0.x; fac[i][1] = f0.y; fac[i][2] = f0.z; fac[i][3] = f0.w;
+            fac[i][4] = f1.x; fac[i][5] = f1.y; fac[i][6] = f1.z; fac[i][7] = f1.w;
+            const float2 s2 = *(const float2 *)(w_sf + i * 16 + 2 * g);
+            sxa[i] = s2.x;
+            sxb[i] = s2.y;
+        }
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            const uint4 h = cur[t].h;
             const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
             const float d16 = d * 0.0625f;
             const uint32_t sc_lo = h.y & 0x3F3F3F3Fu, mn_lo = h.z & 0x3F3F3F3Fu;
             const uint32_t sc_hi = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
             const uint32_t mn_hi = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
-            floatx4 accb = {0.f, 0.f, 0.f, 0.f};
-            const uint4 *xs = l_xp + ((b * 8) * 4 + g) * NC + j; // + step * 4 * NC
 #pragma unroll
             for (int p = 0; p < 2; p++) {
-                const uint4 w = p ? qb : qa;
+                const uint4 w = p ? cur[t].qb : cur[t].qa;
                 const uint32_t scw = p ? sc_hi : sc_lo;
 #pragma unroll
-                for (int u = 0; u < 2; u++) { // u = 0: dwords x,y (chunk 2p)   u = 1: dwords z,w (chunk 2p+1)
+                for (int u = 0; u < 2; u++) { // dwords x,y = chunk 2p; dwords z,w = chunk 2p+1
                     const uint32_t w0 = u ? w.z : w.x, w1 = u ? w.w : w.y;
                     const uint32_t w0s = w0 >> 8, w1s = w1 >> 8;
 #pragma unroll
-                    for (int hn = 0; hn < 2; hn++) { // low nibbles (sub-block 4p+2u), high nibbles (4p+2u+1)
+                    for (int hn = 0; hn < 2; hn++) { // low nibbles = sub-block 4p+2u, high nibbles = 4p+2u+1 (x16)
                         const uint32_t msk = hn ? HI : LO;
-                        uint4 bo = make_uint4(w0 & msk, w0s & msk, w1 & msk, w1s & msk);
-                        const int jj = 2 * u + hn; // sub-block within the p half
-                        uint4 ao = make_uint4(0, 0, 0, 0);
-                        if (j < NC) ao = xs[(4 * p + jj) * 4 * NC];
-                        half8 av, bv;
-                        __builtin_memcpy(&av, &ao, 16);
+                        const uint4 bo = make_uint4(w0 & msk, w0s & msk, w1 & msk, w1s & msk);
+                        half8 bv;
                         __builtin_memcpy(&bv, &bo, 16);
-                        floatx4 z = {0.f, 0.f, 0.f, 0.f};
-                        floatx4 dd = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, z, 0, 0, 0);
+                        const int jj = 2 * u + hn, sb = 4 * p + jj;
+                        const floatx4 z = {0.f, 0.f, 0.f, 0.f};
+                        const floatx4 dd = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[sb], bv, z, 0, 0, 0);
                         const float scf = (float)((scw >> (8 * jj)) & 0xFFu) * (hn ? d16 : d);
-                        accb[0] = fmaf(dd[0], scf, accb[0]);
-                        accb[1] = fmaf(dd[1], scf, accb[1]);
-                        if (NC > 2) {
-                            accb[2] = fmaf(dd[2], scf, accb[2]);
-                            accb[3] = fmaf(dd[3], scf, accb[3]);
+#pragma unroll
+                        for (int i = 0; i < M; i++) {
+                            const float tm = scf * fac[i][sb];
+                            acc[t][2 * i] = fmaf(dd[2 * i], tm, acc[t][2 * i]);
+                            acc[t][2 * i + 1] = fmaf(dd[2 * i + 1], tm, acc[t][2 * i + 1]);
                         }
                     }
                 }
             }
-            // undo the block normalisation (and the 2^-24 of the codes); only g == 0 lanes carry data
-#pragma unroll
-            for (int r = 0; r < NC; r++) acc[r] = fmaf(accb[r], l_fs[(r >> 1) * kb + b], acc[r]);
             // min term: lane group g covers sub-blocks 2g, 2g+1
             const uint32_t mw = (g & 2) ? mn_hi : mn_lo;
             const int sh = (g & 1) * 16;
             const float ma = (float)((mw >> sh) & 0xFFu) * dmin, mb = (float)((mw >> (sh + 8)) & 0xFFu) * dmin;
 #pragma unroll
             for (int i = 0; i < M; i++) {
-                const float2 s2 = *(const float2 *)(l_sx + i * k32 + b * 8 + 2 * g);
-                mins[i] = fmaf(ma, s2.x, mins[i]);
-                mins[i] = fmaf(mb, s2.y, mins[i]);
+                mins[t][i] = fmaf(ma, sxa[i], mins[t][i]);
+                mins[t][i] = fmaf(mb, sxb[i], mins[t][i]);
             }
         }
 #pragma unroll
+        for (int t = 0; t < TT; t++) cur[t] = nxt[t];
+#pragma unroll
+        for (int i = 0; i < M; i++) xc[i] = xn[i];
+    }
+    // ---- reduce over the k ranges of the S wavefronts
+#pragma unroll
+    for (int t = 0; t < TT; t++)
+#pragma unroll
         for (int i = 0; i < M; i++) {
-            float mt = mins[i];
+            float mt = mins[t][i];
             mt += __shfl_xor(mt, 16, 64);
             mt += __shfl_xor(mt, 32, 64);
-            outv[t][i] = (acc[2 * i] + acc[2 * i + 1]) - mt; // meaningful in lanes 0..15 (g == 0)
+            const float v = (acc[t][2 * i] + acc[t][2 * i + 1]) - mt; // meaningful in lanes 0..15
+            if (lane < 16) l_red[((wave * TT + t) * M + i) * 16 + lane] = v;
         }
-    }
-    // cross-wavefront reduction over the k ranges
-    if (lane < 16) {
-#pragma unroll
-        for (int t = 0; t < NT; t++)
-#pragma unroll
-            for (int i = 0; i < M; i++) l_red[((wave * NT + t) * M + i) * 16 + lane] = outv[t][i];
-    }
     __syncthreads();
-    if (tid < 16 * M) {
-        const int i = tid >> 4, jr = tid & 15;
-        float v[NT];
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            float s = 0.f;
-            for (int w = 0; w < S; w++) s += l_red[((w * NT + t) * M + i) * 16 + jr];
-            v[t] = s;
+    if (tid < T * M * 16) {
+        const int t = tid / (M * 16), i = (tid / 16) % M, jr = tid & 15;
+        float v0 = 0.f, v1 = 0.f;
+        for (int w = 0; w < S; w++) {
+            v0 += l_red[((w * TT + t) * M + i) * 16 + jr];
+            if (NT == 2) v1 += l_red[((w * TT + t + T) * M + i) * 16 + jr];
         }
-        const int64_t nout = EPI == FH_EPI_SWIGLU ? q.n / 2 : q.n;
-        const int64_t row = (int64_t)blockIdx.x * 16 + jr;
+        const int64_t row = ((int64_t)blockIdx.x * T + t) * 16 + jr;
         if (row < nout) {
             const int64_t o = (int64_t)i * nout + row;
-            float r = v[0];
+            float r = v0;
             if (EPI == FH_EPI_ADD2) r = (r + ea[o]) + eb[o];
-            if (EPI == FH_EPI_SWIGLU) r = (r / (__expf(-r) + 1.0f)) * v[NT - 1];
+            if (EPI == FH_EPI_SWIGLU) r = (r / (__expf(-r) + 1.0f)) * v1;
             y[o] = r;
         }
     }
 }
 
-static size_t q4k_lds_bytes(int64_t kb, int nc, int S, int nt) {
-    int m = nc / 2;
-    return (size_t)kb * 8 * 4 * nc * 16 + (size_t)m * kb * 8 * 4 + (size_t)m * kb * 4 + (size_t)S * nt * m * 16 * 4;
+template <int M, int T>
+static fh_status launch_q4k_t(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b,
+                              int S, int per, unsigned grid, size_t lds) {
+    hipStream_t st = q->dev->stream;
+    QView v = fh_view(q);
+#define FH_Q4K_LAUNCH(EPI_)                                                                                     \
+    do {                                                                                                        \
+        static bool attr_done = false;                                                                          \
+        if (!attr_done) {                                                                                       \
+            FH_HIP(hipFuncSetAttribute((const void *)k_qmv_q4k_mfma<M, T, EPI_>,                                \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));                \
+            attr_done = true;                                                                                   \
+        }                                                                                                       \
+        k_qmv_q4k_mfma<M, T, EPI_><<<dim3(grid), dim3(64 * S), lds, st>>>(v, x, y, a, b, S, per);                \
+    } while (0)
+    if (epi == FH_EPI_NONE) FH_Q4K_LAUNCH(FH_EPI_NONE);
+    else if (epi == FH_EPI_ADD2) FH_Q4K_LAUNCH(FH_EPI_ADD2);
+    else FH_Q4K_LAUNCH(FH_EPI_SWIGLU);
+#undef FH_Q4K_LAUNCH
+    FH_HIP(hipGetLastError());
+    return FH_OK;
 }
 
 static fh_status launch_q4k_mfma(const fh_qmatrix *q, const float *x, int m, float *y, int epi, const float *a,
                                  const float *b) {
     fh_device *dev = q->dev;
-    const int nc = 2 * m;
-    const int64_t k = q->k, kb = q->kb;
+    const int64_t kb = q->kb;
     const int64_t nout = epi == FH_EPI_SWIGLU ? q->n / 2 : q->n;
     const int nt = epi == FH_EPI_SWIGLU ? 2 : 1;
     const int64_t tiles = (nout + 15) / 16;
-    // staging buffer: xp | sx | fs
-    size_t xp_bytes = (size_t)(k / 32) * 4 * nc * 16, sx_bytes = (size_t)m * (k / 32) * 4, fs_bytes = (size_t)m * kb * 4;
-    size_t sx_off = (xp_bytes + 255) & ~(size_t)255, fs_off = (sx_off + sx_bytes + 255) & ~(size_t)255;
-    FH_TRY(fh_dev_scratch(dev, &dev->act_buf, &dev->act_cap, fs_off + fs_bytes + 256));
-    uint8_t *ab = (uint8_t *)dev->act_buf;
-    {
-        int64_t waves = (int64_t)m * kb;
-        k_act_prep32<<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, dev->stream>>>(
-            x, m, (int)k, nc, (_Float16 *)ab, (float *)(ab + sx_off), (float *)(ab + fs_off));
-        FH_HIP(hipGetLastError());
-    }
-    // wavefronts per tile: enough to put ~12 wavefronts on each CU, at least one block each
-    int S = dev->opt_matvec_waves > 0 ? (int)dev->opt_matvec_waves : 0;
-    if (!S) {
-        int64_t want = ((int64_t)dev->compute_units * 12 + tiles - 1) / tiles;
-        S = (int)(want < 1 ? 1 : want);
-        if (S > 16) S = 16;
-        if (nt == 2 && S > 8) S = 8;
-    }
+    int T = (int)dev->opt_matvec_tiles;
+    if (T != 1 && T != 2 && T != 4) T = tiles >= 1024 ? 4 : (tiles >= 512 ? 2 : 1);
+    if (nt == 2 && T == 4) T = 2; // at most 4 tile streams per wavefront
+    const int smax = T * nt >= 2 ? 8 : 16; // the multi-tile variants keep two register sets of T tiles
+    int S = dev->opt_matvec_waves > 0 ? (int)dev->opt_matvec_waves : smax;
+    if (S > smax) S = smax;
     if (S > kb) S = (int)kb;
-    if (S > 16) S = 16;
-    size_t lds = q4k_lds_bytes(kb, nc, S, nt);
-    if (lds > 160 * 1024) return FH_ERR_UNSUPPORTED; // caller falls back
-    dim3 grid((unsigned)tiles), block(64 * S);
-    QView v = fh_view(q);
-    const uint4 *xp = (const uint4 *)ab;
-    const float *sx = (const float *)(ab + sx_off), *fs = (const float *)(ab + fs_off);
-#define FH_Q4K_LAUNCH(NC_, EPI_)                                                                              \
-    do {                                                                                                      \
-        static bool attr_done = false;                                                                        \
-        if (!attr_done) {                                                                                     \
-            FH_HIP(hipFuncSetAttribute((const void *)k_qmv_q4k_mfma<NC_, EPI_>,                               \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));              \
-            attr_done = true;                                                                                 \
-        }                                                                                                     \
-        k_qmv_q4k_mfma<NC_, EPI_><<<grid, block, lds, dev->stream>>>(v, xp, sx, fs, y, a, b, S);              \
-    } while (0)
-    if (nc == 2) {
-        if (epi == FH_EPI_NONE) FH_Q4K_LAUNCH(2, FH_EPI_NONE);
-        else if (epi == FH_EPI_ADD2) FH_Q4K_LAUNCH(2, FH_EPI_ADD2);
-        else FH_Q4K_LAUNCH(2, FH_EPI_SWIGLU);
-    } else {
-        if (epi == FH_EPI_NONE) FH_Q4K_LAUNCH(4, FH_EPI_NONE);
-        else if (epi == FH_EPI_ADD2) FH_Q4K_LAUNCH(4, FH_EPI_ADD2);
-        else FH_Q4K_LAUNCH(4, FH_EPI_SWIGLU);
+    const int per = (int)((kb + S - 1) / S);
+    S = (int)((kb + per - 1) / per);
+    const int nc = 2 * m;
+    size_t lds = (size_t)S * (32 * nc + 4 * m) * 16 + (size_t)S * T * nt * m * 16 * 4;
+    if (lds > 160 * 1024) return FH_ERR_UNSUPPORTED;
+    unsigned grid = (unsigned)((tiles + T - 1) / T);
+    if (m == 1) {
+        if (T == 1) return launch_q4k_t<1, 1>(q, x, y, epi, a, b, S, per, grid, lds);
+        if (T == 2) return launch_q4k_t<1, 2>(q, x, y, epi, a, b, S, per, grid, lds);
+        return launch_q4k_t<1, 4>(q, x, y, epi, a, b, S, per, grid, lds);
     }
-#undef FH_Q4K_LAUNCH
-    FH_HIP(hipGetLastError());
-    return FH_OK;
+    if (T == 1) return launch_q4k_t<2, 1>(q, x, y, epi, a, b, S, per, grid, lds);
+    if (T == 2) return launch_q4k_t<2, 2>(q, x, y, epi, a, b, S, per, grid, lds);
+    return launch_q4k_t<2, 4>(q, x, y, epi, a, b, S, per, grid, lds);
 }
 
 // ------------------------------------------------------------------------------ dispatch
@@ -329,6 +355,10 @@ fh_status fh_launch_qmatvec(const fh_qmatrix *q, const float *x, int m, float *y
     fh_device *dev = q->dev;
     if (epi == FH_EPI_SWIGLU) FH_REQUIRE(q->n % 32 == 0, "SwiGLU epilogue needs n %% 32 == 0 (n = %lld)", (long long)q->n);
     int kernel = (int)dev->opt_matvec_kernel;
+    if (kernel != 1 && kernel != 3 && q->type == FH_Q4_K && m == 1) {
+        fh_status st = fh_launch_q4k_m1(q, x, y, epi, a, b);
+        if (st != FH_ERR_UNSUPPORTED) return st;
+    }
     if (kernel != 1 && q->type == FH_Q4_K && m <= 2) {
         fh_status st = launch_q4k_mfma(q, x, m, y, epi, a, b);
         if (st != FH_ERR_UNSUPPORTED) return st;

@@ -1,0 +1,251 @@
+// Q4_K decode matvec for ONE activation row (the batch-1 token loop): y[n] = sum_k x[k] * deq(W)[n, k].
+// Reference: fusor-ml/cpu/src/quantized.rs:246-675 (semantics); the factorised form
+//   y = d * sum_j sc_j * (q . x)_j  -  dmin * sum_j m_j * (sum x)_j      (j = 32-element sub-block)
+// is the one the reference's own GPU kernel uses (fusor-ml/tile-ir-kernels/src/kernels/qgemv_q4k_ggml.rs:64-158).
+//
+// Mapping onto v_mfma_f32_16x16x32_f16.  B operand: 16 weight rows x 32 k of one sub-block; the 4-bit
+// codes become f16 SUBNORMAL integers (code * 2^-24, or code * 16 * 2^-24 for the high nibbles) with one
+// AND per two codes.  A operand: 16 rows x 32 k where row (2*s + part) holds the hi (part 0) or lo (part 1)
+// half of the exact two-term f16 split of the normalised activations of sub-block s and is ZERO for the
+// other sub-blocks.  Chaining the 8 steps of a 256-block through the accumulator therefore leaves
+// D[2s + part][row] = (q . x_part)_s for all eight sub-blocks at once: lane (row j, group g) holds the four
+// values of sub-blocks 2g and 2g+1 of its own row and applies that row's d * sc_s * 2^(24-e_s) itself.
+//
+// Workgroup = TS tile streams (TW row tiles; twice that with the SwiGLU epilogue: gate tiles and the matching
+// up tiles) x SW k-slices of PER blocks; wavefront = (stream, slice).  All PER x 2304 B of a wavefront are
+// requested before anything else; meanwhile the workgroup stages x for the whole k once (block b by wavefront
+// b mod waves): each 32-group is normalised by a power of two to [2^14, 2^15) (odd groups 16x lower, which
+// folds the x16 of the high nibbles), split into f16 hi + lo and stored in operand order, with the group sums
+// of the original x and the factors beside them.
+#include "fh_blocks.h"
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+struct Q4KRegs {
+    uint4 h, qa, qb;
+};
+
+// Cross-lane moves inside a row of 16 lanes as DPP modifiers (one VALU op, no LDS round trip).
+#define DPP_XOR1 0xB1        // quad_perm [1,0,3,2]
+#define DPP_XOR2 0x4E        // quad_perm [2,3,0,1]
+#define DPP_HALF_MIRROR 0x141 // lane i <- lane 7-i within each group of 8
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
+#define Q4K_IMG 65 // uint4 per block image: 8 steps x 4 groups x (hi, lo) + one all-zero slot
+
+template <int TS, int PER, int EPI>
+__global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__restrict__ x, float *__restrict__ y,
+                                                      const float *__restrict__ ea, const float *__restrict__ eb,
+                                                      int SW) {
+    constexpr int NT = EPI == FH_EPI_SWIGLU ? 2 : 1;
+    constexpr int TW = TS / NT;
+    constexpr int XB = (PER + TS - 1) / TS; // blocks of x each wavefront stages: kb / (TS * SW) with SW * PER == kb
+    extern __shared__ uint4 lds[];
+    const int kb = (int)q.kb;
+    uint4 *img = lds;
+    float *sf = (float *)(lds + kb * Q4K_IMG); // per block: [0..7] group sums, [8..15] factors
+    float *l_red = sf + kb * 16;               // [TS][SW][16]
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, g = lane >> 4;
+    const int nwaves = TS * SW;
+    const int stream = wave / SW, slice = wave - stream * SW;
+    const int64_t nout = EPI == FH_EPI_SWIGLU ? q.n / 2 : q.n;
+    const int64_t tiles_out = (nout + 15) / 16;
+    const int64_t to = (int64_t)blockIdx.x * TW + (stream % TW);
+    const bool tvalid = to < tiles_out;
+    const int64_t tile = to + (int64_t)(stream / TW) * (nout / 16); // up tiles follow the gate tiles
+    const int b0 = slice * PER;
+
+    // ---- 0. the activations this wavefront stages (blocks wave, wave + nwaves, ...) are requested first:
+    // they are needed first and are short
+    float4 xv[XB];
+#pragma unroll
+    for (int i = 0; i < XB; i++) {
+        const int b = wave + i * nwaves;
+        xv[i] = *(const float4 *)(x + (int64_t)(b < kb ? b : 0) * 256 + lane * 4);
+    }
+    // ---- 1. every weight byte of this wavefront goes in flight.  A tile past the end re-reads the last
+    // tile (its rows are never stored); the host guarantees SW * PER == kb, so no block is out of range.
+    Q4KRegs w[PER];
+    {
+        const int64_t tl = tvalid ? tile : tile - (to - (tiles_out - 1));
+        const uint8_t *rec = q.data + (tl * q.recs + b0) * 2304;
+        const uint8_t *ph = rec + 16 * j, *pq = rec + 256 + lane * 16;
+#pragma unroll
+        for (int r = 0; r < PER; r++) {
+            w[r].h = *(const uint4 *)(ph + r * 2304);
+            w[r].qa = *(const uint4 *)(pq + r * 2304);
+            w[r].qb = *(const uint4 *)(pq + r * 2304 + 1024);
+        }
+    }
+    // ---- 2. stage x (lane owns k = 256*b + 4*lane .. +3)
+#pragma unroll
+    for (int i = 0; i < XB; i++) {
+        const int b = wave + i * nwaves;
+        if (b >= kb) break;
+        const float4 v = xv[i];
+        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        amax = fmaxf(amax, dpp_f32<DPP_XOR1>(amax));
+        amax = fmaxf(amax, dpp_f32<DPP_XOR2>(amax));
+        amax = fmaxf(amax, dpp_f32<DPP_HALF_MIRROR>(amax)); // quads are uniform now: lane 7-i is in the other quad
+        const int s = lane >> 3, gg = (lane >> 1) & 3, half = lane & 1;
+        // e = 14 - floor(log2(amax)) from the exponent field (zero / subnormal / inf / nan just clamp)
+        int e = 141 - (int)((__float_as_uint(amax) >> 23) & 0xFFu);
+        e = e > 100 ? 100 : (e < -100 ? -100 : e);
+        const int eo = e - 4 * (s & 1); // odd sub-blocks meet codes scaled by 16
+        const float sc = __uint_as_float((uint32_t)(eo + 127) << 23);
+        const float xs[4] = {v.x * sc, v.y * sc, v.z * sc, v.w * sc};
+        _Float16 hi[4], lo[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            hi[c] = (_Float16)xs[c];
+            lo[c] = (_Float16)(xs[c] - (float)hi[c]);
+        }
+        const _Float16 oh[4] = {hi[0], hi[2], hi[1], hi[3]}, ol[4] = {lo[0], lo[2], lo[1], lo[3]};
+        uint2 ph, pl;
+        __builtin_memcpy(&ph, oh, 8);
+        __builtin_memcpy(&pl, ol, 8);
+        uint2 *dst = (uint2 *)(img + b * Q4K_IMG + (s * 4 + gg) * 2);
+        dst[half] = ph;     // hi
+        dst[2 + half] = pl; // lo
+        if (lane == 0) img[b * Q4K_IMG + 64] = make_uint4(0, 0, 0, 0);
+        float s4 = (v.x + v.y) + (v.z + v.w);
+        s4 += dpp_f32<DPP_XOR1>(s4);
+        s4 += dpp_f32<DPP_XOR2>(s4);
+        s4 += dpp_f32<DPP_HALF_MIRROR>(s4);
+        if ((lane & 7) == 0) {
+            sf[b * 16 + s] = s4;
+            sf[b * 16 + 8 + s] = __uint_as_float((uint32_t)(24 - e + 127) << 23);
+        }
+    }
+    __syncthreads();
+    // ---- 3. eight chained MFMA steps per block
+    const int mysb = j >> 1, part = j & 1;
+    const uint4 *pa[8]; // per-lane operand address of each step: its own sub-block's (hi|lo) or the zero slot
+#pragma unroll
+    for (int st = 0; st < 8; st++) pa[st] = img + b0 * Q4K_IMG + (st == mysb ? (st * 4 + g) * 2 + part : 64);
+    const float *psf = sf + b0 * 16 + 2 * g;
+    const uint32_t LO = 0x000F000Fu, HI = 0x00F000F0u;
+    // lane group g applies sub-blocks 2g, 2g+1: bytes (g&1)*2, +1 of the low (g < 2) or high (g >= 2) scale word
+    const uint32_t selhi = (g & 2) ? 0xFFFFFFFFu : 0u;
+    const int sh = (g & 1) * 16;
+    float acc = 0.f, mins = 0.f;
+#pragma unroll
+    for (int r = 0; r < PER; r++) {
+        floatx4 dd = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int st = 0; st < 8; st++) {
+            const uint4 wq = (st & 4) ? w[r].qb : w[r].qa;
+            const uint32_t w0 = (st & 2) ? wq.z : wq.x, w1 = (st & 2) ? wq.w : wq.y;
+            const uint32_t msk = (st & 1) ? HI : LO;
+            const uint4 bo = make_uint4(w0 & msk, (w0 >> 8) & msk, w1 & msk, (w1 >> 8) & msk);
+            const uint4 ao = pa[st][r * Q4K_IMG];
+            half8 av, bv;
+            __builtin_memcpy(&av, &ao, 16);
+            __builtin_memcpy(&bv, &bo, 16);
+            dd = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, dd, 0, 0, 0);
+        }
+        const uint4 h = w[r].h;
+        const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
+        const uint32_t sc_l = h.y & 0x3F3F3F3Fu, sc_h = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
+        const uint32_t mn_l = h.z & 0x3F3F3F3Fu, mn_h = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
+        const uint32_t scw = ((sc_l & ~selhi) | (sc_h & selhi)) >> sh;
+        const uint32_t mnw = ((mn_l & ~selhi) | (mn_h & selhi)) >> sh;
+        const float sca = (float)(scw & 0xFFu), scb = (float)((scw >> 8) & 0xFFu);
+        const float mna = (float)(mnw & 0xFFu), mnb = (float)((mnw >> 8) & 0xFFu);
+        const float2 sx = *(const float2 *)(psf + r * 16);
+        const float2 fc = *(const float2 *)(psf + r * 16 + 8);
+        const float sa = (sca * d) * fc.x, sb = (scb * d) * fc.y;
+        acc = fmaf(dd[0] + dd[1], sa, acc);
+        acc = fmaf(dd[2] + dd[3], sb, acc);
+        mins = fmaf(mna * dmin, sx.x, mins);
+        mins = fmaf(mnb * dmin, sx.y, mins);
+    }
+    float v = acc - mins;
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    if (lane < 16) l_red[(stream * SW + slice) * 16 + lane] = v;
+    __syncthreads();
+    if (tid < TW * 16) {
+        const int t = tid >> 4, jr = tid & 15;
+        float v0 = 0.f, v1 = 0.f;
+        for (int s = 0; s < SW; s++) {
+            v0 += l_red[(t * SW + s) * 16 + jr];
+            if (NT == 2) v1 += l_red[((t + TW) * SW + s) * 16 + jr];
+        }
+        const int64_t row = ((int64_t)blockIdx.x * TW + t) * 16 + jr;
+        if (row < nout) {
+            float rr = v0;
+            if (EPI == FH_EPI_ADD2) rr = (rr + ea[row]) + eb[row];
+            if (EPI == FH_EPI_SWIGLU) rr = (rr / (__expf(-rr) + 1.0f)) * v1;
+            y[row] = rr;
+        }
+    }
+}
+
+template <int TS, int PER, int EPI>
+static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b, int SW,
+                               unsigned grid, size_t lds) {
+    static bool attr_done = false;
+    if (!attr_done) {
+        FH_HIP(hipFuncSetAttribute((const void *)k_qmv_q4k_m1<TS, PER, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024));
+        attr_done = true;
+    }
+    k_qmv_q4k_m1<TS, PER, EPI><<<dim3(grid), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+template <int TS, int EPI>
+static fh_status q4k_m1_per(int per, const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b,
+                            int SW, unsigned grid, size_t lds) {
+    if (per == 1) return q4k_m1_launch<TS, 1, EPI>(q, x, y, a, b, SW, grid, lds);
+    if (per == 2) return q4k_m1_launch<TS, 2, EPI>(q, x, y, a, b, SW, grid, lds);
+    return q4k_m1_launch<TS, 4, EPI>(q, x, y, a, b, SW, grid, lds);
+}
+
+// Returns FH_ERR_UNSUPPORTED when the shape does not fit this kernel (the caller falls back).
+fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b) {
+    fh_device *dev = q->dev;
+    const int kb = (int)q->kb;
+    const int nt = epi == FH_EPI_SWIGLU ? 2 : 1;
+    const int64_t nout = epi == FH_EPI_SWIGLU ? q->n / 2 : q->n;
+    const int64_t tiles = (nout + 15) / 16;
+    // blocks per wavefront (all requested up front); 2 measured best for the large shapes, 1 for the small ones
+    int per = (int)dev->opt_matvec_per;
+    if (per != 1 && per != 2 && per != 4) per = tiles >= 512 ? 2 : (kb > 16 ? 2 : 1); // measured best on MI355X
+    while (per > 1 && kb % per) per /= 2; // the kernel wants SW * PER == kb
+    int SW = kb / per;
+    while (SW > 16 && per < 4 && kb % (per * 2) == 0) {
+        per *= 2;
+        SW = kb / per;
+    }
+    if (SW > 16) return FH_ERR_UNSUPPORTED;
+    // row tiles per workgroup share one staging of x
+    int TW = (int)dev->opt_matvec_tiles;
+    if (TW != 1 && TW != 2 && TW != 4) TW = tiles >= 512 ? 2 : 1;
+    while (TW > 1 && TW * nt * SW > 16) TW /= 2;
+    const int TS = TW * nt;
+    if (TS * SW > 16 || (TS != 1 && TS != 2 && TS != 4)) return FH_ERR_UNSUPPORTED;
+    size_t lds = (size_t)kb * Q4K_IMG * 16 + (size_t)kb * 64 + (size_t)TS * SW * 64;
+    if (lds > 160 * 1024) return FH_ERR_UNSUPPORTED;
+    unsigned grid = (unsigned)((tiles + TW - 1) / TW);
+#define Q4K_M1_GO(TS_, EPI_) return q4k_m1_per<TS_, EPI_>(per, q, x, y, a, b, SW, grid, lds)
+    if (epi == FH_EPI_SWIGLU) {
+        if (TS == 2) Q4K_M1_GO(2, FH_EPI_SWIGLU);
+        Q4K_M1_GO(4, FH_EPI_SWIGLU);
+    }
+    if (epi == FH_EPI_ADD2) {
+        if (TS == 1) Q4K_M1_GO(1, FH_EPI_ADD2);
+        if (TS == 2) Q4K_M1_GO(2, FH_EPI_ADD2);
+        Q4K_M1_GO(4, FH_EPI_ADD2);
+    }
+    if (TS == 1) Q4K_M1_GO(1, FH_EPI_NONE);
+    if (TS == 2) Q4K_M1_GO(2, FH_EPI_NONE);
+    Q4K_M1_GO(4, FH_EPI_NONE);
+#undef Q4K_M1_GO
+}

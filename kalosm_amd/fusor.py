@@ -71,6 +71,15 @@ class Device:
         check(self._lib.fh_timer_stop(self._h, C.byref(ms)))
         return ms.value
 
+    # -- record / replay (the reference's lazy graph + single submit)
+    def graph_begin(self) -> None:
+        check(self._lib.fh_graph_begin(self._h))
+
+    def graph_end(self) -> "Graph":
+        h = C.c_void_p()
+        check(self._lib.fh_graph_end(self._h, C.byref(h)))
+        return Graph(self, h)
+
     # -- memory
     def alloc(self, nbytes: int) -> int:
         p = C.c_void_p()
@@ -84,6 +93,21 @@ class Device:
         if self._h is not None:
             self._lib.fh_device_destroy(self._h)
             self._h = None
+
+
+class Graph:
+    def __init__(self, device: Device, handle):
+        self.device, self._h = device, handle
+
+    def launch(self) -> None:
+        check(self.device._lib.fh_graph_launch(self._h))
+
+    def __del__(self):
+        try:
+            if self._h and self.device._h is not None:
+                self.device._lib.fh_graph_free(self._h)
+        except Exception:
+            pass
 
 
 class Tensor:
