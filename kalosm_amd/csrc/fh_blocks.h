@@ -20,16 +20,27 @@ __device__ __host__ __forceinline__ int q4k_qs_off(int j, int i) { // i: byte 0.
     int p = i >> 6, w = i & 63, c2 = w >> 5, o = w & 31, g = o >> 3, r = o & 7;
     return 256 + p * 1024 + (g * 16 + j) * 16 + c2 * 8 + r;
 }
-// Q6_K: record 3360 B
-__device__ __host__ __forceinline__ int q6k_ql_off(int j, int i) { // i: 0..127
-    int p = i >> 6, o = i & 63, g = o >> 4, r = o & 15;
-    return p * 1024 + (g * 16 + j) * 16 + r;
+// Q6_K: record 3360 B.  Element e (0..255, dequantised order) of row j: step t = e/32, lane group
+// g = (e/8)%4, value v = e%8 of lane (g*16 + j).  The 6-bit code is stored as a low nibble in an L word
+// (one per lane and step) and two high bits in an H word (one per lane and step pair), placed so that
+// the f16 operand pair (v = 2p, v = 2p+1) of MFMA operand dword p comes out of one shift+AND each:
+//   L word  = byte offset (t/4)*1024 + (g*16+j)*16 + (t%4)*4; nibble p + 4*(v%2)
+//   H word  = byte offset 2048 + (g*16+j)*16 + (t/2)*4; bit position q6k_hbit(t, p) + 16*(v%2)
+//   scales  = byte 3072 + ((G%8)/2*16 + j)*4 + 2*(G/8) + (G%2) for 16-element group G = e/16
+//   d       = byte 3328 + 2*j
+__device__ __host__ __forceinline__ int q6k_lword_off(int j, int t, int g) {
+    return (t >> 2) * 1024 + (g * 16 + j) * 16 + (t & 3) * 4;
 }
-__device__ __host__ __forceinline__ int q6k_qh_off(int j, int i) { // i: 0..63
-    int p = i >> 5, o = i & 31, g = o >> 3, r = o & 7;
-    return 2048 + p * 512 + (g * 16 + j) * 8 + r;
+__device__ __host__ __forceinline__ int q6k_hword_off(int j, int t, int g) {
+    return 2048 + (g * 16 + j) * 16 + (t >> 1) * 4;
 }
-__device__ __host__ __forceinline__ int q6k_sc_off(int j, int i) { return 3072 + 16 * j + i; }
+__device__ __host__ __forceinline__ int q6k_hbit(int t, int p) {
+    // even step of the pair: (H >> 2p) & 0x00300030;  odd step: (H << 4), (H << 2), (H >> 8), (H >> 10)
+    return (t & 1) ? (p < 2 ? 2 * p : 8 + 2 * p) : 4 + 2 * p;
+}
+__device__ __host__ __forceinline__ int q6k_sc_off(int j, int G) {
+    return 3072 + (((G & 7) >> 1) * 16 + j) * 4 + 2 * (G >> 3) + (G & 1);
+}
 __device__ __host__ __forceinline__ int q6k_d_off(int j) { return 3328 + 2 * j; }
 // Q8_0: record 1088 B = two blocks
 __device__ __host__ __forceinline__ int q80_q_off(int j, int u, int i) { // u: block in record, i: 0..31
@@ -102,12 +113,13 @@ __device__ __forceinline__ float deq_elem_q6_k(const QView &q, int64_t row, int6
     int e = (int)(k & 255);
     const uint8_t *rec = q.data + ((row >> 4) * q.recs + b) * (int64_t)q.rec_bytes;
     int j = (int)(row & 15);
-    int n = e >> 7, jj = (e >> 5) & 3, l = e & 31;
-    uint8_t lo = rec[q6k_ql_off(j, 64 * n + l + ((jj & 1) ? 32 : 0))];
-    uint8_t hi = rec[q6k_qh_off(j, 32 * n + l)];
-    int nib = (jj & 2) ? (lo >> 4) : (lo & 0x0F);
-    int v = (int)(int8_t)((((hi >> (2 * jj)) & 3) << 4) | nib) - 32;
-    int sc = (int)(int8_t)rec[q6k_sc_off(j, 8 * n + 2 * jj + (l >> 4))];
+    int t = e >> 5, g = (e >> 3) & 3, vv = e & 7, p = vv >> 1, odd = vv & 1;
+    uint32_t lw = *(const uint32_t *)(rec + q6k_lword_off(j, t, g));
+    uint32_t hw = *(const uint32_t *)(rec + q6k_hword_off(j, t, g));
+    int nib = (int)((lw >> (4 * (p + 4 * odd))) & 15u);
+    int hb = (int)((hw >> (q6k_hbit(t, p) + 16 * odd)) & 3u);
+    int v = ((hb << 4) | nib) - 32;
+    int sc = (int)(int8_t)rec[q6k_sc_off(j, e >> 4)];
     float d = fh_h2f(fh_ld16(rec + q6k_d_off(j)));
     float ds = d * (float)sc;
     return ds * (float)v;

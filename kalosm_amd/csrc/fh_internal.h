@@ -72,9 +72,12 @@ fh_status fh_dev_scratch(fh_device *dev, void **buf, size_t *cap, size_t need);
 //   [256,2304)   quants: for p in {0,1}, lane l = g*16 + j (g in 0..3):
 //                16 B at 256 + p*1024 + l*16 = qs_j[64p + 8g .. +8] ++ qs_j[64p + 32 + 8g .. +8]
 // FH_Q6_K (record = one 256-block of 16 rows, 3360 B)
-//   [0,2048)     ql: for p in {0,1}, lane l = g*16 + j: 16 B at p*1024 + l*16 = ql_j[64p + 16g .. +16]
-//   [2048,3072)  qh: for p in {0,1}, lane l: 8 B at 2048 + p*512 + l*8 = qh_j[32p + 8g .. +8]
-//   [3072,3328)  scales: row j at 3072 + 16*j (16 x i8)
+//   element e of row j belongs to MFMA step t = e/32, lane l = ((e/8)%4)*16 + j, value v = e%8
+//   [0,2048)     low nibbles: lane l holds 16 B at (t/4)*1024 + l*16, one 32-bit word per step t%4; value v
+//                sits in nibble v/2 + 4*(v%2), so (word >> 4p) & 0x000F000F is the f16 pair (v=2p, v=2p+1)
+//   [2048,3072)  high 2 bits: lane l holds 16 B at 2048 + l*16, one word per step PAIR; bit positions chosen
+//                so that one shift and one AND with 0x00300030 drop them onto bits 4-5 of the same pair
+//   [3072,3328)  scales: lane l holds 4 x i8 at 3072 + l*4: groups 2g, 2g+1 of each half block (g = l/16)
 //   [3328,3360)  d: row j at 3328 + 2*j (f16)
 // FH_Q8_0 (record = two 32-blocks of 16 rows, 1088 B; kb padded to even with zero blocks)
 //   [0,1024)     quants: lane l = g*16 + j: 16 B at l*16 = q_j[blk 2r][8g .. +8] ++ q_j[blk 2r+1][8g .. +8]
@@ -136,6 +139,7 @@ fh_status fh_launch_qmatvec(const fh_qmatrix *q, const float *x, int m, float *y
 fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y);
 enum { FH_EPI_NONE = 0, FH_EPI_ADD2 = 1, FH_EPI_SWIGLU = 2 };
 fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b);
+fh_status fh_launch_q6k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b);
 
 struct fh_kvcache {
     fh_device *dev = nullptr;

@@ -25,9 +25,27 @@ __global__ void k_repack_q6_k(const uint8_t *__restrict__ src, uint8_t *__restri
     const uint8_t *s = src + idx * 210;
     uint8_t *rec = dst + ((row >> 4) * recs + b) * 3360;
     int j = (int)(row & 15);
-    for (int i = 0; i < 128; i++) rec[q6k_ql_off(j, i)] = s[i];
-    for (int i = 0; i < 64; i++) rec[q6k_qh_off(j, i)] = s[128 + i];
-    for (int i = 0; i < 16; i++) rec[q6k_sc_off(j, i)] = s[192 + i];
+    // 6-bit codes in dequantised element order (fusor-ml/gguf/src/lib.rs:2034-2085), then re-packed
+    for (int t = 0; t < 8; t++)
+        for (int g = 0; g < 4; g++) {
+            uint32_t lw = 0, hbits = 0;
+            for (int vv = 0; vv < 8; vv++) {
+                int e = 32 * t + 8 * g + vv;
+                int n = e >> 7, jj = (e >> 5) & 3, l = e & 31;
+                uint8_t lo = s[64 * n + l + ((jj & 1) ? 32 : 0)];
+                uint8_t hi = s[128 + 32 * n + l];
+                uint32_t nib = (jj & 2) ? (lo >> 4) : (lo & 0x0F);
+                uint32_t hb = (hi >> (2 * jj)) & 3u;
+                int p = vv >> 1, odd = vv & 1;
+                lw |= nib << (4 * (p + 4 * odd));
+                hbits |= hb << (q6k_hbit(t, p) + 16 * odd);
+            }
+            *(uint32_t *)(rec + q6k_lword_off(j, t, g)) = lw;
+            uint32_t *hw = (uint32_t *)(rec + q6k_hword_off(j, t, g));
+            if (t & 1) *hw |= hbits; // steps 2u and 2u+1 share a word; this thread owns the whole word
+            else *hw = hbits;
+        }
+    for (int G = 0; G < 16; G++) rec[q6k_sc_off(j, G)] = s[192 + G];
     rec[q6k_d_off(j)] = s[208];
     rec[q6k_d_off(j) + 1] = s[209];
 }

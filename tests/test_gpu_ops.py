@@ -1,0 +1,237 @@
+"""GPU parity of the row / pointwise operators, attention and the KV cache against the CPU checker."""
+import numpy as np
+import pytest
+
+import refgen
+from refgen import assert_close
+from kalosm_amd.fusor import Device, FusorHipError, KvCache, MaskKind, RopeCache, Tensor
+
+pytestmark = pytest.mark.gpu
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+# ----------------------------------------------------------------------------- rms_norm
+@pytest.mark.parametrize("shape", [(1, 4096), (3, 17, 257), (2, 16, 255), (5, 64)])
+@pytest.mark.parametrize("residual", [False, True])
+def test_rms_norm(dev, oracle, shape, residual):
+    """conformance normalization_ops.rs:45-80: weights 1 + (i % 5) * 0.25, eps 1e-5, tol 1e-4; fuzz shapes
+    [2..3, 16..17, 255..257]."""
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal(shape).astype(np.float32)
+    r = rng.standard_normal(shape).astype(np.float32) if residual else None
+    w = (1 + (np.arange(shape[-1]) % 5) * 0.25).astype(np.float32)
+    xt, wt = Tensor.from_slice(dev, x), Tensor.from_slice(dev, w)
+    got = (xt.rms_norm_residual_fused(Tensor.from_slice(dev, r), wt, None, 1e-5) if residual
+           else xt.rms_norm_fused(wt, None, 1e-5)).as_slice()
+    want = oracle.rms_norm(x, w, 1e-5, residual=r)
+    assert_close(got, want, abs_tol=1e-4, rel_tol=1e-4, what="rms_norm")
+    # the formula of the reference's host check (conformance common/mod.rs:426-449) in float64
+    t = (x + r if residual else x).astype(np.float64)
+    ref = t / np.sqrt((t * t).mean(-1, keepdims=True) + 1e-5) * w
+    assert_close(got, ref, abs_tol=1e-4, rel_tol=1e-4, what="rms_norm vs float64 formula")
+
+
+def test_rms_norm_bias(dev, oracle):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((4, 300)).astype(np.float32)
+    w = rng.standard_normal(300).astype(np.float32)
+    b = rng.standard_normal(300).astype(np.float32)
+    got = Tensor.from_slice(dev, x).rms_norm_fused(Tensor.from_slice(dev, w), Tensor.from_slice(dev, b), 1e-6).as_slice()
+    assert_close(got, oracle.rms_norm(x, w, 1e-6, bias=b), abs_tol=1e-4, rel_tol=1e-4, what="rms_norm + bias")
+
+
+# ----------------------------------------------------------------------------- rope
+def test_rope_tables_golden(dev, oracle):
+    """models/kalosm-llama/src/raw/rope.rs:295-310: head_dim 2, theta 5000, 6 positions."""
+    rc = RopeCache.new(2, 6, 5000.0, dev)
+    cos, sin = rc.cos.as_slice().reshape(-1), rc.sin.as_slice().reshape(-1)
+    assert np.abs(cos - np.float32([1.0000, 0.5403, -0.4161, -0.9900, -0.6536, 0.2837])).max() < 1e-4
+    assert np.abs(sin - np.float32([0.0000, 0.8415, 0.9093, 0.1411, -0.7568, -0.9589])).max() < 1e-4
+    oc, os_ = oracle.rope_tables(128, 512, 500000.0)
+    rc = RopeCache.new(128, 512, 500000.0, dev)
+    assert np.array_equal(bits(rc.cos.as_slice()), bits(oc)) and np.array_equal(bits(rc.sin.as_slice()), bits(os_))
+
+
+@pytest.mark.parametrize("interleaved", [True, False])
+@pytest.mark.parametrize("start_pos", [0, 5])
+def test_rope_pair(dev, oracle, interleaved, start_pos):
+    """conformance rope_ops.rs: both pairings, a start position, and q arriving as the transposed view
+    [b, s, h, d] -> [b, h, s, d] (attention_layer.rs:371-374)."""
+    b, hq, hk, s, d = 2, 8, 2, 7, 64
+    rng = np.random.default_rng(start_pos + 10 * interleaved)
+    q_bshd = rng.standard_normal((b, s, hq, d)).astype(np.float32)
+    k_bshd = rng.standard_normal((b, s, hk, d)).astype(np.float32)
+    cos, sin = oracle.rope_tables(d, 32, 10000.0)
+    rc = RopeCache.from_parts(Tensor.from_slice(dev, cos), Tensor.from_slice(dev, sin))
+    qt = Tensor.from_slice(dev, q_bshd).reshape((b, hq, s, d))   # logical shape; physical layout is [b, s, h, d]
+    kt = Tensor.from_slice(dev, k_bshd).reshape((b, hk, s, d))
+    fn = rc.forward_interleaved if interleaved else rc.forward
+    qo, ko = fn(qt, kt, start_pos, q_strides=(s * hq * d, d, hq * d), k_strides=(s * hk * d, d, hk * d))
+    wq = oracle.rope(q_bshd.transpose(0, 2, 1, 3), cos, sin, start_pos, interleaved)
+    wk = oracle.rope(k_bshd.transpose(0, 2, 1, 3), cos, sin, start_pos, interleaved)
+    assert np.array_equal(bits(qo.as_slice()), bits(wq)) and np.array_equal(bits(ko.as_slice()), bits(wk))
+    with pytest.raises(FusorHipError):
+        fn(qt, kt, 30)  # positions beyond the table
+
+
+# ----------------------------------------------------------------------------- pointwise
+def test_swiglu_add_argmax_casts(dev, oracle):
+    rng = np.random.default_rng(5)
+    g = (rng.standard_normal(5000) * 4).astype(np.float32)
+    u = rng.standard_normal(5000).astype(np.float32)
+    got = Tensor.from_slice(dev, g).silu_mul(Tensor.from_slice(dev, u)).as_slice()
+    assert_close(got, oracle.swiglu(g, u), abs_tol=1e-6, rel_tol=1e-6, what="silu*up")
+    a, b, c = (rng.standard_normal(777).astype(np.float32) for _ in range(3))
+    got = Tensor.from_slice(dev, a).add(Tensor.from_slice(dev, b), Tensor.from_slice(dev, c)).as_slice()
+    assert np.array_equal(bits(got), bits(oracle.add3(a, b, c)))
+    x = rng.standard_normal((6, 5, 8)).astype(np.float32)
+    assert np.array_equal(Tensor.from_slice(dev, x).transpose_shd().as_slice(), x.transpose(1, 0, 2))
+    h = Tensor.from_slice(dev, g).cast("f16").as_slice()
+    assert np.array_equal(h.view(np.uint16), g.astype(np.float16).view(np.uint16))
+    from kalosm_amd import synth
+    bf = Tensor.from_slice(dev, g).cast("bf16").as_slice()
+    assert np.array_equal(bf, synth.to_bf16_bits(g))
+    # greedy pick: ties go to the larger id, non-finite values are skipped (fusor/src/lib.rs:416-447)
+    v = rng.standard_normal(128256).astype(np.float32)
+    assert Tensor.from_slice(dev, v).top_k_pairs_1() == oracle.argmax(v) == int(np.argmax(v))
+    v[[7, 70000, 128255]] = v.max() + 1
+    assert Tensor.from_slice(dev, v).top_k_pairs_1() == oracle.argmax(v) == 128255
+    v[128255] = np.inf
+    v[3] = np.nan
+    assert Tensor.from_slice(dev, v).top_k_pairs_1() == oracle.argmax(v) == 70000
+    assert Tensor.from_slice(dev, np.full(100, np.nan, np.float32)).top_k_pairs_1() == oracle.argmax(np.full(100, np.nan)) == -1
+
+
+# ----------------------------------------------------------------------------- attention
+def run_attn(dev, q, k, v, scale, mask=None, dtype="f32"):
+    cast = (lambda a: a.astype(np.float16)) if dtype == "f16" else (lambda a: a)
+    qt, kt, vt = (Tensor.from_slice(dev, cast(a), dtype) for a in (q, k, v))
+    return qt.flash_attention(kt, vt, scale, mask).as_slice().astype(np.float32)
+
+
+@pytest.mark.parametrize("L", [129, 192, 256, 257, 384, 511, 512, 569, 1025])
+def test_attention_decode_tile_boundaries(dev, oracle, L):
+    """conformance flash_attention_ops.rs:310-343: H=16, H_kv=2, d=128, one query, KV lengths around the tile
+    sizes, each run 4 times (races show as run-to-run differences)."""
+    h, hkv, d = 16, 2, 128
+    q = refgen.attn_pattern(h * d, 0.1).reshape(1, h, 1, d)
+    k = refgen.attn_pattern(hkv * L * d, -0.15).reshape(1, hkv, L, d)
+    v = refgen.attn_pattern(hkv * L * d, 0.35).reshape(1, hkv, L, d)
+    want = oracle.flash_attention(q, k, v, 1 / np.sqrt(d))
+    first = None
+    for _ in range(4):
+        got = run_attn(dev, q, k, v, 1 / np.sqrt(d))
+        assert_close(got, want, abs_tol=1e-4, rel_tol=1e-4, what=f"decode L={L}")
+        first = got if first is None else first
+        assert np.array_equal(got, first)
+
+
+@pytest.mark.parametrize("sq,skv,d", [(64, 64, 8), (72, 80, 16), (65, 35, 8), (128, 128, 24), (96, 100, 64), (5, 3000, 128)])
+@pytest.mark.parametrize("kind", ["none", "causal", "additive"])
+def test_attention_prefill_shapes(dev, oracle, sq, skv, d, kind):
+    """core/tests/attention.rs:152-325 and flash_attention_ops.rs:761-828: sin inputs, GQA, causal (with a
+    KV longer or shorter than the queries), additive mask i % 7 == 0 ? -1.5 : 0.25, long-KV streaming."""
+    if kind == "causal" and skv < sq:
+        pytest.skip("a causal mask with fewer keys than queries leaves fully masked rows (NaN in the reference too)")
+    h, hkv = 4, 2
+    q = refgen.attn_sin(h * sq * d, 0.13).reshape(1, h, sq, d)
+    k = refgen.attn_sin(hkv * skv * d, 0.07).reshape(1, hkv, skv, d)
+    v = refgen.attn_sin(hkv * skv * d, 0.11).reshape(1, hkv, skv, d)
+    scale = 1 / np.sqrt(d)
+    mask_np, mask, okind = None, None, oracle.MASK_NONE
+    if kind == "causal":
+        mask, okind = MaskKind.Causal, oracle.MASK_CAUSAL
+    elif kind == "additive":
+        mask_np = np.where(np.arange(sq * skv) % 7 == 0, -1.5, 0.25).astype(np.float32).reshape(sq, skv)
+        mask, okind = (Tensor.from_slice(dev, mask_np), MaskKind.QKMask), oracle.MASK_ADDITIVE
+    got = run_attn(dev, q, k, v, scale, mask)
+    want = oracle.flash_attention(q, k, v, scale, okind, mask_np)
+    assert_close(got, want, abs_tol=1e-4, rel_tol=1e-4, what=f"attention {kind} {sq}x{skv}x{d}")
+    ref = refgen.np_attention(q, k, v, scale, causal=(kind == "causal"), mask=mask_np)
+    assert_close(got, ref, abs_tol=1e-4, rel_tol=1e-4, what="attention vs float64 textbook")
+
+
+def test_attention_invariants(dev, oracle):
+    """rows of P sum to 1 (V = const -> out = const), causal row 0 -> out = v_0, uniform K -> mean(V),
+    GQA == repeated KV heads, all-zero additive mask == no mask (flash_attention_ops.rs:640-647)."""
+    rng = np.random.default_rng(8)
+    h, hkv, s, d = 32, 8, 10, 128
+    q = rng.standard_normal((1, h, s, d)).astype(np.float32)
+    k = rng.standard_normal((1, hkv, s, d)).astype(np.float32)
+    v = rng.standard_normal((1, hkv, s, d)).astype(np.float32)
+    sc = 1 / np.sqrt(d)
+    out = run_attn(dev, q, k, np.full_like(v, 0.75), sc)
+    assert np.abs(out - 0.75).max() < 1e-5
+    out = run_attn(dev, q, k, v, sc, MaskKind.Causal)
+    assert np.abs(out[0, :, 0, :] - np.repeat(v[0, :, 0, :], h // hkv, axis=0)).max() < 1e-6
+    out = run_attn(dev, q, np.ones_like(k), v, sc)
+    assert np.abs(out - np.repeat(v.mean(2, keepdims=True), h // hkv, axis=1)).max() < 1e-5
+    rep = run_attn(dev, q, np.repeat(k, h // hkv, axis=1), np.repeat(v, h // hkv, axis=1), sc)
+    assert_close(run_attn(dev, q, k, v, sc), rep, abs_tol=1e-6, rel_tol=1e-6, what="GQA vs repeated heads")
+    zero = Tensor.zeros(dev, (s, s))
+    assert_close(run_attn(dev, q, k, v, sc, (zero, MaskKind.QKMask)), run_attn(dev, q, k, v, sc), abs_tol=1e-6,
+                 rel_tol=1e-6, what="zero mask")
+    with pytest.raises(FusorHipError, match="divisible"):
+        Tensor.from_slice(dev, q[:, :30]).flash_attention(Tensor.from_slice(dev, k), Tensor.from_slice(dev, v), sc)
+
+
+@pytest.mark.parametrize("L", [200, 1024, 4096])
+def test_attention_f16_decode(dev, oracle, L):
+    """Benchmark configuration 3 (decode): f16 Q/K/V ~ N(0,1), 32 / 8 heads, d = 128.  The checker works in f32 on
+    the f16-rounded inputs; the GPU result is rounded to f16 on output (tolerance 1e-2 as the reference's f16 cases)."""
+    rng = np.random.default_rng(L)
+    h, hkv, d = 32, 8, 128
+    q, k, v = (rng.standard_normal(s).astype(np.float16).astype(np.float32) for s in ((1, h, 1, d), (1, hkv, L, d), (1, hkv, L, d)))
+    got = run_attn(dev, q, k, v, 1 / np.sqrt(d), dtype="f16")
+    want = oracle.flash_attention(q, k, v, 1 / np.sqrt(d))
+    assert_close(got, want, abs_tol=1e-2, rel_tol=1e-3, what=f"f16 decode L={L}")
+
+
+def test_attention_transposed_q(dev, oracle):
+    """flash_attention_ops.rs:354-419: q given as a [b, s, h, d] buffer viewed as [b, h, s, d]."""
+    rng = np.random.default_rng(9)
+    b, h, hkv, s, d = 1, 8, 2, 6, 64
+    q_bshd = rng.standard_normal((b, s, h, d)).astype(np.float32)
+    k = rng.standard_normal((b, hkv, 40, d)).astype(np.float32)
+    v = rng.standard_normal((b, hkv, 40, d)).astype(np.float32)
+    qt = Tensor.from_slice(dev, q_bshd).reshape((b, h, s, d))
+    got = qt.flash_attention(Tensor.from_slice(dev, k), Tensor.from_slice(dev, v), 0.125, MaskKind.Causal,
+                             q_strides=(s * h * d, d, h * d)).as_slice()
+    want = oracle.flash_attention(q_bshd.transpose(0, 2, 1, 3), k, v, 0.125, oracle.MASK_CAUSAL)
+    assert_close(got, want, abs_tol=1e-4, rel_tol=1e-4, what="transposed q")
+
+
+# ----------------------------------------------------------------------------- KV cache
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_kv_cache_growth_append_reset(dev, dtype):
+    """conformance cache_ops.rs:83-268 and tensor_cache.rs:315-338: capacity 256 -> 512 ..., contents preserved
+    across growth, reset, max_len cap and overflow."""
+    layers, hk, d = 2, 2, 64
+    c = KvCache(dev, layers, hk, d, max_len=600, dtype=dtype)
+    rng = np.random.default_rng(11)
+    hist = [[np.zeros((hk, 0, d), np.float32) for _ in range(2)] for _ in range(layers)]
+    expected_caps = []
+    for s in (1, 64, 191, 1, 300):
+        for l in range(layers):
+            k = rng.standard_normal((hk, s, d)).astype(np.float32)
+            v = rng.standard_normal((hk, s, d)).astype(np.float32)
+            c.append(l, Tensor.from_slice(dev, k), Tensor.from_slice(dev, v))
+            hist[l][0] = np.concatenate([hist[l][0], k], 1)
+            hist[l][1] = np.concatenate([hist[l][1], v], 1)
+        ln, cap, kt, vt = c.view(0)
+        expected_caps.append(cap)
+        for l in range(layers):
+            ln, cap, kt, vt = c.view(l)
+            assert ln == hist[l][0].shape[1]
+            want_k = hist[l][0].astype(np.float16).astype(np.float32) if dtype == "f16" else hist[l][0]
+            assert np.array_equal(kt.as_slice()[:, :ln].astype(np.float32), want_k)
+            want_v = hist[l][1].astype(np.float16).astype(np.float32) if dtype == "f16" else hist[l][1]
+            assert np.array_equal(vt.as_slice()[:, :ln].astype(np.float32), want_v)
+    assert expected_caps == [256, 256, 256, 512, 600]  # gpu_allocation_seq_len: pow2, min 256, capped at max_len
+    with pytest.raises(FusorHipError, match="overflow"):
+        c.append(0, Tensor.zeros(dev, (hk, 100, d)), Tensor.zeros(dev, (hk, 100, d)))
+    c.reset()
+    assert c.view(0)[0] == 0
