@@ -267,7 +267,7 @@ static fh_status decode_launch(fh_device *dev, const void *q, int64_t q_sb, int6
                                int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int b, int hq, int hkv, int skv,
                                const int *len_dev, float scale, const float *mask, void *out) {
     // with a device-side length the grid is sized for the capacity, so keep the chunks small
-    int chunk = len_dev ? 64 : pick_chunk(dev, skv, hkv, b);
+    int chunk = len_dev ? 32 : pick_chunk(dev, skv, hkv, b);
     int splits = (skv + chunk - 1) / chunk;
     size_t part_bytes = (size_t)b * hq * splits * (D + 2) * 4;
     FH_TRY(fh_dev_scratch(dev, (void **)&dev->part_buf, &dev->part_cap, part_bytes));

@@ -49,6 +49,7 @@ extern "C" fh_status fh_device_create(int32_t ordinal, fh_device **out) {
     FH_HIP(hipStreamCreate(&d->stream));
     FH_HIP(hipEventCreate(&d->ev_start));
     FH_HIP(hipEventCreate(&d->ev_stop));
+    FH_HIP(hipMalloc(&d->small_buf, 64 * 1024));
     *out = d;
     return FH_OK;
 }
@@ -59,6 +60,7 @@ extern "C" fh_status fh_device_destroy(fh_device *dev) {
     (void)hipStreamSynchronize(dev->stream);
     if (dev->act_buf) (void)hipFree(dev->act_buf);
     if (dev->part_buf) (void)hipFree(dev->part_buf);
+    if (dev->small_buf) (void)hipFree(dev->small_buf);
     (void)hipEventDestroy(dev->ev_start);
     (void)hipEventDestroy(dev->ev_stop);
     (void)hipStreamDestroy(dev->stream);

@@ -45,13 +45,63 @@ __global__ __launch_bounds__(1024) void k_rms_norm(const float *__restrict__ x, 
     }
 }
 
+// Same arithmetic for rows of at most 4096 columns (a multiple of 4): 256 threads keep the row in registers
+// (up to four float4 each), so x and the residual are read once.
+__global__ __launch_bounds__(256) void k_rms_norm_reg(const float *__restrict__ x, const float *__restrict__ res,
+                                                       const float *__restrict__ w, const float *__restrict__ bias,
+                                                       float eps, int cols, float *__restrict__ y) {
+    __shared__ float sh[16];
+    const int64_t off = (int64_t)blockIdx.x * cols;
+    const int n4 = cols >> 2;
+    float4 v[4];
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int c4 = threadIdx.x + i * 256;
+        v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c4 < n4) {
+            v[i] = *(const float4 *)(x + off + 4 * c4);
+            if (res) {
+                const float4 r = *(const float4 *)(res + off + 4 * c4);
+                v[i].x = v[i].x + r.x; v[i].y = v[i].y + r.y; v[i].z = v[i].z + r.z; v[i].w = v[i].w + r.w;
+            }
+            acc = fmaf(v[i].x, v[i].x, acc);
+            acc = fmaf(v[i].y, v[i].y, acc);
+            acc = fmaf(v[i].z, v[i].z, acc);
+            acc = fmaf(v[i].w, v[i].w, acc);
+        }
+    }
+    const float total = block_sum(acc, sh);
+    const float rms = sqrtf(total / (float)cols + eps);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int c4 = threadIdx.x + i * 256;
+        if (c4 < n4) {
+            const float4 ww = *(const float4 *)(w + 4 * c4);
+            float4 o = make_float4((v[i].x / rms) * ww.x, (v[i].y / rms) * ww.y, (v[i].z / rms) * ww.z, (v[i].w / rms) * ww.w);
+            if (bias) {
+                const float4 bb = *(const float4 *)(bias + 4 * c4);
+                o.x = o.x + bb.x; o.y = o.y + bb.y; o.z = o.z + bb.z; o.w = o.w + bb.w;
+            }
+            *(float4 *)(y + off + 4 * c4) = o;
+        }
+    }
+}
+
 extern "C" fh_status fh_rms_norm(fh_device *dev, const float *x_dev, const float *residual_dev, const float *w_dev,
                                  const float *bias_dev, float eps, int32_t rows, int32_t cols, float *y_dev) {
     FH_REQUIRE(dev && x_dev && w_dev && y_dev, "NULL argument");
     FH_REQUIRE(rows > 0 && cols > 0, "empty input [%d, %d]", rows, cols);
-    int threads = cols >= 4096 ? 1024 : (cols >= 1024 ? 256 : 64);
-    k_rms_norm<<<dim3((unsigned)rows), dim3(threads), 0, dev->stream>>>(x_dev, residual_dev, w_dev, bias_dev, eps, cols,
-                                                                       y_dev);
+    const bool aligned = (((uintptr_t)x_dev | (uintptr_t)y_dev | (uintptr_t)w_dev | (uintptr_t)residual_dev |
+                           (uintptr_t)bias_dev) & 15) == 0;
+    if (cols % 4 == 0 && cols <= 4096 && cols >= 256 && aligned) {
+        k_rms_norm_reg<<<dim3((unsigned)rows), dim3(256), 0, dev->stream>>>(x_dev, residual_dev, w_dev, bias_dev, eps,
+                                                                           cols, y_dev);
+    } else {
+        int threads = cols >= 4096 ? 1024 : (cols >= 1024 ? 256 : 64);
+        k_rms_norm<<<dim3((unsigned)rows), dim3(threads), 0, dev->stream>>>(x_dev, residual_dev, w_dev, bias_dev, eps,
+                                                                           cols, y_dev);
+    }
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
@@ -258,14 +308,21 @@ __device__ __forceinline__ void amax_merge(float &v, uint32_t &id, float ov, uin
         id = oid;
     }
 }
-__global__ __launch_bounds__(1024) void k_argmax(const float *__restrict__ x, int64_t n, uint32_t *__restrict__ out) {
+// Stage 1 (pv != NULL): workgroup b scans its slice of x and writes its best (value, id) to pv/pi[b].
+// Stage 2 (pv == NULL in the launch of one workgroup): x is the partial values, xi their ids.
+__global__ __launch_bounds__(1024) void k_argmax(const float *__restrict__ x, const uint32_t *__restrict__ xi, int64_t n,
+                                                  uint32_t *__restrict__ out, float *__restrict__ pv,
+                                                  uint32_t *__restrict__ pi) {
     __shared__ float sv[16];
     __shared__ uint32_t si[16];
     float v = 0.f;
     uint32_t id = 0xFFFFFFFFu;
-    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+    const int64_t per = (n + gridDim.x - 1) / gridDim.x;
+    const int64_t lo = (int64_t)blockIdx.x * per, hi = lo + per < n ? lo + per : n;
+    for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
         float t = x[i];
-        if (isfinite(t)) amax_merge(v, id, t, (uint32_t)i);
+        uint32_t tid_ = xi ? xi[i] : (uint32_t)i;
+        if (isfinite(t) && tid_ != 0xFFFFFFFFu) amax_merge(v, id, t, tid_);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
@@ -281,13 +338,26 @@ __global__ __launch_bounds__(1024) void k_argmax(const float *__restrict__ x, in
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int i = 1; i < (int)(blockDim.x >> 6); i++) amax_merge(v, id, sv[i], si[i]);
-        *out = id;
+        if (pv) {
+            pv[blockIdx.x] = v;
+            pi[blockIdx.x] = id;
+        } else {
+            *out = id;
+        }
     }
 }
 extern "C" fh_status fh_argmax(fh_device *dev, const float *x_dev, int64_t count, uint32_t *id_dev) {
     FH_REQUIRE(dev && x_dev && id_dev, "NULL argument");
     FH_REQUIRE(count > 0 && count < 0xFFFFFFFFll, "count %lld out of range", (long long)count);
-    k_argmax<<<dim3(1), dim3(1024), 0, dev->stream>>>(x_dev, count, id_dev);
+    if (count <= 8192) {
+        k_argmax<<<dim3(1), dim3(1024), 0, dev->stream>>>(x_dev, nullptr, count, id_dev, nullptr, nullptr);
+    } else {
+        const int parts = 128;
+        float *pv = (float *)dev->small_buf;
+        uint32_t *pi = (uint32_t *)(pv + parts);
+        k_argmax<<<dim3(parts), dim3(256), 0, dev->stream>>>(x_dev, nullptr, count, nullptr, pv, pi);
+        k_argmax<<<dim3(1), dim3(128), 0, dev->stream>>>(pv, pi, parts, id_dev, nullptr, nullptr);
+    }
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
@@ -455,6 +525,64 @@ extern "C" fh_status fh_kvcache_append(fh_kvcache *c, int32_t layer, const float
 // Graph-replayed decode step: position read from len_dev; the host mirrors the length afterwards.
 fh_status fh_kvcache_append_devpos(fh_kvcache *c, int layer, const float *k, const float *v, int64_t sh) {
     return kv_append_launch(c, layer, k, sh, 0, v, sh, 0, 1, 0, c->len_dev);
+}
+
+// One-token decode step: interleaved RoPE of q and k at position *pos_dev, the rotated k and the raw v written
+// straight into the cache row (RopeCache::forward_interleaved + KvCache::append in one launch).
+// q, k, v are [heads, d] with head stride d.
+template <typename TO>
+__global__ __launch_bounds__(256) void k_rope_kv_decode(const float *__restrict__ q, const float *__restrict__ k,
+                                                         const float *__restrict__ v, int hq, int hk, int d,
+                                                         const float *__restrict__ cs, const float *__restrict__ sn,
+                                                         int table_rows, const int *__restrict__ pos_dev,
+                                                         float *__restrict__ qo, TO *__restrict__ kc,
+                                                         TO *__restrict__ vc, int cap) {
+    const int half = d >> 1;
+    const int npair = (hq + hk) * half, nv = hk * d;
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= npair + nv) return;
+    int pos = *pos_dev;
+    if (pos >= cap) return; // the host reserves capacity before the step
+    if (idx < npair) {
+        const int i = idx % half, h = idx / half;
+        const int tp = pos < table_rows ? pos : table_rows - 1;
+        const float c = cs[(int64_t)tp * half + i], s = sn[(int64_t)tp * half + i];
+        const bool isk = h >= hq;
+        const float *src = isk ? k + (h - hq) * d : q + h * d;
+        const float x0 = src[2 * i], x1 = src[2 * i + 1];
+        const float ac = x0 * c, bs = x1 * s, as = x0 * s, bc = x1 * c;
+        const float y0 = ac - bs, y1 = as + bc;
+        if (isk) {
+            TO *dst = kc + ((int64_t)(h - hq) * cap + pos) * d;
+            dst[2 * i] = (TO)y0;
+            dst[2 * i + 1] = (TO)y1;
+        } else {
+            qo[h * d + 2 * i] = y0;
+            qo[h * d + 2 * i + 1] = y1;
+        }
+    } else {
+        const int e = idx - npair, h = e / d, c = e % d;
+        vc[((int64_t)h * cap + pos) * d + c] = (TO)v[h * d + c];
+    }
+}
+
+fh_status fh_rope_kv_decode(fh_kvcache *c, int layer, const float *q, const float *k, const float *v, int hq,
+                            const float *cos_t, const float *sin_t, int table_rows, float *q_out) {
+    const int hk = c->kv_heads, d = c->head_dim;
+    const size_t plane = (size_t)hk * c->capacity * d;
+    const int total = (hq + hk) * (d / 2) + hk * d;
+    dim3 grid((unsigned)((total + 255) / 256));
+    hipStream_t s = c->dev->stream;
+    if (c->dtype == FH_F32)
+        k_rope_kv_decode<float><<<grid, 256, 0, s>>>(q, k, v, hq, hk, d, cos_t, sin_t, table_rows, c->len_dev, q_out,
+                                                     (float *)c->k + layer * plane, (float *)c->v + layer * plane,
+                                                     c->capacity);
+    else
+        k_rope_kv_decode<fh_half><<<grid, 256, 0, s>>>(q, k, v, hq, hk, d, cos_t, sin_t, table_rows, c->len_dev, q_out,
+                                                       (fh_half *)c->k + layer * plane, (fh_half *)c->v + layer * plane,
+                                                       c->capacity);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
 }
 
 // End of a graph-replayed decode step: advance the device-side length.

@@ -46,6 +46,8 @@ struct fh_device {
     // split-K partial sums
     float *part_buf = nullptr;
     size_t part_cap = 0;
+    // 64 KB that never moves: partial results of small reductions (argmax)
+    void *small_buf = nullptr;
     // options (fh_set_option)
     int64_t opt_matvec_kernel = 0;   // 0 auto, 1 generic VALU, 2 MFMA
     int64_t opt_matvec_splitk = 0;   // 0 auto, else forced split count
@@ -153,6 +155,8 @@ fh_status fh_kvcache_reserve(fh_kvcache *c, int required);
 // append reading the write position from c->len_dev (graph friendly), s == 1
 fh_status fh_kvcache_append_devpos(fh_kvcache *c, int layer, const float *k, const float *v, int64_t sh);
 fh_status fh_kvcache_advance_dev(fh_kvcache *c);
+fh_status fh_rope_kv_decode(fh_kvcache *c, int layer, const float *q, const float *k, const float *v, int hq,
+                            const float *cos_t, const float *sin_t, int table_rows, float *q_out);
 fh_status fh_kvcache_append_kv(fh_kvcache *c, int layer, const float *k, int64_t k_sh, int64_t k_st, const float *v,
                                int64_t v_sh, int64_t v_st, int s, int pos);
 fh_status fh_kvcache_set_len_dev(fh_kvcache *c, int len);

@@ -255,8 +255,7 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
         }
         const int64_t q_st = row ? row : QD, k_st = row ? row : KD;
         if (dev_pos) {
-            FH_TRY(fh_rope_pair_devpos(dev, qp, kp, H, HK, hd, m->cos_t, m->sin_t, c.ctx, m->cache->len_dev, m->qrot, m->krot));
-            FH_TRY(fh_kvcache_append_devpos(m->cache, li, m->krot, vp, hd));
+            FH_TRY(fh_rope_kv_decode(m->cache, li, qp, kp, vp, H, m->cos_t, m->sin_t, c.ctx, m->qrot));
             size_t plane = (size_t)HK * m->cache->capacity * hd * fh_dtype_size(c.kv_dtype);
             const uint8_t *kc = (const uint8_t *)m->cache->k + li * plane, *vc = (const uint8_t *)m->cache->v + li * plane;
             FH_TRY(fh_attention_decode_devlen(dev, c.kv_dtype, m->qrot, kc, vc, (int64_t)m->cache->capacity * hd, hd, H, HK,

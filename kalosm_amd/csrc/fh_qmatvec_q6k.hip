@@ -221,7 +221,8 @@ fh_status fh_launch_q6k_m1(const fh_qmatrix *q, const float *x, float *y, int ep
     const int64_t nout = epi == FH_EPI_SWIGLU ? q->n / 2 : q->n;
     const int64_t tiles = (nout + 15) / 16;
     int per = (int)dev->opt_matvec_per;
-    if (per != 1 && per != 2 && per != 4) per = tiles >= 512 ? 2 : (kb > 16 ? 2 : 1);
+    // measured on MI355X: vocabulary-sized matrices want 4 blocks per wavefront, layer-sized ones 2
+    if (per != 1 && per != 2 && per != 4) per = tiles >= 4096 ? 4 : (tiles >= 512 ? 2 : (kb > 16 ? 2 : 1));
     while (per > 1 && kb % per) per /= 2; // the kernel wants SW * PER == kb
     int SW = kb / per;
     while (SW > 16 && per < 4 && kb % (per * 2) == 0) {
@@ -230,7 +231,7 @@ fh_status fh_launch_q6k_m1(const fh_qmatrix *q, const float *x, float *y, int ep
     }
     if (SW > 16) return FH_ERR_UNSUPPORTED;
     int TW = (int)dev->opt_matvec_tiles;
-    if (TW != 1 && TW != 2 && TW != 4) TW = tiles >= 512 ? 2 : 1;
+    if (TW != 1 && TW != 2 && TW != 4) TW = (tiles >= 512 && tiles < 4096) ? 2 : 1;
     while (TW > 1 && TW * nt * SW > 16) TW /= 2;
     const int TS = TW * nt;
     if (TS * SW > 16 || (TS != 1 && TS != 2 && TS != 4)) return FH_ERR_UNSUPPORTED;
