@@ -26,6 +26,10 @@ sys.path.insert(0, ROOT)
 SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]  # (n, k)
 HBM_PEAK_GBS = 8000.0
 ROTATE_BYTES = 640 << 20  # > 2x the 256 MB Infinity Cache
+# HBM bytes per launch (average of the four shapes) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this
+# workload at batch 1, scaled by what the same counters read for a 256 MiB device copy (FETCH_SIZE x2.000,
+# WRITE_SIZE x1.000); a measured constant, to be re-measured when the kernel changes.
+TRAFFIC_BYTES_PER_LAUNCH = 19768986
 
 
 def main() -> int:
@@ -36,6 +40,8 @@ def main() -> int:
     ap.add_argument("--m", type=int, default=1, help="activation rows (decode batch)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--e2e", action="store_true", help="also run the 8B-architecture decoder (tok/s) and report it")
+    ap.add_argument("--no-graph", action="store_true", help="launch on the stream instead of replaying a recorded graph")
+    ap.add_argument("--calib-copy", action="store_true", help="append 4 device copies of 256 MiB (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (nothing in it uses a second); run with --gpus 1",
@@ -72,17 +78,30 @@ def main() -> int:
     for s in sets:
         run_shape(s, args.warmup)
     dev.sync()
-    graphs = []
-    for s in sets:
-        dev.graph_begin()
-        run_shape(s, args.steps, offset=args.warmup)
-        graphs.append(dev.graph_end())
     per_shape_ms = []
-    t_wall0 = time.perf_counter()
-    for g in graphs:
-        dev.timer_start()
-        g.launch()
-        per_shape_ms.append(dev.timer_stop())
+    if args.no_graph:  # plain stream launches (for runs under a kernel tracer, which does not follow graph replays)
+        t_wall0 = time.perf_counter()
+        for s in sets:
+            dev.timer_start()
+            run_shape(s, args.steps, offset=args.warmup)
+            per_shape_ms.append(dev.timer_stop())
+    else:
+        graphs = []
+        for s in sets:
+            dev.graph_begin()
+            run_shape(s, args.steps, offset=args.warmup)
+            graphs.append(dev.graph_end())
+        t_wall0 = time.perf_counter()
+        for g in graphs:
+            dev.timer_start()
+            g.launch()
+            per_shape_ms.append(dev.timer_stop())
+    if args.calib_copy:  # a device-to-device copy of known size, to scale the FETCH_SIZE / WRITE_SIZE counters
+        nbytes = 256 << 20
+        a, b = Tensor(dev, (nbytes,), "u8"), Tensor(dev, (nbytes,), "u8")
+        import ctypes as C
+        for _ in range(4):
+            dev._lib.fh_copy(dev._h, C.c_void_p(b.ptr), C.c_void_p(a.ptr), nbytes)
     dev.sync()
     wall_ms = (time.perf_counter() - t_wall0) * 1e3
     total_ms = float(sum(per_shape_ms))
@@ -94,9 +113,9 @@ def main() -> int:
         shapes_out.append({"n": s["n"], "k": s["k"], "us_per_launch": round(us, 3),
                            "GBps": round(s["bytes"] / (us * 1e-6) / 1e9, 1),
                            "frac_hbm_peak": round(s["bytes"] / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
-    # dominant kernel: the Q4_K MFMA matvec; its launches are the step's four, so the per-launch average is
-    # (bytes of the four shapes / 4) over (device time / launches).  The device time also contains the small
-    # activation-staging kernel that precedes every matvec, so this understates the kernel itself.
+    # dominant kernel: the Q4_K MFMA matvec k_qmv_q4k_m1, one launch per matvec (activation staging is inside it);
+    # its launches are the step's four, so the per-launch average is (bytes of the four shapes / 4) over
+    # (device time / launches).  Device time between events includes the dispatch gap between dependent launches.
     launches = args.steps * len(sets)
     avg_us = total_ms * 1e3 / launches
     achieved = (step_bytes / len(sets)) / (avg_us * 1e-6) / 1e9
@@ -113,8 +132,8 @@ def main() -> int:
         "shapes": shapes_out,
         "wall_ms_timed_region": round(wall_ms, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_qmv_q4k_mfma", "avg_launch_us": round(avg_us, 3),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH if m == 1 else None,
+                     "kernel": "k_qmv_q4k_m1", "avg_launch_us": round(avg_us, 3),
                      "algorithmic_bytes_per_launch": step_bytes // len(sets)},
     }
 
