@@ -55,7 +55,7 @@ struct fh_device {
     int64_t opt_matvec_tiles = 0;    // 0 auto, else 1 / 2 / 4 row tiles per workgroup
     int64_t opt_matvec_per = 0;      // 0 auto, else 1 / 2 / 4 blocks per wavefront
     int64_t opt_attn_splits = 0;     // 0 auto
-    int64_t opt_matmul_kernel = 0;   // 0 auto, 1 generic
+    int64_t opt_matmul_kernel = 0;   // 0 auto, 1 generic for every m, 2 MFMA tile kernel for every m
 };
 
 fh_status fh_dev_scratch(fh_device *dev, void **buf, size_t *cap, size_t need);

@@ -4,25 +4,6 @@
 // fusor-ml/gguf/src/lib.rs:1150-1230 (BlockQ8_0::quantize), :1315-1358 (vec_dot).
 #include "fh_blocks.h"
 
-// ------------------------------------------------------------------------------ bf16 -> f32
-__global__ void k_bf16_f32(const uint16_t *__restrict__ x, float *__restrict__ y, int64_t n) {
-    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) y[i] = __uint_as_float((uint32_t)x[i] << 16);
-}
-
-fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y) {
-    fh_device *dev = q->dev;
-    const float *xf = (const float *)x;
-    if (x_is_bf16) {
-        int64_t n = (int64_t)m * q->k;
-        FH_TRY(fh_dev_scratch(dev, (void **)&dev->part_buf, &dev->part_cap, (size_t)n * 4));
-        k_bf16_f32<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, dev->stream>>>((const uint16_t *)x, dev->part_buf, n);
-        FH_HIP(hipGetLastError());
-        xf = dev->part_buf;
-    }
-    return fh_launch_qmatvec(q, xf, m, y, FH_EPI_NONE, nullptr, nullptr);
-}
-
 extern "C" fh_status fh_qmatmul_bf16(const fh_qmatrix *q, const uint16_t *x_bf16_dev, int32_t m, float *y_dev) {
     FH_REQUIRE(q && x_bf16_dev && y_dev, "NULL argument");
     FH_REQUIRE(m >= 1, "m = %d", m);

@@ -1,0 +1,284 @@
+// Quantized matmul for many activation rows (prefill, and decode batches above 2) on the matrix cores:
+//   Y[m, n] = sum_k X[m, k] * deq(W)[n, k]          (fusor-ml/cpu/src/quantized.rs:246-675)
+//
+// Tile kernel: a workgroup owns TN weight rows x TM activation rows and walks k in steps of 32.  Per step the
+// 32-wide slab of the weight tile is decoded from the tiled GGUF layout with exactly the arithmetic of
+// GgufBlock::dequantize (f32), split into an f16 pair hi + lo (w = hi + lo to 2^-22), and put in LDS; the
+// activation slab comes from f16 planes prepared once per call (k_act_split: each row scaled by a power of
+// two into the f16 range, hi + lo for f32 input, a single exact term for bf16 input).  The contraction runs on
+// v_mfma_f32_32x32x16_f16 as  w_hi*x_hi + w_lo*x_hi (+ w_hi*x_lo)  with f32 accumulation, so the only
+// deviation from the f32 reference is the summation order and the 2^-22 residues.
+#include "fh_blocks.h"
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+#define QMM_LDK 40 // halfs per LDS row: 32 + 8 padding (80 B stride: 16-byte reads of 16 rows hit 16 distinct chunks)
+
+// ------------------------------------------------------------------------------ activation planes
+// One workgroup per row.  xh / xl are [m, k] f16, rs[m] = 2^-e undoes the normalisation at the store.
+template <bool BF16>
+__global__ __launch_bounds__(256) void k_act_split(const void *__restrict__ xin, int k, _Float16 *__restrict__ xh,
+                                                    _Float16 *__restrict__ xl, float *__restrict__ rs) {
+    __shared__ float sh[4];
+    const int64_t off = (int64_t)blockIdx.x * k;
+    auto ld = [&](int c) -> float {
+        if (BF16) return __uint_as_float((uint32_t)((const uint16_t *)xin)[off + c] << 16);
+        return ((const float *)xin)[off + c];
+    };
+    float amax = 0.f;
+    for (int c = threadIdx.x; c < k; c += 256) amax = fmaxf(amax, fabsf(ld(c)));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+    int e = 141 - (int)((__float_as_uint(amax) >> 23) & 0xFFu); // 14 - floor(log2 amax); zero / inf / nan clamp
+    e = e > 100 ? 100 : (e < -100 ? -100 : e);
+    const float sc = __uint_as_float((uint32_t)(e + 127) << 23);
+    for (int c = threadIdx.x; c < k; c += 256) {
+        const float v = ld(c) * sc;
+        const _Float16 h = (_Float16)v;
+        xh[off + c] = h;
+        if (!BF16) xl[off + c] = (_Float16)(v - (float)h);
+    }
+    if (threadIdx.x == 0) rs[blockIdx.x] = __uint_as_float((uint32_t)(127 - e) << 23);
+}
+
+// ------------------------------------------------------------------------------ weight slab decode
+// Eight dequantised weights of row (tile16*16 + j), lane group g, k-step ks (32 wide).  pos[i] is the position
+// of w[i] inside the step.  Arithmetic as in fh_blocks.h (bit-exact f32 decode).
+template <int T>
+__device__ __forceinline__ void decode8(const QView &q, int64_t tile16, int j, int g, int ks, float *w, int &p0, int &p1) {
+    p0 = 8 * g;     // position of w[0..3]
+    p1 = 8 * g + 4; // position of w[4..7]
+    if (T == FH_Q8_0) {
+        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 1)) * 1088;
+        const int u = ks & 1;
+        const uint2 c = *(const uint2 *)(rec + (g * 16 + j) * 16 + 8 * u);
+        const float d = fh_h2f(fh_ld16(rec + 1024 + 4 * j + 2 * u));
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[i] = (float)(int)(int8_t)(c.x >> (8 * i)) * d;
+            w[4 + i] = (float)(int)(int8_t)(c.y >> (8 * i)) * d;
+        }
+    } else if (T == FH_Q4_0) {
+        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 2)) * 1152;
+        const int u = ks & 3;
+        const uint32_t c = *(const uint32_t *)(rec + (g * 16 + j) * 16 + 4 * u);
+        const float d = fh_h2f(fh_ld16(rec + 1024 + 8 * j + 2 * u));
+        p0 = 4 * g;
+        p1 = 16 + 4 * g;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[i] = (float)((int)((c >> (8 * i)) & 15u) - 8) * d;
+            w[4 + i] = (float)((int)((c >> (8 * i + 4)) & 15u) - 8) * d;
+        }
+    } else if (T == FH_Q4_K) {
+        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 3)) * 2304;
+        const int sb = ks & 7, p = sb >> 2, u = (sb >> 1) & 1, hn = sb & 1;
+        const uint2 c = *(const uint2 *)(rec + 256 + p * 1024 + (g * 16 + j) * 16 + 8 * u);
+        const uint4 h = *(const uint4 *)(rec + 16 * j);
+        const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
+        const uint32_t scw = sb < 4 ? (h.y & 0x3F3F3F3Fu) : ((h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u));
+        const uint32_t mnw = sb < 4 ? (h.z & 0x3F3F3F3Fu) : (((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u));
+        const float scale = (float)((scw >> (8 * (sb & 3))) & 0xFFu) * d;
+        const float off = (float)((mnw >> (8 * (sb & 3))) & 0xFFu) * dmin;
+        const int sh = 4 * hn;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float a = scale * (float)((c.x >> (8 * i + sh)) & 15u);
+            const float b = scale * (float)((c.y >> (8 * i + sh)) & 15u);
+            w[i] = a - off;
+            w[4 + i] = b - off;
+        }
+    } else { // FH_Q6_K
+        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 3)) * 3360;
+        const int t = ks & 7;
+        const uint32_t lw = *(const uint32_t *)(rec + q6k_lword_off(j, t, g));
+        const uint32_t hw = *(const uint32_t *)(rec + q6k_hword_off(j, t, g));
+        const int sc = (int)(int8_t)rec[q6k_sc_off(j, 2 * t + (g >> 1))];
+        const float ds = fh_h2f(fh_ld16(rec + q6k_d_off(j))) * (float)sc;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int pp = i >> 1, odd = i & 1;
+            const int nib = (int)((lw >> (4 * (pp + 4 * odd))) & 15u);
+            const int hb = (int)((hw >> (q6k_hbit(t, pp) + 16 * odd)) & 3u);
+            w[i] = ds * (float)(((hb << 4) | nib) - 32);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------ tile kernel
+// Wavefronts are arranged WGN x WGM; each owns FN x FM MFMA tiles of 32 x 32.  NTERM = 1: single activation
+// term (bf16 input); 2: hi + lo (f32 input).
+template <int T, int NTERM, int WGN, int WGM, int FN, int FM>
+__global__ __launch_bounds__(64 * WGN * WGM) void k_qmm_tile(QView q, const _Float16 *__restrict__ xh,
+                                                              const _Float16 *__restrict__ xl,
+                                                              const float *__restrict__ rs, int m,
+                                                              float *__restrict__ y) {
+    constexpr int TN = WGN * FN * 32, TM = WGM * FM * 32, NTH = 64 * WGN * WGM;
+    __shared__ __attribute__((aligned(16))) _Float16 s_ah[TN * QMM_LDK], s_al[TN * QMM_LDK], s_bh[TM * QMM_LDK];
+    __shared__ __attribute__((aligned(16))) _Float16 s_bl[NTERM == 2 ? TM * QMM_LDK : 8];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int wn = wave / WGM, wm = wave % WGM;
+    const int64_t n0 = (int64_t)blockIdx.x * TN;
+    const int m0 = blockIdx.y * TM;
+    const int K = (int)q.k, ksteps = K / 32;
+    const int64_t tiles16 = (q.n + 15) / 16;
+    floatx16 acc[FN][FM];
+#pragma unroll
+    for (int a = 0; a < FN; a++)
+#pragma unroll
+        for (int b = 0; b < FM; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
+
+    for (int ks = 0; ks < ksteps; ks++) {
+        __syncthreads(); // the previous step's operands are consumed
+        // ---- weights: TN * 4 (row, group) pairs of 8
+#pragma unroll
+        for (int i = 0; i < (TN * 4 + NTH - 1) / NTH; i++) {
+            const int p = tid + i * NTH;
+            if (p < TN * 4) {
+                const int t16 = p >> 6, l = p & 63, g = l >> 4, j = l & 15;
+                int64_t tile = (n0 >> 4) + t16;
+                if (tile >= tiles16) tile = tiles16 - 1; // rows past the end decode a valid tile and are never stored
+                float w[8];
+                int p0, p1;
+                decode8<T>(q, tile, j, g, ks, w, p0, p1);
+                _Float16 hi[8], lo[8];
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    hi[c] = (_Float16)w[c];
+                    lo[c] = (_Float16)(w[c] - (float)hi[c]);
+                }
+                const int row = t16 * 16 + j;
+                uint2 a0, a1, b0, b1;
+                __builtin_memcpy(&a0, hi, 8);
+                __builtin_memcpy(&a1, hi + 4, 8);
+                __builtin_memcpy(&b0, lo, 8);
+                __builtin_memcpy(&b1, lo + 4, 8);
+                *(uint2 *)(s_ah + row * QMM_LDK + p0) = a0;
+                *(uint2 *)(s_ah + row * QMM_LDK + p1) = a1;
+                *(uint2 *)(s_al + row * QMM_LDK + p0) = b0;
+                *(uint2 *)(s_al + row * QMM_LDK + p1) = b1;
+            }
+        }
+        // ---- activations: TM rows x 32 halfs (two 16-byte pieces per row... four 16-byte pieces: 64 B)
+#pragma unroll
+        for (int i = 0; i < (TM * 4 + NTH - 1) / NTH; i++) {
+            const int p = tid + i * NTH;
+            if (p < TM * 4) {
+                const int row = p >> 2, c = p & 3;
+                const int mm = m0 + row;
+                uint4 vh = make_uint4(0, 0, 0, 0), vl = make_uint4(0, 0, 0, 0);
+                if (mm < m) {
+                    vh = *(const uint4 *)(xh + (int64_t)mm * K + ks * 32 + c * 8);
+                    if (NTERM == 2) vl = *(const uint4 *)(xl + (int64_t)mm * K + ks * 32 + c * 8);
+                }
+                *(uint4 *)(s_bh + row * QMM_LDK + c * 8) = vh;
+                if (NTERM == 2) *(uint4 *)(s_bl + row * QMM_LDK + c * 8) = vl;
+            }
+        }
+        __syncthreads();
+        // ---- contraction
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+            const int ko = kk * 16 + 8 * (lane >> 5), li = lane & 31;
+            half8 ah[FN], al[FN], bh[FM], bl[FM];
+#pragma unroll
+            for (int a = 0; a < FN; a++) {
+                const int row = (wn * FN + a) * 32 + li;
+                ah[a] = *(const half8 *)(s_ah + row * QMM_LDK + ko);
+                al[a] = *(const half8 *)(s_al + row * QMM_LDK + ko);
+            }
+#pragma unroll
+            for (int b = 0; b < FM; b++) {
+                const int row = (wm * FM + b) * 32 + li;
+                bh[b] = *(const half8 *)(s_bh + row * QMM_LDK + ko);
+                if (NTERM == 2) bl[b] = *(const half8 *)(s_bl + row * QMM_LDK + ko);
+            }
+#pragma unroll
+            for (int a = 0; a < FN; a++)
+#pragma unroll
+                for (int b = 0; b < FM; b++) {
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[a], bh[b], acc[a][b], 0, 0, 0);
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[a], bh[b], acc[a][b], 0, 0, 0);
+                    if (NTERM == 2) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[a], bl[b], acc[a][b], 0, 0, 0);
+                }
+        }
+    }
+    // ---- store: lane holds column m = lane % 32 and rows n = 8*(r/4) + 4*(lane/32) + r%4 of each 32 x 32 tile
+    const bool vec = (q.n & 3) == 0;
+#pragma unroll
+    for (int b = 0; b < FM; b++) {
+        const int mm = m0 + (wm * FM + b) * 32 + (lane & 31);
+        if (mm >= m) continue;
+        const float s = rs[mm];
+#pragma unroll
+        for (int a = 0; a < FN; a++) {
+            const int64_t nb = n0 + (wn * FN + a) * 32 + 4 * (lane >> 5);
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+                const int64_t nn = nb + 8 * r4;
+                float4 v = make_float4(acc[a][b][4 * r4] * s, acc[a][b][4 * r4 + 1] * s, acc[a][b][4 * r4 + 2] * s,
+                                       acc[a][b][4 * r4 + 3] * s);
+                float *dst = y + (int64_t)mm * q.n + nn;
+                if (vec && nn + 3 < q.n) {
+                    *(float4 *)dst = v;
+                } else {
+                    if (nn < q.n) dst[0] = v.x;
+                    if (nn + 1 < q.n) dst[1] = v.y;
+                    if (nn + 2 < q.n) dst[2] = v.z;
+                    if (nn + 3 < q.n) dst[3] = v.w;
+                }
+            }
+        }
+    }
+}
+
+template <int T, int NTERM>
+static fh_status qmm_launch_t(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const float *rs, int m,
+                              float *y) {
+    hipStream_t s = q->dev->stream;
+    QView v = fh_view(q);
+    if (m <= 32) {
+        dim3 grid((unsigned)((q->n + 127) / 128), 1);
+        k_qmm_tile<T, NTERM, 4, 1, 1, 1><<<grid, 256, 0, s>>>(v, xh, xl, rs, m, y);
+    } else if (m <= 64) {
+        dim3 grid((unsigned)((q->n + 127) / 128), 1);
+        k_qmm_tile<T, NTERM, 2, 2, 2, 1><<<grid, 256, 0, s>>>(v, xh, xl, rs, m, y);
+    } else {
+        dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + 127) / 128));
+        k_qmm_tile<T, NTERM, 2, 2, 2, 2><<<grid, 256, 0, s>>>(v, xh, xl, rs, m, y);
+    }
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y) {
+    fh_device *dev = q->dev;
+    const int64_t K = q->k;
+    FH_REQUIRE((m + 127) / 128 <= 65535, "m = %d too large for one launch", m);
+    // planes: xh | xl | rs
+    const size_t plane = ((size_t)m * K * 2 + 255) & ~(size_t)255;
+    const size_t need = plane * (x_is_bf16 ? 1 : 2) + (size_t)m * 4 + 256;
+    FH_TRY(fh_dev_scratch(dev, &dev->act_buf, &dev->act_cap, need));
+    _Float16 *xh = (_Float16 *)dev->act_buf;
+    _Float16 *xl = x_is_bf16 ? nullptr : (_Float16 *)((uint8_t *)dev->act_buf + plane);
+    float *rs = (float *)((uint8_t *)dev->act_buf + plane * (x_is_bf16 ? 1 : 2));
+    if (x_is_bf16) k_act_split<true><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, (int)K, xh, xl, rs);
+    else k_act_split<false><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, (int)K, xh, xl, rs);
+    FH_HIP(hipGetLastError());
+#define QMM_GO(T_)                                                              \
+    return x_is_bf16 ? qmm_launch_t<T_, 1>(q, xh, xl, rs, m, y) : qmm_launch_t<T_, 2>(q, xh, xl, rs, m, y)
+    switch (q->type) {
+    case FH_Q4_0: QMM_GO(FH_Q4_0);
+    case FH_Q8_0: QMM_GO(FH_Q8_0);
+    case FH_Q4_K: QMM_GO(FH_Q4_K);
+    case FH_Q6_K: QMM_GO(FH_Q6_K);
+    }
+#undef QMM_GO
+    FH_FAIL(FH_ERR_UNSUPPORTED, "unsupported type %u", q->type);
+}

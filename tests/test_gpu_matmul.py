@@ -1,0 +1,124 @@
+"""GPU parity: the prefill-side quantized matmul (matrix-core tile kernel) against the CPU checker.
+
+Tolerance of the north star for floating point: 1e-3 relative or 1e-2 absolute per element, f32 accumulation.
+"""
+import numpy as np
+import pytest
+
+from refgen import Q4_0, Q4_K, Q6_K, Q8_0, assert_close
+from kalosm_amd import synth
+from kalosm_amd.fusor import QMatrix, Tensor
+
+pytestmark = pytest.mark.gpu
+ALL = [Q4_0, Q8_0, Q4_K, Q6_K]
+NAMES = synth.TYPE_NAMES
+
+
+def bf16_round(x):
+    """f32 -> bf16 bits (round to nearest even) and the f32 value those bits stand for."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    return r, (r.astype(np.uint32) << 16).view(np.float32)
+
+
+def tile_matmul(dev, x, q, force=True):
+    out = Tensor.filled_bytes(dev, (x.shape[0], q.n), 0xFF)  # poisoned: unwritten elements show as NaN
+    dev.set_option("matmul_kernel", 2 if force else 0)
+    try:
+        return Tensor.from_slice(dev, x).q_mat_mul(q, out=out).as_slice()
+    finally:
+        dev.set_option("matmul_kernel", 0)
+
+
+@pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("m,n,k", [(17, 272, 2048), (33, 130, 1024), (64, 128, 512), (65, 100, 768), (130, 300, 1024),
+                                   (256, 256, 256), (3, 37, 512)])
+def test_tile_matmul_f32_vs_checker(dev, oracle, ty, m, n, k):
+    """Ragged m (tile edges 32 / 64 / 128), ragged n (not a multiple of 4, 16 or 128), k of 1..8 super-blocks."""
+    raw = synth.random_weight(ty, n, k, seed=50 + ty)
+    x = synth.random_activation(m, k, seed=60 + m)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    got = tile_matmul(dev, x, q)
+    want = oracle.q_mat_mul(ty, x, raw, n, fast=True)
+    assert_close(got, want, what=f"{NAMES[ty]} {n}x{k} m={m}")
+
+
+@pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
+def test_tile_matmul_matches_decode_kernels(dev, oracle, ty):
+    """The same product through the decode matvec (row by row) and through the tile kernel."""
+    n, k, m = 272, 2048, 40
+    raw = synth.random_weight(ty, n, k, seed=70 + ty)
+    x = synth.random_activation(m, k, seed=71)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    yt = tile_matmul(dev, x, q)
+    for r in (0, 17, 39):
+        yr = Tensor.from_slice(dev, x[r:r + 1]).q_mat_mul(q).as_slice()
+        assert_close(yt[r:r + 1], yr, abs_tol=1e-2, rel_tol=1e-3, what=f"row {r}")
+
+
+@pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
+def test_tile_matmul_invariants(dev, oracle, ty):
+    """One-hot rows pick single weights exactly (tests.rs:951-995); zero rows give exact zeros (:450-476);
+    rows of very different magnitude do not disturb each other (each row carries its own scale); linearity."""
+    n, k, m = 96, 1024, 48
+    raw = synth.random_weight(ty, n, k, seed=80 + ty)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    w = oracle.dequantize(ty, raw).reshape(n, k)
+    x = np.zeros((m, k), np.float32)
+    cols = (np.arange(m) * 37 + 5) % k
+    x[np.arange(m), cols] = 0.125
+    x[7] = 0.0
+    y = tile_matmul(dev, x, q)
+    for r in range(m):
+        want = np.zeros(n, np.float32) if r == 7 else np.float32(0.125) * w[:, cols[r]]
+        assert_close(y[r], want, abs_tol=1e-6, rel_tol=1e-6, what=f"one-hot row {r}")
+    assert not y[7].any()
+    xs = synth.random_activation(m, k, seed=81)
+    xs[3] *= np.float32(1e20)
+    xs[4] *= np.float32(1e-20)
+    xs[5, 100] = 3.0e4  # one outlier in a row of N(0,1)
+    got = tile_matmul(dev, xs, q)
+    want = oracle.q_mat_mul(ty, xs, raw, n, fast=True)
+    scale = np.ones((m, 1), np.float32)
+    scale[3], scale[4] = 1e-20, 1e20
+    assert_close(got * scale, want * scale, what="rows of mixed magnitude")
+    y2 = tile_matmul(dev, xs * np.float32(2.0), q)
+    assert np.array_equal(y2, got * np.float32(2.0)), "scaling the input by 2 must scale the output exactly"
+
+
+@pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("m", [1, 20, 130])
+def test_tile_matmul_bf16_activations(dev, oracle, ty, m):
+    """bf16 activations (the prefill configuration): the checker gets the f32 values of the same bf16 bits."""
+    n, k = 272, 1024
+    raw = synth.random_weight(ty, n, k, seed=90 + ty)
+    xb, xf = bf16_round(synth.random_activation(m, k, seed=91 + m))
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    out = Tensor.filled_bytes(dev, (m, n), 0xFF)
+    got = Tensor.from_slice(dev, xb, dtype="bf16").q_mat_mul(q, out=out).as_slice()
+    want = oracle.q_mat_mul(ty, xf, raw, n, fast=True)
+    assert_close(got, want, what=f"bf16 {NAMES[ty]} m={m}")
+
+
+@pytest.mark.parametrize("ty", [Q6_K, Q8_0], ids=lambda t: NAMES[t])
+def test_prefill_shape_spot_check(dev, oracle, ty):
+    """Full prefill shape (m = 512, k = 4096, n = 14336, bf16 activations): 64 output columns spread over the matrix
+    against the checker, and the sum over all outputs of a row against x . (sum of weight rows) -- a checksum that
+    every output element enters."""
+    m, k, n = 512, 4096, 14336
+    raw = synth.random_weight(ty, n, k, seed=100 + ty)
+    xb, xf = bf16_round(synth.random_activation(m, k, seed=101))
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    got = Tensor.from_slice(dev, xb, dtype="bf16").q_mat_mul(q).as_slice()
+    assert np.isfinite(got).all()
+    rows = (np.arange(64) * 223 + 11) % n
+    bpr = len(raw) // n
+    sub = np.concatenate([raw[r * bpr:(r + 1) * bpr] for r in rows])
+    want = oracle.q_mat_mul(ty, xf, sub, 64, fast=True)
+    assert_close(got[:, rows], want, what="sampled columns")
+    w = oracle.dequantize(ty, raw).reshape(n, k).astype(np.float64)
+    colsum = w.sum(axis=0)
+    want_sum = xf.astype(np.float64) @ colsum
+    got_sum = got.astype(np.float64).sum(axis=1)
+    norm = np.sqrt((xf.astype(np.float64) ** 2).sum(axis=1) * (w ** 2).sum())
+    assert np.all(np.abs(got_sum - want_sum) <= 1e-5 * norm)
