@@ -49,7 +49,7 @@ struct fh_device {
     // 64 KB that never moves: partial results of small reductions (argmax)
     void *small_buf = nullptr;
     // options (fh_set_option)
-    int64_t opt_matvec_kernel = 0;   // 0 auto, 1 generic VALU, 2 MFMA
+    int64_t opt_matvec_kernel = 0;   // 0 auto, 1 generic VALU, 2 MFMA, 3 first-generation Q4_K MFMA, 4 batch MFMA
     int64_t opt_matvec_splitk = 0;   // 0 auto, else forced split count
     int64_t opt_matvec_waves = 0;    // 0 auto
     int64_t opt_matvec_tiles = 0;    // 0 auto, else 1 / 2 / 4 row tiles per workgroup
@@ -138,6 +138,9 @@ static inline QView fh_view(const fh_qmatrix *q) {
 // ---------------------------------------------------------------- launches implemented per file
 fh_status fh_launch_qmatvec(const fh_qmatrix *q, const float *x, int m, float *y, int epilogue,
                             const float *a, const float *b);
+bool fh_qmatvec_batch_supports(const fh_qmatrix *q, int m, int epi);
+fh_status fh_launch_qmatvec_batch(const fh_qmatrix *q, const float *x, int m, float *y, int epi, const float *a,
+                                  const float *b);
 fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y);
 enum { FH_EPI_NONE = 0, FH_EPI_ADD2 = 1, FH_EPI_SWIGLU = 2 };
 fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b);

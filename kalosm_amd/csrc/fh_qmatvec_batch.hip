@@ -1,0 +1,411 @@
+// Decode-side quantized matmul for 1..16 activation rows, all four block formats, on the matrix cores.
+//   Y[m, n] = sum_k X[m, k] * deq(W)[n, k]          (fusor-ml/cpu/src/quantized.rs:246-675)
+//
+// One v_mfma_f32_16x16x32_f16 multiplies 16 activation rows (A operand: row m = lane % 16, k = 8 * (lane / 16) .. +8)
+// with 16 weight rows (B operand: column n = lane % 16, same k), so a lane ends up with the outputs of ONE weight
+// row and FOUR activation rows (m = 4 * (lane / 16) + i): the per-block weight scale is a per-lane scalar.
+//
+// Exactness: a weight code c (4, 6 or 8 bits) is used as the f16 subnormal c * 2^-24 straight from a mask of the
+// packed bytes; each 256-element chunk of an activation row is scaled by a power of two into the f16 range and
+// split into f16 hi + lo, so code * activation products are exact and accumulate in f32.  The block scale
+// (d * sc, d) multiplies the per-block MFMA result, the block offset (dmin * m, 32 * d * sc, 8 * d, 128 * d)
+// multiplies the f32 sum of the block's activations: the same algebra as GgufBlock::dequantize followed by the
+// dot product, re-associated.
+//
+// A workgroup of TW x TS wavefronts owns TW row tiles (16 rows each) and all of k: in round r wavefront (tw, ts)
+// multiplies tile tw with the 256-element chunk r * TS + ts.  The TS chunks of a round are staged once in LDS for
+// all tiles (double buffered, one barrier per round); every wavefront keeps the weights of its next D chunks in
+// flight (the kernel is bound by memory latency, not by arithmetic).  The slices are added through LDS in a fixed
+// order and the epilogue is applied at the store.
+#include "fh_blocks.h"
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+#define QB_DPP_XOR1 0xB1         // quad_perm [1,0,3,2]
+#define QB_DPP_XOR2 0x4E         // quad_perm [2,3,0,1]
+#define QB_DPP_HALF_MIRROR 0x141 // lane i <- lane 7-i within each group of 8
+template <int CTRL>
+__device__ __forceinline__ float qb_dpp(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
+// LDS image of one staged chunk (bytes): activation planes [plane][MR rows][ROW], group sums [NG][16], factors [16].
+// MFMA rows m >= MR read row m % MR: they produce values that are never stored.
+template <int T, int MR>
+struct QbLds {
+    static constexpr int NG = T == FH_Q6_K ? 16 : 8;     // offset groups per chunk
+    static constexpr int ROW = T == FH_Q6_K ? 520 : 264; // halfs per plane row (dword stride = 4 mod 64)
+    static constexpr int PLANES = T == FH_Q6_K ? 1 : 2;  // Q6_K interleaves hi | lo per 16-group
+    static constexpr int PLANE = MR * ROW;               // halfs
+    static constexpr int S_OFF = PLANES * PLANE * 2, F_OFF = S_OFF + NG * 16 * 4, BYTES = F_OFF + 64;
+};
+
+// ------------------------------------------------------------------------------ weights of one (tile, chunk)
+template <int T>
+struct QbW;
+template <>
+struct QbW<FH_Q4_K> {
+    uint4 a, b, h;
+    __device__ __forceinline__ void load(const QView &q, int64_t tile, int c, int lane) {
+        const uint8_t *rec = q.data + (tile * q.recs + c) * 2304;
+        h = *(const uint4 *)(rec + 16 * (lane & 15));
+        a = *(const uint4 *)(rec + 256 + lane * 16);
+        b = *(const uint4 *)(rec + 1280 + lane * 16);
+    }
+};
+template <>
+struct QbW<FH_Q6_K> {
+    uint4 l0, l1, hh;
+    uint32_t sc[4];
+    uint32_t d;
+    __device__ __forceinline__ void load(const QView &q, int64_t tile, int c, int lane) {
+        const uint8_t *rec = q.data + (tile * q.recs + c) * 3360;
+        const int j = lane & 15;
+        l0 = *(const uint4 *)(rec + lane * 16);
+        l1 = *(const uint4 *)(rec + 1024 + lane * 16);
+        hh = *(const uint4 *)(rec + 2048 + lane * 16);
+#pragma unroll
+        for (int qd = 0; qd < 4; qd++) sc[qd] = *(const uint32_t *)(rec + 3072 + (qd * 16 + j) * 4);
+        d = fh_ld16(rec + 3328 + 2 * j);
+    }
+};
+template <>
+struct QbW<FH_Q8_0> {
+    uint4 w[4];
+    uint32_t d[4];
+    __device__ __forceinline__ void load(const QView &q, int64_t tile, int c, int lane) {
+        const uint8_t *rec = q.data + (tile * q.recs + 4 * c) * 1088;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            w[r] = *(const uint4 *)(rec + r * 1088 + lane * 16);
+            d[r] = *(const uint32_t *)(rec + r * 1088 + 1024 + 4 * (lane & 15));
+        }
+    }
+};
+template <>
+struct QbW<FH_Q4_0> {
+    uint4 w[2];
+    uint2 d[2];
+    __device__ __forceinline__ void load(const QView &q, int64_t tile, int c, int lane) {
+        const uint8_t *rec = q.data + (tile * q.recs + 2 * c) * 1152;
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            w[r] = *(const uint4 *)(rec + r * 1152 + lane * 16);
+            d[r] = *(const uint2 *)(rec + r * 1152 + 1024 + 8 * (lane & 15));
+        }
+    }
+};
+
+__device__ __forceinline__ half8 qb_h8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    const uint4 u = make_uint4(a, b, c, d);
+    half8 v;
+    __builtin_memcpy(&v, &u, 16);
+    return v;
+}
+
+// ------------------------------------------------------------------------------ one chunk of one tile
+// yacc[i] += factor[m] * sum_blocks scale * (codes . x_scaled) - sum_blocks offset * sum(x), m = 4g + i.
+template <int T, int MR>
+__device__ __forceinline__ void qb_chunk(const QbW<T> &W, const uint8_t *img, int lane, float *yacc) {
+    typedef QbLds<T, MR> L;
+    const int j = lane & 15, g = lane >> 4;
+    const _Float16 *xa = (const _Float16 *)img + (j & (MR - 1)) * L::ROW + 8 * g;
+    const float *S = (const float *)(img + L::S_OFF) + 4 * g;
+    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+    float tot[4] = {0.f, 0.f, 0.f, 0.f}, off[4] = {0.f, 0.f, 0.f, 0.f};
+    const uint32_t LO = 0x000F000Fu, HI = 0x00F000F0u;
+    if constexpr (T == FH_Q4_K) {
+        const float d = fh_h2f((uint16_t)(W.h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(W.h.x >> 16));
+        const uint32_t sc_l = W.h.y & 0x3F3F3F3Fu, sc_h = (W.h.w & 0x0F0F0F0Fu) | ((W.h.y >> 2) & 0x30303030u);
+        const uint32_t mn_l = W.h.z & 0x3F3F3F3Fu, mn_h = ((W.h.w >> 4) & 0x0F0F0F0Fu) | ((W.h.z >> 2) & 0x30303030u);
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            const uint4 wq = (s & 4) ? W.b : W.a;
+            const uint32_t w0 = (s & 2) ? wq.z : wq.x, w1 = (s & 2) ? wq.w : wq.y;
+            const uint32_t msk = (s & 1) ? HI : LO;
+            const half8 bv = qb_h8(w0 & msk, (w0 >> 8) & msk, w1 & msk, (w1 >> 8) & msk);
+            const half8 ah = *(const half8 *)(xa + 32 * s), al = *(const half8 *)(xa + L::PLANE + 32 * s);
+            floatx4 r = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bv, zero, 0, 0, 0);
+            r = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, bv, r, 0, 0, 0);
+            const float sc = (float)(((s < 4 ? sc_l : sc_h) >> (8 * (s & 3))) & 0xFFu);
+            const float mn = (float)(((s < 4 ? mn_l : mn_h) >> (8 * (s & 3))) & 0xFFu);
+            const float sw = (sc * d) * ((s & 1) ? 0.0625f : 1.0f), ow = mn * dmin; // high nibbles carry a factor 16
+            const float4 sv = *(const float4 *)(S + 16 * s);
+            tot[0] = fmaf(sw, r[0], tot[0]); tot[1] = fmaf(sw, r[1], tot[1]);
+            tot[2] = fmaf(sw, r[2], tot[2]); tot[3] = fmaf(sw, r[3], tot[3]);
+            off[0] = fmaf(ow, sv.x, off[0]); off[1] = fmaf(ow, sv.y, off[1]);
+            off[2] = fmaf(ow, sv.z, off[2]); off[3] = fmaf(ow, sv.w, off[3]);
+        }
+    } else if constexpr (T == FH_Q6_K) {
+        const float d = fh_h2f((uint16_t)W.d);
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            const uint4 lq = (t & 4) ? W.l1 : W.l0;
+            const uint32_t lw = (t & 3) == 0 ? lq.x : (t & 3) == 1 ? lq.y : (t & 3) == 2 ? lq.z : lq.w;
+            const uint32_t hw = (t >> 1) == 0 ? W.hh.x : (t >> 1) == 1 ? W.hh.y : (t >> 1) == 2 ? W.hh.z : W.hh.w;
+            uint32_t o[4];
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                const int hs = q6k_hbit(t, p) - 4; // bring the two high bits of the pair to bits 4-5
+                const uint32_t hb = hs >= 0 ? (hw >> hs) : (hw << (-hs));
+                o[p] = ((lw >> (4 * p)) & LO) | (hb & 0x00300030u);
+            }
+            // lanes 0-31 hold the codes of group 2t, lanes 32-63 those of group 2t+1.  One operand per group with
+            // its codes in both halves: they meet hi in lanes 0-31 and lo in lanes 32-63 of the activation operand
+            // (v_permlane32_swap: first result = lanes 0-31 of the source in both halves, second = lanes 32-63).
+            uint32_t oa[4], ob[4];
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                auto sw2 = __builtin_amdgcn_permlane32_swap(o[p], o[p], false, false);
+                oa[p] = sw2[0];
+                ob[p] = sw2[1];
+            }
+            const half8 ba = qb_h8(oa[0], oa[1], oa[2], oa[3]), bb = qb_h8(ob[0], ob[1], ob[2], ob[3]);
+            const half8 a0 = *(const half8 *)(xa + 64 * t), a1 = *(const half8 *)(xa + 64 * t + 32);
+            const floatx4 r0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, ba, zero, 0, 0, 0);
+            const floatx4 r1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bb, zero, 0, 0, 0);
+            const uint32_t scw = W.sc[t & 3] >> (16 * (t >> 2));
+            const float s0 = d * (float)(int)(int8_t)(scw & 0xFFu), s1 = d * (float)(int)(int8_t)((scw >> 8) & 0xFFu);
+            const float4 v0 = *(const float4 *)(S + 32 * t), v1 = *(const float4 *)(S + 32 * t + 16);
+            tot[0] = fmaf(s0, r0[0], tot[0]); tot[1] = fmaf(s0, r0[1], tot[1]);
+            tot[2] = fmaf(s0, r0[2], tot[2]); tot[3] = fmaf(s0, r0[3], tot[3]);
+            tot[0] = fmaf(s1, r1[0], tot[0]); tot[1] = fmaf(s1, r1[1], tot[1]);
+            tot[2] = fmaf(s1, r1[2], tot[2]); tot[3] = fmaf(s1, r1[3], tot[3]);
+            const float o0 = 32.f * s0, o1 = 32.f * s1;
+            off[0] = fmaf(o0, v0.x, off[0]); off[1] = fmaf(o0, v0.y, off[1]);
+            off[2] = fmaf(o0, v0.z, off[2]); off[3] = fmaf(o0, v0.w, off[3]);
+            off[0] = fmaf(o1, v1.x, off[0]); off[1] = fmaf(o1, v1.y, off[1]);
+            off[2] = fmaf(o1, v1.z, off[2]); off[3] = fmaf(o1, v1.w, off[3]);
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            half8 bv;
+            float sw, ow;
+            if constexpr (T == FH_Q8_0) {
+                const uint4 wq = W.w[s >> 1];
+                const uint32_t w0 = ((s & 1) ? wq.z : wq.x) ^ 0x80808080u, w1 = ((s & 1) ? wq.w : wq.y) ^ 0x80808080u;
+                bv = qb_h8(__builtin_amdgcn_perm(0, w0, 0x0C010C00u), __builtin_amdgcn_perm(0, w0, 0x0C030C02u),
+                           __builtin_amdgcn_perm(0, w1, 0x0C010C00u), __builtin_amdgcn_perm(0, w1, 0x0C030C02u));
+                const uint32_t dd = W.d[s >> 1];
+                sw = fh_h2f((uint16_t)((s & 1) ? (dd >> 16) : (dd & 0xFFFF)));
+                ow = 128.f * sw; // codes are q + 128
+            } else {
+                const uint4 wq = W.w[s >> 2];
+                const uint32_t w0 = (s & 3) == 0 ? wq.x : (s & 3) == 1 ? wq.y : (s & 3) == 2 ? wq.z : wq.w;
+                bv = qb_h8(w0 & LO, (w0 >> 8) & LO, (w0 >> 4) & LO, (w0 >> 12) & LO);
+                const uint2 dd = W.d[s >> 2];
+                const uint32_t dw = (s & 2) ? dd.y : dd.x;
+                sw = fh_h2f((uint16_t)((s & 1) ? (dw >> 16) : (dw & 0xFFFF)));
+                ow = 8.f * sw;
+            }
+            const half8 ah = *(const half8 *)(xa + 32 * s), al = *(const half8 *)(xa + L::PLANE + 32 * s);
+            floatx4 r = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bv, zero, 0, 0, 0);
+            r = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, bv, r, 0, 0, 0);
+            const float4 sv = *(const float4 *)(S + 16 * s);
+            tot[0] = fmaf(sw, r[0], tot[0]); tot[1] = fmaf(sw, r[1], tot[1]);
+            tot[2] = fmaf(sw, r[2], tot[2]); tot[3] = fmaf(sw, r[3], tot[3]);
+            off[0] = fmaf(ow, sv.x, off[0]); off[1] = fmaf(ow, sv.y, off[1]);
+            off[2] = fmaf(ow, sv.z, off[2]); off[3] = fmaf(ow, sv.w, off[3]);
+        }
+    }
+    const float4 fv = *(const float4 *)((const float *)(img + L::F_OFF) + 4 * g);
+    yacc[0] += fv.x * tot[0] - off[0];
+    yacc[1] += fv.y * tot[1] - off[1];
+    yacc[2] += fv.z * tot[2] - off[2];
+    yacc[3] += fv.w * tot[3] - off[3];
+}
+
+// ------------------------------------------------------------------------------ staging of one activation row chunk
+// The wavefront holds row m of the chunk, lane c elements 4c .. 4c+3.  Positions inside the LDS row follow the
+// order in which the format's code masks deliver the weights of a lane (see qb_chunk).
+template <int T, int MR>
+__device__ __forceinline__ void qb_stage(uint8_t *img, int m, int lane, float4 v) {
+    typedef QbLds<T, MR> L;
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, qb_dpp<QB_DPP_XOR1>(amax));
+    amax = fmaxf(amax, qb_dpp<QB_DPP_XOR2>(amax));
+    amax = fmaxf(amax, qb_dpp<QB_DPP_HALF_MIRROR>(amax));
+    amax = fmaxf(amax, __shfl_xor(amax, 8, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+    int e = 141 - (int)((__float_as_uint(amax) >> 23) & 0xFFu); // 14 - floor(log2 amax); zero / inf / nan clamp
+    e = e > 100 ? 100 : (e < -100 ? -100 : e);
+    const float sc = __uint_as_float((uint32_t)(e + 127) << 23);
+    const float xs[4] = {v.x * sc, v.y * sc, v.z * sc, v.w * sc};
+    _Float16 hi[4], lo[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        hi[c] = (_Float16)xs[c];
+        lo[c] = (_Float16)(xs[c] - (float)hi[c]);
+    }
+    const bool swap = T == FH_Q4_K || T == FH_Q4_0; // nibble masks deliver bytes 0,2 then 1,3 of a word
+    const _Float16 oh[4] = {hi[0], swap ? hi[2] : hi[1], swap ? hi[1] : hi[2], hi[3]};
+    const _Float16 ol[4] = {lo[0], swap ? lo[2] : lo[1], swap ? lo[1] : lo[2], lo[3]};
+    uint2 ph, pl;
+    __builtin_memcpy(&ph, oh, 8);
+    __builtin_memcpy(&pl, ol, 8);
+    _Float16 *row = (_Float16 *)img + m * L::ROW;
+    float s4 = (v.x + v.y) + (v.z + v.w);
+    s4 += qb_dpp<QB_DPP_XOR1>(s4);
+    s4 += qb_dpp<QB_DPP_XOR2>(s4);
+    float *S = (float *)(img + L::S_OFF);
+    if (T == FH_Q6_K) {
+        const int G = lane >> 2, e0 = 4 * (lane & 3);
+        *(uint2 *)(row + 32 * G + e0) = ph;
+        *(uint2 *)(row + 32 * G + 16 + e0) = pl;
+        if ((lane & 3) == 0) S[G * 16 + m] = s4;
+    } else {
+        int pos = 4 * lane;
+        if (T == FH_Q4_0) { // low nibbles are elements 0..15 of a block, high nibbles 16..31; a lane group has 4 + 4
+            const int c = lane & 7;
+            pos = 32 * (lane >> 3) + (c < 4 ? 8 * c : 8 * (c - 4) + 4);
+        }
+        *(uint2 *)(row + pos) = ph;
+        *(uint2 *)(row + L::PLANE + pos) = pl;
+        s4 += qb_dpp<QB_DPP_HALF_MIRROR>(s4);
+        if ((lane & 7) == 0) S[(lane >> 3) * 16 + m] = s4;
+    }
+    if (lane == 0) ((float *)(img + L::F_OFF))[m] = __uint_as_float((uint32_t)(24 - e + 127) << 23);
+}
+
+// ------------------------------------------------------------------------------ kernel
+// MR: activation rows held per image (4 or 16, m <= MR); TW x TS = 8 wavefronts; D weight chunks in flight.
+template <int T, int MR, int TW, int TS, int EPI>
+__global__ __launch_bounds__(512) void k_qmv_batch(QView q, const float *__restrict__ x, int M, float *__restrict__ y,
+                                                   const float *__restrict__ ea, const float *__restrict__ eb) {
+    typedef QbLds<T, MR> L;
+    static_assert(TW * TS == 8, "eight wavefronts");
+    constexpr int NT = EPI == FH_EPI_SWIGLU ? 2 : 1, TWO = TW / NT; // output tiles per workgroup
+    constexpr int D = T == FH_Q6_K ? 2 : 4; // chunks of weights in flight per wavefront (register budget)
+    constexpr int RPW = TS * MR / 8, NE = 256 * TW;
+    constexpr int IMG = (L::BYTES + 15) & ~15, ROUND = TS * IMG;
+    constexpr int OUT_BYTES = 8 * 16 * 17 * 4;
+    constexpr int LDS_BYTES = 2 * ROUND > OUT_BYTES ? 2 * ROUND : OUT_BYTES;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[LDS_BYTES];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, g = lane >> 4;
+    const int tw = wave / TS, ts = wave % TS;
+    const int64_t K = q.k;
+    const int C = (int)(K >> 8), R = (C + TS - 1) / TS;
+    const int64_t nout = NT == 2 ? q.n / 2 : q.n;
+    const int64_t tiles_out = (nout + 15) / 16;
+    int64_t to = (int64_t)blockIdx.x * TWO + (tw % TWO);
+    if (to >= tiles_out) to = tiles_out - 1; // a tile past the end re-reads the last one; its rows are never stored
+    const int64_t tile = to + (int64_t)(tw / TWO) * (nout / 16); // up tiles follow the gate tiles
+
+    // staging duty of this wavefront in every round: items i = wave + 8r -> (chunk slot i % TS, row i / TS)
+    float4 xr[2][RPW];
+    auto load_x = [&](float4 *xv, int rr) {
+#pragma unroll
+        for (int r = 0; r < RPW; r++) {
+            const int i = wave + 8 * r, slot = i % TS, m = i / TS, c = rr * TS + slot;
+            xv[r] = (m < M && c < C) ? *(const float4 *)(x + (int64_t)m * K + (int64_t)c * 256 + lane * 4)
+                                     : make_float4(0, 0, 0, 0);
+        }
+    };
+    auto stage = [&](const float4 *xv, int rr) {
+        uint8_t *base = lds + (rr & 1) * ROUND;
+#pragma unroll
+        for (int r = 0; r < RPW; r++) {
+            const int i = wave + 8 * r, slot = i % TS, m = i / TS;
+            if (m < M) qb_stage<T, MR>(base + slot * IMG, m, lane, xv[r]);
+        }
+    };
+    auto chunk_of = [&](int rr) {
+        const int c = rr * TS + ts;
+        return c < C ? c : C - 1; // a slice without a chunk in the last round re-reads the last one and skips the math
+    };
+    load_x(xr[0], 0);
+    QbW<T> wr[D];
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if (d < R) wr[d].load(q, tile, chunk_of(d), lane);
+    if (R > 1) load_x(xr[1], 1);
+    stage(xr[0], 0);
+    float yacc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int r0 = 0; r0 < R; r0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            const int rr = r0 + d;
+            if (rr < R) {
+                __syncthreads(); // image rr is complete; the other buffer is no longer read
+                if (rr + 2 < R) load_x(xr[d & 1], rr + 2);
+                if (rr * TS + ts < C) qb_chunk<T, MR>(wr[d], lds + (rr & 1) * ROUND + ts * IMG, lane, yacc);
+                if (rr + D < R) wr[d].load(q, tile, chunk_of(rr + D), lane);
+                if (rr + 1 < R) stage(xr[(d + 1) & 1], rr + 1);
+            }
+        }
+    }
+    // ---- add the slices through LDS in a fixed order, then epilogue and store: element e = (tile, m, n)
+    __syncthreads();
+    float *o = (float *)lds; // [ts][tw][16][17]
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[((ts * TW + tw) * 16 + 4 * g + i) * 17 + j] = yacc[i];
+    __syncthreads();
+    auto total = [&](int e) {
+        const int at = ((e >> 8) * 16 + ((e >> 4) & 15)) * 17 + (e & 15);
+        float s = 0.f;
+#pragma unroll
+        for (int k2 = 0; k2 < TS; k2++) s += o[k2 * TW * 16 * 17 + at];
+        return s;
+    };
+    for (int e = tid; e < NE / NT; e += 512) {
+        const int t2 = e >> 8, m = (e >> 4) & 15, jn = e & 15;
+        const int64_t n = ((int64_t)blockIdx.x * TWO + t2) * 16 + jn;
+        if (m < M && n < nout) {
+            float rr = total(e);
+            const int64_t at = (int64_t)m * nout + n;
+            if (EPI == FH_EPI_ADD2) rr = (rr + ea[at]) + eb[at];
+            if (EPI == FH_EPI_SWIGLU) rr = (rr / (__expf(-rr) + 1.0f)) * total(e + NE / 2);
+            y[at] = rr;
+        }
+    }
+}
+
+template <int T, int MR, int TW, int TS, int EPI>
+static fh_status qb_launch(const fh_qmatrix *q, const float *x, int m, float *y, const float *a, const float *b) {
+    constexpr int TWO = EPI == FH_EPI_SWIGLU ? TW / 2 : TW;
+    const int64_t nout = EPI == FH_EPI_SWIGLU ? q->n / 2 : q->n;
+    const int64_t groups = ((nout + 15) / 16 + TWO - 1) / TWO;
+    FH_REQUIRE(groups <= 0x7FFFFFFF, "matrix too large for one launch");
+    k_qmv_batch<T, MR, TW, TS, EPI><<<dim3((unsigned)groups), dim3(512), 0, q->dev->stream>>>(fh_view(q), x, m, y, a, b);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+// m <= 4: one tile (SwiGLU: gate + up tile) per workgroup, k over 8 (4) slices.  m <= 16: four tiles, two slices:
+// the staged activations (4 bytes per element and row) are then shared by enough weight rows.
+template <int T, int EPI>
+static fh_status qb_shape(const fh_qmatrix *q, const float *x, int m, float *y, const float *a, const float *b) {
+    if (m <= 4) {
+        if constexpr (EPI == FH_EPI_SWIGLU) return qb_launch<T, 4, 2, 4, EPI>(q, x, m, y, a, b);
+        else return qb_launch<T, 4, 1, 8, EPI>(q, x, m, y, a, b);
+    }
+    return qb_launch<T, 16, 4, 2, EPI>(q, x, m, y, a, b);
+}
+
+template <int T>
+static fh_status qb_epi(const fh_qmatrix *q, const float *x, int m, float *y, int epi, const float *a, const float *b) {
+    if (epi == FH_EPI_ADD2) return qb_shape<T, FH_EPI_ADD2>(q, x, m, y, a, b);
+    if (epi == FH_EPI_SWIGLU) return qb_shape<T, FH_EPI_SWIGLU>(q, x, m, y, a, b);
+    return qb_shape<T, FH_EPI_NONE>(q, x, m, y, a, b);
+}
+
+bool fh_qmatvec_batch_supports(const fh_qmatrix *q, int m, int epi) {
+    if (m < 1 || m > 16 || q->k % 256 != 0) return false;
+    if (epi == FH_EPI_SWIGLU && (q->n % 32) != 0) return false;
+    return true;
+}
+
+fh_status fh_launch_qmatvec_batch(const fh_qmatrix *q, const float *x, int m, float *y, int epi, const float *a,
+                                  const float *b) {
+    FH_REQUIRE(fh_qmatvec_batch_supports(q, m, epi), "shape not supported by the batch kernel");
+    switch (q->type) {
+    case FH_Q4_0: return qb_epi<FH_Q4_0>(q, x, m, y, epi, a, b);
+    case FH_Q8_0: return qb_epi<FH_Q8_0>(q, x, m, y, epi, a, b);
+    case FH_Q4_K: return qb_epi<FH_Q4_K>(q, x, m, y, epi, a, b);
+    case FH_Q6_K: return qb_epi<FH_Q6_K>(q, x, m, y, epi, a, b);
+    }
+    FH_FAIL(FH_ERR_UNSUPPORTED, "unsupported type %u", q->type);
+}

@@ -122,3 +122,77 @@ def test_prefill_shape_spot_check(dev, oracle, ty):
     got_sum = got.astype(np.float64).sum(axis=1)
     norm = np.sqrt((xf.astype(np.float64) ** 2).sum(axis=1) * (w ** 2).sum())
     assert np.all(np.abs(got_sum - want_sum) <= 1e-5 * norm)
+
+
+# ---------------------------------------------------------------------------------------------- batch kernel (m <= 16)
+@pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("m", [1, 3, 4, 7, 16])
+@pytest.mark.parametrize("n,k", [(272, 2048), (37, 256), (300, 3328), (64, 14336)])
+def test_batch_matvec_vs_checker(dev, oracle, ty, m, n, k):
+    """The 16-row matrix-core matvec: k of 1, 8, 13 and 56 chunks (fewer chunks than slices, a last round with idle
+    slices, more rounds than chunks in flight); n with a partial last tile and a partial last tile group."""
+    raw = synth.random_weight(ty, n, k, seed=120 + ty)
+    x = synth.random_activation(m, k, seed=130 + m)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    want = oracle.q_mat_mul(ty, x, raw, n)
+    dev.set_option("matvec_kernel", 4)
+    try:
+        out = Tensor.filled_bytes(dev, (m, n), 0xFF)
+        got = Tensor.from_slice(dev, x).q_mat_mul(q, out=out).as_slice()
+        assert_close(got, want, what=f"{NAMES[ty]} {n}x{k} m={m}")
+    finally:
+        dev.set_option("matvec_kernel", 0)
+
+
+@pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
+def test_batch_matvec_invariants(dev, oracle, ty):
+    """One-hot rows pick single weights (tests.rs:951-995), zero rows give exact zeros (:450-476), chunks of very
+    different magnitude in one row keep their own scale, ragged n (37 rows: three tiles, the last with 5 rows)."""
+    n, k, m = 37, 1024, 6
+    raw = synth.random_weight(ty, n, k, seed=140 + ty)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    w = oracle.dequantize(ty, raw).reshape(n, k)
+    x = np.zeros((m, k), np.float32)
+    cols = np.array([0, 255, 256, 700, 1023, 31])
+    x[np.arange(m), cols] = 0.125
+    x[3] = 0.0
+    dev.set_option("matvec_kernel", 4)
+    try:
+        y = Tensor.from_slice(dev, x).q_mat_mul(q, out=Tensor.filled_bytes(dev, (m, n), 0xFF)).as_slice()
+        for r in range(m):
+            want = np.zeros(n, np.float32) if r == 3 else np.float32(0.125) * w[:, cols[r]]
+            assert_close(y[r], want, abs_tol=1e-6, rel_tol=1e-6, what=f"one-hot row {r}")
+        assert not y[3].any()
+        xs = synth.random_activation(m, k, seed=141)
+        xs[1, :256] *= np.float32(1e12)
+        xs[2, 512:768] *= np.float32(1e-12)
+        got = Tensor.from_slice(dev, xs).q_mat_mul(q).as_slice()
+        want = oracle.q_mat_mul(ty, xs, raw, n)
+        scale = np.ones((m, 1), np.float32)
+        scale[1] = 1e-12
+        assert_close(got * scale, want * scale, what="chunks of mixed magnitude")
+    finally:
+        dev.set_option("matvec_kernel", 0)
+
+
+@pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("m", [1, 5, 16])
+def test_batch_matvec_epilogues(dev, oracle, ty, m):
+    """SwiGLU over stacked gate|up rows and the two-residual add (raw/attention_layer.rs:147-196), several rows."""
+    n, k = 96, 1024
+    raw_g = synth.random_weight(ty, n, k, seed=150 + ty, sigma=2e-3)
+    raw_u = synth.random_weight(ty, n, k, seed=151 + ty, sigma=2e-3)
+    x = synth.random_activation(m, k, seed=152)
+    g, u = QMatrix.from_raw_bytes(dev, (n, k), raw_g, ty), QMatrix.from_raw_bytes(dev, (n, k), raw_u, ty)
+    gu = QMatrix.concat_rows([g, u])
+    xt = Tensor.from_slice(dev, x)
+    a, b = synth.random_activation(m, n, seed=153), synth.random_activation(m, n, seed=154)
+    yg, yu = oracle.q_mat_mul(ty, x, raw_g, n), oracle.q_mat_mul(ty, x, raw_u, n)
+    dev.set_option("matvec_kernel", 4)
+    try:
+        got = xt.q_mat_mul_swiglu(gu).as_slice()
+        assert_close(got, oracle.swiglu(yg, yu), what=f"swiglu m={m}")
+        got = xt.q_mat_mul_add2(g, Tensor.from_slice(dev, a), Tensor.from_slice(dev, b)).as_slice()
+        assert_close(got, oracle.add3(yg, a, b), what=f"add2 m={m}")
+    finally:
+        dev.set_option("matvec_kernel", 0)
