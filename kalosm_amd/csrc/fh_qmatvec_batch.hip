@@ -272,8 +272,20 @@ __device__ __forceinline__ void qb_stage(uint8_t *img, int m, int lane, float4 v
 
 // ------------------------------------------------------------------------------ kernel
 // MR: activation rows held per image (4 or 16, m <= MR); TW x TS = 8 wavefronts; D weight chunks in flight.
-template <int T, int MR, int TW, int TS, int EPI>
-__global__ __launch_bounds__(512) void k_qmv_batch(QView q, const float *__restrict__ x, int M, float *__restrict__ y,
+// One wavefront per (chunk, row): the LDS image of every chunk, written to global memory [chunk][image bytes].
+template <int T, int MR>
+__global__ __launch_bounds__(256) void k_qb_prep(const float *__restrict__ x, int M, int64_t K, uint8_t *__restrict__ out) {
+    typedef QbLds<T, MR> L;
+    constexpr int IMG = (L::BYTES + 15) & ~15;
+    const int lane = threadIdx.x & 63, m = blockIdx.y * 4 + (threadIdx.x >> 6), c = blockIdx.x;
+    if (m >= M) return;
+    const float4 v = *(const float4 *)(x + (int64_t)m * K + (int64_t)c * 256 + lane * 4);
+    qb_stage<T, MR>(out + (int64_t)c * IMG, m, lane, v);
+}
+
+template <int T, int MR, int TW, int TS, int EPI, bool PRE>
+__global__ __launch_bounds__(512) void k_qmv_batch(QView q, const float *__restrict__ x,
+                                                   const uint8_t *__restrict__ ximg, int M, float *__restrict__ y,
                                                    const float *__restrict__ ea, const float *__restrict__ eb) {
     typedef QbLds<T, MR> L;
     static_assert(TW * TS == 8, "eight wavefronts");
@@ -294,22 +306,44 @@ __global__ __launch_bounds__(512) void k_qmv_batch(QView q, const float *__restr
     if (to >= tiles_out) to = tiles_out - 1; // a tile past the end re-reads the last one; its rows are never stored
     const int64_t tile = to + (int64_t)(tw / TWO) * (nout / 16); // up tiles follow the gate tiles
 
-    // staging duty of this wavefront in every round: items i = wave + 8r -> (chunk slot i % TS, row i / TS)
-    float4 xr[2][RPW];
+    // Round images come either from f32 activations converted here (PRE = false; staging duty of this wavefront in
+    // every round: items i = wave + 8r -> chunk slot i % TS, row i / TS) or as copies of images k_qb_prep wrote
+    // (PRE = true: the conversion is done once per call instead of once per workgroup).
+    constexpr int CPT = (ROUND / 16 + 511) / 512; // 16-byte pieces per thread and round
+    constexpr int NXR = PRE ? CPT : RPW;
+    float4 xr[2][NXR];
     auto load_x = [&](float4 *xv, int rr) {
+        if constexpr (PRE) {
+            const int valid = (C - rr * TS < TS ? C - rr * TS : TS) * (IMG / 16);
+            const float4 *src = (const float4 *)ximg + (int64_t)rr * (ROUND / 16);
 #pragma unroll
-        for (int r = 0; r < RPW; r++) {
-            const int i = wave + 8 * r, slot = i % TS, m = i / TS, c = rr * TS + slot;
-            xv[r] = (m < M && c < C) ? *(const float4 *)(x + (int64_t)m * K + (int64_t)c * 256 + lane * 4)
-                                     : make_float4(0, 0, 0, 0);
+            for (int r = 0; r < CPT; r++) {
+                const int i = tid + 512 * r;
+                xv[r] = i < valid ? src[i] : make_float4(0, 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < RPW; r++) {
+                const int i = wave + 8 * r, slot = i % TS, m = i / TS, c = rr * TS + slot;
+                xv[r] = (m < M && c < C) ? *(const float4 *)(x + (int64_t)m * K + (int64_t)c * 256 + lane * 4)
+                                         : make_float4(0, 0, 0, 0);
+            }
         }
     };
     auto stage = [&](const float4 *xv, int rr) {
         uint8_t *base = lds + (rr & 1) * ROUND;
+        if constexpr (PRE) {
 #pragma unroll
-        for (int r = 0; r < RPW; r++) {
-            const int i = wave + 8 * r, slot = i % TS, m = i / TS;
-            if (m < M) qb_stage<T, MR>(base + slot * IMG, m, lane, xv[r]);
+            for (int r = 0; r < CPT; r++) {
+                const int i = tid + 512 * r;
+                if (i < ROUND / 16) ((float4 *)base)[i] = xv[r];
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < RPW; r++) {
+                const int i = wave + 8 * r, slot = i % TS, m = i / TS;
+                if (m < M) qb_stage<T, MR>(base + slot * IMG, m, lane, xv[r]);
+            }
         }
     };
     auto chunk_of = [&](int rr) {
@@ -369,7 +403,23 @@ static fh_status qb_launch(const fh_qmatrix *q, const float *x, int m, float *y,
     const int64_t nout = EPI == FH_EPI_SWIGLU ? q->n / 2 : q->n;
     const int64_t groups = ((nout + 15) / 16 + TWO - 1) / TWO;
     FH_REQUIRE(groups <= 0x7FFFFFFF, "matrix too large for one launch");
-    k_qmv_batch<T, MR, TW, TS, EPI><<<dim3((unsigned)groups), dim3(512), 0, q->dev->stream>>>(fh_view(q), x, m, y, a, b);
+    fh_device *dev = q->dev;
+    // Converting the activations costs about as much as multiplying one tile by them: with many workgroups or
+    // many rows it is done once, in a launch of its own.
+    const int64_t pre_opt = dev->opt_matvec_per; // 0 auto, 1 never, 2 always
+    const bool pre = pre_opt == 2 || (pre_opt == 0 && m > 2);
+    if (pre) {
+        constexpr int IMG = (QbLds<T, MR>::BYTES + 15) & ~15;
+        const int chunks = (int)(q->k / 256);
+        FH_TRY(fh_dev_scratch(dev, &dev->act_buf, &dev->act_cap, (size_t)chunks * IMG));
+        k_qb_prep<T, MR><<<dim3((unsigned)chunks, (unsigned)((m + 3) / 4)), dim3(256), 0, dev->stream>>>(
+            x, m, q->k, (uint8_t *)dev->act_buf);
+        k_qmv_batch<T, MR, TW, TS, EPI, true><<<dim3((unsigned)groups), dim3(512), 0, dev->stream>>>(
+            fh_view(q), x, (const uint8_t *)dev->act_buf, m, y, a, b);
+    } else {
+        k_qmv_batch<T, MR, TW, TS, EPI, false><<<dim3((unsigned)groups), dim3(512), 0, dev->stream>>>(
+            fh_view(q), x, nullptr, m, y, a, b);
+    }
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
@@ -378,10 +428,16 @@ static fh_status qb_launch(const fh_qmatrix *q, const float *x, int m, float *y,
 // the staged activations (4 bytes per element and row) are then shared by enough weight rows.
 template <int T, int EPI>
 static fh_status qb_shape(const fh_qmatrix *q, const float *x, int m, float *y, const float *a, const float *b) {
+    const int64_t tiles = (q->n + 15) / 16;
+    const int64_t force = q->dev->opt_matvec_tiles; // 0 auto, else tiles per workgroup
     if (m <= 4) {
         if constexpr (EPI == FH_EPI_SWIGLU) return qb_launch<T, 4, 2, 4, EPI>(q, x, m, y, a, b);
-        else return qb_launch<T, 4, 1, 8, EPI>(q, x, m, y, a, b);
+        else {
+            if (force == 2 || (force == 0 && tiles >= 512)) return qb_launch<T, 4, 2, 4, EPI>(q, x, m, y, a, b);
+            return qb_launch<T, 4, 1, 8, EPI>(q, x, m, y, a, b);
+        }
     }
+    if (force == 2 || (force == 0 && tiles <= 512)) return qb_launch<T, 16, 2, 4, EPI>(q, x, m, y, a, b);
     return qb_launch<T, 16, 4, 2, EPI>(q, x, m, y, a, b);
 }
 

@@ -137,11 +137,14 @@ def test_batch_matvec_vs_checker(dev, oracle, ty, m, n, k):
     want = oracle.q_mat_mul(ty, x, raw, n)
     dev.set_option("matvec_kernel", 4)
     try:
-        out = Tensor.filled_bytes(dev, (m, n), 0xFF)
-        got = Tensor.from_slice(dev, x).q_mat_mul(q, out=out).as_slice()
-        assert_close(got, want, what=f"{NAMES[ty]} {n}x{k} m={m}")
+        for pre in (1, 2):  # activations converted inside the kernel / once by a launch of its own
+            dev.set_option("matvec_per", pre)
+            out = Tensor.filled_bytes(dev, (m, n), 0xFF)
+            got = Tensor.from_slice(dev, x).q_mat_mul(q, out=out).as_slice()
+            assert_close(got, want, what=f"{NAMES[ty]} {n}x{k} m={m} pre={pre}")
     finally:
         dev.set_option("matvec_kernel", 0)
+        dev.set_option("matvec_per", 0)
 
 
 @pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
