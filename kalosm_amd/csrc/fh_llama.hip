@@ -236,11 +236,19 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
     FH_TRY(fh_embed_rows(m->embd, m->ids, nullptr, s, m->x));
     for (int li = 0; li < c.n_layers; li++) {
         fh_llama_layer &l = m->layers[li];
-        FH_TRY(fh_rms_norm(dev, m->x, nullptr, l.attn_norm, nullptr, c.eps, s, D, m->xn));
+        // Decode steps fold each rms_norm into the matvec that consumes it (one launch instead of two).
+        const bool fuse = dev_pos && s == 1 && dev->opt_fuse_norm == 0 && dev->opt_matvec_kernel == 0;
+        bool qkv_done = false;
+        if (fuse && l.qkv && l.qkv->type == FH_Q4_K) {
+            fh_status st = fh_launch_q4k_m1_norm(l.qkv, m->x, nullptr, l.attn_norm, c.eps, m->qkv, FH_EPI_NONE, nullptr, nullptr);
+            if (st != FH_ERR_UNSUPPORTED) FH_TRY(st);
+            qkv_done = st == FH_OK;
+        }
+        if (!qkv_done) FH_TRY(fh_rms_norm(dev, m->x, nullptr, l.attn_norm, nullptr, c.eps, s, D, m->xn));
         const float *qp, *kp, *vp;
         int64_t row;
         if (l.qkv) {
-            FH_TRY(fh_qmatmul(l.qkv, m->xn, s, m->qkv));
+            if (!qkv_done) FH_TRY(fh_qmatmul(l.qkv, m->xn, s, m->qkv));
             row = QD + 2 * KD;
             qp = m->qkv;
             kp = m->qkv + QD;
@@ -278,8 +286,16 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
             att_in = m->att_t;
         }
         FH_TRY(fh_qmatmul(l.wo, att_in, s, m->attn_out));
-        FH_TRY(fh_rms_norm(dev, m->attn_out, m->x, l.ffn_norm, nullptr, c.eps, s, D, m->xn));
-        if (l.gate_up && s <= 2) {
+        bool ffn_done = false;
+        if (fuse && l.gate_up && l.gate_up->type == FH_Q4_K) {
+            fh_status st = fh_launch_q4k_m1_norm(l.gate_up, m->attn_out, m->x, l.ffn_norm, c.eps, m->act, FH_EPI_SWIGLU,
+                                                 nullptr, nullptr);
+            if (st != FH_ERR_UNSUPPORTED) FH_TRY(st);
+            ffn_done = st == FH_OK;
+        }
+        if (!ffn_done) FH_TRY(fh_rms_norm(dev, m->attn_out, m->x, l.ffn_norm, nullptr, c.eps, s, D, m->xn));
+        if (ffn_done) {
+        } else if (l.gate_up && s <= 2) {
             FH_TRY(fh_qmatmul_swiglu(l.gate_up, m->xn, s, m->act));
         } else if (l.gate_up) {
             FH_TRY(fh_qmatmul(l.gate_up, m->xn, s, m->gu)); // [s, 2F]: gate | up per row

@@ -40,7 +40,8 @@ __device__ __forceinline__ float dpp_f32(float v) {
 template <int TS, int PER, int EPI>
 __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__restrict__ x, float *__restrict__ y,
                                                       const float *__restrict__ ea, const float *__restrict__ eb,
-                                                      int SW) {
+                                                      int SW, const float *__restrict__ xres,
+                                                      const float *__restrict__ nw, float eps) {
     constexpr int NT = EPI == FH_EPI_SWIGLU ? 2 : 1;
     constexpr int TW = TS / NT;
     constexpr int XB = (PER + TS - 1) / TS; // blocks of x each wavefront stages: kb / (TS * SW) with SW * PER == kb
@@ -49,6 +50,7 @@ __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__res
     uint4 *img = lds;
     float *sf = (float *)(lds + kb * Q4K_IMG); // per block: [0..7] group sums, [8..15] factors
     float *l_red = sf + kb * 16;               // [TS][SW][16]
+    float *l_ss = l_red + 16 * 16;             // per wavefront: sum of squares of the blocks it staged
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, g = lane >> 4;
     const int nwaves = TS * SW;
     const int stream = wave / SW, slice = wave - stream * SW;
@@ -61,11 +63,16 @@ __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__res
 
     // ---- 0. the activations this wavefront stages (blocks wave, wave + nwaves, ...) are requested first:
     // they are needed first and are short
-    float4 xv[XB];
+    // With nw the input is rms_norm(x [+ xres]) * nw (composite/normalization.rs:287-401): the weight nw is
+    // folded into the staged values and the common factor 1 / rms is applied to the finished dot product.
+    float4 xv[XB], rv[XB], wv[XB];
 #pragma unroll
     for (int i = 0; i < XB; i++) {
         const int b = wave + i * nwaves;
-        xv[i] = *(const float4 *)(x + (int64_t)(b < kb ? b : 0) * 256 + lane * 4);
+        const int64_t at = (int64_t)(b < kb ? b : 0) * 256 + lane * 4;
+        xv[i] = *(const float4 *)(x + at);
+        if (xres) rv[i] = *(const float4 *)(xres + at);
+        if (nw) wv[i] = *(const float4 *)(nw + at);
     }
     // ---- 1. every weight byte of this wavefront goes in flight.  A tile past the end re-reads the last
     // tile (its rows are never stored); the host guarantees SW * PER == kb, so no block is out of range.
@@ -82,11 +89,17 @@ __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__res
         }
     }
     // ---- 2. stage x (lane owns k = 256*b + 4*lane .. +3)
+    float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < XB; i++) {
         const int b = wave + i * nwaves;
         if (b >= kb) break;
-        const float4 v = xv[i];
+        float4 v = xv[i];
+        if (xres) v = make_float4(v.x + rv[i].x, v.y + rv[i].y, v.z + rv[i].z, v.w + rv[i].w);
+        if (nw) {
+            ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
+            v = make_float4(v.x * wv[i].x, v.y * wv[i].y, v.z * wv[i].z, v.w * wv[i].w);
+        }
         float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
         amax = fmaxf(amax, dpp_f32<DPP_XOR1>(amax));
         amax = fmaxf(amax, dpp_f32<DPP_XOR2>(amax));
@@ -120,6 +133,11 @@ __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__res
             sf[b * 16 + s] = s4;
             sf[b * 16 + 8 + s] = __uint_as_float((uint32_t)(24 - e + 127) << 23);
         }
+    }
+    if (nw) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        if (lane == 0) l_ss[wave] = ss;
     }
     __syncthreads();
     // ---- 3. eight chained MFMA steps per block
@@ -176,6 +194,13 @@ __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__res
             v0 += l_red[(t * SW + s) * 16 + jr];
             if (NT == 2) v1 += l_red[((t + TW) * SW + s) * 16 + jr];
         }
+        if (nw) {
+            float tot = 0.f;
+            for (int w2 = 0; w2 < nwaves; w2++) tot += l_ss[w2];
+            const float rms = sqrtf(tot / (float)q.k + eps);
+            v0 = v0 / rms;
+            v1 = v1 / rms;
+        }
         const int64_t row = ((int64_t)blockIdx.x * TW + t) * 16 + jr;
         if (row < nout) {
             float rr = v0;
@@ -188,28 +213,35 @@ __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__res
 
 template <int TS, int PER, int EPI>
 static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b, int SW,
-                               unsigned grid, size_t lds) {
+                               unsigned grid, size_t lds, const float *xres, const float *nw, float eps) {
     static bool attr_done = false;
     if (!attr_done) {
         FH_HIP(hipFuncSetAttribute((const void *)k_qmv_q4k_m1<TS, PER, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    160 * 1024));
         attr_done = true;
     }
-    k_qmv_q4k_m1<TS, PER, EPI><<<dim3(grid), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW);
+    k_qmv_q4k_m1<TS, PER, EPI><<<dim3(grid), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, xres,
+                                                                                             nw, eps);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
 
 template <int TS, int EPI>
 static fh_status q4k_m1_per(int per, const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b,
-                            int SW, unsigned grid, size_t lds) {
-    if (per == 1) return q4k_m1_launch<TS, 1, EPI>(q, x, y, a, b, SW, grid, lds);
-    if (per == 2) return q4k_m1_launch<TS, 2, EPI>(q, x, y, a, b, SW, grid, lds);
-    return q4k_m1_launch<TS, 4, EPI>(q, x, y, a, b, SW, grid, lds);
+                            int SW, unsigned grid, size_t lds, const float *xres, const float *nw, float eps) {
+    if (per == 1) return q4k_m1_launch<TS, 1, EPI>(q, x, y, a, b, SW, grid, lds, xres, nw, eps);
+    if (per == 2) return q4k_m1_launch<TS, 2, EPI>(q, x, y, a, b, SW, grid, lds, xres, nw, eps);
+    return q4k_m1_launch<TS, 4, EPI>(q, x, y, a, b, SW, grid, lds, xres, nw, eps);
 }
 
 // Returns FH_ERR_UNSUPPORTED when the shape does not fit this kernel (the caller falls back).
 fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b) {
+    return fh_launch_q4k_m1_norm(q, x, nullptr, nullptr, 0.f, y, epi, a, b);
+}
+
+// The same product with the input taken as rms_norm(x [+ xres]) * nw when nw is given.
+fh_status fh_launch_q4k_m1_norm(const fh_qmatrix *q, const float *x, const float *xres, const float *nw, float eps,
+                                float *y, int epi, const float *a, const float *b) {
     fh_device *dev = q->dev;
     const int kb = (int)q->kb;
     const int nt = epi == FH_EPI_SWIGLU ? 2 : 1;
@@ -231,10 +263,10 @@ fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int ep
     while (TW > 1 && TW * nt * SW > 16) TW /= 2;
     const int TS = TW * nt;
     if (TS * SW > 16 || (TS != 1 && TS != 2 && TS != 4)) return FH_ERR_UNSUPPORTED;
-    size_t lds = (size_t)kb * Q4K_IMG * 16 + (size_t)kb * 64 + (size_t)TS * SW * 64;
+    size_t lds = (size_t)kb * Q4K_IMG * 16 + (size_t)kb * 64 + 16 * 64 + 64;
     if (lds > 160 * 1024) return FH_ERR_UNSUPPORTED;
     unsigned grid = (unsigned)((tiles + TW - 1) / TW);
-#define Q4K_M1_GO(TS_, EPI_) return q4k_m1_per<TS_, EPI_>(per, q, x, y, a, b, SW, grid, lds)
+#define Q4K_M1_GO(TS_, EPI_) return q4k_m1_per<TS_, EPI_>(per, q, x, y, a, b, SW, grid, lds, xres, nw, eps)
     if (epi == FH_EPI_SWIGLU) {
         if (TS == 2) Q4K_M1_GO(2, FH_EPI_SWIGLU);
         Q4K_M1_GO(4, FH_EPI_SWIGLU);
