@@ -37,8 +37,8 @@ __device__ __forceinline__ float dpp_f32(float v) {
 
 #define Q4K_IMG 65 // uint4 per block image: 8 steps x 4 groups x (hi, lo) + one all-zero slot
 
-template <int TS, int PER, int EPI>
-__global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__restrict__ x, float *__restrict__ y,
+template <int TS, int PER, int EPI, bool NORM>
+__device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict__ x, float *__restrict__ y,
                                                       const float *__restrict__ ea, const float *__restrict__ eb,
                                                       int SW, const float *__restrict__ xres,
                                                       const float *__restrict__ nw, float eps) {
@@ -71,8 +71,8 @@ __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__res
         const int b = wave + i * nwaves;
         const int64_t at = (int64_t)(b < kb ? b : 0) * 256 + lane * 4;
         xv[i] = *(const float4 *)(x + at);
-        if (xres) rv[i] = *(const float4 *)(xres + at);
-        if (nw) wv[i] = *(const float4 *)(nw + at);
+        if (NORM && xres) rv[i] = *(const float4 *)(xres + at);
+        if (NORM) wv[i] = *(const float4 *)(nw + at);
     }
     // ---- 1. every weight byte of this wavefront goes in flight.  A tile past the end re-reads the last
     // tile (its rows are never stored); the host guarantees SW * PER == kb, so no block is out of range.
@@ -95,8 +95,8 @@ __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__res
         const int b = wave + i * nwaves;
         if (b >= kb) break;
         float4 v = xv[i];
-        if (xres) v = make_float4(v.x + rv[i].x, v.y + rv[i].y, v.z + rv[i].z, v.w + rv[i].w);
-        if (nw) {
+        if (NORM && xres) v = make_float4(v.x + rv[i].x, v.y + rv[i].y, v.z + rv[i].z, v.w + rv[i].w);
+        if (NORM) {
             ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
             v = make_float4(v.x * wv[i].x, v.y * wv[i].y, v.z * wv[i].z, v.w * wv[i].w);
         }
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__res
             sf[b * 16 + 8 + s] = __uint_as_float((uint32_t)(24 - e + 127) << 23);
         }
     }
-    if (nw) {
+    if (NORM) {
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
         if (lane == 0) l_ss[wave] = ss;
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__res
             v0 += l_red[(t * SW + s) * 16 + jr];
             if (NT == 2) v1 += l_red[((t + TW) * SW + s) * 16 + jr];
         }
-        if (nw) {
+        if (NORM) {
             float tot = 0.f;
             for (int w2 = 0; w2 < nwaves; w2++) tot += l_ss[w2];
             const float rms = sqrtf(tot / (float)q.k + eps);
@@ -211,17 +211,34 @@ __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(QView q, const float *__res
     }
 }
 
+// The kernel proper.  With at most two blocks per wavefront the register budget of two resident workgroups
+// (64 VGPRs) is enforced: the kernel lives on the number of bytes in flight per compute unit.
+#define Q4K_M1_PARAMS                                                                                              \
+    QView q, const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ ea,                    \
+        const float *__restrict__ eb, int SW, const float *__restrict__ xres, const float *__restrict__ nw, float eps
+template <int TS, int PER, int EPI, bool NORM>
+__global__ __launch_bounds__(1024) void k_qmv_q4k_m1(Q4K_M1_PARAMS) {
+    qmv_q4k_m1_body<TS, PER, EPI, NORM>(q, x, y, ea, eb, SW, xres, nw, eps);
+}
+template <int TS, int PER, int EPI, bool NORM>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_qmv_q4k_m1_w8(Q4K_M1_PARAMS) {
+    qmv_q4k_m1_body<TS, PER, EPI, NORM>(q, x, y, ea, eb, SW, xres, nw, eps);
+}
+
 template <int TS, int PER, int EPI>
 static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b, int SW,
                                unsigned grid, size_t lds, const float *xres, const float *nw, float eps) {
-    static bool attr_done = false;
-    if (!attr_done) {
-        FH_HIP(hipFuncSetAttribute((const void *)k_qmv_q4k_m1<TS, PER, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   160 * 1024));
-        attr_done = true;
+    typedef void (*kern_t)(QView, const float *, float *, const float *, const float *, int, const float *, const float *,
+                           float);
+    kern_t kern;
+    if constexpr (PER <= 2) kern = nw ? k_qmv_q4k_m1_w8<TS, PER, EPI, true> : k_qmv_q4k_m1_w8<TS, PER, EPI, false>;
+    else kern = nw ? k_qmv_q4k_m1<TS, PER, EPI, true> : k_qmv_q4k_m1<TS, PER, EPI, false>;
+    static bool attr_done[2] = {false, false};
+    if (!attr_done[nw ? 1 : 0]) {
+        FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_done[nw ? 1 : 0] = true;
     }
-    k_qmv_q4k_m1<TS, PER, EPI><<<dim3(grid), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, xres,
-                                                                                             nw, eps);
+    kern<<<dim3(grid), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, xres, nw, eps);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
