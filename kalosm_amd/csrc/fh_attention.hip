@@ -351,7 +351,7 @@ extern "C" fh_status fh_flash_attention(fh_device *dev, int32_t dtype, const voi
 
 // Decode step with the KV length on the device (for graph replay): keys [0, *len_dev] are visible.
 // The grid is sized for max_len; splits past the live length write m = -inf, l = 0 and are ignored.
-fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
+fh_status fh_attention_decode_devlen_v1(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
                                      int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale,
                                      const int *len_dev, int max_len, float *out) {
     const int G = hq / hkv;

@@ -1,0 +1,266 @@
+// Attention of ONE query position against a KV cache whose length lives on the device (graph-replayed decode
+// steps): softmax(q . K^T * scale) . V with grouped-query heads.
+// Reference: fusor-ml/fusor/src/composite/flash_attention.rs:58-236 (semantics, no mask for a single query:
+// models/kalosm-llama/src/raw/mod.rs:969-972).
+//
+// grid (S splits, kv heads).  A workgroup owns the keys [split * chunk, (split + 1) * chunk) of one KV head, with
+// chunk = ceil(len / S) rounded up to 16 computed from the device-side length, and the G query heads that share
+// the KV head: K and V rows are read once for all of them.  A key row is spread over D / 8 lanes (32 bytes of f32
+// or 16 bytes of f16 each); the first four rows of every lane group, K and V, are requested before any arithmetic
+// so that one memory latency covers the usual chunk.  Partial results go to [q head][split][D + 4]:
+// unnormalised output, running max, running sum; k_attn_combine_dl (or the consumer of the partials) merges them.
+#include "fh_internal.h"
+
+typedef _Float16 fh_half;
+
+template <typename T>
+__device__ __forceinline__ void ad_load8(const T *p, float *o);
+template <>
+__device__ __forceinline__ void ad_load8<float>(const float *p, float *o) {
+    const float4 a = *(const float4 *)p, b = *(const float4 *)(p + 4);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+template <>
+__device__ __forceinline__ void ad_load8<fh_half>(const fh_half *p, float *o) {
+    const uint4 r = *(const uint4 *)p;
+    fh_half h[8];
+    __builtin_memcpy(h, &r, 16);
+#pragma unroll
+    for (int i = 0; i < 8; i++) o[i] = (float)h[i];
+}
+
+template <int CTRL>
+__device__ __forceinline__ float ad_dpp(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+// sum over the 16 lanes of a DPP row (all lanes get it): xor 1, xor 2, then mirrors of 8 and 16 over uniform groups
+__device__ __forceinline__ float ad_row16_sum(float a) {
+    a += ad_dpp<0xB1>(a);
+    a += ad_dpp<0x4E>(a);
+    a += ad_dpp<0x141>(a);
+    a += ad_dpp<0x140>(a);
+    return a;
+}
+// sum over the four rows of 16 lanes of a wavefront (lane i of every row gets it)
+__device__ __forceinline__ float ad_rows_sum(float a) {
+    const uint32_t u = __float_as_uint(a);
+    auto s16 = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    a = __uint_as_float(s16[0]) + __uint_as_float(s16[1]);
+    const uint32_t w = __float_as_uint(a);
+    auto s32 = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    return __uint_as_float(s32[0]) + __uint_as_float(s32[1]);
+}
+
+template <typename TKV, int D, int G, int NWV>
+__global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__restrict__ q, const TKV *__restrict__ k,
+                                                              const TKV *__restrict__ v, int64_t kv_sh, int64_t kv_st,
+                                                              const int *__restrict__ len_dev, float scale,
+                                                              int chunk_max, float *__restrict__ part) {
+    constexpr int LP = D / 8, RPW = 64 / LP, RW = NWV * RPW, U = 4;
+    static_assert(NWV >= G, "one wavefront per query head for the softmax statistics");
+    extern __shared__ float sm[];
+    float *s_sc = sm;                  // [G][chunk_max]
+    float *s_red = sm + G * chunk_max; // [NWV][G][D]
+    __shared__ float s_stat[2 * G];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, grp = lane / LP, c = lane % LP;
+    const int split = blockIdx.x, S = gridDim.x, kh = blockIdx.y;
+    const int skv = *len_dev + 1; // the step's own key is already appended at index len
+    int chunk = ((skv + S - 1) / S + 15) & ~15;
+    if (chunk > chunk_max) chunk = chunk_max;
+    const int c0 = split * chunk;
+    const int nk = min(skv, c0 + chunk) - c0; // <= 0 for trailing splits
+    const TKV *kb = k + kh * kv_sh + (int64_t)c0 * kv_st + 8 * c, *vb = v + kh * kv_sh + (int64_t)c0 * kv_st + 8 * c;
+    const int trow = wave * RPW + grp; // row of this lane group inside an iteration of RW rows
+
+    float kpre[U][8], vpre[U][8];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int t = u * RW + trow;
+        if (t < nk) ad_load8<TKV>(kb + (int64_t)t * kv_st, kpre[u]);
+        else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) kpre[u][i] = 0.f;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int t = u * RW + trow;
+        if (t < nk) ad_load8<TKV>(vb + (int64_t)t * kv_st, vpre[u]);
+        else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) vpre[u][i] = 0.f;
+        }
+    }
+    float qr[G][8];
+#pragma unroll
+    for (int h = 0; h < G; h++) {
+        const float4 a = *(const float4 *)(q + (int64_t)(kh * G + h) * D + 8 * c);
+        const float4 b = *(const float4 *)(q + (int64_t)(kh * G + h) * D + 8 * c + 4);
+        qr[h][0] = a.x; qr[h][1] = a.y; qr[h][2] = a.z; qr[h][3] = a.w;
+        qr[h][4] = b.x; qr[h][5] = b.y; qr[h][6] = b.z; qr[h][7] = b.w;
+    }
+    // ---- scores
+    auto score = [&](const float *kv8, int t) {
+#pragma unroll
+        for (int h = 0; h < G; h++) {
+            float a = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) a = fmaf(qr[h][i], kv8[i], a);
+            a = ad_row16_sum(a);
+            if (c == 0 && t < nk) s_sc[h * chunk_max + t] = a * scale;
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < U; u++)
+        if (u * RW < nk) score(kpre[u], u * RW + trow);
+    for (int t0 = U * RW; t0 < nk; t0 += RW) {
+        const int t = t0 + trow;
+        float kv8[8];
+        if (t < nk) ad_load8<TKV>(kb + (int64_t)t * kv_st, kv8);
+        else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) kv8[i] = 0.f;
+        }
+        score(kv8, t);
+    }
+    __syncthreads();
+    // ---- softmax statistics: wavefront h owns query head h
+    if (wave < G) {
+        const int h = wave;
+        float mx = -INFINITY;
+        for (int t = lane; t < nk; t += 64) mx = fmaxf(mx, s_sc[h * chunk_max + t]);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        float sum = 0.f;
+        for (int t = lane; t < nk; t += 64) {
+            const float p = __expf(s_sc[h * chunk_max + t] - mx);
+            s_sc[h * chunk_max + t] = p;
+            sum += p;
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+        if (lane == 0) {
+            s_stat[2 * h] = mx;
+            s_stat[2 * h + 1] = sum;
+        }
+    }
+    __syncthreads();
+    // ---- o[h][8c .. 8c+8) += p[h][t] * v[t][8c .. 8c+8)
+    float o[G][8];
+#pragma unroll
+    for (int h = 0; h < G; h++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[h][i] = 0.f;
+    auto accum = [&](const float *v8, int t) {
+        if (t < nk) {
+#pragma unroll
+            for (int h = 0; h < G; h++) {
+                const float p = s_sc[h * chunk_max + t];
+#pragma unroll
+                for (int i = 0; i < 8; i++) o[h][i] = fmaf(p, v8[i], o[h][i]);
+            }
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < U; u++)
+        if (u * RW < nk) accum(vpre[u], u * RW + trow);
+    for (int t0 = U * RW; t0 < nk; t0 += RW) {
+        const int t = t0 + trow;
+        float v8[8];
+        if (t < nk) {
+            ad_load8<TKV>(vb + (int64_t)t * kv_st, v8);
+            accum(v8, t);
+        }
+    }
+    // ---- add the row groups of the wavefront, then the wavefronts
+#pragma unroll
+    for (int h = 0; h < G; h++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[h][i] = ad_rows_sum(o[h][i]);
+    if (grp == 0) {
+#pragma unroll
+        for (int h = 0; h < G; h++) {
+            float *dst = s_red + (wave * G + h) * D + 8 * c;
+            *(float4 *)dst = make_float4(o[h][0], o[h][1], o[h][2], o[h][3]);
+            *(float4 *)(dst + 4) = make_float4(o[h][4], o[h][5], o[h][6], o[h][7]);
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < G * D; idx += 64 * NWV) {
+        const int h = idx / D, dd = idx % D;
+        float a = 0.f;
+#pragma unroll
+        for (int w = 0; w < NWV; w++) a += s_red[(w * G + h) * D + dd];
+        float *pp = part + ((int64_t)(kh * G + h) * S + split) * (D + 4);
+        pp[dd] = a;
+        if (dd == 0) {
+            pp[D] = nk > 0 ? s_stat[2 * h] : -INFINITY;
+            pp[D + 1] = nk > 0 ? s_stat[2 * h + 1] : 0.f;
+        }
+    }
+}
+
+template <int D>
+__global__ __launch_bounds__(D) void k_attn_combine_dl(const float *__restrict__ part, int splits, float *__restrict__ out) {
+    const int64_t h = blockIdx.x;
+    const float *pp = part + h * splits * (D + 4);
+    float mx = -INFINITY;
+    for (int s = 0; s < splits; s++) mx = fmaxf(mx, pp[s * (D + 4) + D]);
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < splits; s++) {
+        const float m = pp[s * (D + 4) + D];
+        const float w = (m == -INFINITY) ? 0.f : __expf(m - mx);
+        num = fmaf(pp[s * (D + 4) + threadIdx.x], w, num);
+        den = fmaf(pp[s * (D + 4) + D + 1], w, den);
+    }
+    out[h * D + threadIdx.x] = num / den;
+}
+
+template <typename TKV, int G>
+static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const void *v, int64_t kv_sh, int64_t kv_st,
+                           int hq, int hkv, float scale, const int *len_dev, int max_len, float *out, int *splits_out) {
+    constexpr int D = 128, NWV = 16;
+    // splits: about 256 keys of capacity each, between 4 and 16 (the consumer of the partials reads all of them)
+    int S = dev->opt_attn_splits > 0 ? (int)dev->opt_attn_splits : (max_len + 255) / 256;
+    S = S < 4 ? 4 : (S > 16 ? 16 : S);
+    const int chunk_max = ((max_len + S - 1) / S + 15) & ~15;
+    const size_t lds = ((size_t)G * chunk_max + (size_t)NWV * G * D) * 4;
+    FH_REQUIRE(lds <= 150 * 1024, "KV capacity %d too large for the decode attention kernel", max_len);
+    FH_TRY(fh_dev_scratch(dev, (void **)&dev->part_buf, &dev->part_cap, (size_t)hq * S * (D + 4) * 4));
+    static bool attr_done = false;
+    if (!attr_done) {
+        FH_HIP(hipFuncSetAttribute((const void *)k_attn_decode_dl<TKV, D, G, NWV>,
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024));
+        attr_done = true;
+    }
+    k_attn_decode_dl<TKV, D, G, NWV><<<dim3((unsigned)S, (unsigned)hkv), dim3(64 * NWV), lds, dev->stream>>>(
+        q, (const TKV *)k, (const TKV *)v, kv_sh, kv_st, len_dev, scale, chunk_max, dev->part_buf);
+    FH_HIP(hipGetLastError());
+    if (splits_out) *splits_out = S;
+    if (out) {
+        k_attn_combine_dl<D><<<dim3((unsigned)hq), dim3(D), 0, dev->stream>>>(dev->part_buf, S, out);
+        FH_HIP(hipGetLastError());
+    }
+    return FH_OK;
+}
+
+// out != NULL: the attention output [hq, d].  out == NULL: the partials stay in the device's scratch
+// ([hq][*splits_out][d + 4]) for a consumer that merges them itself.
+fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
+                                     int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale,
+                                     const int *len_dev, int max_len, float *out, int *splits_out) {
+    const int G = hq / hkv;
+    if (d != 128 || (G != 1 && G != 2 && G != 4 && G != 8) || kv_st % 8 || kv_sh % 8) return FH_ERR_UNSUPPORTED;
+#define AD_GO(TKV_)                                                                                                   \
+    switch (G) {                                                                                                      \
+    case 1: return ad_launch<TKV_, 1>(dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out);  \
+    case 2: return ad_launch<TKV_, 2>(dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out);  \
+    case 4: return ad_launch<TKV_, 4>(dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out);  \
+    default: return ad_launch<TKV_, 8>(dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out); \
+    }
+    if (kv_dtype == FH_F16) {
+        AD_GO(fh_half)
+    }
+    AD_GO(float)
+#undef AD_GO
+}

@@ -181,6 +181,7 @@ extern "C" fh_status fh_set_option(fh_device *dev, const char *key, int64_t valu
     else if (!strcmp(key, "matvec_tiles")) dev->opt_matvec_tiles = value;
     else if (!strcmp(key, "matvec_per")) dev->opt_matvec_per = value;
     else if (!strcmp(key, "attn_splits")) dev->opt_attn_splits = value;
+    else if (!strcmp(key, "attn_kernel")) dev->opt_attn_kernel = value;
     else if (!strcmp(key, "matmul_kernel")) dev->opt_matmul_kernel = value;
     else if (!strcmp(key, "fuse_norm")) dev->opt_fuse_norm = value;
     else FH_FAIL(FH_ERR_INVALID, "unknown option '%s'", key);

@@ -55,6 +55,7 @@ struct fh_device {
     int64_t opt_matvec_tiles = 0;    // 0 auto, else 1 / 2 / 4 row tiles per workgroup
     int64_t opt_matvec_per = 0;      // 0 auto, else 1 / 2 / 4 blocks per wavefront
     int64_t opt_attn_splits = 0;     // 0 auto
+    int64_t opt_attn_kernel = 0;     // 0 auto, 1 first-generation decode attention
     int64_t opt_fuse_norm = 0;       // 0: decode steps fold rms_norm into the consuming matvec, 1: separate launches
     int64_t opt_matmul_kernel = 0;   // 0 auto, 1 generic for every m, 2 MFMA tile kernel for every m
 };
@@ -168,9 +169,12 @@ fh_status fh_kvcache_append_kv(fh_kvcache *c, int layer, const float *k, int64_t
 fh_status fh_kvcache_set_len_dev(fh_kvcache *c, int len);
 fh_status fh_swiglu_rows(fh_device *dev, const float *gu, int rows, int f, float *y);
 // decode attention reading the KV length from a device int (graph friendly)
-fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *q, const void *k,
+fh_status fh_attention_decode_devlen_v1(fh_device *dev, int kv_dtype, const float *q, const void *k,
                                      const void *v, int64_t kv_sh, int64_t kv_st, int hq, int hkv,
                                      int d, float scale, const int *len_dev, int max_len, float *out);
+fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
+                                     int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale,
+                                     const int *len_dev, int max_len, float *out, int *splits_out);
 fh_status fh_rope_pair_devpos(fh_device *dev, const float *q, const float *k, int hq, int hk, int d,
                               const float *cos_t, const float *sin_t, int table_rows,
                               const int *pos_dev, float *q_out, float *k_out);

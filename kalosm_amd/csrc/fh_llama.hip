@@ -266,8 +266,15 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
             FH_TRY(fh_rope_kv_decode(m->cache, li, qp, kp, vp, H, m->cos_t, m->sin_t, c.ctx, m->qrot));
             size_t plane = (size_t)HK * m->cache->capacity * hd * fh_dtype_size(c.kv_dtype);
             const uint8_t *kc = (const uint8_t *)m->cache->k + li * plane, *vc = (const uint8_t *)m->cache->v + li * plane;
-            FH_TRY(fh_attention_decode_devlen(dev, c.kv_dtype, m->qrot, kc, vc, (int64_t)m->cache->capacity * hd, hd, H, HK,
-                                              hd, scale, m->cache->len_dev, m->cache->capacity, m->att));
+            fh_status ast = dev->opt_attn_kernel == 1
+                                ? FH_ERR_UNSUPPORTED
+                                : fh_attention_decode_devlen(dev, c.kv_dtype, m->qrot, kc, vc, (int64_t)m->cache->capacity * hd,
+                                                             hd, H, HK, hd, scale, m->cache->len_dev, m->cache->capacity,
+                                                             m->att, nullptr);
+            if (ast == FH_ERR_UNSUPPORTED)
+                ast = fh_attention_decode_devlen_v1(dev, c.kv_dtype, m->qrot, kc, vc, (int64_t)m->cache->capacity * hd, hd, H,
+                                                    HK, hd, scale, m->cache->len_dev, m->cache->capacity, m->att);
+            FH_TRY(ast);
         } else {
             FH_TRY(fh_rope_pair(dev, qp, 0, hd, q_st, kp, 0, hd, k_st, 1, H, HK, s, hd, m->cos_t, m->sin_t, c.ctx, pos, 1,
                                 m->qrot, m->krot));
