@@ -244,6 +244,13 @@ static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const 
     return FH_OK;
 }
 
+// Merge the partials fh_attention_decode_devlen left in the device's scratch (head_dim 128).
+fh_status fh_attention_combine_dl(fh_device *dev, int hq, int splits, float *out) {
+    k_attn_combine_dl<128><<<dim3((unsigned)hq), dim3(128), 0, dev->stream>>>(dev->part_buf, splits, out);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
 // out != NULL: the attention output [hq, d].  out == NULL: the partials stay in the device's scratch
 // ([hq][*splits_out][d + 4]) for a consumer that merges them itself.
 fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,

@@ -148,6 +148,8 @@ enum { FH_EPI_NONE = 0, FH_EPI_ADD2 = 1, FH_EPI_SWIGLU = 2 };
 fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b);
 fh_status fh_launch_q4k_m1_norm(const fh_qmatrix *q, const float *x, const float *xres, const float *nw, float eps,
                                 float *y, int epi, const float *a, const float *b);
+fh_status fh_launch_q4k_m1_attn(const fh_qmatrix *q, const float *part, int nsplit, float *y);
+fh_status fh_attention_combine_dl(fh_device *dev, int hq, int splits, float *out);
 fh_status fh_launch_q6k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b);
 
 struct fh_kvcache {

@@ -238,7 +238,7 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
         fh_llama_layer &l = m->layers[li];
         // Decode steps fold each rms_norm into the matvec that consumes it (one launch instead of two).
         const bool fuse = dev_pos && s == 1 && dev->opt_fuse_norm == 0 && dev->opt_matvec_kernel == 0;
-        bool qkv_done = false;
+        bool qkv_done = false, wo_done = false;
         if (fuse && l.qkv && l.qkv->type == FH_Q4_K) {
             fh_status st = fh_launch_q4k_m1_norm(l.qkv, m->x, nullptr, l.attn_norm, c.eps, m->qkv, FH_EPI_NONE, nullptr, nullptr);
             if (st != FH_ERR_UNSUPPORTED) FH_TRY(st);
@@ -266,14 +266,24 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
             FH_TRY(fh_rope_kv_decode(m->cache, li, qp, kp, vp, H, m->cos_t, m->sin_t, c.ctx, m->qrot));
             size_t plane = (size_t)HK * m->cache->capacity * hd * fh_dtype_size(c.kv_dtype);
             const uint8_t *kc = (const uint8_t *)m->cache->k + li * plane, *vc = (const uint8_t *)m->cache->v + li * plane;
+            // The partial results of the attention splits are merged by the output projection itself when it is a
+            // Q4_K matrix (no launch for the merge); otherwise by a small kernel.
+            const bool merge_in_wo = fuse && l.wo->type == FH_Q4_K && hd == 128;
+            int nsplit = 0;
             fh_status ast = dev->opt_attn_kernel == 1
                                 ? FH_ERR_UNSUPPORTED
                                 : fh_attention_decode_devlen(dev, c.kv_dtype, m->qrot, kc, vc, (int64_t)m->cache->capacity * hd,
                                                              hd, H, HK, hd, scale, m->cache->len_dev, m->cache->capacity,
-                                                             m->att, nullptr);
+                                                             merge_in_wo ? nullptr : m->att, &nsplit);
             if (ast == FH_ERR_UNSUPPORTED)
                 ast = fh_attention_decode_devlen_v1(dev, c.kv_dtype, m->qrot, kc, vc, (int64_t)m->cache->capacity * hd, hd, H,
                                                     HK, hd, scale, m->cache->len_dev, m->cache->capacity, m->att);
+            else if (ast == FH_OK && merge_in_wo) {
+                fh_status st = fh_launch_q4k_m1_attn(l.wo, dev->part_buf, nsplit, m->attn_out);
+                if (st == FH_ERR_UNSUPPORTED) st = fh_attention_combine_dl(dev, H, nsplit, m->att);
+                else wo_done = st == FH_OK;
+                ast = st;
+            }
             FH_TRY(ast);
         } else {
             FH_TRY(fh_rope_pair(dev, qp, 0, hd, q_st, kp, 0, hd, k_st, 1, H, HK, s, hd, m->cos_t, m->sin_t, c.ctx, pos, 1,
@@ -292,7 +302,7 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
             FH_TRY(fh_transpose_shd(dev, m->att, H, s, hd, m->att_t));
             att_in = m->att_t;
         }
-        FH_TRY(fh_qmatmul(l.wo, att_in, s, m->attn_out));
+        if (!wo_done) FH_TRY(fh_qmatmul(l.wo, att_in, s, m->attn_out));
         bool ffn_done = false;
         if (fuse && l.gate_up && l.gate_up->type == FH_Q4_K) {
             fh_status st = fh_launch_q4k_m1_norm(l.gate_up, m->attn_out, m->x, l.ffn_norm, c.eps, m->act, FH_EPI_SWIGLU,

@@ -37,11 +37,11 @@ __device__ __forceinline__ float dpp_f32(float v) {
 
 #define Q4K_IMG 65 // uint4 per block image: 8 steps x 4 groups x (hi, lo) + one all-zero slot
 
-template <int TS, int PER, int EPI, bool NORM>
+template <int TS, int PER, int EPI, int IN>
 __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict__ x, float *__restrict__ y,
                                                       const float *__restrict__ ea, const float *__restrict__ eb,
                                                       int SW, const float *__restrict__ xres,
-                                                      const float *__restrict__ nw, float eps) {
+                                                      const float *__restrict__ nw, float eps, int nsplit) {
     constexpr int NT = EPI == FH_EPI_SWIGLU ? 2 : 1;
     constexpr int TW = TS / NT;
     constexpr int XB = (PER + TS - 1) / TS; // blocks of x each wavefront stages: kb / (TS * SW) with SW * PER == kb
@@ -65,14 +65,24 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     // they are needed first and are short
     // With nw the input is rms_norm(x [+ xres]) * nw (composite/normalization.rs:287-401): the weight nw is
     // folded into the staged values and the common factor 1 / rms is applied to the finished dot product.
-    float4 xv[XB], rv[XB], wv[XB];
+    float4 xv[XB], rv[XB], wv[XB], pacc[IN == 2 ? XB : 1][8];
+    float2 pm[IN == 2 ? XB : 1][8];
 #pragma unroll
     for (int i = 0; i < XB; i++) {
         const int b = wave + i * nwaves;
         const int64_t at = (int64_t)(b < kb ? b : 0) * 256 + lane * 4;
-        xv[i] = *(const float4 *)(x + at);
-        if (NORM && xres) rv[i] = *(const float4 *)(xres + at);
-        if (NORM) wv[i] = *(const float4 *)(nw + at);
+        if (IN != 2) xv[i] = *(const float4 *)(x + at);
+        if (IN == 1 && xres) rv[i] = *(const float4 *)(xres + at);
+        if (IN == 1) wv[i] = *(const float4 *)(nw + at);
+        if (IN == 2) { // x holds attention partials [head][nsplit][128 + 4]: unnormalised output, max, sum
+            const float *pp = x + (at >> 7) * nsplit * 132;
+#pragma unroll
+            for (int s = 0; s < 8; s++)
+                if (s < nsplit) {
+                    pacc[i][s] = *(const float4 *)(pp + s * 132 + (at & 127));
+                    pm[i][s] = *(const float2 *)(pp + s * 132 + 128);
+                }
+        }
     }
     // ---- 1. every weight byte of this wavefront goes in flight.  A tile past the end re-reads the last
     // tile (its rows are never stored); the host guarantees SW * PER == kb, so no block is out of range.
@@ -95,8 +105,25 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         const int b = wave + i * nwaves;
         if (b >= kb) break;
         float4 v = xv[i];
-        if (NORM && xres) v = make_float4(v.x + rv[i].x, v.y + rv[i].y, v.z + rv[i].z, v.w + rv[i].w);
-        if (NORM) {
+        if (IN == 2) { // merge the splits: softmax weights exp(m_s - max), then num / den
+            float mx = -INFINITY;
+#pragma unroll
+            for (int s = 0; s < 8; s++)
+                if (s < nsplit) mx = fmaxf(mx, pm[i][s].x);
+            float den = 0.f;
+            v = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int s = 0; s < 8; s++)
+                if (s < nsplit) {
+                    const float w = pm[i][s].x == -INFINITY ? 0.f : __expf(pm[i][s].x - mx);
+                    den = fmaf(pm[i][s].y, w, den);
+                    v.x = fmaf(pacc[i][s].x, w, v.x); v.y = fmaf(pacc[i][s].y, w, v.y);
+                    v.z = fmaf(pacc[i][s].z, w, v.z); v.w = fmaf(pacc[i][s].w, w, v.w);
+                }
+            v = make_float4(v.x / den, v.y / den, v.z / den, v.w / den);
+        }
+        if (IN == 1 && xres) v = make_float4(v.x + rv[i].x, v.y + rv[i].y, v.z + rv[i].z, v.w + rv[i].w);
+        if (IN == 1) {
             ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
             v = make_float4(v.x * wv[i].x, v.y * wv[i].y, v.z * wv[i].z, v.w * wv[i].w);
         }
@@ -134,7 +161,7 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
             sf[b * 16 + 8 + s] = __uint_as_float((uint32_t)(24 - e + 127) << 23);
         }
     }
-    if (NORM) {
+    if (IN == 1) {
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
         if (lane == 0) l_ss[wave] = ss;
@@ -194,7 +221,7 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
             v0 += l_red[(t * SW + s) * 16 + jr];
             if (NT == 2) v1 += l_red[((t + TW) * SW + s) * 16 + jr];
         }
-        if (NORM) {
+        if (IN == 1) {
             float tot = 0.f;
             for (int w2 = 0; w2 < nwaves; w2++) tot += l_ss[w2];
             const float rms = sqrtf(tot / (float)q.k + eps);
@@ -215,40 +242,45 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
 // (64 VGPRs) is enforced: the kernel lives on the number of bytes in flight per compute unit.
 #define Q4K_M1_PARAMS                                                                                              \
     QView q, const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ ea,                    \
-        const float *__restrict__ eb, int SW, const float *__restrict__ xres, const float *__restrict__ nw, float eps
-template <int TS, int PER, int EPI, bool NORM>
+        const float *__restrict__ eb, int SW, const float *__restrict__ xres, const float *__restrict__ nw, float eps, int nsplit
+template <int TS, int PER, int EPI, int IN>
 __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(Q4K_M1_PARAMS) {
-    qmv_q4k_m1_body<TS, PER, EPI, NORM>(q, x, y, ea, eb, SW, xres, nw, eps);
+    qmv_q4k_m1_body<TS, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit);
 }
-template <int TS, int PER, int EPI, bool NORM>
+template <int TS, int PER, int EPI, int IN>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_qmv_q4k_m1_w8(Q4K_M1_PARAMS) {
-    qmv_q4k_m1_body<TS, PER, EPI, NORM>(q, x, y, ea, eb, SW, xres, nw, eps);
+    qmv_q4k_m1_body<TS, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit);
 }
 
 template <int TS, int PER, int EPI>
 static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b, int SW,
-                               unsigned grid, size_t lds, const float *xres, const float *nw, float eps) {
+                               unsigned grid, size_t lds, const float *xres, const float *nw, float eps, int nsplit) {
     typedef void (*kern_t)(QView, const float *, float *, const float *, const float *, int, const float *, const float *,
-                           float);
+                           float, int);
     kern_t kern;
-    if constexpr (PER <= 2) kern = nw ? k_qmv_q4k_m1_w8<TS, PER, EPI, true> : k_qmv_q4k_m1_w8<TS, PER, EPI, false>;
-    else kern = nw ? k_qmv_q4k_m1<TS, PER, EPI, true> : k_qmv_q4k_m1<TS, PER, EPI, false>;
-    static bool attr_done[2] = {false, false};
-    if (!attr_done[nw ? 1 : 0]) {
-        FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_done[nw ? 1 : 0] = true;
+    const int in = nsplit > 0 ? 2 : (nw ? 1 : 0); // input: plain, rms_norm, attention partials
+    if constexpr (PER <= 2) {
+        kern = in == 2 ? k_qmv_q4k_m1<TS, PER, EPI, 2>
+                       : (in == 1 ? k_qmv_q4k_m1_w8<TS, PER, EPI, 1> : k_qmv_q4k_m1_w8<TS, PER, EPI, 0>);
+    } else {
+        kern = in == 2 ? k_qmv_q4k_m1<TS, PER, EPI, 2> : (in == 1 ? k_qmv_q4k_m1<TS, PER, EPI, 1> : k_qmv_q4k_m1<TS, PER, EPI, 0>);
     }
-    kern<<<dim3(grid), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, xres, nw, eps);
+    static bool attr_done[3] = {false, false, false};
+    if (!attr_done[in]) {
+        FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_done[in] = true;
+    }
+    kern<<<dim3(grid), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, xres, nw, eps, nsplit);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
 
 template <int TS, int EPI>
 static fh_status q4k_m1_per(int per, const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b,
-                            int SW, unsigned grid, size_t lds, const float *xres, const float *nw, float eps) {
-    if (per == 1) return q4k_m1_launch<TS, 1, EPI>(q, x, y, a, b, SW, grid, lds, xres, nw, eps);
-    if (per == 2) return q4k_m1_launch<TS, 2, EPI>(q, x, y, a, b, SW, grid, lds, xres, nw, eps);
-    return q4k_m1_launch<TS, 4, EPI>(q, x, y, a, b, SW, grid, lds, xres, nw, eps);
+                            int SW, unsigned grid, size_t lds, const float *xres, const float *nw, float eps, int nsplit) {
+    if (per == 1) return q4k_m1_launch<TS, 1, EPI>(q, x, y, a, b, SW, grid, lds, xres, nw, eps, nsplit);
+    if (per == 2) return q4k_m1_launch<TS, 2, EPI>(q, x, y, a, b, SW, grid, lds, xres, nw, eps, nsplit);
+    return q4k_m1_launch<TS, 4, EPI>(q, x, y, a, b, SW, grid, lds, xres, nw, eps, nsplit);
 }
 
 // Returns FH_ERR_UNSUPPORTED when the shape does not fit this kernel (the caller falls back).
@@ -256,9 +288,24 @@ fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int ep
     return fh_launch_q4k_m1_norm(q, x, nullptr, nullptr, 0.f, y, epi, a, b);
 }
 
+static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const float *xres, const float *nw, float eps, int nsplit,
+                            float *y, int epi, const float *a, const float *b);
+
+// The same product with the input merged from the partial results of the decode-step attention
+// (x = [head][nsplit][128 + 4]; head_dim 128, nsplit <= 8).
+fh_status fh_launch_q4k_m1_attn(const fh_qmatrix *q, const float *part, int nsplit, float *y) {
+    if (nsplit < 1 || nsplit > 8 || q->k % 128) return FH_ERR_UNSUPPORTED;
+    return q4k_m1_any(q, part, nullptr, nullptr, 0.f, nsplit, y, FH_EPI_NONE, nullptr, nullptr);
+}
+
 // The same product with the input taken as rms_norm(x [+ xres]) * nw when nw is given.
 fh_status fh_launch_q4k_m1_norm(const fh_qmatrix *q, const float *x, const float *xres, const float *nw, float eps,
                                 float *y, int epi, const float *a, const float *b) {
+    return q4k_m1_any(q, x, xres, nw, eps, 0, y, epi, a, b);
+}
+
+static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const float *xres, const float *nw, float eps, int nsplit,
+                            float *y, int epi, const float *a, const float *b) {
     fh_device *dev = q->dev;
     const int kb = (int)q->kb;
     const int nt = epi == FH_EPI_SWIGLU ? 2 : 1;
@@ -283,7 +330,7 @@ fh_status fh_launch_q4k_m1_norm(const fh_qmatrix *q, const float *x, const float
     size_t lds = (size_t)kb * Q4K_IMG * 16 + (size_t)kb * 64 + 16 * 64 + 64;
     if (lds > 160 * 1024) return FH_ERR_UNSUPPORTED;
     unsigned grid = (unsigned)((tiles + TW - 1) / TW);
-#define Q4K_M1_GO(TS_, EPI_) return q4k_m1_per<TS_, EPI_>(per, q, x, y, a, b, SW, grid, lds, xres, nw, eps)
+#define Q4K_M1_GO(TS_, EPI_) return q4k_m1_per<TS_, EPI_>(per, q, x, y, a, b, SW, grid, lds, xres, nw, eps, nsplit)
     if (epi == FH_EPI_SWIGLU) {
         if (TS == 2) Q4K_M1_GO(2, FH_EPI_SWIGLU);
         Q4K_M1_GO(4, FH_EPI_SWIGLU);
