@@ -144,7 +144,7 @@ bool fh_qmatvec_batch_supports(const fh_qmatrix *q, int m, int epi);
 fh_status fh_launch_qmatvec_batch(const fh_qmatrix *q, const float *x, int m, float *y, int epi, const float *a,
                                   const float *b);
 fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y);
-enum { FH_EPI_NONE = 0, FH_EPI_ADD2 = 1, FH_EPI_SWIGLU = 2 };
+enum { FH_EPI_NONE = 0, FH_EPI_ADD2 = 1, FH_EPI_SWIGLU = 2, FH_EPI_ROPEKV = 3 };
 fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b);
 fh_status fh_launch_q4k_m1_norm(const fh_qmatrix *q, const float *x, const float *xres, const float *nw, float eps,
                                 float *y, int epi, const float *a, const float *b);
@@ -164,6 +164,9 @@ fh_status fh_kvcache_reserve(fh_kvcache *c, int required);
 // append reading the write position from c->len_dev (graph friendly), s == 1
 fh_status fh_kvcache_append_devpos(fh_kvcache *c, int layer, const float *k, const float *v, int64_t sh);
 fh_status fh_kvcache_advance_dev(fh_kvcache *c);
+fh_status fh_launch_q4k_m1_ropekv(const fh_qmatrix *q, const float *x, const float *nw, float eps, fh_kvcache *c,
+                                  int layer, int hq, const float *cos_t, const float *sin_t, int table_rows,
+                                  float *q_out);
 fh_status fh_rope_kv_decode(fh_kvcache *c, int layer, const float *q, const float *k, const float *v, int hq,
                             const float *cos_t, const float *sin_t, int table_rows, float *q_out);
 fh_status fh_kvcache_append_kv(fh_kvcache *c, int layer, const float *k, int64_t k_sh, int64_t k_st, const float *v,

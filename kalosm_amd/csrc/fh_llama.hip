@@ -239,8 +239,14 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
         // Decode steps fold each rms_norm into the matvec that consumes it (one launch instead of two).
         const bool fuse = dev_pos && s == 1 && dev->opt_fuse_norm == 0 && dev->opt_matvec_kernel == 0;
         bool qkv_done = false, wo_done = false;
+        bool rope_done = false;
         if (fuse && l.qkv && l.qkv->type == FH_Q4_K) {
-            fh_status st = fh_launch_q4k_m1_norm(l.qkv, m->x, nullptr, l.attn_norm, c.eps, m->qkv, FH_EPI_NONE, nullptr, nullptr);
+            // norm + projection + rope + cache append in one launch; without the rope epilogue as second choice
+            fh_status st = fh_launch_q4k_m1_ropekv(l.qkv, m->x, l.attn_norm, c.eps, m->cache, li, H, m->cos_t, m->sin_t, c.ctx,
+                                                   m->qrot);
+            rope_done = st == FH_OK;
+            if (st == FH_ERR_UNSUPPORTED)
+                st = fh_launch_q4k_m1_norm(l.qkv, m->x, nullptr, l.attn_norm, c.eps, m->qkv, FH_EPI_NONE, nullptr, nullptr);
             if (st != FH_ERR_UNSUPPORTED) FH_TRY(st);
             qkv_done = st == FH_OK;
         }
@@ -263,7 +269,7 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
         }
         const int64_t q_st = row ? row : QD, k_st = row ? row : KD;
         if (dev_pos) {
-            FH_TRY(fh_rope_kv_decode(m->cache, li, qp, kp, vp, H, m->cos_t, m->sin_t, c.ctx, m->qrot));
+            if (!rope_done) FH_TRY(fh_rope_kv_decode(m->cache, li, qp, kp, vp, H, m->cos_t, m->sin_t, c.ctx, m->qrot));
             size_t plane = (size_t)HK * m->cache->capacity * hd * fh_dtype_size(c.kv_dtype);
             const uint8_t *kc = (const uint8_t *)m->cache->k + li * plane, *vc = (const uint8_t *)m->cache->v + li * plane;
             // The partial results of the attention splits are merged by the output projection itself when it is a

@@ -35,13 +35,32 @@ __device__ __forceinline__ float dpp_f32(float v) {
     return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
 }
 
+// Arguments of the rope + KV-append epilogue (the fused q|k|v projection of a decode step): rows [0, qd) are query
+// rows (rotated, written to qo), [qd, qd + kd) key rows (rotated, written to the cache row of the device-side
+// position), the rest value rows (copied to the cache).  RopeCache::forward_interleaved + KvCache::append
+// (fusor/src/composite/rope.rs:300-329, fusor/src/cache/kv_cache.rs:49-63).
+struct FhRopeArgs {
+    const float *cs, *sn;
+    const int *pos;
+    float *qo;
+    void *kc, *vc;
+    int qd, kd, hd, cap, table_rows, f16;
+};
+struct Q4kExtra {
+    const float *xres = nullptr, *nw = nullptr;
+    float eps = 0.f;
+    int nsplit = 0;
+    FhRopeArgs rk = {};
+};
+
 #define Q4K_IMG 65 // uint4 per block image: 8 steps x 4 groups x (hi, lo) + one all-zero slot
 
 template <int TS, int PER, int EPI, int IN>
 __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict__ x, float *__restrict__ y,
                                                       const float *__restrict__ ea, const float *__restrict__ eb,
                                                       int SW, const float *__restrict__ xres,
-                                                      const float *__restrict__ nw, float eps, int nsplit) {
+                                                      const float *__restrict__ nw, float eps, int nsplit,
+                                                      FhRopeArgs rk) {
     constexpr int NT = EPI == FH_EPI_SWIGLU ? 2 : 1;
     constexpr int TW = TS / NT;
     constexpr int XB = (PER + TS - 1) / TS; // blocks of x each wavefront stages: kb / (TS * SW) with SW * PER == kb
@@ -229,7 +248,32 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
             v1 = v1 / rms;
         }
         const int64_t row = ((int64_t)blockIdx.x * TW + t) * 16 + jr;
-        if (row < nout) {
+        if (EPI == FH_EPI_ROPEKV) {
+            const float other = __shfl_xor(v0, 1, 64); // the pair (2i, 2i+1) sits in neighbouring lanes
+            const int pos = *rk.pos;
+            if (row < nout && pos < rk.cap) {
+                const int r = (int)row;
+                if (r < rk.qd + rk.kd) {
+                    const int rh = r < rk.qd ? r : r - rk.qd, e = rh % rk.hd, i = e >> 1, half = rk.hd >> 1;
+                    const int tp = pos < rk.table_rows ? pos : rk.table_rows - 1;
+                    const float c = rk.cs[(int64_t)tp * half + i], sn = rk.sn[(int64_t)tp * half + i];
+                    const float x0 = (r & 1) ? other : v0, x1 = (r & 1) ? v0 : other;
+                    const float ac = x0 * c, bs = x1 * sn, as = x0 * sn, bc = x1 * c;
+                    const float yv = (r & 1) ? as + bc : ac - bs;
+                    if (r < rk.qd) rk.qo[r] = yv;
+                    else {
+                        const int64_t at = ((int64_t)(rh / rk.hd) * rk.cap + pos) * rk.hd + e;
+                        if (rk.f16) ((_Float16 *)rk.kc)[at] = (_Float16)yv;
+                        else ((float *)rk.kc)[at] = yv;
+                    }
+                } else {
+                    const int rh = r - rk.qd - rk.kd;
+                    const int64_t at = ((int64_t)(rh / rk.hd) * rk.cap + pos) * rk.hd + rh % rk.hd;
+                    if (rk.f16) ((_Float16 *)rk.vc)[at] = (_Float16)v0;
+                    else ((float *)rk.vc)[at] = v0;
+                }
+            }
+        } else if (row < nout) {
             float rr = v0;
             if (EPI == FH_EPI_ADD2) rr = (rr + ea[row]) + eb[row];
             if (EPI == FH_EPI_SWIGLU) rr = (rr / (__expf(-rr) + 1.0f)) * v1;
@@ -242,23 +286,23 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
 // (64 VGPRs) is enforced: the kernel lives on the number of bytes in flight per compute unit.
 #define Q4K_M1_PARAMS                                                                                              \
     QView q, const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ ea,                    \
-        const float *__restrict__ eb, int SW, const float *__restrict__ xres, const float *__restrict__ nw, float eps, int nsplit
+        const float *__restrict__ eb, int SW, const float *__restrict__ xres, const float *__restrict__ nw, float eps, int nsplit, FhRopeArgs rk
 template <int TS, int PER, int EPI, int IN>
 __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(Q4K_M1_PARAMS) {
-    qmv_q4k_m1_body<TS, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit);
+    qmv_q4k_m1_body<TS, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
 template <int TS, int PER, int EPI, int IN>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_qmv_q4k_m1_w8(Q4K_M1_PARAMS) {
-    qmv_q4k_m1_body<TS, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit);
+    qmv_q4k_m1_body<TS, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
 
 template <int TS, int PER, int EPI>
 static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b, int SW,
-                               unsigned grid, size_t lds, const float *xres, const float *nw, float eps, int nsplit) {
+                               unsigned grid, size_t lds, const Q4kExtra &ex) {
     typedef void (*kern_t)(QView, const float *, float *, const float *, const float *, int, const float *, const float *,
-                           float, int);
+                           float, int, FhRopeArgs);
     kern_t kern;
-    const int in = nsplit > 0 ? 2 : (nw ? 1 : 0); // input: plain, rms_norm, attention partials
+    const int in = ex.nsplit > 0 ? 2 : (ex.nw ? 1 : 0); // input: plain, rms_norm, attention partials
     if constexpr (PER <= 2) {
         kern = in == 2 ? k_qmv_q4k_m1<TS, PER, EPI, 2>
                        : (in == 1 ? k_qmv_q4k_m1_w8<TS, PER, EPI, 1> : k_qmv_q4k_m1_w8<TS, PER, EPI, 0>);
@@ -270,17 +314,18 @@ static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, co
         FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         attr_done[in] = true;
     }
-    kern<<<dim3(grid), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, xres, nw, eps, nsplit);
+    kern<<<dim3(grid), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, ex.xres, ex.nw, ex.eps,
+                                                                  ex.nsplit, ex.rk);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
 
 template <int TS, int EPI>
 static fh_status q4k_m1_per(int per, const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b,
-                            int SW, unsigned grid, size_t lds, const float *xres, const float *nw, float eps, int nsplit) {
-    if (per == 1) return q4k_m1_launch<TS, 1, EPI>(q, x, y, a, b, SW, grid, lds, xres, nw, eps, nsplit);
-    if (per == 2) return q4k_m1_launch<TS, 2, EPI>(q, x, y, a, b, SW, grid, lds, xres, nw, eps, nsplit);
-    return q4k_m1_launch<TS, 4, EPI>(q, x, y, a, b, SW, grid, lds, xres, nw, eps, nsplit);
+                            int SW, unsigned grid, size_t lds, const Q4kExtra &ex) {
+    if (per == 1) return q4k_m1_launch<TS, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
+    if (per == 2) return q4k_m1_launch<TS, 2, EPI>(q, x, y, a, b, SW, grid, lds, ex);
+    return q4k_m1_launch<TS, 4, EPI>(q, x, y, a, b, SW, grid, lds, ex);
 }
 
 // Returns FH_ERR_UNSUPPORTED when the shape does not fit this kernel (the caller falls back).
@@ -288,24 +333,46 @@ fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int ep
     return fh_launch_q4k_m1_norm(q, x, nullptr, nullptr, 0.f, y, epi, a, b);
 }
 
-static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const float *xres, const float *nw, float eps, int nsplit,
-                            float *y, int epi, const float *a, const float *b);
+static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra &ex, float *y, int epi, const float *a,
+                            const float *b);
 
 // The same product with the input merged from the partial results of the decode-step attention
 // (x = [head][nsplit][128 + 4]; head_dim 128, nsplit <= 8).
 fh_status fh_launch_q4k_m1_attn(const fh_qmatrix *q, const float *part, int nsplit, float *y) {
     if (nsplit < 1 || nsplit > 8 || q->k % 128) return FH_ERR_UNSUPPORTED;
-    return q4k_m1_any(q, part, nullptr, nullptr, 0.f, nsplit, y, FH_EPI_NONE, nullptr, nullptr);
+    Q4kExtra ex;
+    ex.nsplit = nsplit;
+    return q4k_m1_any(q, part, ex, y, FH_EPI_NONE, nullptr, nullptr);
 }
 
 // The same product with the input taken as rms_norm(x [+ xres]) * nw when nw is given.
 fh_status fh_launch_q4k_m1_norm(const fh_qmatrix *q, const float *x, const float *xres, const float *nw, float eps,
                                 float *y, int epi, const float *a, const float *b) {
-    return q4k_m1_any(q, x, xres, nw, eps, 0, y, epi, a, b);
+    Q4kExtra ex;
+    ex.xres = xres;
+    ex.nw = nw;
+    ex.eps = eps;
+    return q4k_m1_any(q, x, ex, y, epi, a, b);
 }
 
-static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const float *xres, const float *nw, float eps, int nsplit,
-                            float *y, int epi, const float *a, const float *b) {
+// The fused q|k|v projection of a decode step: rms_norm(x) * nw as input (nw may be NULL: plain x), rotated
+// query rows to q_out, rotated key rows and value rows into the cache row of the device-side position.
+fh_status fh_launch_q4k_m1_ropekv(const fh_qmatrix *q, const float *x, const float *nw, float eps, fh_kvcache *c,
+                                  int layer, int hq, const float *cos_t, const float *sin_t, int table_rows,
+                                  float *q_out) {
+    const int hd = c->head_dim, qd = hq * hd, kd = c->kv_heads * hd;
+    if (q->n != qd + 2 * kd || hd % 16) return FH_ERR_UNSUPPORTED;
+    const size_t plane = (size_t)c->kv_heads * c->capacity * hd * fh_dtype_size(c->dtype);
+    Q4kExtra ex;
+    ex.nw = nw;
+    ex.eps = eps;
+    ex.rk = FhRopeArgs{cos_t, sin_t, c->len_dev, q_out, (uint8_t *)c->k + layer * plane, (uint8_t *)c->v + layer * plane,
+                       qd, kd, hd, c->capacity, table_rows, c->dtype == FH_F16 ? 1 : 0};
+    return q4k_m1_any(q, x, ex, nullptr, FH_EPI_ROPEKV, nullptr, nullptr);
+}
+
+static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra &ex, float *y, int epi, const float *a,
+                            const float *b) {
     fh_device *dev = q->dev;
     const int kb = (int)q->kb;
     const int nt = epi == FH_EPI_SWIGLU ? 2 : 1;
@@ -330,7 +397,7 @@ static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const float *xr
     size_t lds = (size_t)kb * Q4K_IMG * 16 + (size_t)kb * 64 + 16 * 64 + 64;
     if (lds > 160 * 1024) return FH_ERR_UNSUPPORTED;
     unsigned grid = (unsigned)((tiles + TW - 1) / TW);
-#define Q4K_M1_GO(TS_, EPI_) return q4k_m1_per<TS_, EPI_>(per, q, x, y, a, b, SW, grid, lds, xres, nw, eps, nsplit)
+#define Q4K_M1_GO(TS_, EPI_) return q4k_m1_per<TS_, EPI_>(per, q, x, y, a, b, SW, grid, lds, ex)
     if (epi == FH_EPI_SWIGLU) {
         if (TS == 2) Q4K_M1_GO(2, FH_EPI_SWIGLU);
         Q4K_M1_GO(4, FH_EPI_SWIGLU);
@@ -339,6 +406,11 @@ static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const float *xr
         if (TS == 1) Q4K_M1_GO(1, FH_EPI_ADD2);
         if (TS == 2) Q4K_M1_GO(2, FH_EPI_ADD2);
         Q4K_M1_GO(4, FH_EPI_ADD2);
+    }
+    if (epi == FH_EPI_ROPEKV) {
+        if (TS == 1) Q4K_M1_GO(1, FH_EPI_ROPEKV);
+        if (TS == 2) Q4K_M1_GO(2, FH_EPI_ROPEKV);
+        Q4K_M1_GO(4, FH_EPI_ROPEKV);
     }
     if (TS == 1) Q4K_M1_GO(1, FH_EPI_NONE);
     if (TS == 2) Q4K_M1_GO(2, FH_EPI_NONE);
