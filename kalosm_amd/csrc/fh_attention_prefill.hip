@@ -1,0 +1,229 @@
+// Prefill attention on the matrix cores: softmax(Q . K^T * scale [causal]) . V for many query rows, grouped-query
+// heads, head_dim 64 or 128.
+// Reference: fusor-ml/fusor/src/composite/flash_attention.rs:58-236 (semantics; causal mask as MaskKind::Causal
+// with the queries aligned to the END of the keys), fusor-ml/core/src/row_program.rs:1210-1382 (the fused kernel).
+//
+// grid (query blocks of 128, q heads, batch); 4 wavefronts, each owning 32 query rows.  KV tiles of 64 keys go
+// through LDS as f16: K as [key][d], V transposed to [d][key].  Both products are computed TRANSPOSED with
+// v_mfma_f32_32x32x16_f16 so that a lane always stands for ONE query (the accumulator column):
+//   S^T (keys x queries) = K . Q^T      A = K rows, B = Q^T kept in registers for the whole kernel
+//   O^T (d x queries)    = V^T . P^T    A = V^T rows, B = P^T = the S^T accumulator, exponentiated, as f16
+// The online-softmax statistics (running max, running sum, rescale factor) are then per-lane scalars, and the row
+// maximum is a reduction over the lane's own registers plus one exchange with lane + 32.  MFMA row i of the K
+// operand reads key 16*(i/16) + 8*((i/4)%2) + 4*((i/8)%2) + i%4 of the tile: with that order the 16 accumulator
+// registers of a lane are keys 8g .. 8g+7 and 16 + 8g .. 16 + 8g+7 (g = lane / 32), which is exactly the k-slot
+// order of the B operand of the second product - P^T never leaves the registers.
+// Inputs may be f32 or f16; operands are rounded to f16, all accumulation and the softmax are f32.
+#include "fh_internal.h"
+
+typedef _Float16 fh_half;
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ void ap_load8(const float *p, fh_half *o) {
+    const float4 a = *(const float4 *)p, b = *(const float4 *)(p + 4);
+    o[0] = (fh_half)a.x; o[1] = (fh_half)a.y; o[2] = (fh_half)a.z; o[3] = (fh_half)a.w;
+    o[4] = (fh_half)b.x; o[5] = (fh_half)b.y; o[6] = (fh_half)b.z; o[7] = (fh_half)b.w;
+}
+__device__ __forceinline__ void ap_load8(const fh_half *p, fh_half *o) {
+    const uint4 r = *(const uint4 *)p;
+    __builtin_memcpy(o, &r, 16);
+}
+__device__ __forceinline__ float ap_swap32_max(float v) {
+    const uint32_t u = __float_as_uint(v);
+    auto s = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(s[0]), __uint_as_float(s[1]));
+}
+__device__ __forceinline__ float ap_swap32_sum(float v) {
+    const uint32_t u = __float_as_uint(v);
+    auto s = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(s[0]) + __uint_as_float(s[1]);
+}
+__device__ __forceinline__ void ap_store4(float *p, float a, float b, float c, float d) {
+    *(float4 *)p = make_float4(a, b, c, d);
+}
+__device__ __forceinline__ void ap_store4(fh_half *p, float a, float b, float c, float d) {
+    const fh_half h[4] = {(fh_half)a, (fh_half)b, (fh_half)c, (fh_half)d};
+    uint2 u;
+    __builtin_memcpy(&u, h, 8);
+    *(uint2 *)p = u;
+}
+
+template <typename TQ, typename TKV, int D>
+__global__ __launch_bounds__(256) void k_attn_prefill(const TQ *__restrict__ q, int64_t q_sb, int64_t q_sh, int64_t q_st,
+                                                       const TKV *__restrict__ k, const TKV *__restrict__ v,
+                                                       int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int hq, int hkv,
+                                                       int sq, int skv, float scale, int causal, TQ *__restrict__ out) {
+    constexpr int BN = 64, KS = D + 8, VS = BN + 8, DT = D / 32, KSTEPS = D / 16, CH = D / 8; // CH: 8-element chunks per row
+    __shared__ __attribute__((aligned(16))) fh_half sK[BN * KS];
+    __shared__ __attribute__((aligned(16))) fh_half sV[D * VS];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
+    const int h = blockIdx.y, bi = blockIdx.z, kh = h / (hq / hkv);
+    const int qb0 = blockIdx.x * 128;
+    const int qi = qb0 + wave * 32 + li; // this lane's query row
+    const int off = skv - sq;            // causal: query i sees keys 0 .. i + off
+    const TKV *kb = k + bi * kv_sb + kh * kv_sh, *vb = v + bi * kv_sb + kh * kv_sh;
+
+    // Q^T operand, once: lane (query li, k-slots 8g .. 8g+7 of every 16-wide step of d)
+    half8 qf[KSTEPS];
+    {
+        const TQ *qp = q + bi * q_sb + h * q_sh + (int64_t)(qi < sq ? qi : sq - 1) * q_st + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ks++) {
+            fh_half t[8];
+            ap_load8(qp + 16 * ks, t);
+            __builtin_memcpy(&qf[ks], t, 16);
+        }
+    }
+    const int prow = 16 * (li >> 4) + 8 * ((li >> 2) & 1) + 4 * ((li >> 3) & 1) + (li & 3); // key read by MFMA row li
+    const float sc2 = scale * 1.4426950408889634f;                                        // scores in the log2 domain
+    float m_run = -INFINITY, l_run = 0.f;
+    floatx16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[dt][r] = 0.f;
+
+    int kend = skv;
+    if (causal) {
+        const int last = (qb0 + 127 < sq ? qb0 + 127 : sq - 1) + off + 1;
+        kend = last < skv ? last : skv;
+    }
+    for (int t0 = 0; t0 < kend; t0 += BN) {
+        __syncthreads(); // the previous tile is consumed
+        // ---- K tile -> sK[key][d]
+#pragma unroll
+        for (int i = 0; i < BN * CH / 256; i++) {
+            const int c = tid + 256 * i, key = c / CH, dc = c % CH;
+            fh_half t[8];
+            if (t0 + key < skv) ap_load8(kb + (int64_t)(t0 + key) * kv_st + 8 * dc, t);
+            else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) t[e] = (fh_half)0.f;
+            }
+            uint4 u;
+            __builtin_memcpy(&u, t, 16);
+            *(uint4 *)(sK + key * KS + 8 * dc) = u;
+        }
+        // ---- V tile -> sV[d][key] (a lane keeps one key, so the 2-byte stores of a wavefront are contiguous)
+#pragma unroll
+        for (int i = 0; i < BN * CH / 256; i++) {
+            const int c = tid + 256 * i, key = c % BN, dc = c / BN;
+            fh_half t[8];
+            if (t0 + key < skv) ap_load8(vb + (int64_t)(t0 + key) * kv_st + 8 * dc, t);
+            else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) t[e] = (fh_half)0.f;
+            }
+#pragma unroll
+            for (int e = 0; e < 8; e++) sV[(8 * dc + e) * VS + key] = t[e];
+        }
+        __syncthreads();
+        // ---- S^T = K . Q^T for the two 32-key halves of the tile
+        floatx16 st[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) st[kt][r] = 0.f;
+            const fh_half *ap = sK + (kt * 32 + prow) * KS + 8 * g;
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ks++) {
+                const half8 a = *(const half8 *)(ap + 16 * ks);
+                st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], st[kt], 0, 0, 0);
+            }
+        }
+        // ---- mask, running max: register r of half kt is key t0 + 32 kt + 16 (r / 8) + 8 g + r % 8
+        const int lim = causal ? (qi + off < skv - 1 ? qi + off : skv - 1) : skv - 1; // last visible key
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int key = t0 + 32 * kt + 16 * (r >> 3) + 8 * g + (r & 7);
+                const float s = key <= lim ? st[kt][r] * sc2 : -INFINITY;
+                st[kt][r] = s;
+                mx = fmaxf(mx, s);
+            }
+        mx = ap_swap32_max(mx);
+        const float m_new = fmaxf(m_run, mx);
+        const bool dead = m_new == -INFINITY; // nothing visible yet (only queries past the end)
+        const float alpha = dead ? 1.f : exp2f(m_run - m_new);
+        float ps = 0.f;
+        half8 pb[2][2];
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                fh_half t[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float p = dead ? 0.f : exp2f(st[kt][8 * s2 + e] - m_new);
+                    ps += p;
+                    t[e] = (fh_half)p;
+                }
+                __builtin_memcpy(&pb[kt][s2], t, 16);
+            }
+        l_run = l_run * alpha + ap_swap32_sum(ps);
+        m_run = m_new;
+        // ---- O^T = O^T * alpha + V^T . P^T
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[dt][r] *= alpha;
+            const fh_half *vp = sV + (dt * 32 + li) * VS + 8 * g;
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int s2 = 0; s2 < 2; s2++) {
+                    const half8 a = *(const half8 *)(vp + 32 * kt + 16 * s2);
+                    acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[kt][s2], acc[dt], 0, 0, 0);
+                }
+        }
+    }
+    // ---- store: lane = query, register r of d-tile dt is d = 32 dt + 8 (r / 4) + 4 g + r % 4
+    if (qi < sq) {
+        const float inv = 1.0f / l_run;
+        TQ *op = out + (((int64_t)bi * hq + h) * sq + qi) * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++)
+                ap_store4(op + 32 * dt + 8 * r4 + 4 * g, acc[dt][4 * r4] * inv, acc[dt][4 * r4 + 1] * inv,
+                          acc[dt][4 * r4 + 2] * inv, acc[dt][4 * r4 + 3] * inv);
+    }
+}
+
+template <typename TQ, typename TKV>
+static fh_status ap_launch(fh_device *dev, const void *q, int64_t q_sb, int64_t q_sh, int64_t q_st, const void *k,
+                           const void *v, int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int b, int hq, int hkv, int sq,
+                           int skv, int d, float scale, int causal, void *out) {
+    dim3 grid((unsigned)((sq + 127) / 128), (unsigned)hq, (unsigned)b);
+    if (d == 128)
+        k_attn_prefill<TQ, TKV, 128><<<grid, 256, 0, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k,
+                                                                    (const TKV *)v, kv_sb, kv_sh, kv_st, hq, hkv, sq, skv,
+                                                                    scale, causal, (TQ *)out);
+    else
+        k_attn_prefill<TQ, TKV, 64><<<grid, 256, 0, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k,
+                                                                   (const TKV *)v, kv_sb, kv_sh, kv_st, hq, hkv, sq, skv,
+                                                                   scale, causal, (TQ *)out);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+// FH_ERR_UNSUPPORTED when the shape is not one this kernel is written for (the caller keeps the generic kernel).
+fh_status fh_attention_prefill_mfma(fh_device *dev, int q_dtype, int kv_dtype, const void *q, int64_t q_sb,
+                                    int64_t q_sh, int64_t q_st, const void *k, const void *v, int64_t kv_sb,
+                                    int64_t kv_sh, int64_t kv_st, int b, int hq, int hkv, int sq, int skv, int d,
+                                    float scale, int mask_kind, void *out) {
+    if ((d != 128 && d != 64) || hq % hkv || (mask_kind != FH_MASK_NONE && mask_kind != FH_MASK_CAUSAL)) return FH_ERR_UNSUPPORTED;
+    if (q_st % 8 || q_sh % 8 || q_sb % 8 || kv_st % 8 || kv_sh % 8 || kv_sb % 8 || hq > 65535 || b > 65535) return FH_ERR_UNSUPPORTED;
+    if (mask_kind == FH_MASK_CAUSAL && skv < sq) return FH_ERR_UNSUPPORTED;
+    const int causal = mask_kind == FH_MASK_CAUSAL;
+    if (q_dtype == FH_F16 && kv_dtype == FH_F16)
+        return ap_launch<fh_half, fh_half>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, d, scale, causal, out);
+    if (q_dtype == FH_F32 && kv_dtype == FH_F16)
+        return ap_launch<float, fh_half>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, d, scale, causal, out);
+    if (q_dtype == FH_F32 && kv_dtype == FH_F32)
+        return ap_launch<float, float>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, d, scale, causal, out);
+    return FH_ERR_UNSUPPORTED;
+}

@@ -235,3 +235,44 @@ def test_kv_cache_growth_append_reset(dev, dtype):
         c.append(0, Tensor.zeros(dev, (hk, 100, d)), Tensor.zeros(dev, (hk, 100, d)))
     c.reset()
     assert c.view(0)[0] == 0
+
+
+# ----------------------------------------------------------------------------- prefill attention on the matrix cores
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("sq,skv,causal", [(128, 128, True), (200, 200, True), (64, 300, True), (160, 97, False),
+                                           (512, 512, True), (33, 33, True)])
+def test_attention_prefill_f16(dev, oracle, sq, skv, causal, d):
+    """f16 Q/K/V, 8 query heads on 2 KV heads, query blocks and key tiles with ragged ends, causal with the queries
+    aligned to the end of a longer KV.  The checker gets the f32 values of the same f16 inputs; the output is f16
+    (2^-11 relative) and P is rounded to f16 before the second product: 1e-3 relative or 1e-2 absolute."""
+    h, hkv = 8, 2
+    rng = np.random.default_rng(sq * 1000 + skv + d)
+    q = rng.standard_normal((1, h, sq, d)).astype(np.float16)
+    k = rng.standard_normal((1, hkv, skv, d)).astype(np.float16)
+    v = rng.standard_normal((1, hkv, skv, d)).astype(np.float16)
+    scale = 1 / np.sqrt(d)
+    got = run_attn(dev, q, k, v, scale, MaskKind.Causal if causal else None, dtype="f16")
+    qf, kf, vf = (a.astype(np.float32) for a in (q, k, v))
+    want = oracle.flash_attention(qf, kf, vf, scale, oracle.MASK_CAUSAL if causal else oracle.MASK_NONE, None)
+    assert_close(got, want, abs_tol=1e-2, rel_tol=1e-3, what=f"f16 prefill {sq}x{skv}x{d}")
+    ref = refgen.np_attention(qf, kf, vf, scale, causal=causal, mask=None)
+    assert_close(got, ref, abs_tol=1e-2, rel_tol=1e-3, what="vs float64 textbook")
+
+
+def test_attention_prefill_f32_on_request(dev, oracle):
+    """f32 operands through the same kernel (rounded to f16 inside, f32 out), and the invariants that do not depend
+    on the rounding: V constant -> output constant, causal row 0 -> v_0."""
+    h, hkv, sq, d = 4, 1, 96, 128
+    rng = np.random.default_rng(5)
+    q, k, v = (rng.standard_normal((1, n, sq, d)).astype(np.float32) for n in (h, hkv, hkv))
+    dev.set_option("attn_kernel", 2)
+    try:
+        got = run_attn(dev, q, k, v, 1 / np.sqrt(d), MaskKind.Causal)
+        want = oracle.flash_attention(q, k, v, 1 / np.sqrt(d), oracle.MASK_CAUSAL, None)
+        assert_close(got, want, abs_tol=1e-2, rel_tol=1e-3, what="f32 prefill on the matrix cores")
+        assert_close(got[0, :, 0], np.broadcast_to(v[0, 0, 0], (h, d)), abs_tol=1e-3, rel_tol=1e-3, what="row 0 sees v_0 only")
+        vc = np.full_like(v, 0.75)
+        got = run_attn(dev, q, k, vc, 1 / np.sqrt(d), None)
+        assert_close(got, np.full_like(got, 0.75), abs_tol=1e-3, rel_tol=1e-3, what="constant V")
+    finally:
+        dev.set_option("attn_kernel", 0)
