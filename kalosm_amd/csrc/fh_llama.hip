@@ -330,7 +330,11 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
             FH_TRY(fh_swiglu(dev, m->gu, m->gu + (size_t)s * F, m->act, (int64_t)s * F));
         }
         if (s == 1) { // forward_add_residuals, attention_layer.rs:147-174: (down(act) + attn) + residual
-            FH_TRY(fh_qmatmul_add2(l.down, m->act, 1, m->attn_out, m->x, m->x));
+            fh_status st = FH_ERR_UNSUPPORTED;
+            if (fuse && l.down->type == FH_Q6_K && dev->opt_down_splitk != 1)
+                st = fh_launch_q6k_m1_acc(l.down, m->act, m->x, m->attn_out); // x += down(act) + attn
+            if (st == FH_ERR_UNSUPPORTED) st = fh_qmatmul_add2(l.down, m->act, 1, m->attn_out, m->x, m->x);
+            FH_TRY(st);
         } else {      // raw/mod.rs:1036
             FH_TRY(fh_qmatmul(l.down, m->act, s, m->ff));
             FH_TRY(fh_add3(dev, m->ff, m->attn_out, m->x, m->x, (int64_t)s * D));

@@ -38,7 +38,8 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
     constexpr int TW = TS / NT;
     constexpr int XB = (PER + TS - 1) / TS;
     extern __shared__ uint4 lds[];
-    const int kb = (int)q.kb;
+    // gridDim.y > 1: k is split over workgroups (blocks [boff, boff + kb) here) that add into y with atomics
+    const int kb = (int)q.kb / (int)gridDim.y, boff = (int)blockIdx.y * kb;
     uint4 *img = lds;
     float *sf = (float *)(lds + kb * Q6K_IMG);
     float *l_red = sf + kb * Q6K_SF; // [TS][SW][16]
@@ -57,13 +58,13 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
 #pragma unroll
     for (int i = 0; i < XB; i++) {
         const int b = wave + i * nwaves;
-        xv[i] = *(const float4 *)(x + (int64_t)(b < kb ? b : 0) * 256 + lane * 4);
+        xv[i] = *(const float4 *)(x + (int64_t)(boff + (b < kb ? b : 0)) * 256 + lane * 4);
     }
     // ---- 1. all weight bytes of this wavefront (a tile past the end re-reads the last one; never stored)
     Q6KRegs w[PER];
     {
         const int64_t tl = tvalid ? tile : tile - (to - (tiles_out - 1));
-        const uint8_t *rec = q.data + (tl * q.recs + b0) * 3360;
+        const uint8_t *rec = q.data + (tl * q.recs + boff + b0) * 3360;
 #pragma unroll
         for (int r = 0; r < PER; r++) {
             const uint8_t *p = rec + r * 3360;
@@ -186,21 +187,22 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
             float rr = v0;
             if (EPI == FH_EPI_ADD2) rr = (rr + ea[row]) + eb[row];
             if (EPI == FH_EPI_SWIGLU) rr = (rr / (__expf(-rr) + 1.0f)) * v1;
-            y[row] = rr;
+            if (EPI == FH_EPI_ACC) unsafeAtomicAdd(y + row, blockIdx.y == 0 ? rr + ea[row] : rr);
+            else y[row] = rr;
         }
     }
 }
 
 template <int TS, int PER, int EPI>
 static fh_status q6k_m1_launch(const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b, int SW,
-                               unsigned grid, size_t lds) {
+                               unsigned grid, size_t lds, unsigned ksplit = 1) {
     static bool attr_done = false;
     if (!attr_done) {
         FH_HIP(hipFuncSetAttribute((const void *)k_qmv_q6k_m1<TS, PER, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    160 * 1024));
         attr_done = true;
     }
-    k_qmv_q6k_m1<TS, PER, EPI><<<dim3(grid), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW);
+    k_qmv_q6k_m1<TS, PER, EPI><<<dim3(grid, ksplit), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
@@ -252,4 +254,26 @@ fh_status fh_launch_q6k_m1(const fh_qmatrix *q, const float *x, float *y, int ep
     if (TS == 2) Q6K_M1_GO(2, FH_EPI_NONE);
     Q6K_M1_GO(4, FH_EPI_NONE);
 #undef Q6K_M1_GO
+}
+
+// y += W . x + add with k split over `ksplit` workgroups per row tile (atomic adds, so the summation order - and the
+// last bits of the result - vary from run to run).  For matrices with few row tiles and a long k (the down projection
+// of a decode step accumulating into the residual stream) the smaller workgroups overlap their load and compute phases.
+fh_status fh_launch_q6k_m1_acc(const fh_qmatrix *q, const float *x, float *y_inout, const float *add) {
+    fh_device *dev = q->dev;
+    const int kb = (int)q->kb;
+    int ks = (int)dev->opt_matvec_splitk;
+    if (ks <= 0) ks = 4;
+    if (ks < 2 || kb % ks) return FH_ERR_UNSUPPORTED;
+    const int kbl = kb / ks;
+    int per = (int)dev->opt_matvec_per;
+    if (per != 1 && per != 2 && per != 4) per = 1;
+    while (per > 1 && kbl % per) per /= 2;
+    const int SW = kbl / per;
+    if (SW > 16) return FH_ERR_UNSUPPORTED;
+    const int64_t tiles = (q->n + 15) / 16;
+    size_t lds = (size_t)kbl * Q6K_IMG * 16 + (size_t)kbl * Q6K_SF * 4 + (size_t)SW * 64;
+    if (per == 1) return q6k_m1_launch<1, 1, FH_EPI_ACC>(q, x, y_inout, add, nullptr, SW, (unsigned)tiles, lds, (unsigned)ks);
+    if (per == 2) return q6k_m1_launch<1, 2, FH_EPI_ACC>(q, x, y_inout, add, nullptr, SW, (unsigned)tiles, lds, (unsigned)ks);
+    return q6k_m1_launch<1, 4, FH_EPI_ACC>(q, x, y_inout, add, nullptr, SW, (unsigned)tiles, lds, (unsigned)ks);
 }

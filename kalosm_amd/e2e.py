@@ -11,7 +11,7 @@ from .llama import Model
 
 
 def run(dev, cfg: dict | None = None, prompt_len: int = 512, steps: int = 256, seed: int = 0, sigma: float = 1e-4,
-        kv_dtype: str = "f32", repeats: int = 2, prefill_chunk: int = 16) -> dict:
+        kv_dtype: str = "f32", repeats: int = 2, prefill_chunk: int = 512) -> dict:
     cfg = dict(cfg or synth.LLAMA3_8B)
     t0 = time.perf_counter()
     m = Model.random_init(dev, cfg, seed=seed, sigma=sigma, kv_dtype=kv_dtype)
