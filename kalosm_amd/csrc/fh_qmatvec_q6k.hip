@@ -263,7 +263,7 @@ fh_status fh_launch_q6k_m1_acc(const fh_qmatrix *q, const float *x, float *y_ino
     fh_device *dev = q->dev;
     const int kb = (int)q->kb;
     int ks = (int)dev->opt_matvec_splitk;
-    if (ks <= 0) ks = 4;
+    if (ks <= 0) ks = kb % 4 == 0 ? kb / 4 : 0; // four blocks per workgroup measured best (MI355X, k = 14336)
     if (ks < 2 || kb % ks) return FH_ERR_UNSUPPORTED;
     const int kbl = kb / ks;
     int per = (int)dev->opt_matvec_per;
