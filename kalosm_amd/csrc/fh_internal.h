@@ -56,7 +56,8 @@ struct fh_device {
     int64_t opt_matvec_per = 0;      // 0 auto, else 1 / 2 / 4 blocks per wavefront
     int64_t opt_attn_splits = 0;     // 0 auto
     int64_t opt_attn_kernel = 0;     // 0 auto, 1 first-generation kernels only, 2 matrix-core prefill for f32 too
-    int64_t opt_down_splitk = 0;     // 0: decode steps split k of a Q6_K down projection (atomic adds), 1: never
+    int64_t opt_down_splitk = 0;     // 0: decode steps split k of a Q6_K down projection (atomic adds), 1: never, 3: and SwiGLU in its staging
+    int64_t opt_wo_acc = 0;          // 0: decode steps accumulate the output projection into the residual stream, 1: never
     int64_t opt_fuse_norm = 0;       // 0: decode steps fold rms_norm into the consuming matvec, 1: separate launches
     int64_t opt_matmul_kernel = 0;   // 0 auto, 1 generic for every m, 2 MFMA tile kernel for every m
 };
@@ -150,12 +151,13 @@ fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int ep
 fh_status fh_launch_q4k_m1_norm(const fh_qmatrix *q, const float *x, const float *xres, const float *nw, float eps,
                                 float *y, int epi, const float *a, const float *b);
 fh_status fh_launch_q4k_m1_attn(const fh_qmatrix *q, const float *part, int nsplit, float *y);
+fh_status fh_launch_q4k_m1_attn_acc(const fh_qmatrix *q, const float *part, int nsplit, float *y_inout);
 fh_status fh_attention_combine_dl(fh_device *dev, int hq, int splits, float *out);
 fh_status fh_attention_prefill_mfma(fh_device *dev, int q_dtype, int kv_dtype, const void *q, int64_t q_sb,
                                     int64_t q_sh, int64_t q_st, const void *k, const void *v, int64_t kv_sb,
                                     int64_t kv_sh, int64_t kv_st, int b, int hq, int hkv, int sq, int skv, int d,
                                     float scale, int mask_kind, void *out);
-fh_status fh_launch_q6k_m1_acc(const fh_qmatrix *q, const float *x, float *y_inout, const float *add);
+fh_status fh_launch_q6k_m1_acc(const fh_qmatrix *q, const float *x, const float *xup, float *y_inout, const float *add);
 fh_status fh_launch_q6k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b);
 
 struct fh_kvcache {

@@ -238,7 +238,7 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
         fh_llama_layer &l = m->layers[li];
         // Decode steps fold each rms_norm into the matvec that consumes it (one launch instead of two).
         const bool fuse = dev_pos && s == 1 && dev->opt_fuse_norm == 0 && dev->opt_matvec_kernel == 0;
-        bool qkv_done = false, wo_done = false;
+        bool qkv_done = false, wo_done = false, xacc = false;
         bool rope_done = false;
         if (fuse && l.qkv && l.qkv->type == FH_Q4_K) {
             // norm + projection + rope + cache append in one launch; without the rope epilogue as second choice
@@ -285,7 +285,12 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
                 ast = fh_attention_decode_devlen_v1(dev, c.kv_dtype, m->qrot, kc, vc, (int64_t)m->cache->capacity * hd, hd, H,
                                                     HK, hd, scale, m->cache->len_dev, m->cache->capacity, m->att);
             else if (ast == FH_OK && merge_in_wo) {
-                fh_status st = fh_launch_q4k_m1_attn(l.wo, dev->part_buf, nsplit, m->attn_out);
+                // first choice: x += Wo . att with k split over small workgroups; the residual stream then already
+                // holds x + attn for the FFN norm and the final sum ((ffn + attn) + residual, raw/mod.rs:1036)
+                fh_status st = dev->opt_wo_acc == 1 ? FH_ERR_UNSUPPORTED
+                                                    : fh_launch_q4k_m1_attn_acc(l.wo, dev->part_buf, nsplit, m->x);
+                xacc = st == FH_OK;
+                if (st == FH_ERR_UNSUPPORTED) st = fh_launch_q4k_m1_attn(l.wo, dev->part_buf, nsplit, m->attn_out);
                 if (st == FH_ERR_UNSUPPORTED) st = fh_attention_combine_dl(dev, H, nsplit, m->att);
                 else wo_done = st == FH_OK;
                 ast = st;
@@ -309,14 +314,23 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
             att_in = m->att_t;
         }
         if (!wo_done) FH_TRY(fh_qmatmul(l.wo, att_in, s, m->attn_out));
-        bool ffn_done = false;
+        // input of the FFN norm: attn + residual, or the residual stream alone when it already holds the sum
+        const float *hin = xacc ? m->x : m->attn_out, *hres = xacc ? nullptr : m->x, *hadd = xacc ? nullptr : m->attn_out;
+        bool ffn_done = false, late_swiglu = false;
         if (fuse && l.gate_up && l.gate_up->type == FH_Q4_K) {
-            fh_status st = fh_launch_q4k_m1_norm(l.gate_up, m->attn_out, m->x, l.ffn_norm, c.eps, m->act, FH_EPI_SWIGLU,
-                                                 nullptr, nullptr);
+            // On request (down_splitk = 3; measured slower on MI355X) SwiGLU moves into the staging of a split-k Q6_K down
+            // projection: the gate | up
+            // projection then runs in its plain (fastest) form and writes both halves.
+            late_swiglu = l.down->type == FH_Q6_K && dev->opt_down_splitk == 3 && l.down->kb % 4 == 0 && l.down->kb >= 8;
+            fh_status st = late_swiglu ? fh_launch_q4k_m1_norm(l.gate_up, hin, hres, l.ffn_norm, c.eps, m->gu, FH_EPI_NONE,
+                                                               nullptr, nullptr)
+                                       : fh_launch_q4k_m1_norm(l.gate_up, hin, hres, l.ffn_norm, c.eps, m->act,
+                                                               FH_EPI_SWIGLU, nullptr, nullptr);
             if (st != FH_ERR_UNSUPPORTED) FH_TRY(st);
             ffn_done = st == FH_OK;
+            late_swiglu = late_swiglu && ffn_done;
         }
-        if (!ffn_done) FH_TRY(fh_rms_norm(dev, m->attn_out, m->x, l.ffn_norm, nullptr, c.eps, s, D, m->xn));
+        if (!ffn_done) FH_TRY(fh_rms_norm(dev, hin, hres, l.ffn_norm, nullptr, c.eps, s, D, m->xn));
         if (ffn_done) {
         } else if (l.gate_up && s <= 2) {
             FH_TRY(fh_qmatmul_swiglu(l.gate_up, m->xn, s, m->act));
@@ -331,9 +345,18 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
         }
         if (s == 1) { // forward_add_residuals, attention_layer.rs:147-174: (down(act) + attn) + residual
             fh_status st = FH_ERR_UNSUPPORTED;
-            if (fuse && l.down->type == FH_Q6_K && dev->opt_down_splitk != 1)
-                st = fh_launch_q6k_m1_acc(l.down, m->act, m->x, m->attn_out); // x += down(act) + attn
-            if (st == FH_ERR_UNSUPPORTED) st = fh_qmatmul_add2(l.down, m->act, 1, m->attn_out, m->x, m->x);
+            if (late_swiglu) { // x += down(silu(gate) * up) + attn
+                st = fh_launch_q6k_m1_acc(l.down, m->gu, m->gu + F, m->x, hadd);
+                if (st == FH_ERR_UNSUPPORTED) FH_TRY(fh_swiglu(dev, m->gu, m->gu + F, m->act, F));
+            } else if (fuse && l.down->type == FH_Q6_K && dev->opt_down_splitk != 1) {
+                st = fh_launch_q6k_m1_acc(l.down, m->act, nullptr, m->x, hadd); // x += down(act) [+ attn]
+            }
+            if (st == FH_ERR_UNSUPPORTED && xacc) { // x already holds x + attn
+                FH_TRY(fh_qmatmul(l.down, m->act, 1, m->ff));
+                st = fh_add3(dev, m->ff, m->x, nullptr, m->x, D);
+            } else if (st == FH_ERR_UNSUPPORTED) {
+                st = fh_qmatmul_add2(l.down, m->act, 1, m->attn_out, m->x, m->x);
+            }
             FH_TRY(st);
         } else {      // raw/mod.rs:1036
             FH_TRY(fh_qmatmul(l.down, m->act, s, m->ff));

@@ -51,6 +51,7 @@ struct Q4kExtra {
     float eps = 0.f;
     int nsplit = 0;
     FhRopeArgs rk = {};
+    int ksplit = 1; // workgroups along k (FH_EPI_ACC only)
 };
 
 #define Q4K_IMG 65 // uint4 per block image: 8 steps x 4 groups x (hi, lo) + one all-zero slot
@@ -65,7 +66,8 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     constexpr int TW = TS / NT;
     constexpr int XB = (PER + TS - 1) / TS; // blocks of x each wavefront stages: kb / (TS * SW) with SW * PER == kb
     extern __shared__ uint4 lds[];
-    const int kb = (int)q.kb;
+    // gridDim.y > 1: k is split over workgroups (blocks [boff, boff + kb) here) that add into y with atomics
+    const int kb = (int)q.kb / (int)gridDim.y, boff = (int)blockIdx.y * kb;
     uint4 *img = lds;
     float *sf = (float *)(lds + kb * Q4K_IMG); // per block: [0..7] group sums, [8..15] factors
     float *l_red = sf + kb * 16;               // [TS][SW][16]
@@ -89,7 +91,7 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
 #pragma unroll
     for (int i = 0; i < XB; i++) {
         const int b = wave + i * nwaves;
-        const int64_t at = (int64_t)(b < kb ? b : 0) * 256 + lane * 4;
+        const int64_t at = (int64_t)(boff + (b < kb ? b : 0)) * 256 + lane * 4;
         if (IN != 2) xv[i] = *(const float4 *)(x + at);
         if (IN == 1 && xres) rv[i] = *(const float4 *)(xres + at);
         if (IN == 1) wv[i] = *(const float4 *)(nw + at);
@@ -108,7 +110,7 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     Q4KRegs w[PER];
     {
         const int64_t tl = tvalid ? tile : tile - (to - (tiles_out - 1));
-        const uint8_t *rec = q.data + (tl * q.recs + b0) * 2304;
+        const uint8_t *rec = q.data + (tl * q.recs + boff + b0) * 2304;
         const uint8_t *ph = rec + 16 * j, *pq = rec + 256 + lane * 16;
 #pragma unroll
         for (int r = 0; r < PER; r++) {
@@ -277,7 +279,8 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
             float rr = v0;
             if (EPI == FH_EPI_ADD2) rr = (rr + ea[row]) + eb[row];
             if (EPI == FH_EPI_SWIGLU) rr = (rr / (__expf(-rr) + 1.0f)) * v1;
-            y[row] = rr;
+            if (EPI == FH_EPI_ACC) unsafeAtomicAdd(y + row, (blockIdx.y == 0 && ea) ? rr + ea[row] : rr);
+            else y[row] = rr;
         }
     }
 }
@@ -314,7 +317,7 @@ static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, co
         FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         attr_done[in] = true;
     }
-    kern<<<dim3(grid), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, ex.xres, ex.nw, ex.eps,
+    kern<<<dim3(grid, (unsigned)ex.ksplit), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, ex.xres, ex.nw, ex.eps,
                                                                   ex.nsplit, ex.rk);
     FH_HIP(hipGetLastError());
     return FH_OK;
@@ -343,6 +346,18 @@ fh_status fh_launch_q4k_m1_attn(const fh_qmatrix *q, const float *part, int nspl
     Q4kExtra ex;
     ex.nsplit = nsplit;
     return q4k_m1_any(q, part, ex, y, FH_EPI_NONE, nullptr, nullptr);
+}
+
+// y += W . merged attention partials, k split over `ksplit` workgroups per row tile (atomic adds: the summation
+// order, and with it the last bits, vary from run to run).  The output projection of a decode step accumulating
+// into the residual stream.
+fh_status fh_launch_q4k_m1_attn_acc(const fh_qmatrix *q, const float *part, int nsplit, float *y_inout) {
+    if (nsplit < 1 || nsplit > 8 || q->k % 128) return FH_ERR_UNSUPPORTED;
+    Q4kExtra ex;
+    ex.nsplit = nsplit;
+    ex.ksplit = q->dev->opt_matvec_splitk > 0 ? (int)q->dev->opt_matvec_splitk : (q->kb % 4 == 0 ? (int)(q->kb / 4) : 0);
+    if (ex.ksplit < 2) return FH_ERR_UNSUPPORTED;
+    return q4k_m1_any(q, part, ex, y_inout, FH_EPI_ACC, nullptr, nullptr);
 }
 
 // The same product with the input taken as rms_norm(x [+ xres]) * nw when nw is given.
@@ -374,7 +389,8 @@ fh_status fh_launch_q4k_m1_ropekv(const fh_qmatrix *q, const float *x, const flo
 static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra &ex, float *y, int epi, const float *a,
                             const float *b) {
     fh_device *dev = q->dev;
-    const int kb = (int)q->kb;
+    if (ex.ksplit < 1 || q->kb % ex.ksplit || (ex.ksplit > 1 && (epi != FH_EPI_ACC || ex.nw))) return FH_ERR_UNSUPPORTED;
+    const int kb = (int)q->kb / ex.ksplit; // blocks per workgroup
     const int nt = epi == FH_EPI_SWIGLU ? 2 : 1;
     const int64_t nout = epi == FH_EPI_SWIGLU ? q->n / 2 : q->n;
     const int64_t tiles = (nout + 15) / 16;
@@ -406,6 +422,10 @@ static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra 
         if (TS == 1) Q4K_M1_GO(1, FH_EPI_ADD2);
         if (TS == 2) Q4K_M1_GO(2, FH_EPI_ADD2);
         Q4K_M1_GO(4, FH_EPI_ADD2);
+    }
+    if (epi == FH_EPI_ACC) {
+        if (TS == 1) Q4K_M1_GO(1, FH_EPI_ACC);
+        return FH_ERR_UNSUPPORTED;
     }
     if (epi == FH_EPI_ROPEKV) {
         if (TS == 1) Q4K_M1_GO(1, FH_EPI_ROPEKV);

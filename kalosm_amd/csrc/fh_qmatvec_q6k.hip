@@ -33,7 +33,7 @@ __device__ __forceinline__ float dpp_f32(float v) {
 template <int TS, int PER, int EPI>
 __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__restrict__ x, float *__restrict__ y,
                                                       const float *__restrict__ ea, const float *__restrict__ eb,
-                                                      int SW) {
+                                                      int SW, const float *__restrict__ xup) {
     constexpr int NT = EPI == FH_EPI_SWIGLU ? 2 : 1;
     constexpr int TW = TS / NT;
     constexpr int XB = (PER + TS - 1) / TS;
@@ -54,11 +54,15 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
     const int b0 = slice * PER;
 
     // ---- 0. activations first (short, needed first)
-    float4 xv[XB];
+    // With xup the input is silu(x) * xup (the SwiGLU of a gate | up projection, raw/attention_layer.rs:195),
+    // evaluated while staging.
+    float4 xv[XB], uv[XB];
 #pragma unroll
     for (int i = 0; i < XB; i++) {
         const int b = wave + i * nwaves;
-        xv[i] = *(const float4 *)(x + (int64_t)(boff + (b < kb ? b : 0)) * 256 + lane * 4);
+        const int64_t at = (int64_t)(boff + (b < kb ? b : 0)) * 256 + lane * 4;
+        xv[i] = *(const float4 *)(x + at);
+        if (xup) uv[i] = *(const float4 *)(xup + at);
     }
     // ---- 1. all weight bytes of this wavefront (a tile past the end re-reads the last one; never stored)
     Q6KRegs w[PER];
@@ -80,7 +84,10 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
     for (int i = 0; i < XB; i++) {
         const int b = wave + i * nwaves;
         if (b >= kb) break;
-        const float4 v = xv[i];
+        float4 v = xv[i];
+        if (xup)
+            v = make_float4((v.x / (__expf(-v.x) + 1.0f)) * uv[i].x, (v.y / (__expf(-v.y) + 1.0f)) * uv[i].y,
+                            (v.z / (__expf(-v.z) + 1.0f)) * uv[i].z, (v.w / (__expf(-v.w) + 1.0f)) * uv[i].w);
         float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
         amax = fmaxf(amax, dpp_f32<DPP_XOR1>(amax));
         amax = fmaxf(amax, dpp_f32<DPP_XOR2>(amax));
@@ -187,7 +194,7 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
             float rr = v0;
             if (EPI == FH_EPI_ADD2) rr = (rr + ea[row]) + eb[row];
             if (EPI == FH_EPI_SWIGLU) rr = (rr / (__expf(-rr) + 1.0f)) * v1;
-            if (EPI == FH_EPI_ACC) unsafeAtomicAdd(y + row, blockIdx.y == 0 ? rr + ea[row] : rr);
+            if (EPI == FH_EPI_ACC) unsafeAtomicAdd(y + row, (blockIdx.y == 0 && ea) ? rr + ea[row] : rr);
             else y[row] = rr;
         }
     }
@@ -195,14 +202,14 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
 
 template <int TS, int PER, int EPI>
 static fh_status q6k_m1_launch(const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b, int SW,
-                               unsigned grid, size_t lds, unsigned ksplit = 1) {
+                               unsigned grid, size_t lds, unsigned ksplit = 1, const float *xup = nullptr) {
     static bool attr_done = false;
     if (!attr_done) {
         FH_HIP(hipFuncSetAttribute((const void *)k_qmv_q6k_m1<TS, PER, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    160 * 1024));
         attr_done = true;
     }
-    k_qmv_q6k_m1<TS, PER, EPI><<<dim3(grid, ksplit), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW);
+    k_qmv_q6k_m1<TS, PER, EPI><<<dim3(grid, ksplit), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, xup);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
@@ -259,7 +266,8 @@ fh_status fh_launch_q6k_m1(const fh_qmatrix *q, const float *x, float *y, int ep
 // y += W . x + add with k split over `ksplit` workgroups per row tile (atomic adds, so the summation order - and the
 // last bits of the result - vary from run to run).  For matrices with few row tiles and a long k (the down projection
 // of a decode step accumulating into the residual stream) the smaller workgroups overlap their load and compute phases.
-fh_status fh_launch_q6k_m1_acc(const fh_qmatrix *q, const float *x, float *y_inout, const float *add) {
+// With xup the input is silu(x) * xup.
+fh_status fh_launch_q6k_m1_acc(const fh_qmatrix *q, const float *x, const float *xup, float *y_inout, const float *add) {
     fh_device *dev = q->dev;
     const int kb = (int)q->kb;
     int ks = (int)dev->opt_matvec_splitk;
@@ -273,7 +281,7 @@ fh_status fh_launch_q6k_m1_acc(const fh_qmatrix *q, const float *x, float *y_ino
     if (SW > 16) return FH_ERR_UNSUPPORTED;
     const int64_t tiles = (q->n + 15) / 16;
     size_t lds = (size_t)kbl * Q6K_IMG * 16 + (size_t)kbl * Q6K_SF * 4 + (size_t)SW * 64;
-    if (per == 1) return q6k_m1_launch<1, 1, FH_EPI_ACC>(q, x, y_inout, add, nullptr, SW, (unsigned)tiles, lds, (unsigned)ks);
-    if (per == 2) return q6k_m1_launch<1, 2, FH_EPI_ACC>(q, x, y_inout, add, nullptr, SW, (unsigned)tiles, lds, (unsigned)ks);
-    return q6k_m1_launch<1, 4, FH_EPI_ACC>(q, x, y_inout, add, nullptr, SW, (unsigned)tiles, lds, (unsigned)ks);
+    if (per == 1) return q6k_m1_launch<1, 1, FH_EPI_ACC>(q, x, y_inout, add, nullptr, SW, (unsigned)tiles, lds, (unsigned)ks, xup);
+    if (per == 2) return q6k_m1_launch<1, 2, FH_EPI_ACC>(q, x, y_inout, add, nullptr, SW, (unsigned)tiles, lds, (unsigned)ks, xup);
+    return q6k_m1_launch<1, 4, FH_EPI_ACC>(q, x, y_inout, add, nullptr, SW, (unsigned)tiles, lds, (unsigned)ks, xup);
 }
