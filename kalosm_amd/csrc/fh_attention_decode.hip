@@ -220,8 +220,9 @@ template <typename TKV, int G>
 static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const void *v, int64_t kv_sh, int64_t kv_st,
                            int hq, int hkv, float scale, const int *len_dev, int max_len, float *out, int *splits_out) {
     constexpr int D = 128, NWV = 16;
-    // splits: about 256 keys of capacity each, between 4 and 16 (the consumer of the partials reads all of them)
-    int S = dev->opt_attn_splits > 0 ? (int)dev->opt_attn_splits : (max_len + 255) / 256;
+    // splits: 8 measured best from a few hundred to a few thousand keys (MI355X); it is also the most the output
+    // projection merges while staging its input.  The option allows 4 .. 16.
+    int S = dev->opt_attn_splits > 0 ? (int)dev->opt_attn_splits : 8;
     S = S < 4 ? 4 : (S > 16 ? 16 : S);
     const int chunk_max = ((max_len + S - 1) / S + 15) & ~15;
     const size_t lds = ((size_t)G * chunk_max + (size_t)NWV * G * D) * 4;
