@@ -29,7 +29,49 @@ ROTATE_BYTES = 640 << 20  # > 2x the 256 MB Infinity Cache
 # HBM bytes per launch (average of the four shapes) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this
 # workload at batch 1, scaled by what the same counters read for a 256 MiB device copy (FETCH_SIZE x2.000,
 # WRITE_SIZE x1.000); a measured constant, to be re-measured when the kernel changes.
-TRAFFIC_BYTES_PER_LAUNCH = 19768986
+TRAFFIC_BYTES_PER_LAUNCH = 19772006
+
+
+def prefill_legs(dev) -> dict:
+    """configs[2]: Y = X . W^T with bf16 X [m, 4096] and Q6_K / Q8_0 W [14336, 4096]; configs[3]: causal attention,
+    f16, 32 query heads on 8 KV heads, head_dim 128.  Device time per call from events around 5 calls; TFLOP/s counts
+    2 m n k (matmul) and 4 s^2 d h / 2 (causal attention) against the 2.5 PFLOP/s dense f16 MFMA peak."""
+    from kalosm_amd import synth
+    from kalosm_amd.fusor import MaskKind, QMatrix, Tensor
+
+    res = {"matmul": [], "attention": []}
+    n, k = 14336, 4096
+    for ty, name in ((synth.Q6_K, "Q6_K"), (synth.Q8_0, "Q8_0")):
+        q = QMatrix.from_raw_bytes(dev, (n, k), synth.random_weight(ty, n, k, seed=7), ty)
+        for m in (512, 2048):
+            x = Tensor.from_slice(dev, synth.to_bf16_bits(synth.random_activation(m, k, seed=8)), dtype="bf16")
+            y = Tensor(dev, (m, n), "f32")
+            for _ in range(2):
+                x.q_mat_mul(q, out=y)
+            dev.sync()
+            dev.timer_start()
+            for _ in range(5):
+                x.q_mat_mul(q, out=y)
+            ms = dev.timer_stop() / 5
+            tf = 2.0 * m * n * k / ms / 1e9
+            res["matmul"].append({"weights": name, "m": m, "n": n, "k": k, "us": round(ms * 1e3, 1),
+                                  "TFLOPs": round(tf, 1), "frac_mfma_peak": round(tf / 2500.0, 4)})
+    h, hkv, d = 32, 8, 128
+    for s in (512, 2048, 8192):
+        rng = np.random.default_rng(s)
+        qt, kt, vt = (Tensor.from_slice(dev, rng.standard_normal((1, hh, s, d)).astype(np.float16), "f16")
+                      for hh in (h, hkv, hkv))
+        for _ in range(2):
+            qt.flash_attention(kt, vt, 1 / np.sqrt(d), MaskKind.Causal)
+        dev.sync()
+        dev.timer_start()
+        for _ in range(5):
+            qt.flash_attention(kt, vt, 1 / np.sqrt(d), MaskKind.Causal)
+        ms = dev.timer_stop() / 5
+        tf = 4.0 * s * s * d * h / 2 / ms / 1e9
+        res["attention"].append({"seq": s, "us": round(ms * 1e3, 1), "TFLOPs": round(tf, 1),
+                                 "frac_mfma_peak": round(tf / 2500.0, 4)})
+    return res
 
 
 def main() -> int:
@@ -40,6 +82,10 @@ def main() -> int:
     ap.add_argument("--m", type=int, default=1, help="activation rows (decode batch)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--e2e", action="store_true", help="also run the 8B-architecture decoder (tok/s) and report it")
+    ap.add_argument("--e2e-eager", action="store_true",
+                    help="also run 32 decode steps of the decoder with stream launches (for a kernel tracer)")
+    ap.add_argument("--prefill", action="store_true",
+                    help="also time the prefill matmul (configs[2]) and the causal prefill attention (configs[3])")
     ap.add_argument("--no-graph", action="store_true", help="launch on the stream instead of replaying a recorded graph")
     ap.add_argument("--calib-copy", action="store_true", help="append 4 device copies of 256 MiB (counter calibration)")
     args = ap.parse_args()
@@ -133,7 +179,7 @@ def main() -> int:
         "wall_ms_timed_region": round(wall_ms, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH if m == 1 else None,
-                     "kernel": "k_qmv_q4k_m1", "avg_launch_us": round(avg_us, 3),
+                     "kernel": "k_qmv_q4k_m1 (instances <1,1>, <2,2>, <1,4>)", "avg_launch_us": round(avg_us, 3),
                      "algorithmic_bytes_per_launch": step_bytes // len(sets)},
     }
 
@@ -176,6 +222,11 @@ def main() -> int:
     if args.e2e:
         from kalosm_amd import e2e
         out["e2e"] = e2e.run(dev)
+    if args.e2e_eager:
+        from kalosm_amd import e2e
+        out["e2e_eager"] = e2e.run(dev, steps=32, repeats=1, use_graph=False)
+    if args.prefill:
+        out["prefill"] = prefill_legs(dev)
 
     print(json.dumps(out))
     return 0

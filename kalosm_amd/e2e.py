@@ -11,10 +11,10 @@ from .llama import Model
 
 
 def run(dev, cfg: dict | None = None, prompt_len: int = 512, steps: int = 256, seed: int = 0, sigma: float = 1e-4,
-        kv_dtype: str = "f32", repeats: int = 2, prefill_chunk: int = 512) -> dict:
+        kv_dtype: str = "f32", repeats: int = 2, prefill_chunk: int = 512, use_graph: bool = True) -> dict:
     cfg = dict(cfg or synth.LLAMA3_8B)
     t0 = time.perf_counter()
-    m = Model.random_init(dev, cfg, seed=seed, sigma=sigma, kv_dtype=kv_dtype)
+    m = Model.random_init(dev, cfg, seed=seed, sigma=sigma, kv_dtype=kv_dtype, use_graph=use_graph)
     load_s = time.perf_counter() - t0
     rng = np.random.default_rng(seed + 1)
     prompt = rng.integers(0, cfg["vocab"], prompt_len)
@@ -35,7 +35,7 @@ def run(dev, cfg: dict | None = None, prompt_len: int = 512, steps: int = 256, s
     wbytes = m.weight_bytes()
     tok_s = steps / (best * 1e-3)
     return {"tok_per_s": round(tok_s, 1), "ms_per_token": round(best / steps, 4), "steps": steps,
-            "prompt_len": prompt_len, "prefill_ms_host_clock": round(prefill_ms, 1), "kv_dtype": kv_dtype,
+            "prompt_len": prompt_len, "graph_replay": use_graph, "prefill_ms_host_clock": round(prefill_ms, 1), "kv_dtype": kv_dtype,
             "weight_bytes_per_token": wbytes, "weights_GBps": round(wbytes * tok_s / 1e9, 1),
             "frac_hbm_peak": round(wbytes * tok_s / 8e12, 4), "load_seconds": round(load_s, 1),
             "first_tokens": [int(t) for t in toks[:8]], "config": {k: cfg[k] for k in ("n_layers", "d_model", "ffn", "vocab")}}
