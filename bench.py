@@ -54,8 +54,22 @@ def prefill_legs(dev) -> dict:
                 x.q_mat_mul(q, out=y)
             ms = dev.timer_stop() / 5
             tf = 2.0 * m * n * k / ms / 1e9
-            res["matmul"].append({"weights": name, "m": m, "n": n, "k": k, "us": round(ms * 1e3, 1),
-                                  "TFLOPs": round(tf, 1), "frac_mfma_peak": round(tf / 2500.0, 4)})
+            res["matmul"].append({"weights": name, "activations": "bf16", "m": m, "n": n, "k": k,
+                                  "us": round(ms * 1e3, 1), "TFLOPs": round(tf, 1),
+                                  "frac_mfma_peak": round(tf / 2500.0, 4)})
+            if ty == synth.Q8_0:  # the integer variant: f32 activations quantised per 32 inside the call, int8 MFMA
+                xf = Tensor.from_slice(dev, synth.random_activation(m, k, seed=8))
+                for _ in range(2):
+                    xf.q_mat_mul_q8(q, out=y)
+                dev.sync()
+                dev.timer_start()
+                for _ in range(5):
+                    xf.q_mat_mul_q8(q, out=y)
+                ms = dev.timer_stop() / 5
+                tf = 2.0 * m * n * k / ms / 1e9
+                res["matmul"].append({"weights": name, "activations": "Q8_0 per 32 (int8 MFMA)", "m": m, "n": n, "k": k,
+                                      "us": round(ms * 1e3, 1), "TOPs": round(tf, 1),
+                                      "frac_int8_mfma_peak": round(tf / 5000.0, 4)})
     h, hkv, d = 32, 8, 128
     for s in (512, 2048, 8192):
         rng = np.random.default_rng(s)

@@ -145,6 +145,7 @@ fh_status fh_launch_qmatvec(const fh_qmatrix *q, const float *x, int m, float *y
 bool fh_qmatvec_batch_supports(const fh_qmatrix *q, int m, int epi);
 fh_status fh_launch_qmatvec_batch(const fh_qmatrix *q, const float *x, int m, float *y, int epi, const float *a,
                                   const float *b);
+fh_status fh_launch_qmm_q8_mfma(const fh_qmatrix *q, const float *x, int m, float *y);
 fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y);
 enum { FH_EPI_NONE = 0, FH_EPI_ADD2 = 1, FH_EPI_SWIGLU = 2, FH_EPI_ROPEKV = 3, FH_EPI_ACC = 4 };
 fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b);

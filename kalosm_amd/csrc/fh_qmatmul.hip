@@ -89,6 +89,8 @@ extern "C" fh_status fh_qmatmul_q8(const fh_qmatrix *q, const float *x_dev, int3
     if (q->type != FH_Q8_0 && q->type != FH_Q4_0)
         FH_FAIL(FH_ERR_UNSUPPORTED, "the Q8 activation path exists for Q8_0 and Q4_0 weights only (type %u)", q->type);
     fh_device *dev = q->dev;
+    // Q8_0 weights without a request for the integer block sums: the integer matrix-core kernel
+    if (q->type == FH_Q8_0 && !isums_dev && dev->opt_matmul_kernel != 1) return fh_launch_qmm_q8_mfma(q, x_dev, m, y_dev);
     int64_t nb = (int64_t)m * q->kb;
     FH_TRY(fh_dev_scratch(dev, &dev->act_buf, &dev->act_cap, (size_t)nb * 34 + 64));
     k_q8_0_quantize<<<dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, dev->stream>>>(x_dev, nb, (uint8_t *)dev->act_buf);

@@ -205,10 +205,11 @@ class Tensor:
         check(self.device._lib.fh_qmatmul_swiglu(gate_up._h, C.c_void_p(self.ptr), m, C.c_void_p(out.ptr)))
         return out
 
-    def q_mat_mul_q8(self, w: "QMatrix", want_isums: bool = False):
+    def q_mat_mul_q8(self, w: "QMatrix", want_isums: bool = False, out: Optional["Tensor"] = None):
         """The Q8_0 x Q8 integer variant (per-32 activation quantisation + vec_dot)."""
         m = int(np.prod(self.shape[:-1]))
-        out = Tensor(self.device, (*self.shape[:-1], w.n), "f32")
+        if out is None:
+            out = Tensor(self.device, (*self.shape[:-1], w.n), "f32")
         isums = Tensor(self.device, (m, w.n, w.k // 32), "i32") if want_isums else None
         check(self.device._lib.fh_qmatmul_q8(w._h, C.c_void_p(self.ptr), m, C.c_void_p(out.ptr),
                                              C.c_void_p(isums.ptr) if isums else None))

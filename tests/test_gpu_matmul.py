@@ -199,3 +199,40 @@ def test_batch_matvec_epilogues(dev, oracle, ty, m):
         assert_close(got, oracle.add3(yg, a, b), what=f"add2 m={m}")
     finally:
         dev.set_option("matvec_kernel", 0)
+
+
+# ---------------------------------------------------------------------------------------------- Q8_0 x Q8 on int8 MFMA
+@pytest.mark.parametrize("m,n,k", [(3, 80, 1024), (130, 300, 96), (64, 128, 2048), (257, 100, 320)])
+def test_q8_activation_matmul_mfma(dev, oracle, m, n, k):
+    """Q8_0 weights x per-32 quantised activations on the integer matrix cores: exact block sums and the reference's
+    operation order (f32(isum) * (d_w * d_a), blocks added in k order) give the checker's result bit for bit.  Shapes
+    with ragged tiles and an odd number of blocks (the device record holds two)."""
+    raw = synth.random_weight(Q8_0, n, k, seed=200 + m)
+    x = synth.random_activation(m, k, seed=201)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, Q8_0)
+    got = Tensor.from_slice(dev, x).q_mat_mul_q8(q)
+    want = oracle.q8_0_matmul_q8(x, raw, n)
+    assert np.array_equal(got.as_slice().view(np.uint32), want.view(np.uint32)), \
+        f"max abs diff {np.abs(got.as_slice() - want).max()}"
+    dev.set_option("matmul_kernel", 1)  # the per-output kernel gives the same bits
+    try:
+        old = Tensor.from_slice(dev, x).q_mat_mul_q8(q)
+    finally:
+        dev.set_option("matmul_kernel", 0)
+    assert np.array_equal(old.as_slice().view(np.uint32), want.view(np.uint32))
+
+
+def test_q8_activation_matmul_prefill_shape(dev, oracle):
+    """configs[2], integer variant, full shape (m = 512, k = 4096, n = 14336): 48 sampled weight rows against the
+    checker bit for bit, every output finite."""
+    m, k, n = 512, 4096, 14336
+    raw = synth.random_weight(Q8_0, n, k, seed=210)
+    x = synth.random_activation(m, k, seed=211)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, Q8_0)
+    got = Tensor.from_slice(dev, x).q_mat_mul_q8(q).as_slice()
+    assert np.isfinite(got).all()
+    rows = (np.arange(48) * 299 + 7) % n
+    bpr = len(raw) // n
+    sub = np.concatenate([raw[r * bpr:(r + 1) * bpr] for r in rows])
+    want = oracle.q8_0_matmul_q8(x, sub, 48)
+    assert np.array_equal(got[:, rows].view(np.uint32), want.view(np.uint32))
