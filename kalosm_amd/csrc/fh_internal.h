@@ -59,7 +59,7 @@ struct fh_device {
     int64_t opt_down_splitk = 0;     // 0: decode steps split k of a Q6_K down projection (atomic adds), 1: never, 3: and SwiGLU in its staging
     int64_t opt_wo_acc = 0;          // 0: decode steps accumulate the output projection into the residual stream, 1: never
     int64_t opt_fuse_norm = 0;       // 0: decode steps fold rms_norm into the consuming matvec, 1: separate launches
-    int64_t opt_matmul_kernel = 0;   // 0 auto, 1 generic for every m, 2 MFMA tile kernel for every m
+    int64_t opt_matmul_kernel = 0;   // 0 auto, 1 generic for every m, 2 MFMA tile kernels for every m, 3 / 4 and never / always the 128 x 256 one
 };
 
 fh_status fh_dev_scratch(fh_device *dev, void **buf, size_t *cap, size_t need);

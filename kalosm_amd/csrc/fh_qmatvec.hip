@@ -387,7 +387,7 @@ static fh_status qmm_check(const fh_qmatrix *q, const void *x, int m, const void
 extern "C" fh_status fh_qmatmul(const fh_qmatrix *q, const float *x_dev, int32_t m, float *y_dev) {
     FH_TRY(qmm_check(q, x_dev, m, y_dev));
     const int64_t mk = q->dev->opt_matmul_kernel;
-    if ((m > 16 && mk != 1) || mk == 2) return fh_launch_qmatmul_tile(q, x_dev, 0, m, y_dev);
+    if ((m > 16 && mk != 1) || mk >= 2) return fh_launch_qmatmul_tile(q, x_dev, 0, m, y_dev);
     return fh_launch_qmatvec(q, x_dev, m, y_dev, FH_EPI_NONE, nullptr, nullptr);
 }
 

@@ -238,11 +238,269 @@ __global__ __launch_bounds__(64 * WGN * WGM) void k_qmm_tile(QView q, const _Flo
     }
 }
 
+// ------------------------------------------------------------------------------ pipelined 128 x 256 tile kernel
+// The same product for many activation rows: 8 wavefronts (2 x 4) of 64 x 64 each, so the decode of a weight slab is
+// shared by 256 activation rows.  The raw block bytes and the activation slab of step s+2 are in flight in
+// registers, step s+1 is decoded into the second LDS buffer while the MFMAs of step s (issued first) drain: one
+// barrier per step.
+struct QmmRaw {
+    uint32_t a, b; // code words
+    uint4 h;       // scale material (format dependent)
+};
+
+template <int T>
+__device__ __forceinline__ void qmm_load_raw(const QView &q, int64_t tile16, int j, int g, int ks, QmmRaw &r) {
+    r.a = r.b = 0;
+    r.h = make_uint4(0, 0, 0, 0);
+    if (T == FH_Q8_0) {
+        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 1)) * 1088;
+        const int u = ks & 1;
+        const uint2 c = *(const uint2 *)(rec + (g * 16 + j) * 16 + 8 * u);
+        r.a = c.x;
+        r.b = c.y;
+        r.h.x = fh_ld16(rec + 1024 + 4 * j + 2 * u);
+    } else if (T == FH_Q4_0) {
+        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 2)) * 1152;
+        const int u = ks & 3;
+        r.a = *(const uint32_t *)(rec + (g * 16 + j) * 16 + 4 * u);
+        r.h.x = fh_ld16(rec + 1024 + 8 * j + 2 * u);
+    } else if (T == FH_Q4_K) {
+        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 3)) * 2304;
+        const int sb = ks & 7, p = sb >> 2, u = (sb >> 1) & 1;
+        const uint2 c = *(const uint2 *)(rec + 256 + p * 1024 + (g * 16 + j) * 16 + 8 * u);
+        r.a = c.x;
+        r.b = c.y;
+        r.h = *(const uint4 *)(rec + 16 * j);
+    } else {
+        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 3)) * 3360;
+        const int t = ks & 7;
+        r.a = *(const uint32_t *)(rec + q6k_lword_off(j, t, g));
+        r.b = *(const uint32_t *)(rec + q6k_hword_off(j, t, g));
+        r.h.x = rec[q6k_sc_off(j, 2 * t + (g >> 1))];
+        r.h.y = fh_ld16(rec + q6k_d_off(j));
+    }
+}
+
+// Eight dequantised weights from the raw words (arithmetic of fh_blocks.h), and their positions in the step.
+template <int T>
+__device__ __forceinline__ void qmm_decode_raw(const QmmRaw &r, int g, int ks, float *w, int &p0, int &p1) {
+    p0 = 8 * g;
+    p1 = 8 * g + 4;
+    if (T == FH_Q8_0) {
+        const float d = fh_h2f((uint16_t)r.h.x);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[i] = (float)(int)(int8_t)(r.a >> (8 * i)) * d;
+            w[4 + i] = (float)(int)(int8_t)(r.b >> (8 * i)) * d;
+        }
+    } else if (T == FH_Q4_0) {
+        const float d = fh_h2f((uint16_t)r.h.x);
+        p0 = 4 * g;
+        p1 = 16 + 4 * g;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[i] = (float)((int)((r.a >> (8 * i)) & 15u) - 8) * d;
+            w[4 + i] = (float)((int)((r.a >> (8 * i + 4)) & 15u) - 8) * d;
+        }
+    } else if (T == FH_Q4_K) {
+        const int sb = ks & 7, hn = sb & 1;
+        const uint4 h = r.h;
+        const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
+        const uint32_t scw = sb < 4 ? (h.y & 0x3F3F3F3Fu) : ((h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u));
+        const uint32_t mnw = sb < 4 ? (h.z & 0x3F3F3F3Fu) : (((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u));
+        const float scale = (float)((scw >> (8 * (sb & 3))) & 0xFFu) * d;
+        const float off = (float)((mnw >> (8 * (sb & 3))) & 0xFFu) * dmin;
+        const int sh = 4 * hn;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float a = scale * (float)((r.a >> (8 * i + sh)) & 15u);
+            const float b = scale * (float)((r.b >> (8 * i + sh)) & 15u);
+            w[i] = a - off;
+            w[4 + i] = b - off;
+        }
+    } else {
+        const int t = ks & 7;
+        const float ds = fh_h2f((uint16_t)r.h.y) * (float)(int)(int8_t)r.h.x;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int pp = i >> 1, odd = i & 1;
+            const int nib = (int)((r.a >> (4 * (pp + 4 * odd))) & 15u);
+            const int hb = (int)((r.b >> (q6k_hbit(t, pp) + 16 * odd)) & 3u);
+            w[i] = ds * (float)(((hb << 4) | nib) - 32);
+        }
+    }
+}
+
+template <int T, int NTERM>
+__global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__restrict__ xh,
+                                                   const _Float16 *__restrict__ xl, const float *__restrict__ rs,
+                                                   int m, float *__restrict__ y) {
+    constexpr int TN = 128, TM = 256, FN = 2, FM = 2;
+    constexpr int A_H = TN * QMM_LDK, B_H = TM * QMM_LDK;         // halfs per plane
+    constexpr int BUF = 2 * A_H + NTERM * B_H;                    // halfs per buffer: A hi, A lo, B hi (, B lo)
+    extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int wn = wave >> 2, wm = wave & 3;
+    const int64_t n0 = (int64_t)blockIdx.x * TN;
+    const int m0 = blockIdx.y * TM;
+    const int K = (int)q.k, ksteps = K / 32;
+    const int64_t tiles16 = (q.n + 15) / 16;
+    // this thread's weight duty: row a_row of the tile, lane group a_g (8 weights per step)
+    const int a_row = tid >> 2, a_g = tid & 3, a_j = a_row & 15;
+    int64_t a_tile = (n0 >> 4) + (a_row >> 4);
+    if (a_tile >= tiles16) a_tile = tiles16 - 1; // rows past the end decode a valid tile and are never stored
+    // activation duty: two 16-byte pieces per plane and step
+    // piece i (0, 1): row (tid + 512 i) / 4 of the tile, 16-byte column (tid + 512 i) % 4 = tid % 4
+    const int b_c = tid & 3, b_row0 = tid >> 2, b_row1 = b_row0 + 128;
+    // rows past the end repeat the last one (never stored)
+    const int64_t b_off0 = (int64_t)(m0 + b_row0 < m ? m0 + b_row0 : m - 1) * K + b_c * 8;
+    const int64_t b_off1 = (int64_t)(m0 + b_row1 < m ? m0 + b_row1 : m - 1) * K + b_c * 8;
+    // two register sets (even / odd steps), named so that no indexing survives into the generated code
+    struct Slab {
+        QmmRaw raw;
+        uint4 h0, h1, l0, l1;
+    } s0, s1;
+    auto fetch = [&](Slab &sl, int ks) {
+        qmm_load_raw<T>(q, a_tile, a_j, a_g, ks, sl.raw);
+        sl.h0 = *(const uint4 *)(xh + b_off0 + ks * 32);
+        sl.h1 = *(const uint4 *)(xh + b_off1 + ks * 32);
+        if (NTERM == 2) {
+            sl.l0 = *(const uint4 *)(xl + b_off0 + ks * 32);
+            sl.l1 = *(const uint4 *)(xl + b_off1 + ks * 32);
+        }
+    };
+    auto stage = [&](const Slab &sl, int ks) {
+        _Float16 *buf = smem + (ks & 1) * BUF;
+        float w[8];
+        int p0, p1;
+        qmm_decode_raw<T>(sl.raw, a_g, ks, w, p0, p1);
+        _Float16 hi[8], lo[8];
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            hi[c] = (_Float16)w[c];
+            lo[c] = (_Float16)(w[c] - (float)hi[c]);
+        }
+        uint2 a0, a1, l0, l1;
+        __builtin_memcpy(&a0, hi, 8);
+        __builtin_memcpy(&a1, hi + 4, 8);
+        __builtin_memcpy(&l0, lo, 8);
+        __builtin_memcpy(&l1, lo + 4, 8);
+        *(uint2 *)(buf + a_row * QMM_LDK + p0) = a0;
+        *(uint2 *)(buf + a_row * QMM_LDK + p1) = a1;
+        *(uint2 *)(buf + A_H + a_row * QMM_LDK + p0) = l0;
+        *(uint2 *)(buf + A_H + a_row * QMM_LDK + p1) = l1;
+        *(uint4 *)(buf + 2 * A_H + b_row0 * QMM_LDK + b_c * 8) = sl.h0;
+        *(uint4 *)(buf + 2 * A_H + b_row1 * QMM_LDK + b_c * 8) = sl.h1;
+        if (NTERM == 2) {
+            *(uint4 *)(buf + 2 * A_H + B_H + b_row0 * QMM_LDK + b_c * 8) = sl.l0;
+            *(uint4 *)(buf + 2 * A_H + B_H + b_row1 * QMM_LDK + b_c * 8) = sl.l1;
+        }
+    };
+    floatx16 acc[FN][FM];
+#pragma unroll
+    for (int a = 0; a < FN; a++)
+#pragma unroll
+        for (int b = 0; b < FM; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
+
+    fetch(s0, 0);
+    if (ksteps > 1) fetch(s1, 1);
+    stage(s0, 0);
+    for (int ks0 = 0; ks0 < ksteps; ks0 += 2) {
+#pragma unroll
+        for (int d = 0; d < 2; d++) { // slot d holds step ks0 + d ... the slot index stays a compile-time constant
+            const int ks = ks0 + d;
+            if (ks < ksteps) {
+                __syncthreads(); // buffer ks & 1 is complete; the other one is no longer read
+                // raw[d] was consumed by stage(d, ks) in the previous iteration (or the prologue)
+                if (ks + 2 < ksteps) {
+                    if (d == 0) fetch(s0, ks + 2);
+                    else fetch(s1, ks + 2);
+                }
+                const _Float16 *buf = smem + (ks & 1) * BUF;
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++) {
+                    const int ko = kk * 16 + 8 * (lane >> 5), li = lane & 31;
+                    half8 ah[FN], al[FN], bhv[FM], blv[FM];
+#pragma unroll
+                    for (int a = 0; a < FN; a++) {
+                        const int row = (wn * FN + a) * 32 + li;
+                        ah[a] = *(const half8 *)(buf + row * QMM_LDK + ko);
+                        al[a] = *(const half8 *)(buf + A_H + row * QMM_LDK + ko);
+                    }
+#pragma unroll
+                    for (int b = 0; b < FM; b++) {
+                        const int row = (wm * FM + b) * 32 + li;
+                        bhv[b] = *(const half8 *)(buf + 2 * A_H + row * QMM_LDK + ko);
+                        if (NTERM == 2) blv[b] = *(const half8 *)(buf + 2 * A_H + B_H + row * QMM_LDK + ko);
+                    }
+#pragma unroll
+                    for (int a = 0; a < FN; a++)
+#pragma unroll
+                        for (int b = 0; b < FM; b++) {
+                            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[a], bhv[b], acc[a][b], 0, 0, 0);
+                            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[a], bhv[b], acc[a][b], 0, 0, 0);
+                            if (NTERM == 2)
+                                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[a], blv[b], acc[a][b], 0, 0, 0);
+                        }
+                }
+                if (ks + 1 < ksteps) { // the other register set holds step ks + 1
+                    if (d == 0) stage(s1, ks + 1);
+                    else stage(s0, ks + 1);
+                }
+            }
+        }
+    }
+    const bool vec = (q.n & 3) == 0;
+#pragma unroll
+    for (int b = 0; b < FM; b++) {
+        const int mm = m0 + (wm * FM + b) * 32 + (lane & 31);
+        if (mm >= m) continue;
+        const float s = rs[mm];
+#pragma unroll
+        for (int a = 0; a < FN; a++) {
+            const int64_t nb = n0 + (wn * FN + a) * 32 + 4 * (lane >> 5);
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+                const int64_t nn = nb + 8 * r4;
+                const float4 v = make_float4(acc[a][b][4 * r4] * s, acc[a][b][4 * r4 + 1] * s, acc[a][b][4 * r4 + 2] * s,
+                                             acc[a][b][4 * r4 + 3] * s);
+                float *dst = y + (int64_t)mm * q.n + nn;
+                if (vec && nn + 3 < q.n) {
+                    *(float4 *)dst = v;
+                } else {
+                    if (nn < q.n) dst[0] = v.x;
+                    if (nn + 1 < q.n) dst[1] = v.y;
+                    if (nn + 2 < q.n) dst[2] = v.z;
+                    if (nn + 3 < q.n) dst[3] = v.w;
+                }
+            }
+        }
+    }
+}
+
 template <int T, int NTERM>
 static fh_status qmm_launch_t(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const float *rs, int m,
                               float *y) {
     hipStream_t s = q->dev->stream;
     QView v = fh_view(q);
+    // the 128 x 256 kernel when it still fills most of the device (opt_matmul_kernel = 3: never)
+    const int64_t wgs2 = ((q->n + 127) / 128) * ((m + 255) / 256);
+    const int64_t mk = q->dev->opt_matmul_kernel; // 3: never, 4: always
+    if (mk == 4 || (m > 128 && wgs2 * 5 >= (int64_t)q->dev->compute_units * 4 && mk != 3)) {
+        constexpr size_t lds = 2 * (size_t)(2 * 128 * QMM_LDK + NTERM * 256 * QMM_LDK) * 2;
+        static bool attr_done = false;
+        if (!attr_done) {
+            FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2<T, NTERM>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)lds));
+            attr_done = true;
+        }
+        dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + 255) / 256));
+        k_qmm_tile2<T, NTERM><<<grid, 512, lds, s>>>(v, xh, xl, rs, m, y);
+        FH_HIP(hipGetLastError());
+        return FH_OK;
+    }
     if (m <= 32) {
         dim3 grid((unsigned)((q->n + 127) / 128), 1);
         k_qmm_tile<T, NTERM, 4, 1, 1, 1><<<grid, 256, 0, s>>>(v, xh, xl, rs, m, y);

@@ -21,9 +21,10 @@ def bf16_round(x):
     return r, (r.astype(np.uint32) << 16).view(np.float32)
 
 
-def tile_matmul(dev, x, q, force=True):
+def tile_matmul(dev, x, q, force=2):
+    """force = 2: the tile kernels for every m (128 x 128 or 128 x 256 by size); 4: always the pipelined 128 x 256 one."""
     out = Tensor.filled_bytes(dev, (x.shape[0], q.n), 0xFF)  # poisoned: unwritten elements show as NaN
-    dev.set_option("matmul_kernel", 2 if force else 0)
+    dev.set_option("matmul_kernel", force)
     try:
         return Tensor.from_slice(dev, x).q_mat_mul(q, out=out).as_slice()
     finally:
@@ -34,13 +35,15 @@ def tile_matmul(dev, x, q, force=True):
 @pytest.mark.parametrize("m,n,k", [(17, 272, 2048), (33, 130, 1024), (64, 128, 512), (65, 100, 768), (130, 300, 1024),
                                    (256, 256, 256), (3, 37, 512)])
 def test_tile_matmul_f32_vs_checker(dev, oracle, ty, m, n, k):
-    """Ragged m (tile edges 32 / 64 / 128), ragged n (not a multiple of 4, 16 or 128), k of 1..8 super-blocks."""
+    """Ragged m (tile edges 32 / 64 / 128 / 256), ragged n (not a multiple of 4, 16 or 128), k of 1..8 super-blocks;
+    both tile kernels."""
     raw = synth.random_weight(ty, n, k, seed=50 + ty)
     x = synth.random_activation(m, k, seed=60 + m)
     q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
-    got = tile_matmul(dev, x, q)
     want = oracle.q_mat_mul(ty, x, raw, n, fast=True)
-    assert_close(got, want, what=f"{NAMES[ty]} {n}x{k} m={m}")
+    for force in (2, 4):
+        got = tile_matmul(dev, x, q, force)
+        assert_close(got, want, what=f"{NAMES[ty]} {n}x{k} m={m} kernel option {force}")
 
 
 @pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
@@ -94,10 +97,15 @@ def test_tile_matmul_bf16_activations(dev, oracle, ty, m):
     raw = synth.random_weight(ty, n, k, seed=90 + ty)
     xb, xf = bf16_round(synth.random_activation(m, k, seed=91 + m))
     q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
-    out = Tensor.filled_bytes(dev, (m, n), 0xFF)
-    got = Tensor.from_slice(dev, xb, dtype="bf16").q_mat_mul(q, out=out).as_slice()
     want = oracle.q_mat_mul(ty, xf, raw, n, fast=True)
-    assert_close(got, want, what=f"bf16 {NAMES[ty]} m={m}")
+    for force in (0, 4):
+        dev.set_option("matmul_kernel", force)
+        try:
+            out = Tensor.filled_bytes(dev, (m, n), 0xFF)
+            got = Tensor.from_slice(dev, xb, dtype="bf16").q_mat_mul(q, out=out).as_slice()
+        finally:
+            dev.set_option("matmul_kernel", 0)
+        assert_close(got, want, what=f"bf16 {NAMES[ty]} m={m} kernel option {force}")
 
 
 @pytest.mark.parametrize("ty", [Q6_K, Q8_0], ids=lambda t: NAMES[t])
