@@ -50,7 +50,7 @@ __device__ __forceinline__ void ap_store4(fh_half *p, float a, float b, float c,
 }
 
 template <typename TQ, typename TKV, int D>
-__global__ __launch_bounds__(256) void k_attn_prefill(const TQ *__restrict__ q, int64_t q_sb, int64_t q_sh, int64_t q_st,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_attn_prefill(const TQ *__restrict__ q, int64_t q_sb, int64_t q_sh, int64_t q_st,
                                                        const TKV *__restrict__ k, const TKV *__restrict__ v,
                                                        int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int hq, int hkv,
                                                        int sq, int skv, float scale, int causal, TQ *__restrict__ out) {
@@ -59,7 +59,8 @@ __global__ __launch_bounds__(256) void k_attn_prefill(const TQ *__restrict__ q, 
     __shared__ __attribute__((aligned(16))) fh_half sV[D * VS];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
     const int h = blockIdx.y, bi = blockIdx.z, kh = h / (hq / hkv);
-    const int qb0 = blockIdx.x * 128;
+    // causal: the last query blocks see the most keys; they are dispatched first so that the short ones fill the tail
+    const int qb0 = (causal ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x) * 128;
     const int qi = qb0 + wave * 32 + li; // this lane's query row
     const int off = skv - sq;            // causal: query i sees keys 0 .. i + off
     const TKV *kb = k + bi * kv_sb + kh * kv_sh, *vb = v + bi * kv_sb + kh * kv_sh;
@@ -89,36 +90,47 @@ __global__ __launch_bounds__(256) void k_attn_prefill(const TQ *__restrict__ q, 
         const int last = (qb0 + 127 < sq ? qb0 + 127 : sq - 1) + off + 1;
         kend = last < skv ? last : skv;
     }
+    // The next KV tile is requested (into registers, as f16) before the current one is multiplied.
+    constexpr int NCH = BN * CH / 256; // 16-byte pieces of K (and of V) per thread and tile
+    uint4 kreg[NCH], vreg[NCH];
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int c = tid + 256 * i;
+            fh_half t[8];
+            const int kkey = c / CH, kdc = c % CH; // K: consecutive threads along d (coalesced rows)
+            if (t0 + kkey < skv) ap_load8(kb + (int64_t)(t0 + kkey) * kv_st + 8 * kdc, t);
+            else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) t[e] = (fh_half)0.f;
+            }
+            __builtin_memcpy(&kreg[i], t, 16);
+            const int vkey = c % BN, vdc = c / BN; // V: a lane keeps one key, so its 2-byte LDS stores are contiguous
+            if (t0 + vkey < skv) ap_load8(vb + (int64_t)(t0 + vkey) * kv_st + 8 * vdc, t);
+            else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) t[e] = (fh_half)0.f;
+            }
+            __builtin_memcpy(&vreg[i], t, 16);
+        }
+    };
+    auto stash = [&]() { // K tile -> sK[key][d], V tile -> sV[d][key]
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int c = tid + 256 * i;
+            *(uint4 *)(sK + (c / CH) * KS + 8 * (c % CH)) = kreg[i];
+            fh_half t[8];
+            __builtin_memcpy(t, &vreg[i], 16);
+#pragma unroll
+            for (int e = 0; e < 8; e++) sV[(8 * (c / BN) + e) * VS + (c % BN)] = t[e];
+        }
+    };
+    if (kend > 0) fetch(0);
     for (int t0 = 0; t0 < kend; t0 += BN) {
         __syncthreads(); // the previous tile is consumed
-        // ---- K tile -> sK[key][d]
-#pragma unroll
-        for (int i = 0; i < BN * CH / 256; i++) {
-            const int c = tid + 256 * i, key = c / CH, dc = c % CH;
-            fh_half t[8];
-            if (t0 + key < skv) ap_load8(kb + (int64_t)(t0 + key) * kv_st + 8 * dc, t);
-            else {
-#pragma unroll
-                for (int e = 0; e < 8; e++) t[e] = (fh_half)0.f;
-            }
-            uint4 u;
-            __builtin_memcpy(&u, t, 16);
-            *(uint4 *)(sK + key * KS + 8 * dc) = u;
-        }
-        // ---- V tile -> sV[d][key] (a lane keeps one key, so the 2-byte stores of a wavefront are contiguous)
-#pragma unroll
-        for (int i = 0; i < BN * CH / 256; i++) {
-            const int c = tid + 256 * i, key = c % BN, dc = c / BN;
-            fh_half t[8];
-            if (t0 + key < skv) ap_load8(vb + (int64_t)(t0 + key) * kv_st + 8 * dc, t);
-            else {
-#pragma unroll
-                for (int e = 0; e < 8; e++) t[e] = (fh_half)0.f;
-            }
-#pragma unroll
-            for (int e = 0; e < 8; e++) sV[(8 * dc + e) * VS + key] = t[e];
-        }
+        stash();
         __syncthreads();
+        if (t0 + BN < kend) fetch(t0 + BN);
         // ---- S^T = K . Q^T for the two 32-key halves of the tile
         floatx16 st[2];
 #pragma unroll

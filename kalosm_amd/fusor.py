@@ -242,7 +242,7 @@ class Tensor:
         return out
 
     def flash_attention(self, k: "Tensor", v: "Tensor", scale: float, mask=None,
-                        q_strides: Optional[Sequence[int]] = None) -> "Tensor":
+                        q_strides: Optional[Sequence[int]] = None, out: Optional["Tensor"] = None) -> "Tensor":
         """Tensor<4>::flash_attention(&k, &v, scale, Option<(&mask, MaskKind)>)
         (fusor-ml/fusor/src/composite/flash_attention.rs:58-109).  `mask` is None, MaskKind.Causal, or a
         ([sq, skv] f32 Tensor, MaskKind.QKMask) pair.  q_strides = (batch, head, position) element strides of a
@@ -265,7 +265,8 @@ class Tensor:
         qs = q_strides or (hq * sq * d, sq * d, d)
         qdt = F16 if self.dtype == "f16" else F32
         kdt = F16 if k.dtype == "f16" else F32
-        out = Tensor(self.device, (b, hq, sq, d), self.dtype)
+        if out is None:
+            out = Tensor(self.device, (b, hq, sq, d), self.dtype)
         check(self.device._lib.fh_flash_attention_ex(self.device._h, qdt, kdt, C.c_void_p(self.ptr), qs[0], qs[1], qs[2],
                                                      C.c_void_p(k.ptr), C.c_void_p(v.ptr), hkv * skv * d, skv * d, d, b,
                                                      hq, hkv, sq, skv, d, scale, kind, mptr, C.c_void_p(out.ptr)))
