@@ -67,20 +67,26 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     constexpr int XB = (PER + TS - 1) / TS; // blocks of x each wavefront stages: kb / (TS * SW) with SW * PER == kb
     extern __shared__ uint4 lds[];
     // gridDim.y > 1: k is split over workgroups (blocks [boff, boff + kb) here) that add into y with atomics
-    const int kb = (int)q.kb / (int)gridDim.y, boff = (int)blockIdx.y * kb;
+    const int kb = SW * PER, boff = (int)blockIdx.y * kb; // the host launches with SW * PER * gridDim.y == q.kb
     uint4 *img = lds;
     float *sf = (float *)(lds + kb * Q4K_IMG); // per block: [0..7] group sums, [8..15] factors
     float *l_red = sf + kb * 16;               // [TS][SW][16]
     float *l_ss = l_red + 16 * 16;             // per wavefront: sum of squares of the blocks it staged
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, g = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, j = lane & 15, g = lane >> 4;
+    // the wavefront index as a scalar: everything derived from it (tile, record address) stays on the scalar unit
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nwaves = TS * SW;
-    const int stream = wave / SW, slice = wave - stream * SW;
+    const int stream = wave % TS, slice = wave / TS;
     const int64_t nout = EPI == FH_EPI_SWIGLU ? q.n / 2 : q.n;
     const int64_t tiles_out = (nout + 15) / 16;
     const int64_t to = (int64_t)blockIdx.x * TW + (stream % TW);
     const bool tvalid = to < tiles_out;
     const int64_t tile = to + (int64_t)(stream / TW) * (nout / 16); // up tiles follow the gate tiles
     const int b0 = slice * PER;
+    // A tile past the end re-reads the last tile (its rows are never stored).
+    const int64_t tl = tvalid ? tile : tile - (to - (tiles_out - 1));
+    const uint8_t *rec = q.data + (tl * q.recs + boff + b0) * 2304;
+    const uint8_t *ph = rec + 16 * j, *pq = rec + 256 + lane * 16;
 
     // ---- 0. the activations this wavefront stages (blocks wave, wave + nwaves, ...) are requested first:
     // they are needed first and are short
@@ -90,7 +96,8 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     float2 pm[IN == 2 ? XB : 1][8];
 #pragma unroll
     for (int i = 0; i < XB; i++) {
-        const int b = wave + i * nwaves;
+        // one tile stream: a wavefront stages exactly the blocks it multiplies (no other wavefront needs them)
+        const int b = TS == 1 ? b0 + i : wave + i * nwaves;
         const int64_t at = (int64_t)(boff + (b < kb ? b : 0)) * 256 + lane * 4;
         if (IN != 2) xv[i] = *(const float4 *)(x + at);
         if (IN == 1 && xres) rv[i] = *(const float4 *)(xres + at);
@@ -105,13 +112,20 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
                 }
         }
     }
-    // ---- 1. every weight byte of this wavefront goes in flight.  A tile past the end re-reads the last
-    // tile (its rows are never stored); the host guarantees SW * PER == kb, so no block is out of range.
+    // The activation requests stay ahead of the weight requests: loads return in order, so the staging below can
+    // wait for them alone (vmcnt > 0) while the weights are still in flight.
+    __builtin_amdgcn_sched_barrier(0);
+#ifdef Q4K_XFIRST
+    // A compute unit serves its requests in order: without this rendezvous the activation request of a late
+    // wavefront queues behind the weight requests of the early ones and the staging barrier below waits for nearly
+    // all of the workgroup's weights.  (A bare s_barrier: no wait for the loads just issued.)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+    // ---- 1. every weight byte of this wavefront goes in flight (the host guarantees SW * PER == kb, so no
+    // block is out of range).
     Q4KRegs w[PER];
     {
-        const int64_t tl = tvalid ? tile : tile - (to - (tiles_out - 1));
-        const uint8_t *rec = q.data + (tl * q.recs + boff + b0) * 2304;
-        const uint8_t *ph = rec + 16 * j, *pq = rec + 256 + lane * 16;
 #pragma unroll
         for (int r = 0; r < PER; r++) {
             w[r].h = *(const uint4 *)(ph + r * 2304);
@@ -123,8 +137,10 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < XB; i++) {
-        const int b = wave + i * nwaves;
-        if (b >= kb) break;
+        // no branch here (the compiler would sink the activation loads into it, behind the weight loads): a
+        // wavefront without a block of its own stages block 0 once more, writing the values wavefront 0 writes
+        const bool own = TS == 1 || wave + i * nwaves < kb;
+        const int b = TS == 1 ? b0 + i : (own ? wave + i * nwaves : 0);
         float4 v = xv[i];
         if (IN == 2) { // merge the splits: softmax weights exp(m_s - max), then num / den
             float mx = -INFINITY;
@@ -145,7 +161,9 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         }
         if (IN == 1 && xres) v = make_float4(v.x + rv[i].x, v.y + rv[i].y, v.z + rv[i].z, v.w + rv[i].w);
         if (IN == 1) {
-            ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
+            float s2 = v.x * v.x;
+            s2 = fmaf(v.y, v.y, s2); s2 = fmaf(v.z, v.z, s2); s2 = fmaf(v.w, v.w, s2);
+            ss += own ? s2 : 0.f;
             v = make_float4(v.x * wv[i].x, v.y * wv[i].y, v.z * wv[i].z, v.w * wv[i].w);
         }
         float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
@@ -187,7 +205,7 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
         if (lane == 0) l_ss[wave] = ss;
     }
-    __syncthreads();
+    if (TS > 1) __syncthreads(); // with one tile stream the image a wavefront reads is the one it wrote
     // ---- 3. eight chained MFMA steps per block
     const int mysb = j >> 1, part = j & 1;
     const uint4 *pa[8]; // per-lane operand address of each step: its own sub-block's (hi|lo) or the zero slot

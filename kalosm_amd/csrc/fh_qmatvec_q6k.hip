@@ -53,6 +53,10 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
     const int64_t tile = to + (int64_t)(stream / TW) * (nout / 16);
     const int b0 = slice * PER;
 
+    // a tile past the end re-reads the last one (never stored)
+    const int64_t tl = tvalid ? tile : tile - (to - (tiles_out - 1));
+    const uint8_t *rec = q.data + (tl * q.recs + boff + b0) * 3360;
+
     // ---- 0. activations first (short, needed first)
     // With xup the input is silu(x) * xup (the SwiGLU of a gate | up projection, raw/attention_layer.rs:195),
     // evaluated while staging.
@@ -64,11 +68,12 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
         xv[i] = *(const float4 *)(x + at);
         if (xup) uv[i] = *(const float4 *)(xup + at);
     }
-    // ---- 1. all weight bytes of this wavefront (a tile past the end re-reads the last one; never stored)
+    // The activation requests stay ahead of the weight requests: loads return in order, so the staging can wait
+    // for them alone while the weights are still in flight.
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- 1. all weight bytes of this wavefront
     Q6KRegs w[PER];
     {
-        const int64_t tl = tvalid ? tile : tile - (to - (tiles_out - 1));
-        const uint8_t *rec = q.data + (tl * q.recs + boff + b0) * 3360;
 #pragma unroll
         for (int r = 0; r < PER; r++) {
             const uint8_t *p = rec + r * 3360;
@@ -82,8 +87,9 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
     // ---- 2. stage x: lane owns k = 256*b + 4*lane .. +3, i.e. a quarter of group G = lane / 4
 #pragma unroll
     for (int i = 0; i < XB; i++) {
-        const int b = wave + i * nwaves;
-        if (b >= kb) break;
+        // no branch (the compiler would sink the activation loads into it, behind the weight loads): a wavefront
+        // without a block of its own stages block 0 once more, writing the values wavefront 0 writes
+        const int b = wave + i * nwaves < kb ? wave + i * nwaves : 0;
         float4 v = xv[i];
         if (xup)
             v = make_float4((v.x / (__expf(-v.x) + 1.0f)) * uv[i].x, (v.y / (__expf(-v.y) + 1.0f)) * uv[i].y,
