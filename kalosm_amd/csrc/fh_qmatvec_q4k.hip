@@ -35,6 +35,33 @@ __device__ __forceinline__ float dpp_f32(float v) {
     return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
 }
 
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, CTRL, 0xF, 0xF, true);
+}
+// sum over the four rows of 16 lanes of a wavefront (lane i of every row gets it): two register swaps, no LDS
+__device__ __forceinline__ float rows_sum(float a) {
+    const uint32_t u = __float_as_uint(a);
+    auto s16 = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    a = __uint_as_float(s16[0]) + __uint_as_float(s16[1]);
+    const uint32_t w = __float_as_uint(a);
+    auto s32 = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    return __uint_as_float(s32[0]) + __uint_as_float(s32[1]);
+}
+// LDS addresses as 32-bit integers, so that a per-lane choice between two of them is one v_cndmask on a constant
+// lane mask held in scalar registers.
+__device__ __forceinline__ uint32_t lds_addr(const void *p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
+}
+__device__ __forceinline__ uint4 lds_read16(uint32_t a) {
+    return *(__attribute__((address_space(3))) const uint4 *)(uintptr_t)a;
+}
+__device__ __forceinline__ uint32_t sel_lanes(uint64_t mask, uint32_t yes, uint32_t no) {
+    uint32_t r;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(no), "v"(yes), "s"(mask));
+    return r;
+}
+
 // Arguments of the rope + KV-append epilogue (the fused q|k|v projection of a decode step): rows [0, qd) are query
 // rows (rotated, written to qo), [qd, qd + kd) key rows (rotated, written to the cache row of the device-side
 // position), the rest value rows (copied to the cache).  RopeCache::forward_interleaved + KvCache::append
@@ -167,21 +194,23 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
             v = make_float4(v.x * wv[i].x, v.y * wv[i].y, v.z * wv[i].z, v.w * wv[i].w);
         }
         float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        amax = fmaxf(amax, dpp_f32<DPP_XOR1>(amax));
-        amax = fmaxf(amax, dpp_f32<DPP_XOR2>(amax));
-        amax = fmaxf(amax, dpp_f32<DPP_HALF_MIRROR>(amax)); // quads are uniform now: lane 7-i is in the other quad
+        // non-negative floats order like their bit patterns: the cross-lane maximum is an integer one
+        uint32_t am = __float_as_uint(amax);
+        am = max(am, dpp_u32<DPP_XOR1>(am));
+        am = max(am, dpp_u32<DPP_XOR2>(am));
+        am = max(am, dpp_u32<DPP_HALF_MIRROR>(am)); // quads are uniform now: lane 7-i is in the other quad
         const int s = lane >> 3, gg = (lane >> 1) & 3, half = lane & 1;
         // e = 14 - floor(log2(amax)) from the exponent field (zero / subnormal / inf / nan just clamp)
-        int e = 141 - (int)((__float_as_uint(amax) >> 23) & 0xFFu);
+        int e = 141 - (int)((am >> 23) & 0xFFu);
         e = e > 100 ? 100 : (e < -100 ? -100 : e);
         const int eo = e - 4 * (s & 1); // odd sub-blocks meet codes scaled by 16
         const float sc = __uint_as_float((uint32_t)(eo + 127) << 23);
-        const float xs[4] = {v.x * sc, v.y * sc, v.z * sc, v.w * sc};
+        const float xq[4] = {v.x, v.y, v.z, v.w};
         _Float16 hi[4], lo[4];
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            hi[c] = (_Float16)xs[c];
-            lo[c] = (_Float16)(xs[c] - (float)hi[c]);
+        for (int c = 0; c < 4; c++) { // x * sc is exact (a power of two), so the fused form rounds like the split one
+            hi[c] = (_Float16)(xq[c] * sc);
+            lo[c] = (_Float16)__builtin_fmaf(xq[c], sc, -(float)hi[c]);
         }
         const _Float16 oh[4] = {hi[0], hi[2], hi[1], hi[3]}, ol[4] = {lo[0], lo[2], lo[1], lo[3]};
         uint2 ph, pl;
@@ -208,9 +237,20 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     if (TS > 1) __syncthreads(); // with one tile stream the image a wavefront reads is the one it wrote
     // ---- 3. eight chained MFMA steps per block
     const int mysb = j >> 1, part = j & 1;
-    const uint4 *pa[8]; // per-lane operand address of each step: its own sub-block's (hi|lo) or the zero slot
+    // per-lane operand address of each step: its own sub-block's (hi|lo) in step mysb, the zero slot otherwise.
+    // Lanes with (lane >> 1) % 8 == st are bits 2 st, 2 st + 1 of every 16.
+    uint32_t pa[8];
+    {
+        const uint32_t own = lds_addr(img + b0 * Q4K_IMG + (mysb * 4 + g) * 2 + part);
+        const uint32_t zero = lds_addr(img + b0 * Q4K_IMG + 64);
 #pragma unroll
-    for (int st = 0; st < 8; st++) pa[st] = img + b0 * Q4K_IMG + (st == mysb ? (st * 4 + g) * 2 + part : 64);
+        for (int st = 0; st < 8; st++) pa[st] = sel_lanes(0x0003000300030003ull << (2 * st), own, zero);
+    }
+    // the operands do not depend on the weights: RING of them are always on their way from the LDS
+    constexpr int RING = 4;
+    uint4 ring[RING];
+#pragma unroll
+    for (int t = 0; t < RING; t++) ring[t] = lds_read16(pa[t % 8] + (t / 8) * Q4K_IMG * 16);
     const float *psf = sf + b0 * 16 + 2 * g;
     const uint32_t LO = 0x000F000Fu, HI = 0x00F000F0u;
     // lane group g applies sub-blocks 2g, 2g+1: bytes (g&1)*2, +1 of the low (g < 2) or high (g >= 2) scale word
@@ -226,11 +266,13 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
             const uint32_t w0 = (st & 2) ? wq.z : wq.x, w1 = (st & 2) ? wq.w : wq.y;
             const uint32_t msk = (st & 1) ? HI : LO;
             const uint4 bo = make_uint4(w0 & msk, (w0 >> 8) & msk, w1 & msk, (w1 >> 8) & msk);
-            const uint4 ao = pa[st][r * Q4K_IMG];
+            const int t = r * 8 + st;
+            const uint4 ao = ring[t % RING];
             half8 av, bv;
             __builtin_memcpy(&av, &ao, 16);
             __builtin_memcpy(&bv, &bo, 16);
             dd = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, dd, 0, 0, 0);
+            if (t + RING < PER * 8) ring[t % RING] = lds_read16(pa[(t + RING) % 8] + ((t + RING) / 8) * Q4K_IMG * 16);
         }
         const uint4 h = w[r].h;
         const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
@@ -249,8 +291,7 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         mins = fmaf(mnb * dmin, sx.y, mins);
     }
     float v = acc - mins;
-    v += __shfl_xor(v, 16, 64);
-    v += __shfl_xor(v, 32, 64);
+    v = rows_sum(v);
     if (lane < 16) l_red[(stream * SW + slice) * 16 + lane] = v;
     __syncthreads();
     if (tid < TW * 16) {

@@ -39,13 +39,15 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
     constexpr int XB = (PER + TS - 1) / TS;
     extern __shared__ uint4 lds[];
     // gridDim.y > 1: k is split over workgroups (blocks [boff, boff + kb) here) that add into y with atomics
-    const int kb = (int)q.kb / (int)gridDim.y, boff = (int)blockIdx.y * kb;
+    const int kb = SW * PER, boff = (int)blockIdx.y * kb; // the host launches with SW * PER * gridDim.y == q.kb
     uint4 *img = lds;
     float *sf = (float *)(lds + kb * Q6K_IMG);
     float *l_red = sf + kb * Q6K_SF; // [TS][SW][16]
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, g = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, j = lane & 15, g = lane >> 4;
+    // the wavefront index as a scalar: everything derived from it (tile, record address) stays on the scalar unit
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nwaves = TS * SW;
-    const int stream = wave / SW, slice = wave - stream * SW;
+    const int stream = wave % TS, slice = wave / TS;
     const int64_t nout = EPI == FH_EPI_SWIGLU ? q.n / 2 : q.n;
     const int64_t tiles_out = (nout + 15) / 16;
     const int64_t to = (int64_t)blockIdx.x * TW + (stream % TW);
@@ -63,7 +65,8 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
     float4 xv[XB], uv[XB];
 #pragma unroll
     for (int i = 0; i < XB; i++) {
-        const int b = wave + i * nwaves;
+        // one tile stream: a wavefront stages exactly the blocks it multiplies (no other wavefront needs them)
+        const int b = TS == 1 ? b0 + i : wave + i * nwaves;
         const int64_t at = (int64_t)(boff + (b < kb ? b : 0)) * 256 + lane * 4;
         xv[i] = *(const float4 *)(x + at);
         if (xup) uv[i] = *(const float4 *)(xup + at);
@@ -89,7 +92,7 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
     for (int i = 0; i < XB; i++) {
         // no branch (the compiler would sink the activation loads into it, behind the weight loads): a wavefront
         // without a block of its own stages block 0 once more, writing the values wavefront 0 writes
-        const int b = wave + i * nwaves < kb ? wave + i * nwaves : 0;
+        const int b = TS == 1 ? b0 + i : (wave + i * nwaves < kb ? wave + i * nwaves : 0);
         float4 v = xv[i];
         if (xup)
             v = make_float4((v.x / (__expf(-v.x) + 1.0f)) * uv[i].x, (v.y / (__expf(-v.y) + 1.0f)) * uv[i].y,
@@ -123,7 +126,7 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
             sf[b * Q6K_SF + 16 + (lane >> 2)] = __uint_as_float((uint32_t)(24 - e + 127) << 23);
         }
     }
-    __syncthreads();
+    if (TS > 1) __syncthreads(); // with one tile stream the image a wavefront reads is the one it wrote
     // ---- 3. two chains of four MFMA steps per block
     const int gl = j >> 1, part = j & 1; // this lane's A row is (group gl of a half block, hi | lo)
     const uint4 *pa[8];
