@@ -53,8 +53,10 @@ __device__ __forceinline__ float rows_sum(float a) {
 __device__ __forceinline__ uint32_t lds_addr(const void *p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
 }
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 lds_read16(uint32_t a) {
-    return *(__attribute__((address_space(3))) const uint4 *)(uintptr_t)a;
+    const u32x4 v = *(__attribute__((address_space(3))) const u32x4 *)(uintptr_t)a;
+    return make_uint4(v[0], v[1], v[2], v[3]);
 }
 __device__ __forceinline__ uint32_t sel_lanes(uint64_t mask, uint32_t yes, uint32_t no) {
     uint32_t r;
