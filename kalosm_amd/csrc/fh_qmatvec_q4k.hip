@@ -11,12 +11,12 @@
 // D[2s + part][row] = (q . x_part)_s for all eight sub-blocks at once: lane (row j, group g) holds the four
 // values of sub-blocks 2g and 2g+1 of its own row and applies that row's d * sc_s * 2^(24-e_s) itself.
 //
-// Workgroup = TS tile streams (TW row tiles; twice that with the SwiGLU epilogue: gate tiles and the matching
-// up tiles) x SW k-slices of PER blocks; wavefront = (stream, slice).  All PER x 2304 B of a wavefront are
-// requested before anything else; meanwhile the workgroup stages x for the whole k once (block b by wavefront
-// b mod waves): each 32-group is normalised by a power of two to [2^14, 2^15) (odd groups 16x lower, which
-// folds the x16 of the high nibbles), split into f16 hi + lo and stored in operand order, with the group sums
-// of the original x and the factors beside them.
+// Workgroup = SW wavefronts, one per k-slice of PER blocks; a wavefront multiplies its slice of TPW row tiles
+// (with the SwiGLU epilogue: gate tiles and the matching up tiles).  All TPW x PER x 2304 B of a wavefront are
+// requested before anything else; meanwhile it stages the activations of its own blocks (nobody else needs
+// them, so there is no barrier before the products): each 32-group is normalised by a power of two to
+// [2^14, 2^15) (odd groups 16x lower, which folds the x16 of the high nibbles), split into f16 hi + lo and stored
+// in operand order, with the group sums of the original x and the factors beside them.
 #include "fh_blocks.h"
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -85,49 +85,47 @@ struct Q4kExtra {
 
 #define Q4K_IMG 65 // uint4 per block image: 8 steps x 4 groups x (hi, lo) + one all-zero slot
 
-template <int TS, int PER, int EPI, int IN>
+template <int TPW, int PER, int EPI, int IN>
 __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict__ x, float *__restrict__ y,
                                                       const float *__restrict__ ea, const float *__restrict__ eb,
                                                       int SW, const float *__restrict__ xres,
                                                       const float *__restrict__ nw, float eps, int nsplit,
                                                       FhRopeArgs rk) {
     constexpr int NT = EPI == FH_EPI_SWIGLU ? 2 : 1;
-    constexpr int TW = TS / NT;
-    constexpr int XB = (PER + TS - 1) / TS; // blocks of x each wavefront stages: kb / (TS * SW) with SW * PER == kb
+    constexpr int TOUT = TPW / NT; // output tiles of the workgroup
     extern __shared__ uint4 lds[];
     // gridDim.y > 1: k is split over workgroups (blocks [boff, boff + kb) here) that add into y with atomics
     const int kb = SW * PER, boff = (int)blockIdx.y * kb; // the host launches with SW * PER * gridDim.y == q.kb
     uint4 *img = lds;
     float *sf = (float *)(lds + kb * Q4K_IMG); // per block: [0..7] group sums, [8..15] factors
-    float *l_red = sf + kb * 16;               // [TS][SW][16]
-    float *l_ss = l_red + 16 * 16;             // per wavefront: sum of squares of the blocks it staged
+    float *l_red = sf + kb * 16;               // [TPW][SW][16]
+    float *l_ss = l_red + TPW * 16 * 16;       // per wavefront: sum of squares of the blocks it staged
     const int tid = threadIdx.x, lane = tid & 63, j = lane & 15, g = lane >> 4;
-    // the wavefront index as a scalar: everything derived from it (tile, record address) stays on the scalar unit
+    // the wavefront index as a scalar: everything derived from it (record addresses) stays on the scalar unit
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nwaves = TS * SW;
-    const int stream = wave % TS, slice = wave / TS;
     const int64_t nout = EPI == FH_EPI_SWIGLU ? q.n / 2 : q.n;
     const int64_t tiles_out = (nout + 15) / 16;
-    const int64_t to = (int64_t)blockIdx.x * TW + (stream % TW);
-    const bool tvalid = to < tiles_out;
-    const int64_t tile = to + (int64_t)(stream / TW) * (nout / 16); // up tiles follow the gate tiles
-    const int b0 = slice * PER;
-    // A tile past the end re-reads the last tile (its rows are never stored).
-    const int64_t tl = tvalid ? tile : tile - (to - (tiles_out - 1));
-    const uint8_t *rec = q.data + (tl * q.recs + boff + b0) * 2304;
-    const uint8_t *ph = rec + 16 * j, *pq = rec + 256 + lane * 16;
+    const int b0 = wave * PER;
+    const uint8_t *ph[TPW], *pq[TPW];
+#pragma unroll
+    for (int tp = 0; tp < TPW; tp++) {
+        const int64_t to = (int64_t)blockIdx.x * TOUT + (tp % TOUT);
+        const int64_t tile = to + (int64_t)(tp / TOUT) * (nout / 16); // up tiles follow the gate tiles
+        // a tile past the end re-reads the last tile (its rows are never stored)
+        const int64_t tl = to < tiles_out ? tile : tile - (to - (tiles_out - 1));
+        const uint8_t *rec = q.data + (tl * q.recs + boff + b0) * 2304;
+        ph[tp] = rec + 16 * j;
+        pq[tp] = rec + 256 + lane * 16;
+    }
 
-    // ---- 0. the activations this wavefront stages (blocks wave, wave + nwaves, ...) are requested first:
-    // they are needed first and are short
+    // ---- 0. the activations of this wavefront's blocks are requested first: they are needed first and are short
     // With nw the input is rms_norm(x [+ xres]) * nw (composite/normalization.rs:287-401): the weight nw is
     // folded into the staged values and the common factor 1 / rms is applied to the finished dot product.
-    float4 xv[XB], rv[XB], wv[XB], pacc[IN == 2 ? XB : 1][8];
-    float2 pm[IN == 2 ? XB : 1][8];
+    float4 xv[PER], rv[PER], wv[PER], pacc[IN == 2 ? PER : 1][8];
+    float2 pm[IN == 2 ? PER : 1][8];
 #pragma unroll
-    for (int i = 0; i < XB; i++) {
-        // one tile stream: a wavefront stages exactly the blocks it multiplies (no other wavefront needs them)
-        const int b = TS == 1 ? b0 + i : wave + i * nwaves;
-        const int64_t at = (int64_t)(boff + (b < kb ? b : 0)) * 256 + lane * 4;
+    for (int i = 0; i < PER; i++) {
+        const int64_t at = (int64_t)(boff + b0 + i) * 256 + lane * 4;
         if (IN != 2) xv[i] = *(const float4 *)(x + at);
         if (IN == 1 && xres) rv[i] = *(const float4 *)(xres + at);
         if (IN == 1) wv[i] = *(const float4 *)(nw + at);
@@ -144,32 +142,24 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     // The activation requests stay ahead of the weight requests: loads return in order, so the staging below can
     // wait for them alone (vmcnt > 0) while the weights are still in flight.
     __builtin_amdgcn_sched_barrier(0);
-#ifdef Q4K_XFIRST
-    // A compute unit serves its requests in order: without this rendezvous the activation request of a late
-    // wavefront queues behind the weight requests of the early ones and the staging barrier below waits for nearly
-    // all of the workgroup's weights.  (A bare s_barrier: no wait for the loads just issued.)
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-#endif
     // ---- 1. every weight byte of this wavefront goes in flight (the host guarantees SW * PER == kb, so no
     // block is out of range).
-    Q4KRegs w[PER];
-    {
+    Q4KRegs w[TPW][PER];
 #pragma unroll
-        for (int r = 0; r < PER; r++) {
-            w[r].h = *(const uint4 *)(ph + r * 2304);
-            w[r].qa = *(const uint4 *)(pq + r * 2304);
-            w[r].qb = *(const uint4 *)(pq + r * 2304 + 1024);
+    for (int r = 0; r < PER; r++)
+#pragma unroll
+        for (int tp = 0; tp < TPW; tp++) {
+            w[tp][r].h = *(const uint4 *)(ph[tp] + r * 2304);
+            w[tp][r].qa = *(const uint4 *)(pq[tp] + r * 2304);
+            w[tp][r].qb = *(const uint4 *)(pq[tp] + r * 2304 + 1024);
         }
-    }
-    // ---- 2. stage x (lane owns k = 256*b + 4*lane .. +3)
+    // ---- 2. stage x (lane owns k = 256*b + 4*lane .. +3).  A wavefront stages exactly the blocks it multiplies:
+    // nobody else reads its part of the image, so there is no barrier between this and the products.  (No branch
+    // around it either: the compiler would sink the activation loads into it, behind the weight loads.)
     float ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < XB; i++) {
-        // no branch here (the compiler would sink the activation loads into it, behind the weight loads): a
-        // wavefront without a block of its own stages block 0 once more, writing the values wavefront 0 writes
-        const bool own = TS == 1 || wave + i * nwaves < kb;
-        const int b = TS == 1 ? b0 + i : (own ? wave + i * nwaves : 0);
+    for (int i = 0; i < PER; i++) {
+        const int b = b0 + i;
         float4 v = xv[i];
         if (IN == 2) { // merge the splits: softmax weights exp(m_s - max), then num / den
             float mx = -INFINITY;
@@ -192,7 +182,7 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         if (IN == 1) {
             float s2 = v.x * v.x;
             s2 = fmaf(v.y, v.y, s2); s2 = fmaf(v.z, v.z, s2); s2 = fmaf(v.w, v.w, s2);
-            ss += own ? s2 : 0.f;
+            ss += s2;
             v = make_float4(v.x * wv[i].x, v.y * wv[i].y, v.z * wv[i].z, v.w * wv[i].w);
         }
         float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
@@ -236,8 +226,7 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
         if (lane == 0) l_ss[wave] = ss;
     }
-    if (TS > 1) __syncthreads(); // with one tile stream the image a wavefront reads is the one it wrote
-    // ---- 3. eight chained MFMA steps per block
+    // ---- 3. eight chained MFMA steps per block and tile; the TPW tiles share every operand read
     const int mysb = j >> 1, part = j & 1;
     // per-lane operand address of each step: its own sub-block's (hi|lo) in step mysb, the zero slot otherwise.
     // Lanes with (lane >> 1) % 8 == st are bits 2 st, 2 st + 1 of every 16.
@@ -258,59 +247,72 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     // lane group g applies sub-blocks 2g, 2g+1: bytes (g&1)*2, +1 of the low (g < 2) or high (g >= 2) scale word
     const uint32_t selhi = (g & 2) ? 0xFFFFFFFFu : 0u;
     const int sh = (g & 1) * 16;
-    float acc = 0.f, mins = 0.f;
+    float acc[TPW], mins[TPW];
+#pragma unroll
+    for (int tp = 0; tp < TPW; tp++) acc[tp] = mins[tp] = 0.f;
 #pragma unroll
     for (int r = 0; r < PER; r++) {
-        floatx4 dd = {0.f, 0.f, 0.f, 0.f};
+        floatx4 dd[TPW];
+#pragma unroll
+        for (int tp = 0; tp < TPW; tp++) dd[tp] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int st = 0; st < 8; st++) {
-            const uint4 wq = (st & 4) ? w[r].qb : w[r].qa;
-            const uint32_t w0 = (st & 2) ? wq.z : wq.x, w1 = (st & 2) ? wq.w : wq.y;
-            const uint32_t msk = (st & 1) ? HI : LO;
-            const uint4 bo = make_uint4(w0 & msk, (w0 >> 8) & msk, w1 & msk, (w1 >> 8) & msk);
             const int t = r * 8 + st;
             const uint4 ao = ring[t % RING];
-            half8 av, bv;
+            half8 av;
             __builtin_memcpy(&av, &ao, 16);
-            __builtin_memcpy(&bv, &bo, 16);
-            dd = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, dd, 0, 0, 0);
+#pragma unroll
+            for (int tp = 0; tp < TPW; tp++) {
+                const uint4 wq = (st & 4) ? w[tp][r].qb : w[tp][r].qa;
+                const uint32_t w0 = (st & 2) ? wq.z : wq.x, w1 = (st & 2) ? wq.w : wq.y;
+                const uint32_t msk = (st & 1) ? HI : LO;
+                const uint4 bo = make_uint4(w0 & msk, (w0 >> 8) & msk, w1 & msk, (w1 >> 8) & msk);
+                half8 bv;
+                __builtin_memcpy(&bv, &bo, 16);
+                dd[tp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, dd[tp], 0, 0, 0);
+            }
             if (t + RING < PER * 8) ring[t % RING] = lds_read16(pa[(t + RING) % 8] + ((t + RING) / 8) * Q4K_IMG * 16);
         }
-        const uint4 h = w[r].h;
-        const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
-        const uint32_t sc_l = h.y & 0x3F3F3F3Fu, sc_h = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
-        const uint32_t mn_l = h.z & 0x3F3F3F3Fu, mn_h = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
-        const uint32_t scw = ((sc_l & ~selhi) | (sc_h & selhi)) >> sh;
-        const uint32_t mnw = ((mn_l & ~selhi) | (mn_h & selhi)) >> sh;
-        const float sca = (float)(scw & 0xFFu), scb = (float)((scw >> 8) & 0xFFu);
-        const float mna = (float)(mnw & 0xFFu), mnb = (float)((mnw >> 8) & 0xFFu);
         const float2 sx = *(const float2 *)(psf + r * 16);
         const float2 fc = *(const float2 *)(psf + r * 16 + 8);
-        const float sa = (sca * d) * fc.x, sb = (scb * d) * fc.y;
-        acc = fmaf(dd[0] + dd[1], sa, acc);
-        acc = fmaf(dd[2] + dd[3], sb, acc);
-        mins = fmaf(mna * dmin, sx.x, mins);
-        mins = fmaf(mnb * dmin, sx.y, mins);
+#pragma unroll
+        for (int tp = 0; tp < TPW; tp++) {
+            const uint4 h = w[tp][r].h;
+            const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
+            const uint32_t sc_l = h.y & 0x3F3F3F3Fu, sc_h = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
+            const uint32_t mn_l = h.z & 0x3F3F3F3Fu, mn_h = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
+            const uint32_t scw = ((sc_l & ~selhi) | (sc_h & selhi)) >> sh;
+            const uint32_t mnw = ((mn_l & ~selhi) | (mn_h & selhi)) >> sh;
+            const float sca = (float)(scw & 0xFFu), scb = (float)((scw >> 8) & 0xFFu);
+            const float mna = (float)(mnw & 0xFFu), mnb = (float)((mnw >> 8) & 0xFFu);
+            const float sa = (sca * d) * fc.x, sb = (scb * d) * fc.y;
+            acc[tp] = fmaf(dd[tp][0] + dd[tp][1], sa, acc[tp]);
+            acc[tp] = fmaf(dd[tp][2] + dd[tp][3], sb, acc[tp]);
+            mins[tp] = fmaf(mna * dmin, sx.x, mins[tp]);
+            mins[tp] = fmaf(mnb * dmin, sx.y, mins[tp]);
+        }
     }
-    float v = acc - mins;
-    v = rows_sum(v);
-    if (lane < 16) l_red[(stream * SW + slice) * 16 + lane] = v;
+#pragma unroll
+    for (int tp = 0; tp < TPW; tp++) {
+        const float v = rows_sum(acc[tp] - mins[tp]);
+        if (lane < 16) l_red[(tp * SW + wave) * 16 + lane] = v;
+    }
     __syncthreads();
-    if (tid < TW * 16) {
+    if (tid < TOUT * 16) {
         const int t = tid >> 4, jr = tid & 15;
         float v0 = 0.f, v1 = 0.f;
         for (int s = 0; s < SW; s++) {
             v0 += l_red[(t * SW + s) * 16 + jr];
-            if (NT == 2) v1 += l_red[((t + TW) * SW + s) * 16 + jr];
+            if (NT == 2) v1 += l_red[((t + TOUT) * SW + s) * 16 + jr];
         }
         if (IN == 1) {
             float tot = 0.f;
-            for (int w2 = 0; w2 < nwaves; w2++) tot += l_ss[w2];
+            for (int w2 = 0; w2 < SW; w2++) tot += l_ss[w2];
             const float rms = sqrtf(tot / (float)q.k + eps);
             v0 = v0 / rms;
             v1 = v1 / rms;
         }
-        const int64_t row = ((int64_t)blockIdx.x * TW + t) * 16 + jr;
+        const int64_t row = ((int64_t)blockIdx.x * TOUT + t) * 16 + jr;
         if (EPI == FH_EPI_ROPEKV) {
             const float other = __shfl_xor(v0, 1, 64); // the pair (2i, 2i+1) sits in neighbouring lanes
             const int pos = *rk.pos;
@@ -346,50 +348,60 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     }
 }
 
-// The kernel proper.  With at most two blocks per wavefront the register budget of two resident workgroups
+// The kernel proper.  With at most two block tiles per wavefront the register budget of eight wavefronts per SIMD
 // (64 VGPRs) is enforced: the kernel lives on the number of bytes in flight per compute unit.
 #define Q4K_M1_PARAMS                                                                                              \
     QView q, const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ ea,                    \
         const float *__restrict__ eb, int SW, const float *__restrict__ xres, const float *__restrict__ nw, float eps, int nsplit, FhRopeArgs rk
-template <int TS, int PER, int EPI, int IN>
+template <int TPW, int PER, int EPI, int IN>
 __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(Q4K_M1_PARAMS) {
-    qmv_q4k_m1_body<TS, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
+    qmv_q4k_m1_body<TPW, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
-template <int TS, int PER, int EPI, int IN>
+template <int TPW, int PER, int EPI, int IN>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_qmv_q4k_m1_w8(Q4K_M1_PARAMS) {
-    qmv_q4k_m1_body<TS, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
+    qmv_q4k_m1_body<TPW, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
 
-template <int TS, int PER, int EPI>
+template <int TPW, int PER, int EPI>
 static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b, int SW,
                                unsigned grid, size_t lds, const Q4kExtra &ex) {
     typedef void (*kern_t)(QView, const float *, float *, const float *, const float *, int, const float *, const float *,
                            float, int, FhRopeArgs);
     kern_t kern;
     const int in = ex.nsplit > 0 ? 2 : (ex.nw ? 1 : 0); // input: plain, rms_norm, attention partials
-    if constexpr (PER <= 2) {
-        kern = in == 2 ? k_qmv_q4k_m1<TS, PER, EPI, 2>
-                       : (in == 1 ? k_qmv_q4k_m1_w8<TS, PER, EPI, 1> : k_qmv_q4k_m1_w8<TS, PER, EPI, 0>);
+    if constexpr (TPW * PER <= 2) {
+        kern = in == 2 ? k_qmv_q4k_m1<TPW, PER, EPI, 2>
+                       : (in == 1 ? k_qmv_q4k_m1_w8<TPW, PER, EPI, 1> : k_qmv_q4k_m1_w8<TPW, PER, EPI, 0>);
     } else {
-        kern = in == 2 ? k_qmv_q4k_m1<TS, PER, EPI, 2> : (in == 1 ? k_qmv_q4k_m1<TS, PER, EPI, 1> : k_qmv_q4k_m1<TS, PER, EPI, 0>);
+        if (in == 2) return FH_ERR_UNSUPPORTED; // the merge of the attention partials needs the registers
+        kern = in == 1 ? k_qmv_q4k_m1<TPW, PER, EPI, 1> : k_qmv_q4k_m1<TPW, PER, EPI, 0>;
     }
     static bool attr_done[3] = {false, false, false};
     if (!attr_done[in]) {
         FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         attr_done[in] = true;
     }
-    kern<<<dim3(grid, (unsigned)ex.ksplit), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, ex.xres, ex.nw, ex.eps,
-                                                                  ex.nsplit, ex.rk);
+    kern<<<dim3(grid, (unsigned)ex.ksplit), dim3(64 * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, ex.xres,
+                                                                                  ex.nw, ex.eps, ex.nsplit, ex.rk);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
 
-template <int TS, int EPI>
-static fh_status q4k_m1_per(int per, const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b,
-                            int SW, unsigned grid, size_t lds, const Q4kExtra &ex) {
-    if (per == 1) return q4k_m1_launch<TS, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
-    if (per == 2) return q4k_m1_launch<TS, 2, EPI>(q, x, y, a, b, SW, grid, lds, ex);
-    return q4k_m1_launch<TS, 4, EPI>(q, x, y, a, b, SW, grid, lds, ex);
+// (tiles per wavefront, blocks per wavefront) with at most four block tiles (48 registers of weights) per wavefront
+template <int EPI>
+static fh_status q4k_m1_shape(int tpw, int per, const fh_qmatrix *q, const float *x, float *y, const float *a,
+                              const float *b, int SW, unsigned grid, size_t lds, const Q4kExtra &ex) {
+    if constexpr (EPI != FH_EPI_SWIGLU) {
+        if (tpw == 1 && per == 1) return q4k_m1_launch<1, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
+        if (tpw == 1 && per == 2) return q4k_m1_launch<1, 2, EPI>(q, x, y, a, b, SW, grid, lds, ex);
+        if (tpw == 1 && per == 4) return q4k_m1_launch<1, 4, EPI>(q, x, y, a, b, SW, grid, lds, ex);
+    }
+    if constexpr (EPI != FH_EPI_ACC) {
+        if (tpw == 2 && per == 1) return q4k_m1_launch<2, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
+        if (tpw == 2 && per == 2) return q4k_m1_launch<2, 2, EPI>(q, x, y, a, b, SW, grid, lds, ex);
+        if (tpw == 4 && per == 1) return q4k_m1_launch<4, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
+    }
+    return FH_ERR_UNSUPPORTED;
 }
 
 // Returns FH_ERR_UNSUPPORTED when the shape does not fit this kernel (the caller falls back).
@@ -455,46 +467,32 @@ static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra 
     const int nt = epi == FH_EPI_SWIGLU ? 2 : 1;
     const int64_t nout = epi == FH_EPI_SWIGLU ? q->n / 2 : q->n;
     const int64_t tiles = (nout + 15) / 16;
-    // blocks per wavefront (all requested up front); 2 measured best for the large shapes, 1 for the small ones
+    // tiles per wavefront (they share the staged activations and every operand read): two once there are more
+    // tiles than compute units; the SwiGLU epilogue needs the gate and the up tile in one wavefront
+    int tpw = (int)dev->opt_matvec_tiles;
+    if (tpw != 1 && tpw != 2 && tpw != 4) tpw = tiles > dev->compute_units ? 2 : 1;
+    if (epi == FH_EPI_SWIGLU && tpw < 2) tpw = 2;
+    if (epi == FH_EPI_ACC || ex.nsplit > 0) tpw = 1;
+    // blocks per wavefront (all requested up front): one wavefront per block as long as 16 wavefronts cover k
     int per = (int)dev->opt_matvec_per;
-    if (per != 1 && per != 2 && per != 4) per = tiles >= 512 ? 2 : (kb > 16 ? 2 : 1); // measured best on MI355X
-    while (per > 1 && kb % per) per /= 2; // the kernel wants SW * PER == kb
-    int SW = kb / per;
-    while (SW > 16 && per < 4 && kb % (per * 2) == 0) {
+    if (per != 1 && per != 2 && per != 4) per = 1;
+    while (per > 1 && (kb % per || tpw * per > (ex.nsplit > 0 ? 2 : 4))) per /= 2;
+    while (kb / per > 16 && tpw * per < 4 && kb % (per * 2) == 0) per *= 2; // the kernel wants SW * PER == kb
+    while (kb / per > 16 && tpw > nt && kb % (per * 2) == 0) { // long k: fewer tiles, more blocks per wavefront
+        tpw /= 2;
         per *= 2;
-        SW = kb / per;
     }
-    if (SW > 16) return FH_ERR_UNSUPPORTED;
-    // row tiles per workgroup share one staging of x
-    int TW = (int)dev->opt_matvec_tiles;
-    if (TW != 1 && TW != 2 && TW != 4) TW = tiles >= 512 ? 2 : 1;
-    while (TW > 1 && TW * nt * SW > 16) TW /= 2;
-    const int TS = TW * nt;
-    if (TS * SW > 16 || (TS != 1 && TS != 2 && TS != 4)) return FH_ERR_UNSUPPORTED;
-    size_t lds = (size_t)kb * Q4K_IMG * 16 + (size_t)kb * 64 + 16 * 64 + 64;
+    const int SW = kb / per;
+    if (SW > 16 || kb % per || tpw * per > 4) return FH_ERR_UNSUPPORTED;
+    size_t lds = (size_t)kb * Q4K_IMG * 16 + (size_t)kb * 64 + (size_t)tpw * 16 * 64 + 64;
     if (lds > 160 * 1024) return FH_ERR_UNSUPPORTED;
-    unsigned grid = (unsigned)((tiles + TW - 1) / TW);
-#define Q4K_M1_GO(TS_, EPI_) return q4k_m1_per<TS_, EPI_>(per, q, x, y, a, b, SW, grid, lds, ex)
-    if (epi == FH_EPI_SWIGLU) {
-        if (TS == 2) Q4K_M1_GO(2, FH_EPI_SWIGLU);
-        Q4K_M1_GO(4, FH_EPI_SWIGLU);
+    const int tout = tpw / nt;
+    unsigned grid = (unsigned)((tiles + tout - 1) / tout);
+    switch (epi) {
+    case FH_EPI_SWIGLU: return q4k_m1_shape<FH_EPI_SWIGLU>(tpw, per, q, x, y, a, b, SW, grid, lds, ex);
+    case FH_EPI_ADD2: return q4k_m1_shape<FH_EPI_ADD2>(tpw, per, q, x, y, a, b, SW, grid, lds, ex);
+    case FH_EPI_ACC: return q4k_m1_shape<FH_EPI_ACC>(tpw, per, q, x, y, a, b, SW, grid, lds, ex);
+    case FH_EPI_ROPEKV: return q4k_m1_shape<FH_EPI_ROPEKV>(tpw, per, q, x, y, a, b, SW, grid, lds, ex);
+    default: return q4k_m1_shape<FH_EPI_NONE>(tpw, per, q, x, y, a, b, SW, grid, lds, ex);
     }
-    if (epi == FH_EPI_ADD2) {
-        if (TS == 1) Q4K_M1_GO(1, FH_EPI_ADD2);
-        if (TS == 2) Q4K_M1_GO(2, FH_EPI_ADD2);
-        Q4K_M1_GO(4, FH_EPI_ADD2);
-    }
-    if (epi == FH_EPI_ACC) {
-        if (TS == 1) Q4K_M1_GO(1, FH_EPI_ACC);
-        return FH_ERR_UNSUPPORTED;
-    }
-    if (epi == FH_EPI_ROPEKV) {
-        if (TS == 1) Q4K_M1_GO(1, FH_EPI_ROPEKV);
-        if (TS == 2) Q4K_M1_GO(2, FH_EPI_ROPEKV);
-        Q4K_M1_GO(4, FH_EPI_ROPEKV);
-    }
-    if (TS == 1) Q4K_M1_GO(1, FH_EPI_NONE);
-    if (TS == 2) Q4K_M1_GO(2, FH_EPI_NONE);
-    Q4K_M1_GO(4, FH_EPI_NONE);
-#undef Q4K_M1_GO
 }
