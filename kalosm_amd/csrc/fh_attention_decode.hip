@@ -3,11 +3,12 @@
 // Reference: fusor-ml/fusor/src/composite/flash_attention.rs:58-236 (semantics, no mask for a single query:
 // models/kalosm-llama/src/raw/mod.rs:969-972).
 //
-// grid (S splits, kv heads).  A workgroup owns the keys [split * chunk, (split + 1) * chunk) of one KV head, with
-// chunk = ceil(len / S) rounded up to 16 computed from the device-side length, and the G query heads that share
-// the KV head: K and V rows are read once for all of them.  A key row is spread over D / 8 lanes (32 bytes of f32
-// or 16 bytes of f16 each); the first four rows of every lane group, K and V, are requested before any arithmetic
-// so that one memory latency covers the usual chunk.  Partial results go to [q head][split][D + 4]:
+// grid (S splits, kv heads).  The keys of one KV head are dealt to the splits in granules of 16 (granule i goes
+// to split i mod S), so which rows a workgroup reads does not depend on the device-side length: the first four
+// rows of every lane group, K and V, are requested before the length has arrived (rows past the length are
+// read from the cache allocation and masked afterwards), and one memory latency covers the usual context.  A
+// workgroup serves the G query heads that share its KV head: K and V rows are read once for all of them.  A key
+// row is spread over D / 8 lanes (32 bytes of f32 or 16 bytes of f16 each).  Partial results go to [q head][split][D + 4]:
 // unnormalised output, running max, running sum; k_attn_combine_dl (or the consumer of the partials) merges them.
 #include "fh_internal.h"
 
@@ -41,6 +42,16 @@ __device__ __forceinline__ float ad_row16_sum(float a) {
     a += ad_dpp<0x140>(a);
     return a;
 }
+// lanes 0-31: a[l] + a[l + 32]; lanes 32-63: b[l - 32] + b[l]  (one swap and one add fold two registers)
+__device__ __forceinline__ float ad_fold32(float a, float b) {
+    auto s = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(s[0]) + __uint_as_float(s[1]);
+}
+// rows of 16 lanes (r0, r1, r2, r3) of a and b -> (a.r0 + a.r1, b.r0 + b.r1, a.r2 + a.r3, b.r2 + b.r3)
+__device__ __forceinline__ float ad_fold16(float a, float b) {
+    auto s = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(s[0]) + __uint_as_float(s[1]);
+}
 // sum over the four rows of 16 lanes of a wavefront (lane i of every row gets it)
 __device__ __forceinline__ float ad_rows_sum(float a) {
     const uint32_t u = __float_as_uint(a);
@@ -55,7 +66,7 @@ template <typename TKV, int D, int G, int NWV>
 __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__restrict__ q, const TKV *__restrict__ k,
                                                               const TKV *__restrict__ v, int64_t kv_sh, int64_t kv_st,
                                                               const int *__restrict__ len_dev, float scale,
-                                                              int chunk_max, float *__restrict__ part) {
+                                                              int chunk_max, int cap, float *__restrict__ part) {
     constexpr int LP = D / 8, RPW = 64 / LP, RW = NWV * RPW, U = 4;
     static_assert(NWV >= G, "one wavefront per query head for the softmax statistics");
     extern __shared__ float sm[];
@@ -64,33 +75,46 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
     __shared__ float s_stat[2 * G];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, grp = lane / LP, c = lane % LP;
     const int split = blockIdx.x, S = gridDim.x, kh = blockIdx.y;
-    const int skv = *len_dev + 1; // the step's own key is already appended at index len
-    int chunk = ((skv + S - 1) / S + 15) & ~15;
-    if (chunk > chunk_max) chunk = chunk_max;
-    const int c0 = split * chunk;
-    const int nk = min(skv, c0 + chunk) - c0; // <= 0 for trailing splits
-    const TKV *kb = k + kh * kv_sh + (int64_t)c0 * kv_st + 8 * c, *vb = v + kh * kv_sh + (int64_t)c0 * kv_st + 8 * c;
-    const int trow = wave * RPW + grp; // row of this lane group inside an iteration of RW rows
+    const TKV *kb = k + kh * kv_sh + 8 * c, *vb = v + kh * kv_sh + 8 * c;
+    const int trow = wave * RPW + grp; // local row of this lane group inside an iteration of RW rows
+    // local row -> cache row: granule (local / 16) of this split is granule (local / 16) * S + split of the head
+    auto cache_row = [&](int lr) { return ((lr >> 4) * S + split) * 16 + (lr & 15); };
 
+    // the first U0 rows of every lane group are requested blind (2 * RW local rows = 1024 keys with 8 splits); the
+    // other prefetched rows wait for the length, so that a short context does not pay for requests it drops
+    constexpr int U0 = 2;
     float kpre[U][8], vpre[U][8];
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-        const int t = u * RW + trow;
-        if (t < nk) ad_load8<TKV>(kb + (int64_t)t * kv_st, kpre[u]);
-        else {
+    for (int u = 0; u < U0; u++) {
+        const int t = cache_row(u * RW + trow);
+        ad_load8<TKV>(kb + (int64_t)(t < cap ? t : 0) * kv_st, kpre[u]);
+    }
 #pragma unroll
-            for (int i = 0; i < 8; i++) kpre[u][i] = 0.f;
+    for (int u = 0; u < U0; u++) {
+        const int t = cache_row(u * RW + trow);
+        ad_load8<TKV>(vb + (int64_t)(t < cap ? t : 0) * kv_st, vpre[u]);
+    }
+    __builtin_amdgcn_sched_barrier(0); // the requests above do not wait for the length
+    const int skv = *len_dev + 1;      // the step's own key is already appended at index len
+    // local rows of this split: 16 per whole granule it owns, plus the tail if the last, partial granule is its own
+    const int gfull = skv >> 4;
+    int nk = gfull > split ? ((gfull - split + S - 1) / S) * 16 : 0;
+    if (gfull % S == split) nk += skv & 15;
+    if (nk > chunk_max) nk = chunk_max;
+#pragma unroll
+    for (int u = U0; u < U; u++) {
+        const int lr = u * RW + trow;
+        if (u * RW < nk) {
+            ad_load8<TKV>(kb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st, kpre[u]);
+            ad_load8<TKV>(vb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st, vpre[u]);
         }
     }
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-        const int t = u * RW + trow;
-        if (t < nk) ad_load8<TKV>(vb + (int64_t)t * kv_st, vpre[u]);
-        else {
+    for (int u = 0; u < U; u++)
+        if (u * RW + trow >= nk) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) vpre[u][i] = 0.f;
+            for (int i = 0; i < 8; i++) kpre[u][i] = vpre[u][i] = 0.f;
         }
-    }
     float qr[G][8];
 #pragma unroll
     for (int h = 0; h < G; h++) {
@@ -116,7 +140,7 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
     for (int t0 = U * RW; t0 < nk; t0 += RW) {
         const int t = t0 + trow;
         float kv8[8];
-        if (t < nk) ad_load8<TKV>(kb + (int64_t)t * kv_st, kv8);
+        if (t < nk) ad_load8<TKV>(kb + (int64_t)cache_row(t) * kv_st, kv8);
         else {
 #pragma unroll
             for (int i = 0; i < 8; i++) kv8[i] = 0.f;
@@ -168,21 +192,33 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
         const int t = t0 + trow;
         float v8[8];
         if (t < nk) {
-            ad_load8<TKV>(vb + (int64_t)t * kv_st, v8);
+            ad_load8<TKV>(vb + (int64_t)cache_row(t) * kv_st, v8);
             accum(v8, t);
         }
     }
     // ---- add the row groups of the wavefront, then the wavefronts
+    if constexpr (G == 4) {
+        // four heads x one dim fold into one register: row r of 16 lanes ends with head r's total, so every lane
+        // stores eight sums of "its" head (6 operations per 4 values instead of 6 per value)
+        float f[8];
 #pragma unroll
-    for (int h = 0; h < G; h++)
+        for (int i = 0; i < 8; i++)
+            f[i] = ad_fold16(ad_fold32(o[0][i], o[2][i]), ad_fold32(o[1][i], o[3][i]));
+        float *dst = s_red + (wave * G + grp) * D + 8 * c;
+        *(float4 *)dst = make_float4(f[0], f[1], f[2], f[3]);
+        *(float4 *)(dst + 4) = make_float4(f[4], f[5], f[6], f[7]);
+    } else {
 #pragma unroll
-        for (int i = 0; i < 8; i++) o[h][i] = ad_rows_sum(o[h][i]);
-    if (grp == 0) {
+        for (int h = 0; h < G; h++)
 #pragma unroll
-        for (int h = 0; h < G; h++) {
-            float *dst = s_red + (wave * G + h) * D + 8 * c;
-            *(float4 *)dst = make_float4(o[h][0], o[h][1], o[h][2], o[h][3]);
-            *(float4 *)(dst + 4) = make_float4(o[h][4], o[h][5], o[h][6], o[h][7]);
+            for (int i = 0; i < 8; i++) o[h][i] = ad_rows_sum(o[h][i]);
+        if (grp == 0) {
+#pragma unroll
+            for (int h = 0; h < G; h++) {
+                float *dst = s_red + (wave * G + h) * D + 8 * c;
+                *(float4 *)dst = make_float4(o[h][0], o[h][1], o[h][2], o[h][3]);
+                *(float4 *)(dst + 4) = make_float4(o[h][4], o[h][5], o[h][6], o[h][7]);
+            }
         }
     }
     __syncthreads();
@@ -224,7 +260,7 @@ static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const 
     // projection merges while staging its input.  The option allows 4 .. 16.
     int S = dev->opt_attn_splits > 0 ? (int)dev->opt_attn_splits : 8;
     S = S < 4 ? 4 : (S > 16 ? 16 : S);
-    const int chunk_max = ((max_len + S - 1) / S + 15) & ~15;
+    const int chunk_max = (((max_len + 15) / 16 + S - 1) / S) * 16; // most local rows of a split
     const size_t lds = ((size_t)G * chunk_max + (size_t)NWV * G * D) * 4;
     FH_REQUIRE(lds <= 150 * 1024, "KV capacity %d too large for the decode attention kernel", max_len);
     FH_TRY(fh_dev_scratch(dev, (void **)&dev->part_buf, &dev->part_cap, (size_t)hq * S * (D + 4) * 4));
@@ -235,7 +271,7 @@ static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const 
         attr_done = true;
     }
     k_attn_decode_dl<TKV, D, G, NWV><<<dim3((unsigned)S, (unsigned)hkv), dim3(64 * NWV), lds, dev->stream>>>(
-        q, (const TKV *)k, (const TKV *)v, kv_sh, kv_st, len_dev, scale, chunk_max, dev->part_buf);
+        q, (const TKV *)k, (const TKV *)v, kv_sh, kv_st, len_dev, scale, chunk_max, max_len, dev->part_buf);
     FH_HIP(hipGetLastError());
     if (splits_out) *splits_out = S;
     if (out) {

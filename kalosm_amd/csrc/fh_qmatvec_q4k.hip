@@ -372,6 +372,9 @@ static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, co
     if constexpr (TPW * PER <= 2) {
         kern = in == 2 ? k_qmv_q4k_m1<TPW, PER, EPI, 2>
                        : (in == 1 ? k_qmv_q4k_m1_w8<TPW, PER, EPI, 1> : k_qmv_q4k_m1_w8<TPW, PER, EPI, 0>);
+    } else if constexpr (EPI == FH_EPI_ACC && PER == 1) {
+        kern = in == 2 ? k_qmv_q4k_m1<TPW, PER, EPI, 2>
+                       : (in == 1 ? k_qmv_q4k_m1<TPW, PER, EPI, 1> : k_qmv_q4k_m1<TPW, PER, EPI, 0>);
     } else {
         if (in == 2) return FH_ERR_UNSUPPORTED; // the merge of the attention partials needs the registers
         kern = in == 1 ? k_qmv_q4k_m1<TPW, PER, EPI, 1> : k_qmv_q4k_m1<TPW, PER, EPI, 0>;
@@ -396,10 +399,10 @@ static fh_status q4k_m1_shape(int tpw, int per, const fh_qmatrix *q, const float
         if (tpw == 1 && per == 2) return q4k_m1_launch<1, 2, EPI>(q, x, y, a, b, SW, grid, lds, ex);
         if (tpw == 1 && per == 4) return q4k_m1_launch<1, 4, EPI>(q, x, y, a, b, SW, grid, lds, ex);
     }
+    if (tpw == 2 && per == 1) return q4k_m1_launch<2, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
+    if (tpw == 4 && per == 1) return q4k_m1_launch<4, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
     if constexpr (EPI != FH_EPI_ACC) {
-        if (tpw == 2 && per == 1) return q4k_m1_launch<2, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
         if (tpw == 2 && per == 2) return q4k_m1_launch<2, 2, EPI>(q, x, y, a, b, SW, grid, lds, ex);
-        if (tpw == 4 && per == 1) return q4k_m1_launch<4, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
     }
     return FH_ERR_UNSUPPORTED;
 }
@@ -472,7 +475,11 @@ static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra 
     int tpw = (int)dev->opt_matvec_tiles;
     if (tpw != 1 && tpw != 2 && tpw != 4) tpw = tiles > dev->compute_units ? 2 : 1;
     if (epi == FH_EPI_SWIGLU && tpw < 2) tpw = 2;
-    if (epi == FH_EPI_ACC || ex.nsplit > 0) tpw = 1;
+    if (ex.nsplit > 0) { // merging attention partials: every workgroup merges its slice again, so fewer, fatter ones
+        tpw = (int)dev->opt_wo_tiles;
+        if (tpw != 1 && tpw != 2 && tpw != 4) tpw = 4;
+        if (epi != FH_EPI_ACC) tpw = 1;
+    } else if (epi == FH_EPI_ACC) tpw = 1;
     // blocks per wavefront (all requested up front): one wavefront per block as long as 16 wavefronts cover k
     int per = (int)dev->opt_matvec_per;
     if (per != 1 && per != 2 && per != 4) per = 1;
