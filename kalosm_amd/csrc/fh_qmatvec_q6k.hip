@@ -10,6 +10,7 @@
 // (two accumulator tiles per 256-block).  Lane (row j, group g) then owns groups 2g, 2g+1 of both halves of
 // its own row and applies d * sc_G * 2^(24 - e_G).
 #include "fh_blocks.h"
+#include "fh_mv_lanes.h"
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -20,54 +21,47 @@ struct Q6KRegs {
     uint16_t d;
 };
 
-#define DPP_XOR1 0xB1 // quad_perm [1,0,3,2]
-#define DPP_XOR2 0x4E // quad_perm [2,3,0,1]
-template <int CTRL>
-__device__ __forceinline__ float dpp_f32(float v) {
-    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
-}
-
 #define Q6K_IMG 65 // uint4 per block image: 8 steps x 4 lane groups x (hi, lo) + one all-zero slot
 #define Q6K_SF 32  // floats per block: 16 group sums, 16 factors
 
-template <int TS, int PER, int EPI>
+// Workgroup = SW wavefronts, one per k-slice of PER blocks; a wavefront multiplies its slice of TPW row tiles (with
+// the SwiGLU epilogue: gate tiles and the matching up tiles), stages the activations of its own blocks only (no
+// barrier before the products) and requests all its weight bytes before anything else.
+template <int TPW, int PER, int EPI>
 __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__restrict__ x, float *__restrict__ y,
                                                       const float *__restrict__ ea, const float *__restrict__ eb,
                                                       int SW, const float *__restrict__ xup) {
     constexpr int NT = EPI == FH_EPI_SWIGLU ? 2 : 1;
-    constexpr int TW = TS / NT;
-    constexpr int XB = (PER + TS - 1) / TS;
+    constexpr int TOUT = TPW / NT; // output tiles of the workgroup
     extern __shared__ uint4 lds[];
     // gridDim.y > 1: k is split over workgroups (blocks [boff, boff + kb) here) that add into y with atomics
     const int kb = SW * PER, boff = (int)blockIdx.y * kb; // the host launches with SW * PER * gridDim.y == q.kb
     uint4 *img = lds;
     float *sf = (float *)(lds + kb * Q6K_IMG);
-    float *l_red = sf + kb * Q6K_SF; // [TS][SW][16]
+    float *l_red = sf + kb * Q6K_SF; // [TPW][SW][16]
     const int tid = threadIdx.x, lane = tid & 63, j = lane & 15, g = lane >> 4;
-    // the wavefront index as a scalar: everything derived from it (tile, record address) stays on the scalar unit
+    // the wavefront index as a scalar: everything derived from it (record addresses) stays on the scalar unit
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nwaves = TS * SW;
-    const int stream = wave % TS, slice = wave / TS;
     const int64_t nout = EPI == FH_EPI_SWIGLU ? q.n / 2 : q.n;
     const int64_t tiles_out = (nout + 15) / 16;
-    const int64_t to = (int64_t)blockIdx.x * TW + (stream % TW);
-    const bool tvalid = to < tiles_out;
-    const int64_t tile = to + (int64_t)(stream / TW) * (nout / 16);
-    const int b0 = slice * PER;
-
-    // a tile past the end re-reads the last one (never stored)
-    const int64_t tl = tvalid ? tile : tile - (to - (tiles_out - 1));
-    const uint8_t *rec = q.data + (tl * q.recs + boff + b0) * 3360;
+    const int b0 = wave * PER;
+    const uint8_t *rec[TPW];
+#pragma unroll
+    for (int tp = 0; tp < TPW; tp++) {
+        const int64_t to = (int64_t)blockIdx.x * TOUT + (tp % TOUT);
+        const int64_t tile = to + (int64_t)(tp / TOUT) * (nout / 16); // up tiles follow the gate tiles
+        // a tile past the end re-reads the last one (never stored)
+        const int64_t tl = to < tiles_out ? tile : tile - (to - (tiles_out - 1));
+        rec[tp] = q.data + (tl * q.recs + boff + b0) * 3360;
+    }
 
     // ---- 0. activations first (short, needed first)
     // With xup the input is silu(x) * xup (the SwiGLU of a gate | up projection, raw/attention_layer.rs:195),
     // evaluated while staging.
-    float4 xv[XB], uv[XB];
+    float4 xv[PER], uv[PER];
 #pragma unroll
-    for (int i = 0; i < XB; i++) {
-        // one tile stream: a wavefront stages exactly the blocks it multiplies (no other wavefront needs them)
-        const int b = TS == 1 ? b0 + i : wave + i * nwaves;
-        const int64_t at = (int64_t)(boff + (b < kb ? b : 0)) * 256 + lane * 4;
+    for (int i = 0; i < PER; i++) {
+        const int64_t at = (int64_t)(boff + b0 + i) * 256 + lane * 4;
         xv[i] = *(const float4 *)(x + at);
         if (xup) uv[i] = *(const float4 *)(xup + at);
     }
@@ -75,40 +69,42 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
     // for them alone while the weights are still in flight.
     __builtin_amdgcn_sched_barrier(0);
     // ---- 1. all weight bytes of this wavefront
-    Q6KRegs w[PER];
-    {
+    Q6KRegs w[TPW][PER];
 #pragma unroll
-        for (int r = 0; r < PER; r++) {
-            const uint8_t *p = rec + r * 3360;
-            w[r].l0 = *(const uint4 *)(p + lane * 16);
-            w[r].l1 = *(const uint4 *)(p + 1024 + lane * 16);
-            w[r].h = *(const uint4 *)(p + 2048 + lane * 16);
-            w[r].sc = *(const uint32_t *)(p + 3072 + lane * 4);
-            w[r].d = *(const uint16_t *)(p + 3328 + 2 * j);
+    for (int r = 0; r < PER; r++)
+#pragma unroll
+        for (int tp = 0; tp < TPW; tp++) {
+            const uint8_t *p = rec[tp] + r * 3360;
+            w[tp][r].l0 = *(const uint4 *)(p + lane * 16);
+            w[tp][r].l1 = *(const uint4 *)(p + 1024 + lane * 16);
+            w[tp][r].h = *(const uint4 *)(p + 2048 + lane * 16);
+            w[tp][r].sc = *(const uint32_t *)(p + 3072 + lane * 4);
+            w[tp][r].d = *(const uint16_t *)(p + 3328 + 2 * j);
         }
-    }
-    // ---- 2. stage x: lane owns k = 256*b + 4*lane .. +3, i.e. a quarter of group G = lane / 4
+    // ---- 2. stage x: lane owns k = 256*b + 4*lane .. +3, i.e. a quarter of group G = lane / 4.  A wavefront stages
+    // exactly the blocks it multiplies.  (No branch around this: the compiler would sink the activation loads
+    // into it, behind the weight loads.)
 #pragma unroll
-    for (int i = 0; i < XB; i++) {
-        // no branch (the compiler would sink the activation loads into it, behind the weight loads): a wavefront
-        // without a block of its own stages block 0 once more, writing the values wavefront 0 writes
-        const int b = TS == 1 ? b0 + i : (wave + i * nwaves < kb ? wave + i * nwaves : 0);
+    for (int i = 0; i < PER; i++) {
+        const int b = b0 + i;
         float4 v = xv[i];
         if (xup)
             v = make_float4((v.x / (__expf(-v.x) + 1.0f)) * uv[i].x, (v.y / (__expf(-v.y) + 1.0f)) * uv[i].y,
                             (v.z / (__expf(-v.z) + 1.0f)) * uv[i].z, (v.w / (__expf(-v.w) + 1.0f)) * uv[i].w);
-        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        amax = fmaxf(amax, dpp_f32<DPP_XOR1>(amax));
-        amax = fmaxf(amax, dpp_f32<DPP_XOR2>(amax));
-        int e = 141 - (int)((__float_as_uint(amax) >> 23) & 0xFFu); // 14 - floor(log2 amax); specials clamp
+        const float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        // non-negative floats order like their bit patterns: the cross-lane maximum is an integer one
+        uint32_t am = __float_as_uint(amax);
+        am = max(am, dpp_u32<DPP_XOR1>(am));
+        am = max(am, dpp_u32<DPP_XOR2>(am));
+        int e = 141 - (int)((am >> 23) & 0xFFu); // 14 - floor(log2 amax); specials clamp
         e = e > 100 ? 100 : (e < -100 ? -100 : e);
         const float sc = __uint_as_float((uint32_t)(e + 127) << 23);
-        const float xs[4] = {v.x * sc, v.y * sc, v.z * sc, v.w * sc};
+        const float xq[4] = {v.x, v.y, v.z, v.w};
         _Float16 hi[4], lo[4];
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            hi[c] = (_Float16)xs[c];
-            lo[c] = (_Float16)(xs[c] - (float)hi[c]);
+        for (int c = 0; c < 4; c++) { // x * sc is exact (a power of two), so the fused form rounds like the split one
+            hi[c] = (_Float16)(xq[c] * sc);
+            lo[c] = (_Float16)__builtin_fmaf(xq[c], sc, -(float)hi[c]);
         }
         uint2 ph, pl;
         __builtin_memcpy(&ph, hi, 8);
@@ -126,79 +122,104 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
             sf[b * Q6K_SF + 16 + (lane >> 2)] = __uint_as_float((uint32_t)(24 - e + 127) << 23);
         }
     }
-    if (TS > 1) __syncthreads(); // with one tile stream the image a wavefront reads is the one it wrote
-    // ---- 3. two chains of four MFMA steps per block
-    const int gl = j >> 1, part = j & 1; // this lane's A row is (group gl of a half block, hi | lo)
-    const uint4 *pa[8];
+    // ---- 3. two chains of four MFMA steps per block and tile; the TPW tiles share every operand read
+    // This lane's A row is (group gl of a half block, hi | lo): it holds data in steps m and m + 4 with m = gl / 2
+    // if its lane group covers the k of that group (g / 2 == gl % 2), zeros otherwise.  Those lanes are bits
+    // 4m, 4m + 1 of the rows 0, 1 and bits 4m + 2, 4m + 3 of the rows 2, 3.
+    const int gl = j >> 1, part = j & 1;
+    uint32_t pa[8];
+    {
+        const uint32_t own = lds_addr(img + b0 * Q6K_IMG + ((gl >> 1) * 4 + g) * 2 + part);
+        const uint32_t zero = lds_addr(img + b0 * Q6K_IMG + 64);
 #pragma unroll
-    for (int t = 0; t < 8; t++) {
-        const bool real = ((t & 3) == (gl >> 1)) && ((g >> 1) == (gl & 1));
-        pa[t] = img + b0 * Q6K_IMG + (real ? (t * 4 + g) * 2 + part : 64);
+        for (int t = 0; t < 8; t++) {
+            const int m = t & 3;
+            const uint64_t mask = ((uint64_t)0x00030003u << (4 * m)) | ((uint64_t)0x000C000Cu << (4 * m + 32));
+            pa[t] = sel_lanes(mask, own + (t >> 2) * 32 * 16, zero);
+        }
     }
+    // the operands do not depend on the weights: RING of them are always on their way from the LDS
+    constexpr int RING = 4;
+    uint4 ring[RING];
+#pragma unroll
+    for (int t = 0; t < RING; t++) ring[t] = lds_read16(pa[t % 8] + (t / 8) * Q6K_IMG * 16);
     const float *psf = sf + b0 * Q6K_SF + 2 * g;
     const uint32_t LO = 0x000F000Fu, HB = 0x00300030u;
-    float acc = 0.f, cen = 0.f;
+    float acc[TPW], cen[TPW];
+#pragma unroll
+    for (int tp = 0; tp < TPW; tp++) acc[tp] = cen[tp] = 0.f;
 #pragma unroll
     for (int r = 0; r < PER; r++) {
-        floatx4 dd[2];
+        floatx4 dd[TPW][2];
 #pragma unroll
         for (int hb = 0; hb < 2; hb++) {
-            floatx4 c = {0.f, 0.f, 0.f, 0.f};
-            const uint4 lq = hb ? w[r].l1 : w[r].l0;
+#pragma unroll
+            for (int tp = 0; tp < TPW; tp++) dd[tp][hb] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int tt = 0; tt < 4; tt++) {
-                const int t = 4 * hb + tt;
-                const uint32_t lw = tt == 0 ? lq.x : (tt == 1 ? lq.y : (tt == 2 ? lq.z : lq.w));
-                const uint32_t hsel = (t >> 1) == 0 ? w[r].h.x : ((t >> 1) == 1 ? w[r].h.y : ((t >> 1) == 2 ? w[r].h.z : w[r].h.w));
-                uint4 bo;
-                if ((t & 1) == 0) {
-                    bo.x = (lw & LO) | (hsel & HB);
-                    bo.y = ((lw >> 4) & LO) | ((hsel >> 2) & HB);
-                    bo.z = ((lw >> 8) & LO) | ((hsel >> 4) & HB);
-                    bo.w = ((lw >> 12) & LO) | ((hsel >> 6) & HB);
-                } else {
-                    bo.x = (lw & LO) | ((hsel << 4) & HB);
-                    bo.y = ((lw >> 4) & LO) | ((hsel << 2) & HB);
-                    bo.z = ((lw >> 8) & LO) | ((hsel >> 8) & HB);
-                    bo.w = ((lw >> 12) & LO) | ((hsel >> 10) & HB);
-                }
-                const uint4 ao = pa[t][r * Q6K_IMG];
-                half8 av, bv;
+                const int t = 4 * hb + tt, ti = r * 8 + t;
+                const uint4 ao = ring[ti % RING];
+                half8 av;
                 __builtin_memcpy(&av, &ao, 16);
-                __builtin_memcpy(&bv, &bo, 16);
-                c = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, c, 0, 0, 0);
+#pragma unroll
+                for (int tp = 0; tp < TPW; tp++) {
+                    const uint4 lq = hb ? w[tp][r].l1 : w[tp][r].l0;
+                    const uint4 hq = w[tp][r].h;
+                    const uint32_t lw = tt == 0 ? lq.x : (tt == 1 ? lq.y : (tt == 2 ? lq.z : lq.w));
+                    const uint32_t hsel = (t >> 1) == 0 ? hq.x : ((t >> 1) == 1 ? hq.y : ((t >> 1) == 2 ? hq.z : hq.w));
+                    uint4 bo;
+                    if ((t & 1) == 0) {
+                        bo.x = (lw & LO) | (hsel & HB);
+                        bo.y = ((lw >> 4) & LO) | ((hsel >> 2) & HB);
+                        bo.z = ((lw >> 8) & LO) | ((hsel >> 4) & HB);
+                        bo.w = ((lw >> 12) & LO) | ((hsel >> 6) & HB);
+                    } else {
+                        bo.x = (lw & LO) | ((hsel << 4) & HB);
+                        bo.y = ((lw >> 4) & LO) | ((hsel << 2) & HB);
+                        bo.z = ((lw >> 8) & LO) | ((hsel >> 8) & HB);
+                        bo.w = ((lw >> 12) & LO) | ((hsel >> 10) & HB);
+                    }
+                    half8 bv;
+                    __builtin_memcpy(&bv, &bo, 16);
+                    dd[tp][hb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, dd[tp][hb], 0, 0, 0);
+                }
+                if (ti + RING < PER * 8)
+                    ring[ti % RING] = lds_read16(pa[(ti + RING) % 8] + ((ti + RING) / 8) * Q6K_IMG * 16);
             }
-            dd[hb] = c;
         }
-        const float d = fh_h2f(w[r].d);
-        const int scw = (int)w[r].sc;
-        const float s0 = (float)((scw << 24) >> 24), s1 = (float)((scw << 16) >> 24), s2 = (float)((scw << 8) >> 24),
-                    s3 = (float)(scw >> 24);
         const float2 sx0 = *(const float2 *)(psf + r * Q6K_SF), sx1 = *(const float2 *)(psf + r * Q6K_SF + 8);
         const float2 f0 = *(const float2 *)(psf + r * Q6K_SF + 16), f1 = *(const float2 *)(psf + r * Q6K_SF + 24);
-        acc = fmaf(dd[0][0] + dd[0][1], (s0 * d) * f0.x, acc);
-        acc = fmaf(dd[0][2] + dd[0][3], (s1 * d) * f0.y, acc);
-        acc = fmaf(dd[1][0] + dd[1][1], (s2 * d) * f1.x, acc);
-        acc = fmaf(dd[1][2] + dd[1][3], (s3 * d) * f1.y, acc);
-        float cs = s0 * sx0.x;
-        cs = fmaf(s1, sx0.y, cs);
-        cs = fmaf(s2, sx1.x, cs);
-        cs = fmaf(s3, sx1.y, cs);
-        cen = fmaf(d, cs, cen);
+#pragma unroll
+        for (int tp = 0; tp < TPW; tp++) {
+            const float d = fh_h2f(w[tp][r].d);
+            const int scw = (int)w[tp][r].sc;
+            const float s0 = (float)((scw << 24) >> 24), s1 = (float)((scw << 16) >> 24),
+                        s2 = (float)((scw << 8) >> 24), s3 = (float)(scw >> 24);
+            acc[tp] = fmaf(dd[tp][0][0] + dd[tp][0][1], (s0 * d) * f0.x, acc[tp]);
+            acc[tp] = fmaf(dd[tp][0][2] + dd[tp][0][3], (s1 * d) * f0.y, acc[tp]);
+            acc[tp] = fmaf(dd[tp][1][0] + dd[tp][1][1], (s2 * d) * f1.x, acc[tp]);
+            acc[tp] = fmaf(dd[tp][1][2] + dd[tp][1][3], (s3 * d) * f1.y, acc[tp]);
+            float cs = s0 * sx0.x;
+            cs = fmaf(s1, sx0.y, cs);
+            cs = fmaf(s2, sx1.x, cs);
+            cs = fmaf(s3, sx1.y, cs);
+            cen[tp] = fmaf(d, cs, cen[tp]);
+        }
     }
-    float v = fmaf(-32.0f, cen, acc);
-    v += __shfl_xor(v, 16, 64);
-    v += __shfl_xor(v, 32, 64);
-    if (lane < 16) l_red[(stream * SW + slice) * 16 + lane] = v;
+#pragma unroll
+    for (int tp = 0; tp < TPW; tp++) {
+        const float v = rows_sum(fmaf(-32.0f, cen[tp], acc[tp]));
+        if (lane < 16) l_red[(tp * SW + wave) * 16 + lane] = v;
+    }
     __syncthreads();
-    if (tid < TW * 16) {
+    if (tid < TOUT * 16) {
         const int t = tid >> 4, jr = tid & 15;
         float v0 = 0.f, v1 = 0.f;
         for (int s = 0; s < SW; s++) {
             v0 += l_red[(t * SW + s) * 16 + jr];
-            if (NT == 2) v1 += l_red[((t + TW) * SW + s) * 16 + jr];
+            if (NT == 2) v1 += l_red[((t + TOUT) * SW + s) * 16 + jr];
         }
-        const int64_t row = ((int64_t)blockIdx.x * TW + t) * 16 + jr;
+        const int64_t row = ((int64_t)blockIdx.x * TOUT + t) * 16 + jr;
         if (row < nout) {
             float rr = v0;
             if (EPI == FH_EPI_ADD2) rr = (rr + ea[row]) + eb[row];
@@ -209,26 +230,34 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
     }
 }
 
-template <int TS, int PER, int EPI>
+template <int TPW, int PER, int EPI>
 static fh_status q6k_m1_launch(const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b, int SW,
                                unsigned grid, size_t lds, unsigned ksplit = 1, const float *xup = nullptr) {
     static bool attr_done = false;
     if (!attr_done) {
-        FH_HIP(hipFuncSetAttribute((const void *)k_qmv_q6k_m1<TS, PER, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        FH_HIP(hipFuncSetAttribute((const void *)k_qmv_q6k_m1<TPW, PER, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    160 * 1024));
         attr_done = true;
     }
-    k_qmv_q6k_m1<TS, PER, EPI><<<dim3(grid, ksplit), dim3(64 * TS * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, xup);
+    k_qmv_q6k_m1<TPW, PER, EPI><<<dim3(grid, ksplit), dim3(64 * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, xup);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
 
-template <int TS, int EPI>
-static fh_status q6k_m1_per(int per, const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b,
-                            int SW, unsigned grid, size_t lds) {
-    if (per == 1) return q6k_m1_launch<TS, 1, EPI>(q, x, y, a, b, SW, grid, lds);
-    if (per == 2) return q6k_m1_launch<TS, 2, EPI>(q, x, y, a, b, SW, grid, lds);
-    return q6k_m1_launch<TS, 4, EPI>(q, x, y, a, b, SW, grid, lds);
+// (tiles per wavefront, blocks per wavefront) with at most four block tiles (56 registers of weights) per wavefront
+template <int EPI>
+static fh_status q6k_m1_shape(int tpw, int per, const fh_qmatrix *q, const float *x, float *y, const float *a,
+                              const float *b, int SW, unsigned grid, size_t lds, unsigned ksplit = 1,
+                              const float *xup = nullptr) {
+    if constexpr (EPI != FH_EPI_SWIGLU) {
+        if (tpw == 1 && per == 1) return q6k_m1_launch<1, 1, EPI>(q, x, y, a, b, SW, grid, lds, ksplit, xup);
+        if (tpw == 1 && per == 2) return q6k_m1_launch<1, 2, EPI>(q, x, y, a, b, SW, grid, lds, ksplit, xup);
+        if (tpw == 1 && per == 4) return q6k_m1_launch<1, 4, EPI>(q, x, y, a, b, SW, grid, lds, ksplit, xup);
+    }
+    if (tpw == 2 && per == 1) return q6k_m1_launch<2, 1, EPI>(q, x, y, a, b, SW, grid, lds, ksplit, xup);
+    if (tpw == 2 && per == 2) return q6k_m1_launch<2, 2, EPI>(q, x, y, a, b, SW, grid, lds, ksplit, xup);
+    if (tpw == 4 && per == 1) return q6k_m1_launch<4, 1, EPI>(q, x, y, a, b, SW, grid, lds, ksplit, xup);
+    return FH_ERR_UNSUPPORTED;
 }
 
 // Returns FH_ERR_UNSUPPORTED when the shape does not fit this kernel (the caller falls back).
@@ -238,44 +267,35 @@ fh_status fh_launch_q6k_m1(const fh_qmatrix *q, const float *x, float *y, int ep
     const int nt = epi == FH_EPI_SWIGLU ? 2 : 1;
     const int64_t nout = epi == FH_EPI_SWIGLU ? q->n / 2 : q->n;
     const int64_t tiles = (nout + 15) / 16;
+    // tiles per wavefront (they share the staged activations and every operand read): two once there are more
+    // tiles than compute units; the SwiGLU epilogue needs the gate and the up tile in one wavefront
+    int tpw = (int)dev->opt_matvec_tiles;
+    if (tpw != 1 && tpw != 2 && tpw != 4) tpw = tiles > dev->compute_units ? 2 : 1;
+    if (epi == FH_EPI_SWIGLU && tpw < 2) tpw = 2;
+    // blocks per wavefront (all requested up front): vocabulary-sized matrices want two (measured on MI355X)
     int per = (int)dev->opt_matvec_per;
-    // measured on MI355X: vocabulary-sized matrices want 4 blocks per wavefront, layer-sized ones 2
-    if (per != 1 && per != 2 && per != 4) per = tiles >= 4096 ? 4 : (tiles >= 512 ? 2 : (kb > 16 ? 2 : 1));
-    while (per > 1 && kb % per) per /= 2; // the kernel wants SW * PER == kb
-    int SW = kb / per;
-    while (SW > 16 && per < 4 && kb % (per * 2) == 0) {
+    if (per != 1 && per != 2 && per != 4) per = tiles >= 4096 ? 2 : 1;
+    while (per > 1 && (kb % per || tpw * per > 4)) per /= 2;
+    while (kb / per > 16 && tpw * per < 4 && kb % (per * 2) == 0) per *= 2; // the kernel wants SW * PER == kb
+    while (kb / per > 16 && tpw > nt && kb % (per * 2) == 0) { // long k: fewer tiles, more blocks per wavefront
+        tpw /= 2;
         per *= 2;
-        SW = kb / per;
     }
-    if (SW > 16) return FH_ERR_UNSUPPORTED;
-    int TW = (int)dev->opt_matvec_tiles;
-    if (TW != 1 && TW != 2 && TW != 4) TW = (tiles >= 512 && tiles < 4096) ? 2 : 1;
-    while (TW > 1 && TW * nt * SW > 16) TW /= 2;
-    const int TS = TW * nt;
-    if (TS * SW > 16 || (TS != 1 && TS != 2 && TS != 4)) return FH_ERR_UNSUPPORTED;
-    size_t lds = (size_t)kb * Q6K_IMG * 16 + (size_t)kb * Q6K_SF * 4 + (size_t)TS * SW * 64;
+    const int SW = kb / per;
+    if (SW > 16 || kb % per || tpw * per > 4) return FH_ERR_UNSUPPORTED;
+    size_t lds = (size_t)kb * Q6K_IMG * 16 + (size_t)kb * Q6K_SF * 4 + (size_t)tpw * SW * 64;
     if (lds > 160 * 1024) return FH_ERR_UNSUPPORTED;
-    unsigned grid = (unsigned)((tiles + TW - 1) / TW);
-#define Q6K_M1_GO(TS_, EPI_) return q6k_m1_per<TS_, EPI_>(per, q, x, y, a, b, SW, grid, lds)
-    if (epi == FH_EPI_SWIGLU) {
-        if (TS == 2) Q6K_M1_GO(2, FH_EPI_SWIGLU);
-        Q6K_M1_GO(4, FH_EPI_SWIGLU);
-    }
-    if (epi == FH_EPI_ADD2) {
-        if (TS == 1) Q6K_M1_GO(1, FH_EPI_ADD2);
-        if (TS == 2) Q6K_M1_GO(2, FH_EPI_ADD2);
-        Q6K_M1_GO(4, FH_EPI_ADD2);
-    }
-    if (TS == 1) Q6K_M1_GO(1, FH_EPI_NONE);
-    if (TS == 2) Q6K_M1_GO(2, FH_EPI_NONE);
-    Q6K_M1_GO(4, FH_EPI_NONE);
-#undef Q6K_M1_GO
+    const int tout = tpw / nt;
+    unsigned grid = (unsigned)((tiles + tout - 1) / tout);
+    if (epi == FH_EPI_SWIGLU) return q6k_m1_shape<FH_EPI_SWIGLU>(tpw, per, q, x, y, a, b, SW, grid, lds);
+    if (epi == FH_EPI_ADD2) return q6k_m1_shape<FH_EPI_ADD2>(tpw, per, q, x, y, a, b, SW, grid, lds);
+    return q6k_m1_shape<FH_EPI_NONE>(tpw, per, q, x, y, a, b, SW, grid, lds);
 }
 
-// y += W . x + add with k split over `ksplit` workgroups per row tile (atomic adds, so the summation order - and the
-// last bits of the result - vary from run to run).  For matrices with few row tiles and a long k (the down projection
-// of a decode step accumulating into the residual stream) the smaller workgroups overlap their load and compute phases.
-// With xup the input is silu(x) * xup.
+// y += W . x + add with k split over `ksplit` workgroups per row tile group (atomic adds, so the summation order -
+// and the last bits of the result - vary from run to run).  For matrices with few row tiles and a long k (the down
+// projection of a decode step accumulating into the residual stream) the smaller workgroups overlap their load and
+// compute phases.  With xup the input is silu(x) * xup.
 fh_status fh_launch_q6k_m1_acc(const fh_qmatrix *q, const float *x, const float *xup, float *y_inout, const float *add) {
     fh_device *dev = q->dev;
     const int kb = (int)q->kb;
@@ -283,14 +303,15 @@ fh_status fh_launch_q6k_m1_acc(const fh_qmatrix *q, const float *x, const float 
     if (ks <= 0) ks = kb % 4 == 0 ? kb / 4 : 0; // four blocks per workgroup measured best (MI355X, k = 14336)
     if (ks < 2 || kb % ks) return FH_ERR_UNSUPPORTED;
     const int kbl = kb / ks;
+    int tpw = (int)dev->opt_down_tiles;
+    if (tpw != 1 && tpw != 2 && tpw != 4) tpw = 1;
     int per = (int)dev->opt_matvec_per;
     if (per != 1 && per != 2 && per != 4) per = 1;
-    while (per > 1 && kbl % per) per /= 2;
+    while (per > 1 && (kbl % per || tpw * per > 4)) per /= 2;
     const int SW = kbl / per;
     if (SW > 16) return FH_ERR_UNSUPPORTED;
     const int64_t tiles = (q->n + 15) / 16;
-    size_t lds = (size_t)kbl * Q6K_IMG * 16 + (size_t)kbl * Q6K_SF * 4 + (size_t)SW * 64;
-    if (per == 1) return q6k_m1_launch<1, 1, FH_EPI_ACC>(q, x, y_inout, add, nullptr, SW, (unsigned)tiles, lds, (unsigned)ks, xup);
-    if (per == 2) return q6k_m1_launch<1, 2, FH_EPI_ACC>(q, x, y_inout, add, nullptr, SW, (unsigned)tiles, lds, (unsigned)ks, xup);
-    return q6k_m1_launch<1, 4, FH_EPI_ACC>(q, x, y_inout, add, nullptr, SW, (unsigned)tiles, lds, (unsigned)ks, xup);
+    size_t lds = (size_t)kbl * Q6K_IMG * 16 + (size_t)kbl * Q6K_SF * 4 + (size_t)tpw * SW * 64;
+    const unsigned grid = (unsigned)((tiles + tpw - 1) / tpw);
+    return q6k_m1_shape<FH_EPI_ACC>(tpw, per, q, x, y_inout, add, nullptr, SW, grid, lds, (unsigned)ks, xup);
 }
