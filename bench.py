@@ -29,7 +29,7 @@ ROTATE_BYTES = 640 << 20  # > 2x the 256 MB Infinity Cache
 # HBM bytes per launch (average of the four shapes) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this
 # workload at batch 1, scaled by what the same counters read for a 256 MiB device copy (FETCH_SIZE x2.000,
 # WRITE_SIZE x1.000); a measured constant, to be re-measured when the kernel changes.
-TRAFFIC_BYTES_PER_LAUNCH = 19772006
+TRAFFIC_BYTES_PER_LAUNCH = 19766426
 
 
 def prefill_legs(dev) -> dict:
@@ -194,7 +194,7 @@ def main() -> int:
         "wall_ms_timed_region": round(wall_ms, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH if m == 1 else None,
-                     "kernel": "k_qmv_q4k_m1 (instances <1,1>, <2,2>, <1,4>)", "avg_launch_us": round(avg_us, 3),
+                     "kernel": "k_qmv_q4k_m1 (instances <1,1>, <2,1>, <1,4>: tiles, blocks per wavefront)", "avg_launch_us": round(avg_us, 3),
                      "algorithmic_bytes_per_launch": step_bytes // len(sets)},
     }
 
