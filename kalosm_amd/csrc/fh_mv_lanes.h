@@ -6,6 +6,7 @@
 #define DPP_XOR1 0xB1        // quad_perm [1,0,3,2]
 #define DPP_XOR2 0x4E        // quad_perm [2,3,0,1]
 #define DPP_HALF_MIRROR 0x141 // lane i <- lane 7-i within each group of 8
+#define DPP_ROW_MIRROR 0x140  // lane i <- lane 15-i within each row of 16
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {
     return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));

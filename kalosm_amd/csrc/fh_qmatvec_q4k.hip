@@ -54,7 +54,11 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
                                                       int SW, const float *__restrict__ xres,
                                                       const float *__restrict__ nw, float eps, int nsplit,
                                                       FhRopeArgs rk) {
-    constexpr int NT = EPI == FH_EPI_SWIGLU ? 2 : 1;
+    // SwiGLU with one tile per wavefront: the "tile" is rows 8h .. 8h+7 of a gate tile (columns 0-7 of the MFMA) and
+    // the same rows of the matching up tile (columns 8-15), h = workgroup parity: workgroups half as heavy as with a
+    // whole gate and a whole up tile, which divides the Llama FFN evenly over the compute units
+    constexpr bool HP = EPI == FH_EPI_SWIGLU && TPW == 1;
+    constexpr int NT = (EPI == FH_EPI_SWIGLU && !HP) ? 2 : 1;
     constexpr int TOUT = TPW / NT; // output tiles of the workgroup
     extern __shared__ uint4 lds[];
     // gridDim.y > 1: k is split over workgroups (blocks [boff, boff + kb) here) that add into y with atomics
@@ -70,8 +74,15 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     const int64_t tiles_out = (nout + 15) / 16;
     const int b0 = wave * PER;
     const uint8_t *ph[TPW], *pq[TPW];
+    if constexpr (HP) {
+        const int64_t tile = (int64_t)(blockIdx.x >> 1) + (j < 8 ? 0 : nout / 16);
+        const uint8_t *rec = q.data + (tile * q.recs + boff + b0) * 2304; // per lane: gate or up record
+        const int rr = 8 * (int)(blockIdx.x & 1) + (j & 7);
+        ph[0] = rec + 16 * rr;
+        pq[0] = rec + 256 + (16 * g + rr) * 16;
+    }
 #pragma unroll
-    for (int tp = 0; tp < TPW; tp++) {
+    for (int tp = 0; tp < (HP ? 0 : TPW); tp++) {
         const int64_t to = (int64_t)blockIdx.x * TOUT + (tp % TOUT);
         const int64_t tile = to + (int64_t)(tp / TOUT) * (nout / 16); // up tiles follow the gate tiles
         // a tile past the end re-reads the last tile (its rows are never stored)
@@ -185,8 +196,11 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         }
     }
     if (IN == 1) {
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        ss += dpp_f32<DPP_XOR1>(ss);
+        ss += dpp_f32<DPP_XOR2>(ss);
+        ss += dpp_f32<DPP_HALF_MIRROR>(ss);
+        ss += dpp_f32<DPP_ROW_MIRROR>(ss); // rows of 16 are uniform now
+        ss = rows_sum(ss);
         if (lane == 0) l_ss[wave] = ss;
     }
     // ---- 3. eight chained MFMA steps per block and tile; the TPW tiles share every operand read
@@ -276,7 +290,10 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
             v1 = v1 / rms;
         }
         const int64_t row = ((int64_t)blockIdx.x * TOUT + t) * 16 + jr;
-        if (EPI == FH_EPI_ROPEKV) {
+        if constexpr (HP) {
+            const float up = __shfl_xor(v0, 8, 64); // column j + 8 is the up row of gate row j
+            if (jr < 8) y[(int64_t)blockIdx.x * 8 + jr] = (v0 / (__expf(-v0) + 1.0f)) * up;
+        } else if (EPI == FH_EPI_ROPEKV) {
             const float other = __shfl_xor(v0, 1, 64); // the pair (2i, 2i+1) sits in neighbouring lanes
             const int pos = *rk.pos;
             if (row < nout && pos < rk.cap) {
@@ -357,11 +374,9 @@ static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, co
 template <int EPI>
 static fh_status q4k_m1_shape(int tpw, int per, const fh_qmatrix *q, const float *x, float *y, const float *a,
                               const float *b, int SW, unsigned grid, size_t lds, const Q4kExtra &ex) {
-    if constexpr (EPI != FH_EPI_SWIGLU) {
-        if (tpw == 1 && per == 1) return q4k_m1_launch<1, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
-        if (tpw == 1 && per == 2) return q4k_m1_launch<1, 2, EPI>(q, x, y, a, b, SW, grid, lds, ex);
-        if (tpw == 1 && per == 4) return q4k_m1_launch<1, 4, EPI>(q, x, y, a, b, SW, grid, lds, ex);
-    }
+    if (tpw == 1 && per == 1) return q4k_m1_launch<1, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
+    if (tpw == 1 && per == 2) return q4k_m1_launch<1, 2, EPI>(q, x, y, a, b, SW, grid, lds, ex);
+    if (tpw == 1 && per == 4) return q4k_m1_launch<1, 4, EPI>(q, x, y, a, b, SW, grid, lds, ex);
     if (tpw == 2 && per == 1) return q4k_m1_launch<2, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
     if (tpw == 4 && per == 1) return q4k_m1_launch<4, 1, EPI>(q, x, y, a, b, SW, grid, lds, ex);
     if constexpr (EPI != FH_EPI_ACC) {
@@ -437,7 +452,9 @@ static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra 
     // tiles than compute units; the SwiGLU epilogue needs the gate and the up tile in one wavefront
     int tpw = (int)dev->opt_matvec_tiles;
     if (tpw != 1 && tpw != 2 && tpw != 4) tpw = tiles > dev->compute_units ? 2 : 1;
-    if (epi == FH_EPI_SWIGLU && tpw < 2) tpw = 2;
+    // SwiGLU: half a gate tile and half an up tile per wavefront when the rows allow it (workgroups half as heavy)
+    const bool half_pairs = epi == FH_EPI_SWIGLU && nout % 16 == 0 && dev->opt_matvec_tiles <= 1;
+    if (epi == FH_EPI_SWIGLU) tpw = half_pairs ? 1 : (tpw < 2 ? 2 : tpw);
     if (ex.nsplit > 0) { // merging attention partials: every workgroup merges its slice again, so fewer, fatter ones
         tpw = (int)dev->opt_wo_tiles;
         if (tpw != 1 && tpw != 2 && tpw != 4) tpw = 4;
@@ -445,7 +462,7 @@ static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra 
     } else if (epi == FH_EPI_ACC) tpw = 1;
     // blocks per wavefront (all requested up front): one wavefront per block as long as 16 wavefronts cover k
     int per = (int)dev->opt_matvec_per;
-    if (per != 1 && per != 2 && per != 4) per = 1;
+    if (per != 1 && per != 2 && per != 4) per = half_pairs ? 2 : 1;
     while (per > 1 && (kb % per || tpw * per > (ex.nsplit > 0 ? 2 : 4))) per /= 2;
     while (kb / per > 16 && tpw * per < 4 && kb % (per * 2) == 0) per *= 2; // the kernel wants SW * PER == kb
     while (kb / per > 16 && tpw > nt && kb % (per * 2) == 0) { // long k: fewer tiles, more blocks per wavefront
@@ -456,8 +473,8 @@ static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra 
     if (SW > 16 || kb % per || tpw * per > 4) return FH_ERR_UNSUPPORTED;
     size_t lds = (size_t)kb * Q4K_IMG * 16 + (size_t)kb * 64 + (size_t)tpw * 16 * 64 + 64;
     if (lds > 160 * 1024) return FH_ERR_UNSUPPORTED;
-    const int tout = tpw / nt;
-    unsigned grid = (unsigned)((tiles + tout - 1) / tout);
+    const int tout = half_pairs ? 1 : tpw / nt;
+    unsigned grid = half_pairs ? (unsigned)(2 * tiles) : (unsigned)((tiles + tout - 1) / tout);
     switch (epi) {
     case FH_EPI_SWIGLU: return q4k_m1_shape<FH_EPI_SWIGLU>(tpw, per, q, x, y, a, b, SW, grid, lds, ex);
     case FH_EPI_ADD2: return q4k_m1_shape<FH_EPI_ADD2>(tpw, per, q, x, y, a, b, SW, grid, lds, ex);
