@@ -66,7 +66,8 @@ template <typename TKV, int D, int G, int NWV>
 __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__restrict__ q, const TKV *__restrict__ k,
                                                               const TKV *__restrict__ v, int64_t kv_sh, int64_t kv_st,
                                                               const int *__restrict__ len_dev, float scale,
-                                                              int chunk_max, int cap, float *__restrict__ part) {
+                                                              int chunk_max, int cap, int gtot,
+                                                              float *__restrict__ part) {
     constexpr int LP = D / 8, RPW = 64 / LP, RW = NWV * RPW, U = 4;
     static_assert(NWV >= G, "one wavefront per query head for the softmax statistics");
     extern __shared__ float sm[];
@@ -74,15 +75,16 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
     float *s_red = sm + G * chunk_max; // [NWV][G][D]
     __shared__ float s_stat[2 * G];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, grp = lane / LP, c = lane % LP;
-    const int split = blockIdx.x, S = gridDim.x, kh = blockIdx.y;
+    // blockIdx.z: which G of the gtot query heads of this KV head (the K and V rows are then read once per group)
+    const int split = blockIdx.x, S = gridDim.x, kh = blockIdx.y, h0 = kh * gtot + (int)blockIdx.z * G;
     const TKV *kb = k + kh * kv_sh + 8 * c, *vb = v + kh * kv_sh + 8 * c;
     const int trow = wave * RPW + grp; // local row of this lane group inside an iteration of RW rows
     // local row -> cache row: granule (local / 16) of this split is granule (local / 16) * S + split of the head
     auto cache_row = [&](int lr) { return ((lr >> 4) * S + split) * 16 + (lr & 15); };
 
-    // the first U0 rows of every lane group are requested blind (2 * RW local rows = 1024 keys with 8 splits); the
+    // the first U0 rows of every lane group are requested blind (U0 * RW = 128 local rows = 1024 keys with 8 splits); the
     // other prefetched rows wait for the length, so that a short context does not pay for requests it drops
-    constexpr int U0 = 2;
+    constexpr int U0 = 32 / NWV < U ? 32 / NWV : U;
     float kpre[U][8], vpre[U][8];
 #pragma unroll
     for (int u = 0; u < U0; u++) {
@@ -118,8 +120,8 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
     float qr[G][8];
 #pragma unroll
     for (int h = 0; h < G; h++) {
-        const float4 a = *(const float4 *)(q + (int64_t)(kh * G + h) * D + 8 * c);
-        const float4 b = *(const float4 *)(q + (int64_t)(kh * G + h) * D + 8 * c + 4);
+        const float4 a = *(const float4 *)(q + (int64_t)(h0 + h) * D + 8 * c);
+        const float4 b = *(const float4 *)(q + (int64_t)(h0 + h) * D + 8 * c + 4);
         qr[h][0] = a.x; qr[h][1] = a.y; qr[h][2] = a.z; qr[h][3] = a.w;
         qr[h][4] = b.x; qr[h][5] = b.y; qr[h][6] = b.z; qr[h][7] = b.w;
     }
@@ -207,6 +209,20 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
         float *dst = s_red + (wave * G + grp) * D + 8 * c;
         *(float4 *)dst = make_float4(f[0], f[1], f[2], f[3]);
         *(float4 *)(dst + 4) = make_float4(f[4], f[5], f[6], f[7]);
+    } else if constexpr (G == 2) {
+        // row r ends with head r % 2, dims i + 4 (r / 2)
+        float f[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            f[i] = ad_fold16(ad_fold32(o[0][i], o[0][i + 4]), ad_fold32(o[1][i], o[1][i + 4]));
+        *(float4 *)(s_red + (wave * G + (grp & 1)) * D + 8 * c + 4 * (grp >> 1)) = make_float4(f[0], f[1], f[2], f[3]);
+    } else if constexpr (G == 1) {
+        // row r ends with dims i + 2 r
+        float f[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+            f[i] = ad_fold16(ad_fold32(o[0][i], o[0][i + 4]), ad_fold32(o[0][i + 2], o[0][i + 6]));
+        *(float2 *)(s_red + wave * D + 8 * c + 2 * grp) = make_float2(f[0], f[1]);
     } else {
 #pragma unroll
         for (int h = 0; h < G; h++)
@@ -227,7 +243,7 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
         float a = 0.f;
 #pragma unroll
         for (int w = 0; w < NWV; w++) a += s_red[(w * G + h) * D + dd];
-        float *pp = part + ((int64_t)(kh * G + h) * S + split) * (D + 4);
+        float *pp = part + ((int64_t)(h0 + h) * S + split) * (D + 4);
         pp[dd] = a;
         if (dd == 0) {
             pp[D] = nk > 0 ? s_stat[2 * h] : -INFINITY;
@@ -252,10 +268,11 @@ __global__ __launch_bounds__(D) void k_attn_combine_dl(const float *__restrict__
     out[h * D + threadIdx.x] = num / den;
 }
 
-template <typename TKV, int G>
+template <typename TKV, int G, int NWV>
 static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const void *v, int64_t kv_sh, int64_t kv_st,
-                           int hq, int hkv, float scale, const int *len_dev, int max_len, float *out, int *splits_out) {
-    constexpr int D = 128, NWV = 16;
+                           int hq, int hkv, float scale, const int *len_dev, int max_len, float *out, int *splits_out,
+                           int gtot) {
+    constexpr int D = 128;
     // splits: 8 measured best from a few hundred to a few thousand keys (MI355X); it is also the most the output
     // projection merges while staging its input.  The option allows 4 .. 16.
     int S = dev->opt_attn_splits > 0 ? (int)dev->opt_attn_splits : 8;
@@ -270,8 +287,8 @@ static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const 
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024));
         attr_done = true;
     }
-    k_attn_decode_dl<TKV, D, G, NWV><<<dim3((unsigned)S, (unsigned)hkv), dim3(64 * NWV), lds, dev->stream>>>(
-        q, (const TKV *)k, (const TKV *)v, kv_sh, kv_st, len_dev, scale, chunk_max, max_len, dev->part_buf);
+    k_attn_decode_dl<TKV, D, G, NWV><<<dim3((unsigned)S, (unsigned)hkv, (unsigned)(gtot / G)), dim3(64 * NWV), lds, dev->stream>>>(
+        q, (const TKV *)k, (const TKV *)v, kv_sh, kv_st, len_dev, scale, chunk_max, max_len, gtot, dev->part_buf);
     FH_HIP(hipGetLastError());
     if (splits_out) *splits_out = S;
     if (out) {
@@ -293,18 +310,26 @@ fh_status fh_attention_combine_dl(fh_device *dev, int hq, int splits, float *out
 fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
                                      int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale,
                                      const int *len_dev, int max_len, float *out, int *splits_out) {
-    const int G = hq / hkv;
-    if (d != 128 || (G != 1 && G != 2 && G != 4 && G != 8) || kv_st % 8 || kv_sh % 8) return FH_ERR_UNSUPPORTED;
-#define AD_GO(TKV_)                                                                                                   \
-    switch (G) {                                                                                                      \
-    case 1: return ad_launch<TKV_, 1>(dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out);  \
-    case 2: return ad_launch<TKV_, 2>(dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out);  \
-    case 4: return ad_launch<TKV_, 4>(dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out);  \
-    default: return ad_launch<TKV_, 8>(dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out); \
+    const int gtot = hq / hkv;
+    if (d != 128 || (gtot != 1 && gtot != 2 && gtot != 4 && gtot != 8) || kv_st % 8 || kv_sh % 8) return FH_ERR_UNSUPPORTED;
+    // query heads per workgroup: the arithmetic of a workgroup grows with them, the K and V reads do not; one
+    // (the workgroups of a KV head then share the rows through the L2) measured best on MI355X for 4 heads per KV
+    // head at contexts of some hundred keys: 256 workgroups instead of 64
+    int G = dev->opt_attn_heads > 0 ? (int)dev->opt_attn_heads : 1;
+    while (G > 1 && (gtot % G || (G != 2 && G != 4 && G != 8))) G /= 2;
+    const bool w8 = dev->opt_attn_waves == 8 && G <= 8; // 8 wavefronts per workgroup instead of 16
+#define AD_ARGS dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out, gtot
+#define AD_GO(TKV_)                                                                       \
+    switch (G) {                                                                          \
+    case 1: return w8 ? ad_launch<TKV_, 1, 8>(AD_ARGS) : ad_launch<TKV_, 1, 16>(AD_ARGS); \
+    case 2: return w8 ? ad_launch<TKV_, 2, 8>(AD_ARGS) : ad_launch<TKV_, 2, 16>(AD_ARGS); \
+    case 4: return w8 ? ad_launch<TKV_, 4, 8>(AD_ARGS) : ad_launch<TKV_, 4, 16>(AD_ARGS); \
+    default: return w8 ? ad_launch<TKV_, 8, 8>(AD_ARGS) : ad_launch<TKV_, 8, 16>(AD_ARGS); \
     }
     if (kv_dtype == FH_F16) {
         AD_GO(fh_half)
     }
     AD_GO(float)
 #undef AD_GO
+#undef AD_ARGS
 }

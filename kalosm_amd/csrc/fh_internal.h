@@ -58,6 +58,8 @@ struct fh_device {
     int64_t opt_attn_kernel = 0;     // 0 auto, 1 first-generation kernels only, 2 matrix-core prefill for f32 too
     int64_t opt_down_splitk = 0;     // 0: decode steps split k of a Q6_K down projection (atomic adds), 1: never, 3: and SwiGLU in its staging
     int64_t opt_down_tiles = 0;      // row tiles per wavefront of the accumulating Q6_K down projection (0: 1; 1, 2, 4)
+    int64_t opt_attn_heads = 0;      // query heads per workgroup of the decode attention (0: automatic; 1, 2, 4, 8)
+    int64_t opt_attn_waves = 0;      // wavefronts per workgroup of the decode attention (0: 16; 8)
     int64_t opt_wo_tiles = 0;        // row tiles per wavefront of the accumulating output projection (0: 4; 1, 2, 4)
     int64_t opt_wo_acc = 0;          // 0: decode steps accumulate the output projection into the residual stream, 1: never
     int64_t opt_fuse_norm = 0;       // 0: decode steps fold rms_norm into the consuming matvec, 1: separate launches
