@@ -111,12 +111,8 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
             ad_load8<TKV>(vb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st, vpre[u]);
         }
     }
-#pragma unroll
-    for (int u = 0; u < U; u++)
-        if (u * RW + trow >= nk) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) kpre[u][i] = vpre[u][i] = 0.f;
-        }
+    // (rows past nk hold whatever the cache allocation held: every use below is guarded by the row index)
+    const int niter = (nk + RW - 1) / RW;
     float qr[G][8];
 #pragma unroll
     for (int h = 0; h < G; h++) {
@@ -136,18 +132,19 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
             if (c == 0 && t < nk) s_sc[h * chunk_max + t] = a * scale;
         }
     };
+    // a ring of U rows per lane group: the slot of iteration it is refilled with the row of iteration it + U
+    for (int it0 = 0; it0 < niter; it0 += U) {
 #pragma unroll
-    for (int u = 0; u < U; u++)
-        if (u * RW < nk) score(kpre[u], u * RW + trow);
-    for (int t0 = U * RW; t0 < nk; t0 += RW) {
-        const int t = t0 + trow;
-        float kv8[8];
-        if (t < nk) ad_load8<TKV>(kb + (int64_t)cache_row(t) * kv_st, kv8);
-        else {
-#pragma unroll
-            for (int i = 0; i < 8; i++) kv8[i] = 0.f;
+        for (int u = 0; u < U; u++) {
+            const int it = it0 + u;
+            if (it < niter) {
+                score(kpre[u], it * RW + trow);
+                if ((it + U) * RW < nk) {
+                    const int lr = (it + U) * RW + trow;
+                    ad_load8<TKV>(kb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st, kpre[u]);
+                }
+            }
         }
-        score(kv8, t);
     }
     __syncthreads();
     // ---- softmax statistics: wavefront h owns query head h
@@ -187,15 +184,17 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
             }
         }
     };
+    for (int it0 = 0; it0 < niter; it0 += U) {
 #pragma unroll
-    for (int u = 0; u < U; u++)
-        if (u * RW < nk) accum(vpre[u], u * RW + trow);
-    for (int t0 = U * RW; t0 < nk; t0 += RW) {
-        const int t = t0 + trow;
-        float v8[8];
-        if (t < nk) {
-            ad_load8<TKV>(vb + (int64_t)cache_row(t) * kv_st, v8);
-            accum(v8, t);
+        for (int u = 0; u < U; u++) {
+            const int it = it0 + u;
+            if (it < niter) {
+                accum(vpre[u], it * RW + trow);
+                if ((it + U) * RW < nk) {
+                    const int lr = (it + U) * RW + trow;
+                    ad_load8<TKV>(vb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st, vpre[u]);
+                }
+            }
         }
     }
     // ---- add the row groups of the wavefront, then the wavefronts
