@@ -60,6 +60,7 @@ extern "C" fh_status fh_device_destroy(fh_device *dev) {
     (void)hipStreamSynchronize(dev->stream);
     if (dev->act_buf) (void)hipFree(dev->act_buf);
     if (dev->part_buf) (void)hipFree(dev->part_buf);
+    if (dev->ksplit_buf) (void)hipFree(dev->ksplit_buf);
     if (dev->small_buf) (void)hipFree(dev->small_buf);
     (void)hipEventDestroy(dev->ev_start);
     (void)hipEventDestroy(dev->ev_stop);

@@ -46,6 +46,8 @@ struct fh_device {
     // split-K partial sums
     float *part_buf = nullptr;
     size_t part_cap = 0;
+    float *ksplit_buf = nullptr; // partial planes of a k-split prefill matmul
+    size_t ksplit_cap = 0;
     // 64 KB that never moves: partial results of small reductions (argmax)
     void *small_buf = nullptr;
     // options (fh_set_option)

@@ -331,27 +331,34 @@ __device__ __forceinline__ void qmm_decode_raw(const QmmRaw &r, int g, int ks, f
     }
 }
 
-template <int T, int NTERM>
+// WN x (8 / WN) wavefronts of (32 FN) x (32 FM) outputs each: 128 weight rows x 256, 128 or 64 activation rows.
+template <int T, int NTERM, int WN, int FN, int FM>
 __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__restrict__ xh,
                                                    const _Float16 *__restrict__ xl, const float *__restrict__ rs,
                                                    int m, float *__restrict__ y) {
-    constexpr int TN = 128, TM = 256, FN = 2, FM = 2;
+    constexpr int WM = 8 / WN, TN = WN * FN * 32, TM = WM * FM * 32;
+    static_assert(TN == 128, "512 threads decode 128 weight rows x 4 pieces per step");
+    constexpr int NB = (TM * 4 + 511) / 512; // 16-byte activation pieces per thread, plane and step
     constexpr int A_H = TN * QMM_LDK, B_H = TM * QMM_LDK;         // halfs per plane
     constexpr int BUF = 2 * A_H + NTERM * B_H;                    // halfs per buffer: A hi, A lo, B hi (, B lo)
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int wn = wave >> 2, wm = wave & 3;
+    const int wn = wave / WM, wm = wave % WM;
     const int64_t n0 = (int64_t)blockIdx.x * TN;
     const int m0 = blockIdx.y * TM;
-    const int K = (int)q.k, ksteps = K / 32;
+    // gridDim.z > 1: the k steps are split over workgroups, each writing its partial product to its own [m, n] plane
+    // of y (the host sums the planes); a split holds an even number of steps, so LDS buffer parity is that of ks
+    const int K = (int)q.k, kper = K / 32 / (int)gridDim.z, kbeg = (int)blockIdx.z * kper, ksteps = kbeg + kper;
+    y += (size_t)blockIdx.z * (size_t)m * (size_t)q.n;
     const int64_t tiles16 = (q.n + 15) / 16;
     // this thread's weight duty: row a_row of the tile, lane group a_g (8 weights per step)
     const int a_row = tid >> 2, a_g = tid & 3, a_j = a_row & 15;
     int64_t a_tile = (n0 >> 4) + (a_row >> 4);
     if (a_tile >= tiles16) a_tile = tiles16 - 1; // rows past the end decode a valid tile and are never stored
-    // activation duty: two 16-byte pieces per plane and step
+    // activation duty: NB 16-byte pieces per plane and step
     // piece i (0, 1): row (tid + 512 i) / 4 of the tile, 16-byte column (tid + 512 i) % 4 = tid % 4
-    const int b_c = tid & 3, b_row0 = tid >> 2, b_row1 = b_row0 + 128;
+    // (a 64-row tile has 256 pieces: the upper half of the workgroup repeats the lower half's, same values)
+    const int b_c = tid & 3, b_row0 = (tid >> 2) % TM, b_row1 = (b_row0 + 128) % TM;
     // rows past the end repeat the last one (never stored)
     const int64_t b_off0 = (int64_t)(m0 + b_row0 < m ? m0 + b_row0 : m - 1) * K + b_c * 8;
     const int64_t b_off1 = (int64_t)(m0 + b_row1 < m ? m0 + b_row1 : m - 1) * K + b_c * 8;
@@ -363,10 +370,10 @@ __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__re
     auto fetch = [&](Slab &sl, int ks) {
         qmm_load_raw<T>(q, a_tile, a_j, a_g, ks, sl.raw);
         sl.h0 = *(const uint4 *)(xh + b_off0 + ks * 32);
-        sl.h1 = *(const uint4 *)(xh + b_off1 + ks * 32);
+        sl.h1 = NB == 2 ? *(const uint4 *)(xh + b_off1 + ks * 32) : sl.h0;
         if (NTERM == 2) {
             sl.l0 = *(const uint4 *)(xl + b_off0 + ks * 32);
-            sl.l1 = *(const uint4 *)(xl + b_off1 + ks * 32);
+            sl.l1 = NB == 2 ? *(const uint4 *)(xl + b_off1 + ks * 32) : sl.l0;
         }
     };
     auto stage = [&](const Slab &sl, int ks) {
@@ -390,10 +397,10 @@ __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__re
         *(uint2 *)(buf + A_H + a_row * QMM_LDK + p0) = l0;
         *(uint2 *)(buf + A_H + a_row * QMM_LDK + p1) = l1;
         *(uint4 *)(buf + 2 * A_H + b_row0 * QMM_LDK + b_c * 8) = sl.h0;
-        *(uint4 *)(buf + 2 * A_H + b_row1 * QMM_LDK + b_c * 8) = sl.h1;
+        if (NB == 2) *(uint4 *)(buf + 2 * A_H + b_row1 * QMM_LDK + b_c * 8) = sl.h1;
         if (NTERM == 2) {
             *(uint4 *)(buf + 2 * A_H + B_H + b_row0 * QMM_LDK + b_c * 8) = sl.l0;
-            *(uint4 *)(buf + 2 * A_H + B_H + b_row1 * QMM_LDK + b_c * 8) = sl.l1;
+            if (NB == 2) *(uint4 *)(buf + 2 * A_H + B_H + b_row1 * QMM_LDK + b_c * 8) = sl.l1;
         }
     };
     floatx16 acc[FN][FM];
@@ -404,20 +411,14 @@ __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__re
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
 
-    fetch(s0, 0);
-    if (ksteps > 1) fetch(s1, 1);
-    stage(s0, 0);
-    for (int ks0 = 0; ks0 < ksteps; ks0 += 2) {
-#pragma unroll
-        for (int d = 0; d < 2; d++) { // slot d holds step ks0 + d ... the slot index stays a compile-time constant
-            const int ks = ks0 + d;
+    fetch(s0, kbeg);
+    if (kper > 1) fetch(s1, kbeg + 1);
+    stage(s0, kbeg);
+    // one k step; `mine` is the register set that held step ks (free again), `other` holds step ks + 1
+    auto kstep = [&](int ks, Slab &mine, const Slab &other) {
             if (ks < ksteps) {
                 __syncthreads(); // buffer ks & 1 is complete; the other one is no longer read
-                // raw[d] was consumed by stage(d, ks) in the previous iteration (or the prologue)
-                if (ks + 2 < ksteps) {
-                    if (d == 0) fetch(s0, ks + 2);
-                    else fetch(s1, ks + 2);
-                }
+                if (ks + 2 < ksteps) fetch(mine, ks + 2);
                 const _Float16 *buf = smem + (ks & 1) * BUF;
 #pragma unroll
                 for (int kk = 0; kk < 2; kk++) {
@@ -445,12 +446,12 @@ __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__re
                                 acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[a], blv[b], acc[a][b], 0, 0, 0);
                         }
                 }
-                if (ks + 1 < ksteps) { // the other register set holds step ks + 1
-                    if (d == 0) stage(s1, ks + 1);
-                    else stage(s0, ks + 1);
-                }
+                if (ks + 1 < ksteps) stage(other, ks + 1);
             }
-        }
+    };
+    for (int ks0 = kbeg; ks0 < ksteps; ks0 += 2) { // the register sets alternate: no indexing survives into the code
+        kstep(ks0, s0, s1);
+        kstep(ks0 + 1, s1, s0);
     }
     const bool vec = (q.n & 3) == 0;
 #pragma unroll
@@ -480,32 +481,87 @@ __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__re
     }
 }
 
+// y = sum of the partial planes of a k-split product, in plane order (deterministic)
+__global__ void k_qmm_sum_planes(const float4 *__restrict__ part, int planes, int64_t n4, float4 *__restrict__ y) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    float4 a = part[i];
+    for (int p = 1; p < planes; p++) {
+        const float4 b = part[(int64_t)p * n4 + i];
+        a = make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
+    }
+    y[i] = a;
+}
+
+template <int T, int NTERM, int WN, int FN, int FM>
+static fh_status qmm_launch_tile2(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const float *rs, int m,
+                                  float *y, int ksplit = 1) {
+    constexpr int TM = (8 / WN) * FM * 32;
+    constexpr size_t lds = 2 * (size_t)(2 * 128 * QMM_LDK + NTERM * TM * QMM_LDK) * 2;
+    static bool attr_done = false;
+    if (!attr_done) {
+        FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2<T, NTERM, WN, FN, FM>,
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_done = true;
+    }
+    dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + TM - 1) / TM), (unsigned)ksplit);
+    float *dst = y;
+    if (ksplit > 1) {
+        fh_device *dev = q->dev;
+        FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, (size_t)ksplit * m * q->n * 4));
+        dst = dev->ksplit_buf;
+    }
+    k_qmm_tile2<T, NTERM, WN, FN, FM><<<grid, 512, lds, q->dev->stream>>>(fh_view(q), xh, xl, rs, m, dst);
+    FH_HIP(hipGetLastError());
+    if (ksplit > 1) {
+        const int64_t n4 = (int64_t)m * q->n / 4;
+        k_qmm_sum_planes<<<dim3((unsigned)((n4 + 255) / 256)), 256, 0, q->dev->stream>>>((const float4 *)dst, ksplit, n4,
+                                                                                       (float4 *)y);
+        FH_HIP(hipGetLastError());
+    }
+    return FH_OK;
+}
+
 template <int T, int NTERM>
 static fh_status qmm_launch_t(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const float *rs, int m,
                               float *y) {
     hipStream_t s = q->dev->stream;
     QView v = fh_view(q);
-    // the 128 x 256 kernel when it still fills most of the device (opt_matmul_kernel = 3: never)
-    const int64_t wgs2 = ((q->n + 127) / 128) * ((m + 255) / 256);
-    const int64_t mk = q->dev->opt_matmul_kernel; // 3: never, 4: always
-    if (mk == 4 || (m > 128 && wgs2 * 5 >= (int64_t)q->dev->compute_units * 4 && mk != 3)) {
-        constexpr size_t lds = 2 * (size_t)(2 * 128 * QMM_LDK + NTERM * 256 * QMM_LDK) * 2;
-        static bool attr_done = false;
-        if (!attr_done) {
-            FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2<T, NTERM>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds));
-            attr_done = true;
+    // the pipelined kernel with the tallest activation tile (256, 128, 64 rows) that still fills most of the device
+    // (opt_matmul_kernel = 3: never, 4: always 256)
+    const int64_t tn = (q->n + 127) / 128, cus = q->dev->compute_units;
+    const int64_t mk = q->dev->opt_matmul_kernel;
+    if (mk == 4 || (m > 128 && tn * ((m + 255) / 256) * 5 >= cus * 4 && mk != 3))
+        return qmm_launch_tile2<T, NTERM, 2, 2, 2>(q, xh, xl, rs, m, y);
+    if (m > 64 && mk != 3 && mk != 5) {
+        // too few tiles for the device: split k over workgroups rather than shrink the tile (every tile row of
+        // workgroups decodes the weights again), as long as a split keeps 16 steps; the partial planes are summed
+        // by a second launch
+        const int ksteps = (int)(q->k / 32);
+        auto split_for = [&](int64_t tiles) {
+            int ks = 1;
+            while (tiles * ks * 5 < cus * 4 && ks < 8 && ksteps % (ks * 4) == 0 && ksteps / (ks * 2) >= 16 &&
+                   (q->n & 3) == 0)
+                ks *= 2;
+            return ks;
+        };
+        if (m > 128) {
+            const int ks = split_for(tn * ((m + 255) / 256));
+            if (tn * ((m + 255) / 256) * ks * 5 >= cus * 4) return qmm_launch_tile2<T, NTERM, 2, 2, 2>(q, xh, xl, rs, m, y, ks);
         }
-        dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + 255) / 256));
-        k_qmm_tile2<T, NTERM><<<grid, 512, lds, s>>>(v, xh, xl, rs, m, y);
-        FH_HIP(hipGetLastError());
-        return FH_OK;
+        const int ks = split_for(tn * ((m + 127) / 128));
+        if (tn * ((m + 127) / 128) * ks * 5 >= cus * 4) return qmm_launch_tile2<T, NTERM, 2, 2, 1>(q, xh, xl, rs, m, y, ks);
+        return qmm_launch_tile2<T, NTERM, 4, 1, 1>(q, xh, xl, rs, m, y, split_for(tn * ((m + 63) / 64)));
     }
     if (m <= 32) {
         dim3 grid((unsigned)((q->n + 127) / 128), 1);
         k_qmm_tile<T, NTERM, 4, 1, 1, 1><<<grid, 256, 0, s>>>(v, xh, xl, rs, m, y);
     } else if (m <= 64) {
         dim3 grid((unsigned)((q->n + 127) / 128), 1);
+        k_qmm_tile<T, NTERM, 2, 2, 2, 1><<<grid, 256, 0, s>>>(v, xh, xl, rs, m, y);
+    } else if (((q->n + 127) / 128) * ((m + 127) / 128) < (int64_t)q->dev->compute_units && mk != 5) {
+        // too few 128 x 128 tiles to fill the device: 128 x 64 tiles (the weight slab is decoded twice as often)
+        dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + 63) / 64));
         k_qmm_tile<T, NTERM, 2, 2, 2, 1><<<grid, 256, 0, s>>>(v, xh, xl, rs, m, y);
     } else {
         dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + 127) / 128));

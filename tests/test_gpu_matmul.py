@@ -47,6 +47,28 @@ def test_tile_matmul_f32_vs_checker(dev, oracle, ty, m, n, k):
 
 
 @pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("m,n,k", [(200, 384, 4096), (70, 132, 8192), (512, 4096, 2048), (512, 4096, 4096)])
+def test_tile_matmul_split_k(dev, oracle, ty, m, n, k):
+    """Few output tiles for the device and a long k: the default dispatch splits k over workgroups and sums the
+    partial planes in a second launch (on 256 compute units: 64-row tiles four- and eight-fold, 128-row tiles
+    two-fold, 256-row tiles four-fold); f32 and bf16 activations.  The sum is in plane order, so two runs agree bit
+    for bit.  The large cases are checked on the activation rows around the tile edges."""
+    raw = synth.random_weight(ty, n, k, seed=150 + ty)
+    x = synth.random_activation(m, k, seed=160 + m)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    rows = np.arange(m) if m * n * k < 2 ** 30 else np.array([0, 63, 64, 127, 128, 255, 256, m - 1])
+    got = tile_matmul(dev, x, q, 0)
+    assert_close(got[rows], oracle.q_mat_mul(ty, x[rows], raw, n, fast=True), what=f"{NAMES[ty]} {n}x{k} m={m} split k")
+    assert np.array_equal(got.view(np.uint32), tile_matmul(dev, x, q, 0).view(np.uint32))
+    bits, xb = bf16_round(x)
+    out = Tensor.filled_bytes(dev, (m, n), 0xFF)
+    gb = Tensor.from_slice(dev, bits, dtype="bf16").q_mat_mul(q, out=out).as_slice()
+    assert_close(gb[rows], oracle.q_mat_mul(ty, xb[rows], raw, n, fast=True),
+                 what=f"{NAMES[ty]} {n}x{k} m={m} split k, bf16")
+    assert not np.isnan(gb).any() and not np.isnan(got).any()
+
+
+@pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
 def test_tile_matmul_matches_decode_kernels(dev, oracle, ty):
     """The same product through the decode matvec (row by row) and through the tile kernel."""
     n, k, m = 272, 2048, 40
