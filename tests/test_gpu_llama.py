@@ -78,6 +78,36 @@ def test_decoder_matches_checker(dev, oracle, variant, cfg):
     assert_close(m.forward([want3[-1]]), ref.forward([want3[-1]]), what="logits after 40 device-side steps", **tol)
 
 
+@pytest.mark.parametrize("heads,kv_heads", [(4, 1), (4, 2), (8, 1), (2, 2)], ids=["g4", "g2", "g8", "g1"])
+@pytest.mark.parametrize("opts", [{}, dict(attn_heads=2), dict(attn_heads=4, attn_waves=8), dict(attn_splits=4, wo_tiles=1),
+                                  dict(wo_tiles=2, down_tiles=2, matvec_tiles=2), dict(matvec_per=2, down_tiles=4)],
+                         ids=["default", "heads2", "heads4-waves8", "splits4-wo1", "tiles2", "per2-down4"])
+def test_decode_step_kernel_variants(dev, oracle, heads, kv_heads, opts):
+    """The fused decode step (head_dim 128) with other groupings of query heads per KV head and with the kernel
+    shapes the options select: 70 greedy steps on the device (five granules of 16 keys, so every attention split
+    owns keys and the blind prefetch reads past the length) against the checker's greedy loop, then the logits
+    through the eager path on the cache the device-side steps wrote."""
+    cfg = dict(HD128, n_heads=heads, n_kv_heads=kv_heads, d_model=128 * heads)
+    m, ref = build_pair(dev, oracle, cfg, seed=3)
+    for k, v in opts.items():
+        dev.set_option(k, v)
+    try:
+        prompt = np.random.default_rng(5).integers(0, cfg["vocab"], 11)
+        lg, wl = m.forward(prompt), ref.forward(prompt)
+        assert_close(lg, wl, what="prefill logits")
+        t = int(np.argmax(wl))
+        got, _ = m.decode_greedy(t, 70)
+        want = []
+        for _ in range(70):
+            t = oracle.argmax(ref.forward([t]))
+            want.append(t)
+        assert got.tolist() == want
+        assert_close(m.forward([want[-1]]), ref.forward([want[-1]]), what="logits after 70 device-side steps")
+    finally:
+        for k in opts:
+            dev.set_option(k, 0)
+
+
 def test_decoder_errors(dev):
     from kalosm_amd.fusor import FusorHipError
     m = Model(dev, SMALL)
