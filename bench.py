@@ -70,6 +70,22 @@ def prefill_legs(dev) -> dict:
                 res["matmul"].append({"weights": name, "activations": "Q8_0 per 32 (int8 MFMA)", "m": m, "n": n, "k": k,
                                       "us": round(ms * 1e3, 1), "TOPs": round(tf, 1),
                                       "frac_int8_mfma_peak": round(tf / 5000.0, 4)})
+    # the decoder's own prefill projections with few output tiles (k split over workgroups): f32 activations
+    for ty, name, n2, k2 in ((synth.Q4_K, "Q4_K", 4096, 4096), (synth.Q6_K, "Q6_K", 4096, 14336)):
+        q = QMatrix.from_raw_bytes(dev, (n2, k2), synth.random_weight(ty, n2, k2, seed=9), ty)
+        m = 512
+        xf = Tensor.from_slice(dev, synth.random_activation(m, k2, seed=10))
+        y = Tensor(dev, (m, n2), "f32")
+        for _ in range(2):
+            xf.q_mat_mul(q, out=y)
+        dev.sync()
+        dev.timer_start()
+        for _ in range(5):
+            xf.q_mat_mul(q, out=y)
+        ms = dev.timer_stop() / 5
+        tf = 2.0 * m * n2 * k2 / ms / 1e9
+        res["matmul"].append({"weights": name, "activations": "f32", "m": m, "n": n2, "k": k2, "us": round(ms * 1e3, 1),
+                              "TFLOPs": round(tf, 1), "frac_mfma_peak": round(tf / 2500.0, 4)})
     h, hkv, d = 32, 8, 128
     for s in (512, 2048, 8192):
         rng = np.random.default_rng(s)
