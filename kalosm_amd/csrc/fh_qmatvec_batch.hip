@@ -325,8 +325,8 @@ __global__ __launch_bounds__(512) void k_qmv_batch(QView q, const float *__restr
 #pragma unroll
             for (int r = 0; r < RPW; r++) {
                 const int i = wave + 8 * r, slot = i % TS, m = i / TS, c = rr * TS + slot;
-                xv[r] = (m < M && c < C) ? *(const float4 *)(x + (int64_t)m * K + (int64_t)c * 256 + lane * 4)
-                                         : make_float4(0, 0, 0, 0);
+                // rows past M are not staged and chunks past C not multiplied: their loads repeat the last valid ones
+                xv[r] = *(const float4 *)(x + (int64_t)(m < M ? m : M - 1) * K + (int64_t)(c < C ? c : C - 1) * 256 + lane * 4);
             }
         }
     };
@@ -351,11 +351,14 @@ __global__ __launch_bounds__(512) void k_qmv_batch(QView q, const float *__restr
         return c < C ? c : C - 1; // a slice without a chunk in the last round re-reads the last one and skips the math
     };
     load_x(xr[0], 0);
+    __builtin_amdgcn_sched_barrier(0); // the first activations stay ahead of the weights in the request order
     QbW<T> wr[D];
+    // no branches around the first requests (a wait after a branch becomes a wait for everything in flight): a
+    // slice with fewer than D rounds repeats its last chunk, a single round repeats its activations
 #pragma unroll
-    for (int d = 0; d < D; d++)
-        if (d < R) wr[d].load(q, tile, chunk_of(d), lane);
-    if (R > 1) load_x(xr[1], 1);
+    for (int d = 0; d < D; d++) wr[d].load(q, tile, chunk_of(d < R ? d : R - 1), lane);
+    load_x(xr[1], R > 1 ? 1 : 0);
+    __builtin_amdgcn_sched_barrier(0);
     stage(xr[0], 0);
     float yacc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int r0 = 0; r0 < R; r0 += D) {

@@ -48,7 +48,11 @@ struct Q4kExtra {
 
 #define Q4K_IMG 65 // uint4 per block image: 8 steps x 4 groups x (hi, lo) + one all-zero slot
 
-template <int TPW, int PER, int EPI, int IN>
+// FMT = FH_Q4_0: the same kernel on eight 32-blocks (two records of the tiled Q4_0 layout, 2304 bytes as well) per
+// 256 activations: sub-block s is block s, its scale the block's f16 d, its offset 8 d (gguf/src/lib.rs Q4_0:
+// d * (q - 8)); a byte carries elements i (low nibble) and i + 16 (high nibble), so lane group g multiplies the
+// elements 4g .. 4g+3 and 16+4g .. 16+4g+3 of its block and the staging writes the activations in that order.
+template <int FMT, int TPW, int PER, int EPI, int IN>
 __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict__ x, float *__restrict__ y,
                                                       const float *__restrict__ ea, const float *__restrict__ eb,
                                                       int SW, const float *__restrict__ xres,
@@ -76,10 +80,16 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     const uint8_t *ph[TPW], *pq[TPW];
     if constexpr (HP) {
         const int64_t tile = (int64_t)(blockIdx.x >> 1) + (j < 8 ? 0 : nout / 16);
-        const uint8_t *rec = q.data + (tile * q.recs + boff + b0) * 2304; // per lane: gate or up record
+        // per lane: gate or up record
+        const uint8_t *rec = q.data + tile * q.recs * (FMT == FH_Q4_0 ? 1152 : 2304) + (int64_t)(boff + b0) * 2304;
         const int rr = 8 * (int)(blockIdx.x & 1) + (j & 7);
-        ph[0] = rec + 16 * rr;
-        pq[0] = rec + 256 + (16 * g + rr) * 16;
+        if (FMT == FH_Q4_0) {
+            ph[0] = rec + (g >> 1) * 1152 + 1024 + 8 * rr + 4 * (g & 1);
+            pq[0] = rec + (16 * g + rr) * 16;
+        } else {
+            ph[0] = rec + 16 * rr;
+            pq[0] = rec + 256 + (16 * g + rr) * 16;
+        }
     }
 #pragma unroll
     for (int tp = 0; tp < (HP ? 0 : TPW); tp++) {
@@ -87,9 +97,14 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         const int64_t tile = to + (int64_t)(tp / TOUT) * (nout / 16); // up tiles follow the gate tiles
         // a tile past the end re-reads the last tile (its rows are never stored)
         const int64_t tl = to < tiles_out ? tile : tile - (to - (tiles_out - 1));
-        const uint8_t *rec = q.data + (tl * q.recs + boff + b0) * 2304;
-        ph[tp] = rec + 16 * j;
-        pq[tp] = rec + 256 + lane * 16;
+        const uint8_t *rec = q.data + tl * q.recs * (FMT == FH_Q4_0 ? 1152 : 2304) + (int64_t)(boff + b0) * 2304;
+        if (FMT == FH_Q4_0) { // d of the blocks 2g, 2g+1 of this lane's row; quants of the two records
+            ph[tp] = rec + (g >> 1) * 1152 + 1024 + 8 * j + 4 * (g & 1);
+            pq[tp] = rec + lane * 16;
+        } else {
+            ph[tp] = rec + 16 * j;
+            pq[tp] = rec + 256 + lane * 16;
+        }
     }
 
     // ---- 0. the activations of this wavefront's blocks are requested first: they are needed first and are short
@@ -123,9 +138,15 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     for (int r = 0; r < PER; r++)
 #pragma unroll
         for (int tp = 0; tp < TPW; tp++) {
-            w[tp][r].h = *(const uint4 *)(ph[tp] + r * 2304);
-            w[tp][r].qa = *(const uint4 *)(pq[tp] + r * 2304);
-            w[tp][r].qb = *(const uint4 *)(pq[tp] + r * 2304 + 1024);
+            if (FMT == FH_Q4_0) {
+                w[tp][r].h.x = *(const uint32_t *)(ph[tp] + r * 2304);
+                w[tp][r].qa = *(const uint4 *)(pq[tp] + r * 2304);
+                w[tp][r].qb = *(const uint4 *)(pq[tp] + r * 2304 + 1152);
+            } else {
+                w[tp][r].h = *(const uint4 *)(ph[tp] + r * 2304);
+                w[tp][r].qa = *(const uint4 *)(pq[tp] + r * 2304);
+                w[tp][r].qb = *(const uint4 *)(pq[tp] + r * 2304 + 1024);
+            }
         }
     // ---- 2. stage x (lane owns k = 256*b + 4*lane .. +3).  A wavefront stages exactly the blocks it multiplies:
     // nobody else reads its part of the image, so there is no barrier between this and the products.  (No branch
@@ -165,11 +186,14 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         am = max(am, dpp_u32<DPP_XOR1>(am));
         am = max(am, dpp_u32<DPP_XOR2>(am));
         am = max(am, dpp_u32<DPP_HALF_MIRROR>(am)); // quads are uniform now: lane 7-i is in the other quad
-        const int s = lane >> 3, gg = (lane >> 1) & 3, half = lane & 1;
+        // Q4_K: lanes 2 gg, 2 gg + 1 of a sub-block fill the two halves of operand slot gg; odd sub-blocks are the
+        // high nibbles.  Q4_0: lanes gg and gg + 4 do, the second with the high nibbles' elements.
+        const int s = lane >> 3, gg = FMT == FH_Q4_0 ? lane & 3 : (lane >> 1) & 3;
+        const int half = FMT == FH_Q4_0 ? (lane >> 2) & 1 : lane & 1;
         // e = 14 - floor(log2(amax)) from the exponent field (zero / subnormal / inf / nan just clamp)
         int e = 141 - (int)((am >> 23) & 0xFFu);
         e = e > 100 ? 100 : (e < -100 ? -100 : e);
-        const int eo = e - 4 * (s & 1); // odd sub-blocks meet codes scaled by 16
+        const int eo = e - 4 * (FMT == FH_Q4_0 ? half : s & 1); // high nibbles are codes scaled by 16
         const float sc = __uint_as_float((uint32_t)(eo + 127) << 23);
         const float xq[4] = {v.x, v.y, v.z, v.w};
         _Float16 hi[4], lo[4];
@@ -241,9 +265,15 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
 #pragma unroll
             for (int tp = 0; tp < TPW; tp++) {
                 const uint4 wq = (st & 4) ? w[tp][r].qb : w[tp][r].qa;
-                const uint32_t w0 = (st & 2) ? wq.z : wq.x, w1 = (st & 2) ? wq.w : wq.y;
-                const uint32_t msk = (st & 1) ? HI : LO;
-                const uint4 bo = make_uint4(w0 & msk, (w0 >> 8) & msk, w1 & msk, (w1 >> 8) & msk);
+                uint4 bo;
+                if (FMT == FH_Q4_0) { // one word per block: low nibbles, then high nibbles
+                    const uint32_t w0 = (st & 3) == 0 ? wq.x : ((st & 3) == 1 ? wq.y : ((st & 3) == 2 ? wq.z : wq.w));
+                    bo = make_uint4(w0 & LO, (w0 >> 8) & LO, w0 & HI, (w0 >> 8) & HI);
+                } else {
+                    const uint32_t w0 = (st & 2) ? wq.z : wq.x, w1 = (st & 2) ? wq.w : wq.y;
+                    const uint32_t msk = (st & 1) ? HI : LO;
+                    bo = make_uint4(w0 & msk, (w0 >> 8) & msk, w1 & msk, (w1 >> 8) & msk);
+                }
                 half8 bv;
                 __builtin_memcpy(&bv, &bo, 16);
                 dd[tp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, dd[tp], 0, 0, 0);
@@ -255,6 +285,14 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
 #pragma unroll
         for (int tp = 0; tp < TPW; tp++) {
             const uint4 h = w[tp][r].h;
+            if (FMT == FH_Q4_0) {
+                const float da = fh_h2f((uint16_t)(h.x & 0xFFFF)), db = fh_h2f((uint16_t)(h.x >> 16));
+                acc[tp] = fmaf(dd[tp][0] + dd[tp][1], da * fc.x, acc[tp]);
+                acc[tp] = fmaf(dd[tp][2] + dd[tp][3], db * fc.y, acc[tp]);
+                mins[tp] = fmaf(8.0f * da, sx.x, mins[tp]);
+                mins[tp] = fmaf(8.0f * db, sx.y, mins[tp]);
+                continue;
+            }
             const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
             const uint32_t sc_l = h.y & 0x3F3F3F3Fu, sc_h = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
             const uint32_t mn_l = h.z & 0x3F3F3F3Fu, mn_h = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
@@ -335,11 +373,20 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         const float *__restrict__ eb, int SW, const float *__restrict__ xres, const float *__restrict__ nw, float eps, int nsplit, FhRopeArgs rk
 template <int TPW, int PER, int EPI, int IN>
 __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(Q4K_M1_PARAMS) {
-    qmv_q4k_m1_body<TPW, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
+    qmv_q4k_m1_body<FH_Q4_K, TPW, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
 template <int TPW, int PER, int EPI, int IN>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_qmv_q4k_m1_w8(Q4K_M1_PARAMS) {
-    qmv_q4k_m1_body<TPW, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
+    qmv_q4k_m1_body<FH_Q4_K, TPW, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
+}
+// Q4_0 weights (plain input; epilogues none / add2 / SwiGLU)
+template <int TPW, int PER, int EPI>
+__global__ __launch_bounds__(1024) void k_qmv_q40_m1(Q4K_M1_PARAMS) {
+    qmv_q4k_m1_body<FH_Q4_0, TPW, PER, EPI, 0>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
+}
+template <int TPW, int PER, int EPI>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_qmv_q40_m1_w8(Q4K_M1_PARAMS) {
+    qmv_q4k_m1_body<FH_Q4_0, TPW, PER, EPI, 0>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
 
 template <int TPW, int PER, int EPI>
@@ -349,6 +396,24 @@ static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, co
                            float, int, FhRopeArgs);
     kern_t kern;
     const int in = ex.nsplit > 0 ? 2 : (ex.nw ? 1 : 0); // input: plain, rms_norm, attention partials
+    if (q->type == FH_Q4_0) {
+        if constexpr (EPI == FH_EPI_NONE || EPI == FH_EPI_ADD2 || EPI == FH_EPI_SWIGLU) {
+            if (in != 0) return FH_ERR_UNSUPPORTED;
+            if constexpr (TPW * PER <= 2) kern = k_qmv_q40_m1_w8<TPW, PER, EPI>;
+            else kern = k_qmv_q40_m1<TPW, PER, EPI>;
+            static bool attr40 = false;
+            if (!attr40) {
+                FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+                attr40 = true;
+            }
+            kern<<<dim3(grid, 1), dim3(64 * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, nullptr, nullptr, 0.f, 0,
+                                                                        ex.rk);
+            FH_HIP(hipGetLastError());
+            return FH_OK;
+        } else {
+            return FH_ERR_UNSUPPORTED;
+        }
+    }
     if constexpr (TPW * PER <= 2) {
         kern = in == 2 ? k_qmv_q4k_m1<TPW, PER, EPI, 2>
                        : (in == 1 ? k_qmv_q4k_m1_w8<TPW, PER, EPI, 1> : k_qmv_q4k_m1_w8<TPW, PER, EPI, 0>);
@@ -443,8 +508,10 @@ fh_status fh_launch_q4k_m1_ropekv(const fh_qmatrix *q, const float *x, const flo
 static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra &ex, float *y, int epi, const float *a,
                             const float *b) {
     fh_device *dev = q->dev;
-    if (ex.ksplit < 1 || q->kb % ex.ksplit || (ex.ksplit > 1 && (epi != FH_EPI_ACC || ex.nw))) return FH_ERR_UNSUPPORTED;
-    const int kb = (int)q->kb / ex.ksplit; // blocks per workgroup
+    if (q->type != FH_Q4_K && !(q->type == FH_Q4_0 && q->k % 256 == 0 && ex.ksplit == 1)) return FH_ERR_UNSUPPORTED;
+    const int64_t kb256 = q->k / 256; // 256-element blocks (Q4_0: eight of its 32-blocks, two records)
+    if (ex.ksplit < 1 || kb256 % ex.ksplit || (ex.ksplit > 1 && (epi != FH_EPI_ACC || ex.nw))) return FH_ERR_UNSUPPORTED;
+    const int kb = (int)kb256 / ex.ksplit; // blocks per workgroup
     const int nt = epi == FH_EPI_SWIGLU ? 2 : 1;
     const int64_t nout = epi == FH_EPI_SWIGLU ? q->n / 2 : q->n;
     const int64_t tiles = (nout + 15) / 16;
