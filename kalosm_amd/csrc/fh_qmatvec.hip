@@ -356,7 +356,7 @@ fh_status fh_launch_qmatvec(const fh_qmatrix *q, const float *x, int m, float *y
     if (epi == FH_EPI_SWIGLU) FH_REQUIRE(q->n % 32 == 0, "SwiGLU epilogue needs n %% 32 == 0 (n = %lld)", (long long)q->n);
     int kernel = (int)dev->opt_matvec_kernel;
     if (kernel == 4 && fh_qmatvec_batch_supports(q, m, epi)) return fh_launch_qmatvec_batch(q, x, m, y, epi, a, b);
-    if (kernel != 1 && kernel != 3 && (q->type == FH_Q4_K || (q->type == FH_Q4_0 && q->k % 256 == 0)) && m == 1) {
+    if (kernel != 1 && kernel != 3 && (q->type == FH_Q4_K || ((q->type == FH_Q4_0 || q->type == FH_Q8_0) && q->k % 256 == 0)) && m == 1) {
         fh_status st = fh_launch_q4k_m1(q, x, y, epi, a, b);
         if (st != FH_ERR_UNSUPPORTED) return st;
     }

@@ -24,7 +24,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 struct Q4KRegs {
-    uint4 h, qa, qb;
+    uint4 h, qa, qb, qc, qd; // qc, qd: Q8_0 only (four records per 256 activations)
 };
 
 // Arguments of the rope + KV-append epilogue (the fused q|k|v projection of a decode step): rows [0, qd) are query
@@ -52,6 +52,9 @@ struct Q4kExtra {
 // 256 activations: sub-block s is block s, its scale the block's f16 d, its offset 8 d (gguf/src/lib.rs Q4_0:
 // d * (q - 8)); a byte carries elements i (low nibble) and i + 16 (high nibble), so lane group g multiplies the
 // elements 4g .. 4g+3 and 16+4g .. 16+4g+3 of its block and the staging writes the activations in that order.
+// FMT = FH_Q8_0: eight 32-blocks = four records of 1088 bytes; a code byte q becomes the f16 1152 + q (xor 0x80,
+// then v_perm_b32 sets it under the high byte 0x64: 1024 + (q + 128) exactly), so the offset is 1152 d and the
+// activation factor carries no 2^24.
 template <int FMT, int TPW, int PER, int EPI, int IN>
 __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict__ x, float *__restrict__ y,
                                                       const float *__restrict__ ea, const float *__restrict__ eb,
@@ -77,14 +80,19 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     const int64_t nout = EPI == FH_EPI_SWIGLU ? q.n / 2 : q.n;
     const int64_t tiles_out = (nout + 15) / 16;
     const int b0 = wave * PER;
+    constexpr int REC = FMT == FH_Q4_0 ? 1152 : (FMT == FH_Q8_0 ? 1088 : 2304); // bytes of a tiled record
+    constexpr int CHUNK = FMT == FH_Q8_0 ? 4352 : 2304;                          // bytes per 256 activations and tile
     const uint8_t *ph[TPW], *pq[TPW];
     if constexpr (HP) {
         const int64_t tile = (int64_t)(blockIdx.x >> 1) + (j < 8 ? 0 : nout / 16);
         // per lane: gate or up record
-        const uint8_t *rec = q.data + tile * q.recs * (FMT == FH_Q4_0 ? 1152 : 2304) + (int64_t)(boff + b0) * 2304;
+        const uint8_t *rec = q.data + tile * q.recs * REC + (int64_t)(boff + b0) * CHUNK;
         const int rr = 8 * (int)(blockIdx.x & 1) + (j & 7);
         if (FMT == FH_Q4_0) {
             ph[0] = rec + (g >> 1) * 1152 + 1024 + 8 * rr + 4 * (g & 1);
+            pq[0] = rec + (16 * g + rr) * 16;
+        } else if (FMT == FH_Q8_0) {
+            ph[0] = rec + g * 1088 + 1024 + 4 * rr;
             pq[0] = rec + (16 * g + rr) * 16;
         } else {
             ph[0] = rec + 16 * rr;
@@ -97,9 +105,12 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         const int64_t tile = to + (int64_t)(tp / TOUT) * (nout / 16); // up tiles follow the gate tiles
         // a tile past the end re-reads the last tile (its rows are never stored)
         const int64_t tl = to < tiles_out ? tile : tile - (to - (tiles_out - 1));
-        const uint8_t *rec = q.data + tl * q.recs * (FMT == FH_Q4_0 ? 1152 : 2304) + (int64_t)(boff + b0) * 2304;
+        const uint8_t *rec = q.data + tl * q.recs * REC + (int64_t)(boff + b0) * CHUNK;
         if (FMT == FH_Q4_0) { // d of the blocks 2g, 2g+1 of this lane's row; quants of the two records
             ph[tp] = rec + (g >> 1) * 1152 + 1024 + 8 * j + 4 * (g & 1);
+            pq[tp] = rec + lane * 16;
+        } else if (FMT == FH_Q8_0) { // record g holds the blocks 2g, 2g+1
+            ph[tp] = rec + g * 1088 + 1024 + 4 * j;
             pq[tp] = rec + lane * 16;
         } else {
             ph[tp] = rec + 16 * j;
@@ -142,6 +153,12 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
                 w[tp][r].h.x = *(const uint32_t *)(ph[tp] + r * 2304);
                 w[tp][r].qa = *(const uint4 *)(pq[tp] + r * 2304);
                 w[tp][r].qb = *(const uint4 *)(pq[tp] + r * 2304 + 1152);
+            } else if (FMT == FH_Q8_0) {
+                w[tp][r].h.x = *(const uint32_t *)(ph[tp] + r * 4352);
+                w[tp][r].qa = *(const uint4 *)(pq[tp] + r * 4352);
+                w[tp][r].qb = *(const uint4 *)(pq[tp] + r * 4352 + 1088);
+                w[tp][r].qc = *(const uint4 *)(pq[tp] + r * 4352 + 2176);
+                w[tp][r].qd = *(const uint4 *)(pq[tp] + r * 4352 + 3264);
             } else {
                 w[tp][r].h = *(const uint4 *)(ph[tp] + r * 2304);
                 w[tp][r].qa = *(const uint4 *)(pq[tp] + r * 2304);
@@ -193,7 +210,7 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         // e = 14 - floor(log2(amax)) from the exponent field (zero / subnormal / inf / nan just clamp)
         int e = 141 - (int)((am >> 23) & 0xFFu);
         e = e > 100 ? 100 : (e < -100 ? -100 : e);
-        const int eo = e - 4 * (FMT == FH_Q4_0 ? half : s & 1); // high nibbles are codes scaled by 16
+        const int eo = e - (FMT == FH_Q8_0 ? 0 : 4 * (FMT == FH_Q4_0 ? half : s & 1)); // high nibbles: codes x 16
         const float sc = __uint_as_float((uint32_t)(eo + 127) << 23);
         const float xq[4] = {v.x, v.y, v.z, v.w};
         _Float16 hi[4], lo[4];
@@ -216,7 +233,7 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         s4 += dpp_f32<DPP_HALF_MIRROR>(s4);
         if ((lane & 7) == 0) {
             sf[b * 16 + s] = s4;
-            sf[b * 16 + 8 + s] = __uint_as_float((uint32_t)(24 - e + 127) << 23);
+            sf[b * 16 + 8 + s] = __uint_as_float((uint32_t)((FMT == FH_Q8_0 ? 0 : 24) - e + 127) << 23);
         }
     }
     if (IN == 1) {
@@ -264,9 +281,15 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
             __builtin_memcpy(&av, &ao, 16);
 #pragma unroll
             for (int tp = 0; tp < TPW; tp++) {
-                const uint4 wq = (st & 4) ? w[tp][r].qb : w[tp][r].qa;
+                const uint4 wq = FMT == FH_Q8_0 ? ((st >> 1) == 0 ? w[tp][r].qa : ((st >> 1) == 1 ? w[tp][r].qb : ((st >> 1) == 2 ? w[tp][r].qc : w[tp][r].qd)))
+                                                 : ((st & 4) ? w[tp][r].qb : w[tp][r].qa);
                 uint4 bo;
-                if (FMT == FH_Q4_0) { // one word per block: low nibbles, then high nibbles
+                if (FMT == FH_Q8_0) { // eight code bytes of block st -> f16 1152 + q, pairs in the order of the staging
+                    const uint32_t c0 = ((st & 1) ? wq.z : wq.x) ^ 0x80808080u, c1 = ((st & 1) ? wq.w : wq.y) ^ 0x80808080u;
+                    const uint32_t k64 = 0x64646464u;
+                    bo = make_uint4(__builtin_amdgcn_perm(k64, c0, 0x04020400u), __builtin_amdgcn_perm(k64, c0, 0x04030401u),
+                                    __builtin_amdgcn_perm(k64, c1, 0x04020400u), __builtin_amdgcn_perm(k64, c1, 0x04030401u));
+                } else if (FMT == FH_Q4_0) { // one word per block: low nibbles, then high nibbles
                     const uint32_t w0 = (st & 3) == 0 ? wq.x : ((st & 3) == 1 ? wq.y : ((st & 3) == 2 ? wq.z : wq.w));
                     bo = make_uint4(w0 & LO, (w0 >> 8) & LO, w0 & HI, (w0 >> 8) & HI);
                 } else {
@@ -285,12 +308,13 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
 #pragma unroll
         for (int tp = 0; tp < TPW; tp++) {
             const uint4 h = w[tp][r].h;
-            if (FMT == FH_Q4_0) {
+            if (FMT == FH_Q4_0 || FMT == FH_Q8_0) {
+                const float off = FMT == FH_Q8_0 ? 1152.0f : 8.0f;
                 const float da = fh_h2f((uint16_t)(h.x & 0xFFFF)), db = fh_h2f((uint16_t)(h.x >> 16));
                 acc[tp] = fmaf(dd[tp][0] + dd[tp][1], da * fc.x, acc[tp]);
                 acc[tp] = fmaf(dd[tp][2] + dd[tp][3], db * fc.y, acc[tp]);
-                mins[tp] = fmaf(8.0f * da, sx.x, mins[tp]);
-                mins[tp] = fmaf(8.0f * db, sx.y, mins[tp]);
+                mins[tp] = fmaf(off * da, sx.x, mins[tp]);
+                mins[tp] = fmaf(off * db, sx.y, mins[tp]);
                 continue;
             }
             const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
@@ -379,14 +403,14 @@ template <int TPW, int PER, int EPI, int IN>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_qmv_q4k_m1_w8(Q4K_M1_PARAMS) {
     qmv_q4k_m1_body<FH_Q4_K, TPW, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
-// Q4_0 weights (plain input; epilogues none / add2 / SwiGLU)
-template <int TPW, int PER, int EPI>
+// Q4_0 / Q8_0 weights (plain input; epilogues none / add2 / SwiGLU)
+template <int FMT, int TPW, int PER, int EPI>
 __global__ __launch_bounds__(1024) void k_qmv_q40_m1(Q4K_M1_PARAMS) {
-    qmv_q4k_m1_body<FH_Q4_0, TPW, PER, EPI, 0>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
+    qmv_q4k_m1_body<FMT, TPW, PER, EPI, 0>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
-template <int TPW, int PER, int EPI>
+template <int FMT, int TPW, int PER, int EPI>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_qmv_q40_m1_w8(Q4K_M1_PARAMS) {
-    qmv_q4k_m1_body<FH_Q4_0, TPW, PER, EPI, 0>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
+    qmv_q4k_m1_body<FMT, TPW, PER, EPI, 0>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
 
 template <int TPW, int PER, int EPI>
@@ -396,15 +420,20 @@ static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, co
                            float, int, FhRopeArgs);
     kern_t kern;
     const int in = ex.nsplit > 0 ? 2 : (ex.nw ? 1 : 0); // input: plain, rms_norm, attention partials
-    if (q->type == FH_Q4_0) {
+    if (q->type == FH_Q4_0 || q->type == FH_Q8_0) {
         if constexpr (EPI == FH_EPI_NONE || EPI == FH_EPI_ADD2 || EPI == FH_EPI_SWIGLU) {
             if (in != 0) return FH_ERR_UNSUPPORTED;
-            if constexpr (TPW * PER <= 2) kern = k_qmv_q40_m1_w8<TPW, PER, EPI>;
-            else kern = k_qmv_q40_m1<TPW, PER, EPI>;
-            static bool attr40 = false;
-            if (!attr40) {
+            const bool q8 = q->type == FH_Q8_0;
+            if constexpr (TPW * PER <= 2) { // Q8_0 holds 17 registers of weights per block tile: one fits the budget
+                if constexpr (TPW * PER == 1) kern = q8 ? k_qmv_q40_m1_w8<FH_Q8_0, TPW, PER, EPI> : k_qmv_q40_m1_w8<FH_Q4_0, TPW, PER, EPI>;
+                else kern = q8 ? k_qmv_q40_m1<FH_Q8_0, TPW, PER, EPI> : k_qmv_q40_m1_w8<FH_Q4_0, TPW, PER, EPI>;
+            } else {
+                kern = q8 ? k_qmv_q40_m1<FH_Q8_0, TPW, PER, EPI> : k_qmv_q40_m1<FH_Q4_0, TPW, PER, EPI>;
+            }
+            static bool attr40[2] = {false, false};
+            if (!attr40[q8]) {
                 FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-                attr40 = true;
+                attr40[q8] = true;
             }
             kern<<<dim3(grid, 1), dim3(64 * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, nullptr, nullptr, 0.f, 0,
                                                                         ex.rk);
@@ -508,7 +537,8 @@ fh_status fh_launch_q4k_m1_ropekv(const fh_qmatrix *q, const float *x, const flo
 static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra &ex, float *y, int epi, const float *a,
                             const float *b) {
     fh_device *dev = q->dev;
-    if (q->type != FH_Q4_K && !(q->type == FH_Q4_0 && q->k % 256 == 0 && ex.ksplit == 1)) return FH_ERR_UNSUPPORTED;
+    if (q->type != FH_Q4_K && !((q->type == FH_Q4_0 || q->type == FH_Q8_0) && q->k % 256 == 0 && ex.ksplit == 1))
+        return FH_ERR_UNSUPPORTED;
     const int64_t kb256 = q->k / 256; // 256-element blocks (Q4_0: eight of its 32-blocks, two records)
     if (ex.ksplit < 1 || kb256 % ex.ksplit || (ex.ksplit > 1 && (epi != FH_EPI_ACC || ex.nw))) return FH_ERR_UNSUPPORTED;
     const int kb = (int)kb256 / ex.ksplit; // blocks per workgroup
