@@ -62,6 +62,7 @@ struct fh_device {
     int64_t opt_down_tiles = 0;      // row tiles per wavefront of the accumulating Q6_K down projection (0: 1; 1, 2, 4)
     int64_t opt_attn_heads = 0;      // query heads per workgroup of the decode attention (0: automatic; 1, 2, 4, 8)
     int64_t opt_attn_waves = 0;      // wavefronts per workgroup of the decode attention (0: 16; 8)
+    int64_t opt_matvec_rows = 0;     // 1: 2 .. 4 activation rows never through the single-row Q4_K kernel's row variant
     int64_t opt_wo_tiles = 0;        // row tiles per wavefront of the accumulating output projection (0: 4; 1, 2, 4)
     int64_t opt_wo_acc = 0;          // 0: decode steps accumulate the output projection into the residual stream, 1: never
     int64_t opt_fuse_norm = 0;       // 0: decode steps fold rms_norm into the consuming matvec, 1: separate launches
@@ -154,6 +155,7 @@ fh_status fh_launch_qmatvec_batch(const fh_qmatrix *q, const float *x, int m, fl
 fh_status fh_launch_qmm_q8_mfma(const fh_qmatrix *q, const float *x, int m, float *y);
 fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y);
 enum { FH_EPI_NONE = 0, FH_EPI_ADD2 = 1, FH_EPI_SWIGLU = 2, FH_EPI_ROPEKV = 3, FH_EPI_ACC = 4 };
+fh_status fh_launch_q4k_rows(const fh_qmatrix *q, const float *x, int m, float *y, int epi, const float *a, const float *b);
 fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b);
 fh_status fh_launch_q4k_m1_norm(const fh_qmatrix *q, const float *x, const float *xres, const float *nw, float eps,
                                 float *y, int epi, const float *a, const float *b);

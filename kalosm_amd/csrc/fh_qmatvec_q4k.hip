@@ -55,12 +55,17 @@ struct Q4kExtra {
 // FMT = FH_Q8_0: eight 32-blocks = four records of 1088 bytes; a code byte q becomes the f16 1152 + q (xor 0x80,
 // then v_perm_b32 sets it under the high byte 0x64: 1024 + (q + 128) exactly), so the offset is 1152 d and the
 // activation factor carries no 2^24.
-template <int FMT, int TPW, int PER, int EPI, int IN>
+// MR > 1: MR activation rows (nsplit then carries the number of valid ones; plain input, epilogues none / add2):
+// the weights are unpacked once per step and multiplied with the operand of every row; a wavefront stages its
+// blocks of all rows, images interleaved [block][row] so that every operand address is the base plus a constant.
+template <int FMT, int TPW, int PER, int EPI, int IN, int MR = 1>
 __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict__ x, float *__restrict__ y,
                                                       const float *__restrict__ ea, const float *__restrict__ eb,
                                                       int SW, const float *__restrict__ xres,
                                                       const float *__restrict__ nw, float eps, int nsplit,
                                                       FhRopeArgs rk) {
+    static_assert(MR == 1 || (IN == 0 && (EPI == FH_EPI_NONE || EPI == FH_EPI_ADD2)), "rows: plain input, none / add2");
+    static_assert(MR == 1 || MR == 2 || MR == 4, "rows per launch");
     // SwiGLU with one tile per wavefront: the "tile" is rows 8h .. 8h+7 of a gate tile (columns 0-7 of the MFMA) and
     // the same rows of the matching up tile (columns 8-15), h = workgroup parity: workgroups half as heavy as with a
     // whole gate and a whole up tile, which divides the Llama FFN evenly over the compute units
@@ -71,9 +76,9 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     // gridDim.y > 1: k is split over workgroups (blocks [boff, boff + kb) here) that add into y with atomics
     const int kb = SW * PER, boff = (int)blockIdx.y * kb; // the host launches with SW * PER * gridDim.y == q.kb
     uint4 *img = lds;
-    float *sf = (float *)(lds + kb * Q4K_IMG); // per block: [0..7] group sums, [8..15] factors
-    float *l_red = sf + kb * 16;               // [TPW][SW][16]
-    float *l_ss = l_red + TPW * 16 * 16;       // per wavefront: sum of squares of the blocks it staged
+    float *sf = (float *)(lds + kb * MR * Q4K_IMG); // per block and row: [0..7] group sums, [8..15] factors
+    float *l_red = sf + kb * MR * 16;               // [MR][TPW][SW][16]
+    float *l_ss = l_red + MR * TPW * 16 * 16;       // per wavefront: sum of squares of the blocks it staged
     const int tid = threadIdx.x, lane = tid & 63, j = lane & 15, g = lane >> 4;
     // the wavefront index as a scalar: everything derived from it (record addresses) stays on the scalar unit
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -121,12 +126,15 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     // ---- 0. the activations of this wavefront's blocks are requested first: they are needed first and are short
     // With nw the input is rms_norm(x [+ xres]) * nw (composite/normalization.rs:287-401): the weight nw is
     // folded into the staged values and the common factor 1 / rms is applied to the finished dot product.
-    float4 xv[PER], rv[PER], wv[PER], pacc[IN == 2 ? PER : 1][8];
+    float4 xv[PER * MR], rv[PER], wv[PER], pacc[IN == 2 ? PER : 1][8];
     float2 pm[IN == 2 ? PER : 1][8];
 #pragma unroll
     for (int i = 0; i < PER; i++) {
         const int64_t at = (int64_t)(boff + b0 + i) * 256 + lane * 4;
         if (IN != 2) xv[i] = *(const float4 *)(x + at);
+#pragma unroll
+        for (int mr = 1; mr < MR; mr++) // rows past the valid ones repeat the last (never stored)
+            xv[mr * PER + i] = *(const float4 *)(x + (int64_t)(mr < nsplit ? mr : nsplit - 1) * q.k + at);
         if (IN == 1 && xres) rv[i] = *(const float4 *)(xres + at);
         if (IN == 1) wv[i] = *(const float4 *)(nw + at);
         if (IN == 2) { // x holds attention partials [head][nsplit][128 + 4]: unnormalised output, max, sum
@@ -170,9 +178,10 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     // around it either: the compiler would sink the activation loads into it, behind the weight loads.)
     float ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < PER; i++) {
-        const int b = b0 + i;
-        float4 v = xv[i];
+    for (int ii = 0; ii < PER * MR; ii++) {
+        const int i = ii % PER;
+        const int b = (b0 + i) * MR + ii / PER; // image index: [block][row]
+        float4 v = xv[ii];
         if (IN == 2) { // merge the splits: softmax weights exp(m_s - max), then num / den
             float mx = -INFINITY;
 #pragma unroll
@@ -250,35 +259,47 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     // Lanes with (lane >> 1) % 8 == st are bits 2 st, 2 st + 1 of every 16.
     uint32_t pa[8];
     {
-        const uint32_t own = lds_addr(img + b0 * Q4K_IMG + (mysb * 4 + g) * 2 + part);
-        const uint32_t zero = lds_addr(img + b0 * Q4K_IMG + 64);
+        const uint32_t own = lds_addr(img + b0 * MR * Q4K_IMG + (mysb * 4 + g) * 2 + part);
+        const uint32_t zero = lds_addr(img + b0 * MR * Q4K_IMG + 64);
 #pragma unroll
         for (int st = 0; st < 8; st++) pa[st] = sel_lanes(0x0003000300030003ull << (2 * st), own, zero);
     }
     // the operands do not depend on the weights: RING of them are always on their way from the LDS
     constexpr int RING = 4;
     uint4 ring[RING];
+    // operand number t = (block r, step st, row mr) in the order of use; its image is (r * MR + mr) after the base
+    auto operand = [&](int t) {
+        const int mr = t % MR, st = (t / MR) % 8, r = t / (8 * MR);
+        return lds_read16(pa[st] + (r * MR + mr) * Q4K_IMG * 16);
+    };
 #pragma unroll
-    for (int t = 0; t < RING; t++) ring[t] = lds_read16(pa[t % 8] + (t / 8) * Q4K_IMG * 16);
-    const float *psf = sf + b0 * 16 + 2 * g;
+    for (int t = 0; t < RING; t++) ring[t] = operand(t);
+    const float *psf = sf + b0 * MR * 16 + 2 * g;
     const uint32_t LO = 0x000F000Fu, HI = 0x00F000F0u;
     // lane group g applies sub-blocks 2g, 2g+1: bytes (g&1)*2, +1 of the low (g < 2) or high (g >= 2) scale word
     const uint32_t selhi = (g & 2) ? 0xFFFFFFFFu : 0u;
     const int sh = (g & 1) * 16;
-    float acc[TPW], mins[TPW];
+    float acc[TPW][MR], mins[TPW][MR];
 #pragma unroll
-    for (int tp = 0; tp < TPW; tp++) acc[tp] = mins[tp] = 0.f;
+    for (int tp = 0; tp < TPW; tp++)
+#pragma unroll
+        for (int mr = 0; mr < MR; mr++) acc[tp][mr] = mins[tp][mr] = 0.f;
 #pragma unroll
     for (int r = 0; r < PER; r++) {
-        floatx4 dd[TPW];
+        floatx4 dd[TPW][MR];
 #pragma unroll
-        for (int tp = 0; tp < TPW; tp++) dd[tp] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int tp = 0; tp < TPW; tp++)
+#pragma unroll
+            for (int mr = 0; mr < MR; mr++) dd[tp][mr] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int st = 0; st < 8; st++) {
-            const int t = r * 8 + st;
-            const uint4 ao = ring[t % RING];
-            half8 av;
-            __builtin_memcpy(&av, &ao, 16);
+            const int t = (r * 8 + st) * MR;
+            half8 av[MR];
+#pragma unroll
+            for (int mr = 0; mr < MR; mr++) {
+                const uint4 ao = ring[(t + mr) % RING];
+                __builtin_memcpy(&av[mr], &ao, 16);
+            }
 #pragma unroll
             for (int tp = 0; tp < TPW; tp++) {
                 const uint4 wq = FMT == FH_Q8_0 ? ((st >> 1) == 0 ? w[tp][r].qa : ((st >> 1) == 1 ? w[tp][r].qb : ((st >> 1) == 2 ? w[tp][r].qc : w[tp][r].qd)))
@@ -299,49 +320,58 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
                 }
                 half8 bv;
                 __builtin_memcpy(&bv, &bo, 16);
-                dd[tp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, dd[tp], 0, 0, 0);
+#pragma unroll
+                for (int mr = 0; mr < MR; mr++)
+                    dd[tp][mr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[mr], bv, dd[tp][mr], 0, 0, 0);
             }
-            if (t + RING < PER * 8) ring[t % RING] = lds_read16(pa[(t + RING) % 8] + ((t + RING) / 8) * Q4K_IMG * 16);
+#pragma unroll
+            for (int mr = 0; mr < MR; mr++)
+                if (t + mr + RING < PER * 8 * MR) ring[(t + mr) % RING] = operand(t + mr + RING);
         }
-        const float2 sx = *(const float2 *)(psf + r * 16);
-        const float2 fc = *(const float2 *)(psf + r * 16 + 8);
+#pragma unroll
+        for (int mr = 0; mr < MR; mr++) {
+            const float2 sx = *(const float2 *)(psf + (r * MR + mr) * 16);
+            const float2 fc = *(const float2 *)(psf + (r * MR + mr) * 16 + 8);
+#pragma unroll
+            for (int tp = 0; tp < TPW; tp++) {
+                const uint4 h = w[tp][r].h;
+                if (FMT == FH_Q4_0 || FMT == FH_Q8_0) {
+                    const float off = FMT == FH_Q8_0 ? 1152.0f : 8.0f;
+                    const float da = fh_h2f((uint16_t)(h.x & 0xFFFF)), db = fh_h2f((uint16_t)(h.x >> 16));
+                    acc[tp][mr] = fmaf(dd[tp][mr][0] + dd[tp][mr][1], da * fc.x, acc[tp][mr]);
+                    acc[tp][mr] = fmaf(dd[tp][mr][2] + dd[tp][mr][3], db * fc.y, acc[tp][mr]);
+                    mins[tp][mr] = fmaf(off * da, sx.x, mins[tp][mr]);
+                    mins[tp][mr] = fmaf(off * db, sx.y, mins[tp][mr]);
+                    continue;
+                }
+                const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
+                const uint32_t sc_l = h.y & 0x3F3F3F3Fu, sc_h = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
+                const uint32_t mn_l = h.z & 0x3F3F3F3Fu, mn_h = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
+                const uint32_t scw = ((sc_l & ~selhi) | (sc_h & selhi)) >> sh;
+                const uint32_t mnw = ((mn_l & ~selhi) | (mn_h & selhi)) >> sh;
+                const float sca = (float)(scw & 0xFFu), scb = (float)((scw >> 8) & 0xFFu);
+                const float mna = (float)(mnw & 0xFFu), mnb = (float)((mnw >> 8) & 0xFFu);
+                const float sa = (sca * d) * fc.x, sb = (scb * d) * fc.y;
+                acc[tp][mr] = fmaf(dd[tp][mr][0] + dd[tp][mr][1], sa, acc[tp][mr]);
+                acc[tp][mr] = fmaf(dd[tp][mr][2] + dd[tp][mr][3], sb, acc[tp][mr]);
+                mins[tp][mr] = fmaf(mna * dmin, sx.x, mins[tp][mr]);
+                mins[tp][mr] = fmaf(mnb * dmin, sx.y, mins[tp][mr]);
+            }
+        }
+    }
+#pragma unroll
+    for (int mr = 0; mr < MR; mr++)
 #pragma unroll
         for (int tp = 0; tp < TPW; tp++) {
-            const uint4 h = w[tp][r].h;
-            if (FMT == FH_Q4_0 || FMT == FH_Q8_0) {
-                const float off = FMT == FH_Q8_0 ? 1152.0f : 8.0f;
-                const float da = fh_h2f((uint16_t)(h.x & 0xFFFF)), db = fh_h2f((uint16_t)(h.x >> 16));
-                acc[tp] = fmaf(dd[tp][0] + dd[tp][1], da * fc.x, acc[tp]);
-                acc[tp] = fmaf(dd[tp][2] + dd[tp][3], db * fc.y, acc[tp]);
-                mins[tp] = fmaf(off * da, sx.x, mins[tp]);
-                mins[tp] = fmaf(off * db, sx.y, mins[tp]);
-                continue;
-            }
-            const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
-            const uint32_t sc_l = h.y & 0x3F3F3F3Fu, sc_h = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
-            const uint32_t mn_l = h.z & 0x3F3F3F3Fu, mn_h = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
-            const uint32_t scw = ((sc_l & ~selhi) | (sc_h & selhi)) >> sh;
-            const uint32_t mnw = ((mn_l & ~selhi) | (mn_h & selhi)) >> sh;
-            const float sca = (float)(scw & 0xFFu), scb = (float)((scw >> 8) & 0xFFu);
-            const float mna = (float)(mnw & 0xFFu), mnb = (float)((mnw >> 8) & 0xFFu);
-            const float sa = (sca * d) * fc.x, sb = (scb * d) * fc.y;
-            acc[tp] = fmaf(dd[tp][0] + dd[tp][1], sa, acc[tp]);
-            acc[tp] = fmaf(dd[tp][2] + dd[tp][3], sb, acc[tp]);
-            mins[tp] = fmaf(mna * dmin, sx.x, mins[tp]);
-            mins[tp] = fmaf(mnb * dmin, sx.y, mins[tp]);
+            const float v = rows_sum(acc[tp][mr] - mins[tp][mr]);
+            if (lane < 16) l_red[((mr * TPW + tp) * SW + wave) * 16 + lane] = v;
         }
-    }
-#pragma unroll
-    for (int tp = 0; tp < TPW; tp++) {
-        const float v = rows_sum(acc[tp] - mins[tp]);
-        if (lane < 16) l_red[(tp * SW + wave) * 16 + lane] = v;
-    }
     __syncthreads();
-    if (tid < TOUT * 16) {
-        const int t = tid >> 4, jr = tid & 15;
+    if (tid < TOUT * 16 * MR) {
+        const int t = (tid >> 4) % TOUT, mr = (tid >> 4) / TOUT, jr = tid & 15;
         float v0 = 0.f, v1 = 0.f;
         for (int s = 0; s < SW; s++) {
-            v0 += l_red[(t * SW + s) * 16 + jr];
+            v0 += l_red[((mr * TPW + t) * SW + s) * 16 + jr];
             if (NT == 2) v1 += l_red[((t + TOUT) * SW + s) * 16 + jr];
         }
         if (IN == 1) {
@@ -380,6 +410,11 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
                     else ((float *)rk.vc)[at] = v0;
                 }
             }
+        } else if (MR > 1) {
+            if (row < nout && mr < nsplit) {
+                const int64_t at = (int64_t)mr * nout + row;
+                y[at] = EPI == FH_EPI_ADD2 ? (v0 + ea[at]) + eb[at] : v0;
+            }
         } else if (row < nout) {
             float rr = v0;
             if (EPI == FH_EPI_ADD2) rr = (rr + ea[row]) + eb[row];
@@ -402,6 +437,11 @@ __global__ __launch_bounds__(1024) void k_qmv_q4k_m1(Q4K_M1_PARAMS) {
 template <int TPW, int PER, int EPI, int IN>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_qmv_q4k_m1_w8(Q4K_M1_PARAMS) {
     qmv_q4k_m1_body<FH_Q4_K, TPW, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
+}
+// 2 .. 4 activation rows (Q4_K; plain input; epilogues none / add2); nsplit = number of valid rows
+template <int TPW, int PER, int EPI, int MR>
+__global__ __launch_bounds__(1024) void k_qmv_q4k_mr(Q4K_M1_PARAMS) {
+    qmv_q4k_m1_body<FH_Q4_K, TPW, PER, EPI, 0, MR>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
 // Q4_0 / Q8_0 weights (plain input; epilogues none / add2 / SwiGLU)
 template <int FMT, int TPW, int PER, int EPI>
@@ -477,6 +517,48 @@ static fh_status q4k_m1_shape(int tpw, int per, const fh_qmatrix *q, const float
         if (tpw == 2 && per == 2) return q4k_m1_launch<2, 2, EPI>(q, x, y, a, b, SW, grid, lds, ex);
     }
     return FH_ERR_UNSUPPORTED;
+}
+
+// y[m, n] for m = 2 .. 4 activation rows of a Q4_K matrix (epilogues none / add2): the weights are unpacked once
+// for all rows.  FH_ERR_UNSUPPORTED when the staged images of all rows do not fit the LDS (the caller falls back).
+template <int EPI, int MR>
+static fh_status q4k_mr_go(const fh_qmatrix *q, const float *x, int m, float *y, const float *a, const float *b) {
+    fh_device *dev = q->dev;
+    const int kb = (int)q->kb;
+    int per = 1;
+    while (kb / per > 16 && per < 2 && kb % (per * 2) == 0) per *= 2;
+    const int SW = kb / per;
+    if (SW > 16 || kb % per) return FH_ERR_UNSUPPORTED;
+    const size_t lds = (size_t)kb * MR * Q4K_IMG * 16 + (size_t)kb * MR * 64 + (size_t)MR * 2 * 16 * 64 + 64;
+    if (lds > 160 * 1024) return FH_ERR_UNSUPPORTED;
+    const int64_t tiles = (q->n + 15) / 16;
+    // two row tiles per wavefront (one staging for both) once there are more tiles than compute units
+    int tpw = (int)dev->opt_matvec_tiles;
+    if (tpw != 1 && tpw != 2) tpw = tiles > dev->compute_units ? 2 : 1;
+    if (per == 2) tpw = 1;
+    const unsigned grid = (unsigned)((tiles + tpw - 1) / tpw);
+    typedef void (*kern_t)(QView, const float *, float *, const float *, const float *, int, const float *, const float *,
+                           float, int, FhRopeArgs);
+    const kern_t kern = per == 2 ? (kern_t)k_qmv_q4k_mr<1, 2, EPI, MR>
+                                 : (tpw == 2 ? (kern_t)k_qmv_q4k_mr<2, 1, EPI, MR> : (kern_t)k_qmv_q4k_mr<1, 1, EPI, MR>);
+    static bool attr_done[3] = {false, false, false};
+    const int ki = per == 2 ? 2 : tpw - 1;
+    if (!attr_done[ki]) {
+        FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_done[ki] = true;
+    }
+    kern<<<dim3(grid, 1), dim3(64 * SW), lds, dev->stream>>>(fh_view(q), x, y, a, b, SW, nullptr, nullptr, 0.f, m, FhRopeArgs{});
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_launch_q4k_rows(const fh_qmatrix *q, const float *x, int m, float *y, int epi, const float *a, const float *b) {
+    if (q->type != FH_Q4_K || m < 2 || m > 4 || (epi != FH_EPI_NONE && epi != FH_EPI_ADD2)) return FH_ERR_UNSUPPORTED;
+    // three or four rows of a very tall matrix: the batch kernel (four tiles share one staging) measured better
+    if (m > 2 && (q->n + 15) / 16 > 4 * (int64_t)q->dev->compute_units) return FH_ERR_UNSUPPORTED;
+    if (epi == FH_EPI_ADD2)
+        return m == 2 ? q4k_mr_go<FH_EPI_ADD2, 2>(q, x, m, y, a, b) : q4k_mr_go<FH_EPI_ADD2, 4>(q, x, m, y, a, b);
+    return m == 2 ? q4k_mr_go<FH_EPI_NONE, 2>(q, x, m, y, a, b) : q4k_mr_go<FH_EPI_NONE, 4>(q, x, m, y, a, b);
 }
 
 // Returns FH_ERR_UNSUPPORTED when the shape does not fit this kernel (the caller falls back).
