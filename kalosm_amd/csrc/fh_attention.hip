@@ -332,10 +332,9 @@ extern "C" fh_status fh_flash_attention_ex(fh_device *dev, int32_t q_dtype, int3
     FH_REQUIRE(sq <= 65535 && hq <= 65535 && b <= 65535, "grid dimension too large");
     const bool qh = q_dtype == FH_F16, kh = kv_dtype == FH_F16;
     FH_REQUIRE((qh || q_dtype == FH_F32) && (kh || kv_dtype == FH_F32), "dtype must be FH_F32 or FH_F16");
-    // many query rows of head_dim 64 / 128 without an additive mask: the matrix-core kernel
-    // (f32 operands are rounded to f16 there, so for f32 queries AND f32 keys it is taken on request only)
-    const bool mfma_ok = qh || kh || dev->opt_attn_kernel == 2;
-    if (sq >= 32 && dev->opt_attn_kernel != 1 && mfma_ok) {
+    // many query rows of head_dim 64 / 128 without an additive mask: the matrix-core kernel (all-f32 inputs go
+    // through its split-operand form, which keeps f32 accuracy; attn_kernel = 2 asks for plain f16 rounding)
+    if (sq >= 32 && dev->opt_attn_kernel != 1) {
         fh_status st = fh_attention_prefill_mfma(dev, q_dtype, kv_dtype, q_dev, q_sb, q_sh, q_st, k_dev, v_dev, kv_sb, kv_sh,
                                                  kv_st, b, hq, hkv, sq, skv, d, scale, mask_kind, out_dev);
         if (st != FH_ERR_UNSUPPORTED) return st;

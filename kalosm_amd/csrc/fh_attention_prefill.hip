@@ -14,6 +14,9 @@
 // registers of a lane are keys 8g .. 8g+7 and 16 + 8g .. 16 + 8g+7 (g = lane / 32), which is exactly the k-slot
 // order of the B operand of the second product - P^T never leaves the registers.
 // Inputs may be f32 or f16; operands are rounded to f16, all accumulation and the softmax are f32.
+// SPLIT (f32 Q, K and V): every operand is the exact two-term f16 split hi + lo of the f32 value (2^-22 relative;
+// the values must lie within the f16 range of +-65504) and both products are the three MFMAs
+// hi.hi + lo.hi + hi.lo, so the result keeps f32 accuracy at three times the matrix-core work.
 #include "fh_internal.h"
 
 typedef _Float16 fh_half;
@@ -49,14 +52,23 @@ __device__ __forceinline__ void ap_store4(fh_half *p, float a, float b, float c,
     *(uint2 *)p = u;
 }
 
-template <typename TQ, typename TKV, int D>
+__device__ __forceinline__ void ap_split8(const float *x, fh_half *hi, fh_half *lo) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        hi[e] = (fh_half)x[e];
+        lo[e] = (fh_half)(x[e] - (float)hi[e]);
+    }
+}
+
+template <typename TQ, typename TKV, int D, bool SPLIT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_attn_prefill(const TQ *__restrict__ q, int64_t q_sb, int64_t q_sh, int64_t q_st,
                                                        const TKV *__restrict__ k, const TKV *__restrict__ v,
                                                        int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int hq, int hkv,
                                                        int sq, int skv, float scale, int causal, TQ *__restrict__ out) {
     constexpr int BN = 64, KS = D + 8, VS = BN + 8, DT = D / 32, KSTEPS = D / 16, CH = D / 8; // CH: 8-element chunks per row
-    __shared__ __attribute__((aligned(16))) fh_half sK[BN * KS];
-    __shared__ __attribute__((aligned(16))) fh_half sV[D * VS];
+    constexpr int NP = SPLIT ? 2 : 1; // operand planes: hi (, lo)
+    __shared__ __attribute__((aligned(16))) fh_half sK[NP * BN * KS];
+    __shared__ __attribute__((aligned(16))) fh_half sV[NP * D * VS];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
     const int h = blockIdx.y, bi = blockIdx.z, kh = h / (hq / hkv);
     // causal: the last query blocks see the most keys; they are dispatched first so that the short ones fill the tail
@@ -66,13 +78,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const TKV *kb = k + bi * kv_sb + kh * kv_sh, *vb = v + bi * kv_sb + kh * kv_sh;
 
     // Q^T operand, once: lane (query li, k-slots 8g .. 8g+7 of every 16-wide step of d)
-    half8 qf[KSTEPS];
+    half8 qf[KSTEPS], ql[SPLIT ? KSTEPS : 1];
     {
         const TQ *qp = q + bi * q_sb + h * q_sh + (int64_t)(qi < sq ? qi : sq - 1) * q_st + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ks++) {
             fh_half t[8];
-            ap_load8(qp + 16 * ks, t);
+            if constexpr (SPLIT) {
+                const float4 a = *(const float4 *)(qp + 16 * ks), b = *(const float4 *)(qp + 16 * ks + 4);
+                const float x[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+                fh_half lo[8];
+                ap_split8(x, t, lo);
+                __builtin_memcpy(&ql[ks], lo, 16);
+            } else {
+                ap_load8(qp + 16 * ks, t);
+            }
             __builtin_memcpy(&qf[ks], t, 16);
         }
     }
@@ -91,14 +111,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         kend = last < skv ? last : skv;
     }
     // The next KV tile is requested (into registers, as f16) before the current one is multiplied.
-    constexpr int NCH = BN * CH / 256; // 16-byte pieces of K (and of V) per thread and tile
+    constexpr int NCH = BN * CH / 256; // 8-element pieces of K (and of V) per thread and tile
     uint4 kreg[NCH], vreg[NCH];
+    float4 kraw[SPLIT ? 2 * NCH : 1], vraw[SPLIT ? 2 * NCH : 1]; // SPLIT: the f32 values wait in registers
     auto fetch = [&](int t0) {
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const int c = tid + 256 * i;
             fh_half t[8];
             const int kkey = c / CH, kdc = c % CH; // K: consecutive threads along d (coalesced rows)
+            if constexpr (SPLIT) { // rows past the end repeat the last one: their scores are masked, their P is 0
+                const float *kp = (const float *)kb + (int64_t)(t0 + kkey < skv ? t0 + kkey : skv - 1) * kv_st + 8 * kdc;
+                kraw[2 * i] = *(const float4 *)kp;
+                kraw[2 * i + 1] = *(const float4 *)(kp + 4);
+                const int vk = c % BN, vd = c / BN;
+                const float *vp = (const float *)vb + (int64_t)(t0 + vk < skv ? t0 + vk : skv - 1) * kv_st + 8 * vd;
+                vraw[2 * i] = *(const float4 *)vp;
+                vraw[2 * i + 1] = *(const float4 *)(vp + 4);
+                continue;
+            }
             if (t0 + kkey < skv) ap_load8(kb + (int64_t)(t0 + kkey) * kv_st + 8 * kdc, t);
             else {
 #pragma unroll
@@ -118,6 +149,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const int c = tid + 256 * i;
+            if constexpr (SPLIT) {
+                const float kx[8] = {kraw[2 * i].x, kraw[2 * i].y, kraw[2 * i].z, kraw[2 * i].w,
+                                     kraw[2 * i + 1].x, kraw[2 * i + 1].y, kraw[2 * i + 1].z, kraw[2 * i + 1].w};
+                fh_half hi[8], lo[8];
+                ap_split8(kx, hi, lo);
+                uint4 uh, ul;
+                __builtin_memcpy(&uh, hi, 16);
+                __builtin_memcpy(&ul, lo, 16);
+                *(uint4 *)(sK + (c / CH) * KS + 8 * (c % CH)) = uh;
+                *(uint4 *)(sK + BN * KS + (c / CH) * KS + 8 * (c % CH)) = ul;
+                const float vx[8] = {vraw[2 * i].x, vraw[2 * i].y, vraw[2 * i].z, vraw[2 * i].w,
+                                     vraw[2 * i + 1].x, vraw[2 * i + 1].y, vraw[2 * i + 1].z, vraw[2 * i + 1].w};
+                ap_split8(vx, hi, lo);
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    sV[(8 * (c / BN) + e) * VS + (c % BN)] = hi[e];
+                    sV[D * VS + (8 * (c / BN) + e) * VS + (c % BN)] = lo[e];
+                }
+                continue;
+            }
             *(uint4 *)(sK + (c / CH) * KS + 8 * (c % CH)) = kreg[i];
             fh_half t[8];
             __builtin_memcpy(t, &vreg[i], 16);
@@ -142,6 +193,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             for (int ks = 0; ks < KSTEPS; ks++) {
                 const half8 a = *(const half8 *)(ap + 16 * ks);
                 st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], st[kt], 0, 0, 0);
+                if constexpr (SPLIT) {
+                    const half8 al = *(const half8 *)(ap + BN * KS + 16 * ks);
+                    st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, qf[ks], st[kt], 0, 0, 0);
+                    st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, ql[ks], st[kt], 0, 0, 0);
+                }
             }
         }
         // ---- mask, running max: register r of half kt is key t0 + 32 kt + 16 (r / 8) + 8 g + r % 8
@@ -161,19 +217,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const bool dead = m_new == -INFINITY; // nothing visible yet (only queries past the end)
         const float alpha = dead ? 1.f : exp2f(m_run - m_new);
         float ps = 0.f;
-        half8 pb[2][2];
+        half8 pb[2][2], pl[SPLIT ? 2 : 1][2];
 #pragma unroll
         for (int kt = 0; kt < 2; kt++)
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++) {
-                fh_half t[8];
+                fh_half t[8], tl[8];
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     const float p = dead ? 0.f : exp2f(st[kt][8 * s2 + e] - m_new);
                     ps += p;
                     t[e] = (fh_half)p;
+                    if constexpr (SPLIT) tl[e] = (fh_half)(p - (float)t[e]);
                 }
                 __builtin_memcpy(&pb[kt][s2], t, 16);
+                if constexpr (SPLIT) __builtin_memcpy(&pl[kt][s2], tl, 16);
             }
         l_run = l_run * alpha + ap_swap32_sum(ps);
         m_run = m_new;
@@ -189,6 +247,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 for (int s2 = 0; s2 < 2; s2++) {
                     const half8 a = *(const half8 *)(vp + 32 * kt + 16 * s2);
                     acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[kt][s2], acc[dt], 0, 0, 0);
+                    if constexpr (SPLIT) {
+                        const half8 al = *(const half8 *)(vp + D * VS + 32 * kt + 16 * s2);
+                        acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, pb[kt][s2], acc[dt], 0, 0, 0);
+                        acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pl[kt][s2], acc[dt], 0, 0, 0);
+                    }
                 }
         }
     }
@@ -205,17 +268,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
-template <typename TQ, typename TKV>
+template <typename TQ, typename TKV, bool SPLIT = false>
 static fh_status ap_launch(fh_device *dev, const void *q, int64_t q_sb, int64_t q_sh, int64_t q_st, const void *k,
                            const void *v, int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int b, int hq, int hkv, int sq,
                            int skv, int d, float scale, int causal, void *out) {
     dim3 grid((unsigned)((sq + 127) / 128), (unsigned)hq, (unsigned)b);
     if (d == 128)
-        k_attn_prefill<TQ, TKV, 128><<<grid, 256, 0, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k,
+        k_attn_prefill<TQ, TKV, 128, SPLIT><<<grid, 256, 0, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k,
                                                                     (const TKV *)v, kv_sb, kv_sh, kv_st, hq, hkv, sq, skv,
                                                                     scale, causal, (TQ *)out);
     else
-        k_attn_prefill<TQ, TKV, 64><<<grid, 256, 0, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k,
+        k_attn_prefill<TQ, TKV, 64, SPLIT><<<grid, 256, 0, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k,
                                                                    (const TKV *)v, kv_sb, kv_sh, kv_st, hq, hkv, sq, skv,
                                                                    scale, causal, (TQ *)out);
     FH_HIP(hipGetLastError());
@@ -235,6 +298,8 @@ fh_status fh_attention_prefill_mfma(fh_device *dev, int q_dtype, int kv_dtype, c
         return ap_launch<fh_half, fh_half>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, d, scale, causal, out);
     if (q_dtype == FH_F32 && kv_dtype == FH_F16)
         return ap_launch<float, fh_half>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, d, scale, causal, out);
+    if (q_dtype == FH_F32 && kv_dtype == FH_F32 && dev->opt_attn_kernel != 2) // all f32: split operands, f32 accuracy
+        return ap_launch<float, float, true>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, d, scale, causal, out);
     if (q_dtype == FH_F32 && kv_dtype == FH_F32)
         return ap_launch<float, float>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, d, scale, causal, out);
     return FH_ERR_UNSUPPORTED;

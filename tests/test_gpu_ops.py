@@ -259,6 +259,32 @@ def test_attention_prefill_f16(dev, oracle, sq, skv, causal, d):
     assert_close(got, ref, abs_tol=1e-2, rel_tol=1e-3, what="vs float64 textbook")
 
 
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("sq,skv,causal", [(128, 128, True), (200, 200, True), (64, 300, True), (160, 97, False),
+                                           (512, 512, True), (33, 33, True)])
+def test_attention_prefill_f32_split(dev, oracle, sq, skv, causal, d):
+    """All-f32 Q/K/V take the matrix-core kernel with split operands (every value as the exact two-term f16 split,
+    three MFMAs per product): f32 accuracy, so the tolerance is a tenth of the north star's; inputs of magnitude up
+    to ~10 (scores up to a few tens) and the same ragged shapes as the f16 test; compared with the checker and with
+    the exact row kernel."""
+    h, hkv = 8, 2
+    rng = np.random.default_rng(sq * 1000 + skv + d + 7)
+    q = (rng.standard_normal((1, h, sq, d)) * 2.5).astype(np.float32)
+    k = (rng.standard_normal((1, hkv, skv, d)) * 2.5).astype(np.float32)
+    v = (rng.standard_normal((1, hkv, skv, d)) * 3.0).astype(np.float32)
+    scale = 1 / np.sqrt(d)
+    mask = MaskKind.Causal if causal else None
+    got = run_attn(dev, q, k, v, scale, mask)
+    want = oracle.flash_attention(q, k, v, scale, oracle.MASK_CAUSAL if causal else oracle.MASK_NONE, None)
+    assert_close(got, want, abs_tol=1e-3, rel_tol=1e-4, what=f"f32 split prefill {sq}x{skv}x{d}")
+    dev.set_option("attn_kernel", 1)
+    try:
+        rows = run_attn(dev, q, k, v, scale, mask)
+    finally:
+        dev.set_option("attn_kernel", 0)
+    assert_close(got, rows, abs_tol=1e-3, rel_tol=1e-4, what="vs the exact row kernel")
+
+
 def test_attention_prefill_f32_on_request(dev, oracle):
     """f32 operands through the same kernel (rounded to f16 inside, f32 out), and the invariants that do not depend
     on the rounding: V constant -> output constant, causal row 0 -> v_0."""
