@@ -360,7 +360,7 @@ fh_status fh_launch_qmatvec(const fh_qmatrix *q, const float *x, int m, float *y
         fh_status st = fh_launch_q4k_m1(q, x, y, epi, a, b);
         if (st != FH_ERR_UNSUPPORTED) return st;
     }
-    if (kernel == 0 && q->type == FH_Q4_K && m >= 2 && m <= 4 && dev->opt_matvec_rows != 1) {
+    if (kernel == 0 && q->type != FH_Q6_K && m >= 2 && m <= 4 && dev->opt_matvec_rows != 1) {
         fh_status st = fh_launch_q4k_rows(q, x, m, y, epi, a, b);
         if (st != FH_ERR_UNSUPPORTED) return st;
     }

@@ -438,10 +438,10 @@ template <int TPW, int PER, int EPI, int IN>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_qmv_q4k_m1_w8(Q4K_M1_PARAMS) {
     qmv_q4k_m1_body<FH_Q4_K, TPW, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
-// 2 .. 4 activation rows (Q4_K; plain input; epilogues none / add2); nsplit = number of valid rows
-template <int TPW, int PER, int EPI, int MR>
+// 2 .. 4 activation rows (plain input; epilogues none / add2); nsplit = number of valid rows
+template <int FMT, int TPW, int PER, int EPI, int MR>
 __global__ __launch_bounds__(1024) void k_qmv_q4k_mr(Q4K_M1_PARAMS) {
-    qmv_q4k_m1_body<FH_Q4_K, TPW, PER, EPI, 0, MR>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
+    qmv_q4k_m1_body<FMT, TPW, PER, EPI, 0, MR>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
 // Q4_0 / Q8_0 weights (plain input; epilogues none / add2 / SwiGLU)
 template <int FMT, int TPW, int PER, int EPI>
@@ -521,10 +521,10 @@ static fh_status q4k_m1_shape(int tpw, int per, const fh_qmatrix *q, const float
 
 // y[m, n] for m = 2 .. 4 activation rows of a Q4_K matrix (epilogues none / add2): the weights are unpacked once
 // for all rows.  FH_ERR_UNSUPPORTED when the staged images of all rows do not fit the LDS (the caller falls back).
-template <int EPI, int MR>
+template <int FMT, int EPI, int MR>
 static fh_status q4k_mr_go(const fh_qmatrix *q, const float *x, int m, float *y, const float *a, const float *b) {
     fh_device *dev = q->dev;
-    const int kb = (int)q->kb;
+    const int kb = (int)(q->k / 256);
     int per = 1;
     while (kb / per > 16 && per < 2 && kb % (per * 2) == 0) per *= 2;
     const int SW = kb / per;
@@ -539,8 +539,8 @@ static fh_status q4k_mr_go(const fh_qmatrix *q, const float *x, int m, float *y,
     const unsigned grid = (unsigned)((tiles + tpw - 1) / tpw);
     typedef void (*kern_t)(QView, const float *, float *, const float *, const float *, int, const float *, const float *,
                            float, int, FhRopeArgs);
-    const kern_t kern = per == 2 ? (kern_t)k_qmv_q4k_mr<1, 2, EPI, MR>
-                                 : (tpw == 2 ? (kern_t)k_qmv_q4k_mr<2, 1, EPI, MR> : (kern_t)k_qmv_q4k_mr<1, 1, EPI, MR>);
+    const kern_t kern = per == 2 ? (kern_t)k_qmv_q4k_mr<FMT, 1, 2, EPI, MR>
+                                 : (tpw == 2 ? (kern_t)k_qmv_q4k_mr<FMT, 2, 1, EPI, MR> : (kern_t)k_qmv_q4k_mr<FMT, 1, 1, EPI, MR>);
     static bool attr_done[3] = {false, false, false};
     const int ki = per == 2 ? 2 : tpw - 1;
     if (!attr_done[ki]) {
@@ -552,13 +552,21 @@ static fh_status q4k_mr_go(const fh_qmatrix *q, const float *x, int m, float *y,
     return FH_OK;
 }
 
+template <int FMT>
+static fh_status q4k_rows_fmt(const fh_qmatrix *q, const float *x, int m, float *y, int epi, const float *a, const float *b) {
+    if (epi == FH_EPI_ADD2)
+        return m == 2 ? q4k_mr_go<FMT, FH_EPI_ADD2, 2>(q, x, m, y, a, b) : q4k_mr_go<FMT, FH_EPI_ADD2, 4>(q, x, m, y, a, b);
+    return m == 2 ? q4k_mr_go<FMT, FH_EPI_NONE, 2>(q, x, m, y, a, b) : q4k_mr_go<FMT, FH_EPI_NONE, 4>(q, x, m, y, a, b);
+}
+
 fh_status fh_launch_q4k_rows(const fh_qmatrix *q, const float *x, int m, float *y, int epi, const float *a, const float *b) {
-    if (q->type != FH_Q4_K || m < 2 || m > 4 || (epi != FH_EPI_NONE && epi != FH_EPI_ADD2)) return FH_ERR_UNSUPPORTED;
+    if (m < 2 || m > 4 || (epi != FH_EPI_NONE && epi != FH_EPI_ADD2)) return FH_ERR_UNSUPPORTED;
+    if (q->type != FH_Q4_K && !((q->type == FH_Q4_0 || q->type == FH_Q8_0) && q->k % 256 == 0)) return FH_ERR_UNSUPPORTED;
     // three or four rows of a very tall matrix: the batch kernel (four tiles share one staging) measured better
     if (m > 2 && (q->n + 15) / 16 > 4 * (int64_t)q->dev->compute_units) return FH_ERR_UNSUPPORTED;
-    if (epi == FH_EPI_ADD2)
-        return m == 2 ? q4k_mr_go<FH_EPI_ADD2, 2>(q, x, m, y, a, b) : q4k_mr_go<FH_EPI_ADD2, 4>(q, x, m, y, a, b);
-    return m == 2 ? q4k_mr_go<FH_EPI_NONE, 2>(q, x, m, y, a, b) : q4k_mr_go<FH_EPI_NONE, 4>(q, x, m, y, a, b);
+    if (q->type == FH_Q4_0) return q4k_rows_fmt<FH_Q4_0>(q, x, m, y, epi, a, b);
+    if (q->type == FH_Q8_0) return q4k_rows_fmt<FH_Q8_0>(q, x, m, y, epi, a, b);
+    return q4k_rows_fmt<FH_Q4_K>(q, x, m, y, epi, a, b);
 }
 
 // Returns FH_ERR_UNSUPPORTED when the shape does not fit this kernel (the caller falls back).
