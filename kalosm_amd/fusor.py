@@ -190,18 +190,19 @@ class Tensor:
             check(L.fh_qmatmul(w._h, C.c_void_p(self.ptr), m, C.c_void_p(out.ptr)))
         return out
 
-    def q_mat_mul_add2(self, w: "QMatrix", first: "Tensor", second: "Tensor") -> "Tensor":
+    def q_mat_mul_add2(self, w: "QMatrix", first: "Tensor", second: "Tensor",
+                       out: Optional["Tensor"] = None) -> "Tensor":
         """(x.W^T + first) + second, the decode epilogue of raw/attention_layer.rs:147-174."""
         m = int(np.prod(self.shape[:-1]))
-        out = Tensor(self.device, (*self.shape[:-1], w.n), "f32")
+        out = out or Tensor(self.device, (*self.shape[:-1], w.n), "f32")
         check(self.device._lib.fh_qmatmul_add2(w._h, C.c_void_p(self.ptr), m, C.c_void_p(first.ptr),
                                                C.c_void_p(second.ptr), C.c_void_p(out.ptr)))
         return out
 
-    def q_mat_mul_swiglu(self, gate_up: "QMatrix") -> "Tensor":
+    def q_mat_mul_swiglu(self, gate_up: "QMatrix", out: Optional["Tensor"] = None) -> "Tensor":
         """silu(x.Wg^T) * (x.Wu^T) with gate_up = concat_rows(gate, up), raw/attention_layer.rs:186-196."""
         m = int(np.prod(self.shape[:-1]))
-        out = Tensor(self.device, (*self.shape[:-1], gate_up.n // 2), "f32")
+        out = out or Tensor(self.device, (*self.shape[:-1], gate_up.n // 2), "f32")
         check(self.device._lib.fh_qmatmul_swiglu(gate_up._h, C.c_void_p(self.ptr), m, C.c_void_p(out.ptr)))
         return out
 

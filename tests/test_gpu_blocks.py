@@ -176,6 +176,29 @@ def test_epilogues(dev, oracle):
     assert np.array_equal(bits(got), bits(want))
 
 
+@pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("m", [1, 2, 4])
+@pytest.mark.parametrize("n", [48, 272])
+def test_epilogues_all_formats_auto_dispatch(dev, oracle, ty, m, n):
+    """SwiGLU and add2 through whichever kernel the dispatch picks for 1 .. 4 rows (raw/attention_layer.rs:147-196);
+    the stacked gate|up matrix needs halves of whole 16-row tiles; 3 and 17 tiles per half are both odd counts."""
+    k = 1280
+    raw_g = synth.random_weight(ty, n, k, seed=70 + ty, sigma=2e-3)
+    raw_u = synth.random_weight(ty, n, k, seed=71 + ty, sigma=2e-3)
+    x = synth.random_activation(m, k, seed=72 + m)
+    g, u = QMatrix.from_raw_bytes(dev, (n, k), raw_g, ty), QMatrix.from_raw_bytes(dev, (n, k), raw_u, ty)
+    gu = QMatrix.concat_rows([g, u])
+    xt = Tensor.from_slice(dev, x)
+    a, b = synth.random_activation(m, n, seed=73), synth.random_activation(m, n, seed=74)
+    yg, yu = oracle.q_mat_mul(ty, x, raw_g, n), oracle.q_mat_mul(ty, x, raw_u, n)
+    out = Tensor.filled_bytes(dev, (m, n), 0xFF)
+    got = xt.q_mat_mul_swiglu(gu, out=out).as_slice()
+    assert_close(got, oracle.swiglu(yg, yu), what=f"{NAMES[ty]} swiglu m={m} n={n}")
+    out = Tensor.filled_bytes(dev, (m, n), 0xFF)
+    got = xt.q_mat_mul_add2(g, Tensor.from_slice(dev, a), Tensor.from_slice(dev, b), out=out).as_slice()
+    assert_close(got, oracle.add3(yg, a, b), what=f"{NAMES[ty]} add2 m={m} n={n}")
+
+
 def test_errors_are_status_codes(dev):
     """Programmer errors the reference panics on are FH_ERR_INVALID here (cpu/src/quantized.rs:54-59, :270-274)."""
     raw = synth.random_weight(Q4_K, 16, 256, seed=70)
