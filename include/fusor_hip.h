@@ -43,7 +43,9 @@ enum {
     FH_ERR_HIP = -2,         /* a HIP runtime call failed */
     FH_ERR_UNSUPPORTED = -3, /* GgufReadError::UnsupportedDType (fusor-ml/core/src/quantized/mod.rs:485) */
     FH_ERR_OOM = -4,
-    FH_ERR_NO_DEVICE = -5    /* Device::gpu() failed (fusor-ml/fusor/src/device.rs:29-39) */
+    FH_ERR_NO_DEVICE = -5,   /* Device::gpu() failed (fusor-ml/fusor/src/device.rs:29-39) */
+    FH_ERR_IO = -6,          /* GgufReadError::Io (fusor-ml/gguf/src/lib.rs:224-225): unreadable or truncated file */
+    FH_ERR_NOT_FOUND = -7    /* Error::VarBuilder "Key ... not found" (fusor-ml/fusor/src/varbuilder.rs:81-83) */
 };
 
 /* GgmlType ids, fusor-ml/gguf/src/lib.rs:35-50 */
@@ -60,6 +62,7 @@ typedef struct fh_qmatrix fh_qmatrix;
 typedef struct fh_kvcache fh_kvcache;
 typedef struct fh_llama fh_llama;
 typedef struct fh_graph fh_graph;
+typedef struct fh_gguf fh_gguf;
 
 const char *fh_last_error(void);
 /* Version string of the library, and the gfx target it was built for. */
@@ -106,7 +109,8 @@ fh_status fh_graph_free(fh_graph *g);
  * it is re-laid-out on the device, the host buffer is not referenced after return. */
 fh_status fh_qmatrix_from_gguf_bytes(fh_device *dev, uint32_t ggml_type, int64_t n, int64_t k,
                                      const void *bytes, size_t len, fh_qmatrix **out);
-/* QMatrix::concat_rows, fusor-ml/fusor/src/quantized.rs:102-112 (same type and k). */
+/* QMatrix::concat_rows, fusor-ml/fusor/src/quantized.rs:102-112.  Where the reference returns None (parts of
+ * different type or k, fusor-ml/core/src/quantized/mod.rs:329-337) the status is FH_ERR_UNSUPPORTED. */
 fh_status fh_qmatrix_concat_rows(fh_device *dev, const fh_qmatrix *const *parts, int32_t count,
                                  fh_qmatrix **out);
 fh_status fh_qmatrix_free(fh_qmatrix *q);
@@ -167,6 +171,10 @@ fh_status fh_rms_norm(fh_device *dev, const float *x_dev, const float *residual_
  * host in f32 (powf, mul, cosf/sinf) and uploaded. */
 fh_status fh_rope_tables(fh_device *dev, int32_t head_dim, int32_t ctx, float theta, float *cos_dev,
                          float *sin_dev);
+/* create_inverse_frequency with a `rope_freqs.weight` tensor, models/kalosm-llama/src/raw/rope.rs:41-48:
+ * inverse frequency i is multiplied by freq_weight_host[i] (head_dim/2 host floats; NULL: no weights). */
+fh_status fh_rope_tables_weighted(fh_device *dev, int32_t head_dim, int32_t ctx, float theta,
+                                  const float *freq_weight_host, float *cos_dev, float *sin_dev);
 /* RopeCache::forward{,_interleaved}(&q, &k, start_pos), rope.rs:284-329.  q is [b, hq, s, d] and
  * k is [b, hk, s, d] as VIEWS: element (b, h, t, c) of q lives at q_dev[b*q_sb + h*q_sh + t*q_st + c]
  * (strides in elements), likewise k.  Outputs are contiguous [b, h, s, d].  One launch rotates both. */
@@ -236,6 +244,63 @@ fh_status fh_cast_f32_bf16(fh_device *dev, const float *x_dev, void *y_bf16_dev,
  * larger index, non-finite skipped; *id_dev = 0xFFFFFFFF when nothing is finite. */
 fh_status fh_argmax(fh_device *dev, const float *x_dev, int64_t count, uint32_t *id_dev);
 
+/* -------------------------------------------------------------- GGUF files
+ * GgufMetadata::read, fusor-ml/gguf/src/lib.rs:559-613: versions 1 .. 3, metadata key/values, tensor
+ * directory (dimensions reversed to row-major order, :583), payload start rounded up to
+ * `general.alignment` (default 32, :597-606).  Host code only: no device is needed.  Error mapping of
+ * GgufReadError (:222-241): Io -> FH_ERR_IO, MagicBytesMismatch / InvalidBool / InvalidValueType /
+ * InvalidTensorSize -> FH_ERR_INVALID, UnsupportedVersion / UnsupportedDType -> FH_ERR_UNSUPPORTED.
+ * fh_gguf_open maps the file read-only; fh_gguf_open_memory parses a caller-owned buffer that must outlive
+ * the handle.  Strings are handed out as (pointer, length) into the file image: not NUL-terminated, trailing
+ * NUL bytes already dropped (:330-332), bytes not re-encoded (the reference replaces invalid UTF-8). */
+fh_status fh_gguf_open(const char *path, fh_gguf **out);
+fh_status fh_gguf_open_memory(const void *bytes, size_t len, fh_gguf **out);
+fh_status fh_gguf_close(fh_gguf *g);
+fh_status fh_gguf_info(const fh_gguf *g, uint32_t *version, uint64_t *tensor_count, uint64_t *metadata_count,
+                       uint64_t *alignment, uint64_t *tensor_data_offset);
+/* GgufMetadataValueType ids, fusor-ml/gguf/src/lib.rs:349-379 */
+enum {
+    FH_GGUF_U8 = 0, FH_GGUF_I8 = 1, FH_GGUF_U16 = 2, FH_GGUF_I16 = 3, FH_GGUF_U32 = 4, FH_GGUF_I32 = 5,
+    FH_GGUF_F32 = 6, FH_GGUF_BOOL = 7, FH_GGUF_STRING = 8, FH_GGUF_ARRAY = 9, FH_GGUF_U64 = 10,
+    FH_GGUF_I64 = 11, FH_GGUF_F64 = 12
+};
+/* Metadata entries in file order (a repeated key keeps its last value, as the reference's map insert). */
+fh_status fh_gguf_meta_key(const fh_gguf *g, uint64_t index, const char **key, uint32_t *value_type);
+/* GgufMetadata::get_value, :301-311: a key starting with '.' matches the shortest stored key ending with
+ * it (`.attention.head_count` finds `llama.attention.head_count`).  All getters below look keys up this
+ * way and return FH_ERR_NOT_FOUND for a missing key, FH_ERR_INVALID for a value of another kind. */
+fh_status fh_gguf_meta_find(const fh_gguf *g, const char *key, const char **full_key, uint32_t *value_type);
+/* to_u8 .. to_i64 (:544-551): any integer type, converted like Rust's `as`. */
+fh_status fh_gguf_meta_int(const fh_gguf *g, const char *key, int64_t *out);
+/* to_f32 / to_f64 (:552-553): F32 or F64 only. */
+fh_status fh_gguf_meta_float(const fh_gguf *g, const char *key, double *out);
+fh_status fh_gguf_meta_bool(const fh_gguf *g, const char *key, int32_t *out);
+fh_status fh_gguf_meta_string(const fh_gguf *g, const char *key, const char **bytes, uint64_t *len);
+/* to_array (:556): element type and count; `packed` (optional) points at the little-endian elements of
+ * an array of fixed-size values and is NULL for arrays of strings or arrays. */
+fh_status fh_gguf_meta_array(const fh_gguf *g, const char *key, uint32_t *elem_type, uint64_t *count,
+                             const void **packed);
+fh_status fh_gguf_meta_array_int(const fh_gguf *g, const char *key, uint64_t index, int64_t *out);
+fh_status fh_gguf_meta_array_float(const fh_gguf *g, const char *key, uint64_t index, double *out);
+fh_status fh_gguf_meta_array_string(const fh_gguf *g, const char *key, uint64_t index, const char **bytes,
+                                    uint64_t *len);
+/* GgufTensorMetadata (:254-259): shape in row-major order (outermost first), offset relative to the
+ * payload start. */
+#define FH_GGUF_MAX_RANK 8
+typedef struct {
+    const char *name; /* owned by the handle */
+    uint32_t ggml_type;
+    int32_t rank;
+    int64_t shape[FH_GGUF_MAX_RANK];
+    uint64_t offset;
+} fh_gguf_tensor;
+fh_status fh_gguf_tensor_info(const fh_gguf *g, uint64_t index, fh_gguf_tensor *out);
+fh_status fh_gguf_tensor_find(const fh_gguf *g, const char *name, uint64_t *index);
+/* GgufTensorMetadata::read_tensor_bytes (:262-286): the raw block stream inside the file image. */
+fh_status fh_gguf_tensor_data(const fh_gguf *g, uint64_t index, const void **bytes, size_t *len);
+/* VarBuilder::get, fusor-ml/fusor/src/varbuilder.rs:79-127: the named tensor as a device weight. */
+fh_status fh_qmatrix_from_gguf_tensor(fh_device *dev, const fh_gguf *g, const char *name, fh_qmatrix **out);
+
 /* ----------------------------------------------------------------- decoder
  * Model::forward for the Llama architecture, models/kalosm-llama/src/raw/mod.rs:851-865,
  * :925-1049 (Separate attention variant + Llama feed-forward, interleaved RoPE), with the
@@ -252,7 +317,9 @@ typedef struct {
 fh_status fh_llama_create(fh_device *dev, const fh_llama_config *cfg, fh_llama **out);
 fh_status fh_llama_destroy(fh_llama *m);
 /* Load one GGUF tensor by its GGUF name (`token_embd.weight`, `blk.N.attn_q.weight`, ...,
- * models/kalosm-llama/src/raw/mod.rs:473-604).  ggml_type 0 (F32) for norm vectors. */
+ * models/kalosm-llama/src/raw/mod.rs:473-604).  ggml_type 0 (F32) for norm vectors and for
+ * `rope_freqs.weight` (head_dim / 2 factors the inverse frequencies are multiplied by,
+ * raw/rope.rs:44-48). */
 fh_status fh_llama_load_tensor(fh_llama *m, const char *name, uint32_t ggml_type, int64_t n,
                                int64_t k, const void *bytes, size_t len);
 /* Fuse/concatenate what the config asks for and allocate the step buffers; call once after loading. */
@@ -269,6 +336,13 @@ fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, int32_t step
                                  uint32_t *out_tokens_host, float *elapsed_ms);
 /* Bytes of weights read per decoded token (for roofline reports). */
 fh_status fh_llama_weight_bytes(const fh_llama *m, uint64_t *bytes);
+/* Model parameters from GGUF metadata, models/kalosm-llama/src/raw/mod.rs:377-416 (architecture
+ * `llama` only; kv_dtype f32, fusions and graph replay switched on: adjust before fh_llama_create,
+ * e.g. a smaller ctx than the file's context_length). */
+fh_status fh_llama_config_from_gguf(const fh_gguf *g, fh_llama_config *cfg);
+/* Load every decoder tensor of the file (raw/mod.rs:418-604: token_embd, output_norm, output,
+ * rope_freqs, blk.N.*); f16 vectors are widened to f32.  Call fh_llama_finalize afterwards. */
+fh_status fh_llama_load_gguf(fh_llama *m, const fh_gguf *g);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop

@@ -11,6 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libfusor_hip.so")
 
 FH_OK, FH_ERR_INVALID, FH_ERR_HIP, FH_ERR_UNSUPPORTED, FH_ERR_OOM, FH_ERR_NO_DEVICE = 0, -1, -2, -3, -4, -5
+FH_ERR_IO, FH_ERR_NOT_FOUND = -6, -7
 Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
 MASK_NONE, MASK_CAUSAL, MASK_ADDITIVE = 0, 1, 2
 F32, F16 = 0, 1
@@ -26,6 +27,11 @@ class LlamaConfig(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("n_layers", "d_model", "n_heads", "n_kv_heads", "head_dim", "ffn", "vocab",
                                          "ctx")] + [("eps", C.c_float), ("theta", C.c_float)] + \
                [(n, C.c_int32) for n in ("kv_dtype", "fuse_qkv", "fuse_gate_up", "use_graph")]
+
+
+class GgufTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("ggml_type", C.c_uint32), ("rank", C.c_int32), ("shape", C.c_int64 * 8),
+                ("offset", C.c_uint64)]
 
 
 _p = C.c_void_p
@@ -92,6 +98,27 @@ SIGNATURES = {
     "fh_llama_forward": [_p, _p, _i32, _p, _p],
     "fh_llama_decode_greedy": [_p, _u32, _i32, _p, C.POINTER(_f32)],
     "fh_llama_weight_bytes": [_p, C.POINTER(_u64)],
+    "fh_llama_config_from_gguf": [_p, C.POINTER(LlamaConfig)],
+    "fh_llama_load_gguf": [_p, _p],
+    "fh_rope_tables_weighted": [_p, _i32, _i32, _f32, _p, _p, _p],
+    "fh_gguf_open": [C.c_char_p, _pp],
+    "fh_gguf_open_memory": [_p, _sz, _pp],
+    "fh_gguf_close": [_p],
+    "fh_gguf_info": [_p, C.POINTER(_u32), C.POINTER(_u64), C.POINTER(_u64), C.POINTER(_u64), C.POINTER(_u64)],
+    "fh_gguf_meta_key": [_p, _u64, C.POINTER(C.c_char_p), C.POINTER(_u32)],
+    "fh_gguf_meta_find": [_p, C.c_char_p, C.POINTER(C.c_char_p), C.POINTER(_u32)],
+    "fh_gguf_meta_int": [_p, C.c_char_p, C.POINTER(_i64)],
+    "fh_gguf_meta_float": [_p, C.c_char_p, C.POINTER(C.c_double)],
+    "fh_gguf_meta_bool": [_p, C.c_char_p, C.POINTER(_i32)],
+    "fh_gguf_meta_string": [_p, C.c_char_p, _pp, C.POINTER(_u64)],
+    "fh_gguf_meta_array": [_p, C.c_char_p, C.POINTER(_u32), C.POINTER(_u64), _pp],
+    "fh_gguf_meta_array_int": [_p, C.c_char_p, _u64, C.POINTER(_i64)],
+    "fh_gguf_meta_array_float": [_p, C.c_char_p, _u64, C.POINTER(C.c_double)],
+    "fh_gguf_meta_array_string": [_p, C.c_char_p, _u64, _pp, C.POINTER(_u64)],
+    "fh_gguf_tensor_info": [_p, _u64, C.POINTER(GgufTensor)],
+    "fh_gguf_tensor_find": [_p, C.c_char_p, C.POINTER(_u64)],
+    "fh_gguf_tensor_data": [_p, _u64, _pp, C.POINTER(_sz)],
+    "fh_qmatrix_from_gguf_tensor": [_p, _p, C.c_char_p, _pp],
 }
 STRING_GETTERS = ("fh_last_error", "fh_version")
 

@@ -25,6 +25,7 @@ struct fh_llama {
     bool output_is_embd = false;
     float *out_norm = nullptr;
     float *cos_t = nullptr, *sin_t = nullptr;
+    std::vector<float> rope_freq_weight; // rope_freqs.weight when the file has one
     fh_kvcache *cache = nullptr;
     bool finalized = false;
     int pos = 0;
@@ -118,6 +119,15 @@ extern "C" fh_status fh_llama_load_tensor(fh_llama *m, const char *name, uint32_
     if (!strcmp(name, "token_embd.weight")) return loadq(&m->embd, c.vocab, D);
     if (!strcmp(name, "output.weight")) return loadq(&m->output, c.vocab, D);
     if (!strcmp(name, "output_norm.weight")) return load_f32(m, &m->out_norm, D, n, k, bytes, len, name);
+    if (!strcmp(name, "rope_freqs.weight")) {
+        const int64_t half = c.head_dim / 2, count = n * (k > 0 ? k : 1);
+        FH_REQUIRE(ggml_type == 0 && count == half && len == (size_t)half * 4,
+                   "%s: expected %lld f32 values, got type %u [%lld, %lld] / %zu bytes", name, (long long)half, ggml_type,
+                   (long long)n, (long long)k, len);
+        m->rope_freq_weight.resize((size_t)half);
+        memcpy(m->rope_freq_weight.data(), bytes, len);
+        return FH_OK;
+    }
     int li = -1;
     char field[64] = "";
     if (sscanf(name, "blk.%d.%63s", &li, field) == 2 && li >= 0 && li < c.n_layers) {
@@ -193,7 +203,8 @@ extern "C" fh_status fh_llama_finalize(fh_llama *m) {
     size_t tbl = (size_t)c.ctx * (c.head_dim / 2) * 4;
     FH_TRY(fh_malloc(m->dev, tbl, (void **)&m->cos_t));
     FH_TRY(fh_malloc(m->dev, tbl, (void **)&m->sin_t));
-    FH_TRY(fh_rope_tables(m->dev, c.head_dim, c.ctx, c.theta, m->cos_t, m->sin_t));
+    FH_TRY(fh_rope_tables_weighted(m->dev, c.head_dim, c.ctx, c.theta,
+                                   m->rope_freq_weight.empty() ? nullptr : m->rope_freq_weight.data(), m->cos_t, m->sin_t));
     FH_TRY(fh_kvcache_create(m->dev, c.n_layers, c.n_kv_heads, c.head_dim, c.ctx, c.kv_dtype, &m->cache));
     FH_TRY(fh_malloc(m->dev, (size_t)c.vocab * 4, (void **)&m->logits));
     FH_TRY(fh_malloc(m->dev, 256, (void **)&m->tok_dev));

@@ -172,8 +172,9 @@ extern "C" fh_status fh_qmatrix_concat_rows(fh_device *dev, const fh_qmatrix *co
     int64_t n = 0;
     for (int i = 0; i < count; i++) {
         FH_REQUIRE(parts[i], "part %d is NULL", i);
-        FH_REQUIRE(parts[i]->type == parts[0]->type && parts[i]->k == parts[0]->k,
-                   "concat_rows needs one type and one k (part %d differs)", i);
+        // Option::None in the reference (fusor-ml/core/src/quantized/mod.rs:329-337)
+        if (parts[i]->type != parts[0]->type || parts[i]->k != parts[0]->k)
+            FH_FAIL(FH_ERR_UNSUPPORTED, "concat_rows needs one type and one k (part %d differs)", i);
         if (i + 1 < count && parts[i]->n % 16 != 0)
             FH_FAIL(FH_ERR_UNSUPPORTED, "concat_rows: part %d has %lld rows, not a multiple of 16", i,
                     (long long)parts[i]->n);

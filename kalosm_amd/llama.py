@@ -49,6 +49,25 @@ class Model:
         m.finalize()
         return m
 
+    @staticmethod
+    def from_gguf(device: Device, source, ctx: Optional[int] = None, kv_dtype: str = "f32", fuse_qkv: bool = True,
+                  fuse_gate_up: bool = True, use_graph: bool = True) -> "Model":
+        """Model::from_gguf for the Llama architecture (raw/mod.rs:284-648): parameters from the metadata, every
+        decoder tensor from the file.  `source` is a path or an open `GgufMetadata`; `ctx` caps the context
+        length (and with it the KV cache) below the file's `context_length`."""
+        from .gguf import GgufMetadata
+        g = source if isinstance(source, GgufMetadata) else GgufMetadata.read(source)
+        c = LlamaConfig()
+        check(device._lib.fh_llama_config_from_gguf(g._h, C.byref(c)))
+        cfg = {n: getattr(c, n) for n in ("n_layers", "d_model", "n_heads", "n_kv_heads", "head_dim", "ffn", "vocab",
+                                          "ctx", "eps", "theta")}
+        if ctx is not None:
+            cfg["ctx"] = min(cfg["ctx"], int(ctx))
+        m = Model(device, cfg, kv_dtype=kv_dtype, fuse_qkv=fuse_qkv, fuse_gate_up=fuse_gate_up, use_graph=use_graph)
+        check(device._lib.fh_llama_load_gguf(m._h, g._h))
+        m.finalize()
+        return m
+
     def finalize(self) -> None:
         check(self.device._lib.fh_llama_finalize(self._h))
         self._final = True

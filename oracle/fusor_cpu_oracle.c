@@ -600,10 +600,14 @@ void fo_rms_norm(const float *x, const float *residual, const float *w, const fl
 void fo_rope_inverse_frequency(int dim, float theta, float *inv) {
     for (int i = 0; i < dim; i += 2) inv[i / 2] = 1.0f / powf(theta, (float)i / (float)dim);
 }
-void fo_rope_tables(int dim, int ctx, float theta, float *cosv, float *sinv) {
+/* freq_weight (optional, dim/2 values): the `rope_freqs.weight` tensor of a model file; the inverse
+ * frequencies are MULTIPLIED by it (models/kalosm-llama/src/raw/rope.rs:41-48). */
+void fo_rope_tables_weighted(int dim, int ctx, float theta, const float *freq_weight, float *cosv, float *sinv) {
     int half = dim / 2;
     float *inv = (float *)malloc((size_t)half * sizeof(float));
     fo_rope_inverse_frequency(dim, theta, inv);
+    if (freq_weight)
+        for (int i = 0; i < half; i++) inv[i] = inv[i] * freq_weight[i];
     for (int p = 0; p < ctx; p++)
         for (int i = 0; i < half; i++) {
             float a = (float)p * inv[i];
@@ -611,6 +615,9 @@ void fo_rope_tables(int dim, int ctx, float theta, float *cosv, float *sinv) {
             sinv[(size_t)p * half + i] = sinf(a);
         }
     free(inv);
+}
+void fo_rope_tables(int dim, int ctx, float theta, float *cosv, float *sinv) {
+    fo_rope_tables_weighted(dim, ctx, theta, NULL, cosv, sinv);
 }
 
 /* fusor/src/composite/rope.rs:77-108 (interleaved: pairs (2i, 2i+1)) and :46-68
@@ -701,6 +708,7 @@ typedef struct {
 typedef struct {
     const uint8_t *wq, *wk, *wv, *wo, *gate, *up, *down;
     const float *attn_norm, *ffn_norm;
+    int tq, tk, tv, to, tgate, tup, tdown; /* block type of each weight (model files mix them per layer) */
 } fo_llama_layer;
 
 typedef struct {
@@ -737,6 +745,18 @@ void fo_llama_set_layer(fo_llama *m, int l, const uint8_t *wq, const uint8_t *wk
     y->wq = wq; y->wk = wk; y->wv = wv; y->wo = wo;
     y->gate = gate; y->up = up; y->down = down;
     y->attn_norm = attn_norm; y->ffn_norm = ffn_norm;
+    y->tq = y->tk = y->tv = y->to = m->c.type_attn;
+    y->tgate = y->tup = m->c.type_ffn_gate_up;
+    y->tdown = m->c.type_ffn_down;
+}
+/* types: q, k, v, o, gate, up, down -- call after fo_llama_set_layer */
+void fo_llama_set_layer_types(fo_llama *m, int l, const int *types) {
+    fo_llama_layer *y = &m->layers[l];
+    y->tq = types[0]; y->tk = types[1]; y->tv = types[2]; y->to = types[3];
+    y->tgate = types[4]; y->tup = types[5]; y->tdown = types[6];
+}
+void fo_llama_set_rope_freq_weight(fo_llama *m, const float *w) {
+    fo_rope_tables_weighted(m->c.head_dim, m->c.ctx, m->c.theta, w, m->cosv, m->sinv);
 }
 void fo_llama_set_globals(fo_llama *m, const uint8_t *embd, const float *out_norm, const uint8_t *output) {
     m->embd = embd; m->out_norm = out_norm; m->output = output;
@@ -783,9 +803,9 @@ int fo_llama_forward(fo_llama *m, const uint32_t *tokens, int s, float *logits, 
         fo_llama_layer *y = &m->layers[l];
         /* residual = x; x = attention_norm(x)                      raw/mod.rs:961-964 */
         fo_rms_norm(x, NULL, y->attn_norm, NULL, c->eps, s, D, xn);
-        fo_q_mat_mul_fast(c->type_attn, xn, s, D, y->wq, H * hd, q, L, nt);
-        fo_q_mat_mul_fast(c->type_attn, xn, s, D, y->wk, HK * hd, k, L, nt);
-        fo_q_mat_mul_fast(c->type_attn, xn, s, D, y->wv, HK * hd, v, L, nt);
+        fo_q_mat_mul_fast(y->tq, xn, s, D, y->wq, H * hd, q, L, nt);
+        fo_q_mat_mul_fast(y->tk, xn, s, D, y->wk, HK * hd, k, L, nt);
+        fo_q_mat_mul_fast(y->tv, xn, s, D, y->wv, HK * hd, v, L, nt);
         to_heads(q, s, H, hd, qh);      /* reshape + transpose(1,2), attention_layer.rs:371-374 */
         to_heads(k, s, HK, hd, kh);
         to_heads(v, s, HK, hd, vh);
@@ -801,13 +821,13 @@ int fo_llama_forward(fo_llama *m, const uint32_t *tokens, int s, float *logits, 
         fo_flash_attention(qr, kall, vall, 1, H, HK, s, len, hd, (float)(1.0 / sqrt((double)hd)),
                            s > 1 ? 1 : 0, NULL, ao, nt);
         from_heads(ao, s, H, hd, ao2);  /* transpose(1,2) + reshape, attention_layer.rs:689-691 */
-        fo_q_mat_mul_fast(c->type_attn, ao2, s, H * hd, y->wo, D, att, L, nt);
+        fo_q_mat_mul_fast(y->to, ao2, s, H * hd, y->wo, D, att, L, nt);
         /* x2 = ffn_norm(att + residual)                            raw/mod.rs:1017 */
         fo_rms_norm(att, x, y->ffn_norm, NULL, c->eps, s, D, xn);
-        fo_q_mat_mul_fast(c->type_ffn_gate_up, xn, s, D, y->gate, F, g, L, nt);
-        fo_q_mat_mul_fast(c->type_ffn_gate_up, xn, s, D, y->up, F, u, L, nt);
+        fo_q_mat_mul_fast(y->tgate, xn, s, D, y->gate, F, g, L, nt);
+        fo_q_mat_mul_fast(y->tup, xn, s, D, y->up, F, u, L, nt);
         fo_swiglu(g, u, act, (size_t)s * F);
-        fo_q_mat_mul_fast(c->type_ffn_down, act, s, F, y->down, D, ff, L, nt);
+        fo_q_mat_mul_fast(y->tdown, act, s, F, y->down, D, ff, L, nt);
         fo_add3(ff, att, x, x, sd);     /* (ffn + attn) + residual, raw/mod.rs:1036 */
     }
     fo_rms_norm(x + (size_t)(s - 1) * D, NULL, m->out_norm, NULL, c->eps, 1, D, xn);

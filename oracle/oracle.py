@@ -69,6 +69,9 @@ def lib() -> C.CDLL:
         L.fo_llama_create.argtypes = [C.c_void_p, C.c_int]
         L.fo_llama_set_layer.argtypes = [C.c_void_p, C.c_int] + [u8p] * 7 + [fp, fp]
         L.fo_llama_set_globals.argtypes = [C.c_void_p, u8p, fp, u8p]
+        L.fo_llama_set_layer_types.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int)]
+        L.fo_llama_set_rope_freq_weight.argtypes = [C.c_void_p, fp]
+        L.fo_rope_tables_weighted.argtypes = [C.c_int, C.c_int, C.c_float, fp, fp, fp]
         L.fo_llama_reset.argtypes = [C.c_void_p]
         L.fo_llama_destroy.argtypes = [C.c_void_p]
         L.fo_llama_forward.argtypes = [C.c_void_p, u32p, C.c_int, fp, fp]
@@ -221,6 +224,14 @@ def rope_inverse_frequency(dim: int, theta: float) -> np.ndarray:
     return inv
 
 
+def rope_tables_weighted(dim: int, ctx: int, theta: float, freq_weight):
+    cos = np.empty((ctx, dim // 2), np.float32)
+    sin = np.empty((ctx, dim // 2), np.float32)
+    w = _f32(freq_weight)
+    lib().fo_rope_tables_weighted(dim, ctx, theta, _p(w, C.c_float), _p(cos, C.c_float), _p(sin, C.c_float))
+    return cos, sin
+
+
 def rope_tables(dim: int, ctx: int, theta: float):
     cos = np.empty((ctx, dim // 2), np.float32)
     sin = np.empty((ctx, dim // 2), np.float32)
@@ -305,6 +316,15 @@ class Llama:
                                      u8(p + "ffn_gate.weight"), u8(p + "ffn_up.weight"), u8(p + "ffn_down.weight"),
                                      f32(p + "attn_norm.weight"), f32(p + "ffn_norm.weight"))
         lib().fo_llama_set_globals(self._h, u8("token_embd.weight"), f32("output_norm.weight"), u8("output.weight"))
+        # per-tensor block types (model files mix them from layer to layer): cfg["tensor_types"] = {name: type}
+        types = cfg.get("tensor_types")
+        if types:
+            names = ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down")
+            for l in range(cfg["n_layers"]):
+                arr = (C.c_int * 7)(*[types[f"blk.{l}.{n}.weight"] for n in names])
+                lib().fo_llama_set_layer_types(self._h, l, arr)
+        if "rope_freqs.weight" in weights:
+            lib().fo_llama_set_rope_freq_weight(self._h, f32("rope_freqs.weight"))
 
     def reset(self):
         lib().fo_llama_reset(self._h)

@@ -108,6 +108,76 @@ def test_decode_step_kernel_variants(dev, oracle, heads, kv_heads, opts):
             dev.set_option(k, 0)
 
 
+@pytest.mark.parametrize("variant", [dict(), dict(fuse_qkv=False, fuse_gate_up=False, use_graph=False)],
+                         ids=["fused+graph", "separate+eager"])
+def test_decoder_from_gguf_file(dev, oracle, variant, tmp_path):
+    """Model::from_gguf (raw/mod.rs:284-648) on a small random-init file with what model files really hold:
+    block types that change from layer to layer (so q|k|v and gate|up cannot always be fused), f32 and f16 norm
+    vectors, a rope_freqs.weight tensor, tokenizer metadata beside the model keys.  The checker's decoder is fed
+    from the same file through the plain-Python reader."""
+    from test_gguf_reader import TINY, llama_file
+    from oracle import gguf_ref
+    data, weights, types = llama_file(TINY, seed=5)
+    path = tmp_path / "tiny.gguf"
+    path.write_bytes(data)
+    m = Model.from_gguf(dev, str(path), ctx=80, **variant)
+    assert m.cfg == {**TINY, "ctx": 80, "eps": float(np.float32(1e-5))}
+    r = gguf_ref.GgufRef(data)
+    rw = {}
+    for name, (ty, shape, off) in r.tensors.items():
+        raw = r.tensor_bytes(name)
+        if ty == 0:
+            raw = raw.view(np.float32)
+        elif ty == 1:
+            raw = raw.view(np.float16).astype(np.float32)
+        rw[name.decode()] = raw
+    ocfg = dict(m.cfg, type_attn=synth.Q4_K, type_ffn_gate_up=synth.Q4_K, type_ffn_down=synth.Q6_K, type_embd=synth.Q4_K,
+                type_output=synth.Q6_K, tensor_types={n.decode(): t for n, (t, _, _) in r.tensors.items()})
+    ref = oracle.Llama(ocfg, rw)
+    rng = np.random.default_rng(2)
+    prompt = rng.integers(0, TINY["vocab"], 11)
+    lg, hid = m.forward(prompt, want_hidden=True)
+    wl, wh = ref.forward(prompt, want_hidden=True)
+    assert_close(hid, wh, what="prefill hidden")
+    assert_close(lg, wl, what="prefill logits")
+    tok = oracle.argmax(wl)
+    got, _ = m.decode_greedy(tok, 30)
+    want, t = [], tok
+    for _ in range(30):
+        t = oracle.argmax(ref.forward([t]))
+        want.append(t)
+    assert got.tolist() == want
+    assert_close(m.forward([want[-1]]), ref.forward([want[-1]]), what="logits after 30 device-side steps")
+    # the rope_freqs factors matter: the same file without them gives other logits
+    cos, sin = oracle.rope_tables_weighted(64, 4, 500000.0, weights["rope_freqs.weight"])
+    c0, s0 = oracle.rope_tables(64, 4, 500000.0)
+    assert not np.allclose(cos[3], c0[3]) and np.array_equal(cos[0], c0[0])
+    # weights by name through the VarBuilder
+    from kalosm_amd.gguf import VarBuilder
+    vb = VarBuilder.from_gguf(str(path))
+    q = vb.pp("blk").pp(0).get("attn_v.weight", dev)
+    assert q.shape() == (128, 256) and q.ggml_type == synth.Q6_K
+    want_w = oracle.dequantize(synth.Q6_K, weights["blk.0.attn_v.weight"]).reshape(128, 256)
+    assert np.array_equal(q.dequantize().as_slice().view(np.uint32), want_w.view(np.uint32))
+    with pytest.raises(Exception) as e:
+        vb.get("blk.9.attn_v.weight", dev)
+    assert "not found" in str(e.value)
+    # parts of different block types do not concatenate (None in the reference, core/src/quantized/mod.rs:329-337)
+    from kalosm_amd.fusor import QMatrix
+    assert QMatrix.concat_rows([vb.get("blk.0.attn_k.weight", dev), q]) is None
+
+
+def test_decoder_from_gguf_refuses_other_variants(dev):
+    """Tensors of attention / norm variants this decoder does not implement are refused, not skipped."""
+    from test_gguf_reader import TINY, llama_file
+    from kalosm_amd.gguf import GgufMetadata
+    bias = np.zeros(256, np.float32).view(np.uint8)
+    data, _, _ = llama_file(TINY, extra_tensors=[("blk.0.attn_q.bias", 0, (256,), bias)])
+    with pytest.raises(Exception) as e:
+        Model.from_gguf(dev, GgufMetadata.read_bytes(data))
+    assert "attn_q.bias" in str(e.value)
+
+
 def test_decoder_errors(dev):
     from kalosm_amd.fusor import FusorHipError
     m = Model(dev, SMALL)
