@@ -189,6 +189,7 @@ extern "C" fh_status fh_set_option(fh_device *dev, const char *key, int64_t valu
     else if (!strcmp(key, "wo_acc")) dev->opt_wo_acc = value;
     else if (!strcmp(key, "wo_tiles")) dev->opt_wo_tiles = value;
     else if (!strcmp(key, "matvec_rows")) dev->opt_matvec_rows = value;
+    else if (!strcmp(key, "matvec_direct")) dev->opt_matvec_direct = value;
     else if (!strcmp(key, "attn_waves")) dev->opt_attn_waves = value;
     else if (!strcmp(key, "attn_heads")) dev->opt_attn_heads = value;
     else if (!strcmp(key, "down_tiles")) dev->opt_down_tiles = value;

@@ -63,6 +63,7 @@ struct fh_device {
     int64_t opt_attn_heads = 0;      // query heads per workgroup of the decode attention (0: automatic; 1, 2, 4, 8)
     int64_t opt_attn_waves = 0;      // wavefronts per workgroup of the decode attention (0: 16; 8)
     int64_t opt_matvec_rows = 0;     // 1: 2 .. 4 activation rows never through the single-row Q4_K kernel's row variant
+    int64_t opt_matvec_direct = 0; // 1: 5 .. 16 rows never through the unstaged kernel, 2: 2 .. 4 rows through it as well
     int64_t opt_wo_tiles = 0;        // row tiles per wavefront of the accumulating output projection (0: 4; 1, 2, 4)
     int64_t opt_wo_acc = 0;          // 0: decode steps accumulate the output projection into the residual stream, 1: never
     int64_t opt_fuse_norm = 0;       // 0: decode steps fold rms_norm into the consuming matvec, 1: separate launches

@@ -105,33 +105,45 @@ __device__ __forceinline__ half8 qb_h8(uint32_t a, uint32_t b, uint32_t c, uint3
 }
 
 // ------------------------------------------------------------------------------ one chunk of one tile
-// yacc[i] += factor[m] * sum_blocks scale * (codes . x_scaled) - sum_blocks offset * sum(x), m = 4g + i.
+// Where the activation operands of a chunk come from: `opnd(off)` is the A operand at half offset `off` of the
+// lane's image row, `sum(off)` the four group sums at float offset `off`, `fac()` the four row factors.
 template <int T, int MR>
-__device__ __forceinline__ void qb_chunk(const QbW<T> &W, const uint8_t *img, int lane, float *yacc) {
+struct QbLdsSrc { // a staged image in LDS
     typedef QbLds<T, MR> L;
-    const int j = lane & 15, g = lane >> 4;
-    const _Float16 *xa = (const _Float16 *)img + (j & (MR - 1)) * L::ROW + 8 * g;
-    const float *S = (const float *)(img + L::S_OFF) + 4 * g;
+    const _Float16 *xa;
+    const float *S, *F;
+    __device__ __forceinline__ QbLdsSrc(const uint8_t *img, int lane)
+        : xa((const _Float16 *)img + ((lane & 15) & (MR - 1)) * L::ROW + 8 * (lane >> 4)),
+          S((const float *)(img + L::S_OFF) + 4 * (lane >> 4)), F((const float *)(img + L::F_OFF) + 4 * (lane >> 4)) {}
+    __device__ __forceinline__ half8 opnd(int off) const { return *(const half8 *)(xa + off); }
+    __device__ __forceinline__ float4 sum(int off) const { return *(const float4 *)(S + off); }
+    __device__ __forceinline__ float4 fac() const { return *(const float4 *)F; }
+};
+
+// Steps S0 .. S1-1 of the eight a chunk has (a 32-group each; Q6_K: two 16-groups each):
+// tot[i] += scale * (codes . x_scaled), off[i] += offset * sum(x), for the rows m = 4g + i of the lane.
+template <int T, int MR, int S0, int S1, class Src>
+__device__ __forceinline__ void qb_steps(const QbW<T> &W, const Src &src, float *tot, float *off) {
+    typedef QbLds<T, MR> L;
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-    float tot[4] = {0.f, 0.f, 0.f, 0.f}, off[4] = {0.f, 0.f, 0.f, 0.f};
     const uint32_t LO = 0x000F000Fu, HI = 0x00F000F0u;
     if constexpr (T == FH_Q4_K) {
         const float d = fh_h2f((uint16_t)(W.h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(W.h.x >> 16));
         const uint32_t sc_l = W.h.y & 0x3F3F3F3Fu, sc_h = (W.h.w & 0x0F0F0F0Fu) | ((W.h.y >> 2) & 0x30303030u);
         const uint32_t mn_l = W.h.z & 0x3F3F3F3Fu, mn_h = ((W.h.w >> 4) & 0x0F0F0F0Fu) | ((W.h.z >> 2) & 0x30303030u);
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
+        for (int s = S0; s < S1; s++) {
             const uint4 wq = (s & 4) ? W.b : W.a;
             const uint32_t w0 = (s & 2) ? wq.z : wq.x, w1 = (s & 2) ? wq.w : wq.y;
             const uint32_t msk = (s & 1) ? HI : LO;
             const half8 bv = qb_h8(w0 & msk, (w0 >> 8) & msk, w1 & msk, (w1 >> 8) & msk);
-            const half8 ah = *(const half8 *)(xa + 32 * s), al = *(const half8 *)(xa + L::PLANE + 32 * s);
+            const half8 ah = src.opnd(32 * s), al = src.opnd(L::PLANE + 32 * s);
             floatx4 r = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bv, zero, 0, 0, 0);
             r = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, bv, r, 0, 0, 0);
             const float sc = (float)(((s < 4 ? sc_l : sc_h) >> (8 * (s & 3))) & 0xFFu);
             const float mn = (float)(((s < 4 ? mn_l : mn_h) >> (8 * (s & 3))) & 0xFFu);
             const float sw = (sc * d) * ((s & 1) ? 0.0625f : 1.0f), ow = mn * dmin; // high nibbles carry a factor 16
-            const float4 sv = *(const float4 *)(S + 16 * s);
+            const float4 sv = src.sum(16 * s);
             tot[0] = fmaf(sw, r[0], tot[0]); tot[1] = fmaf(sw, r[1], tot[1]);
             tot[2] = fmaf(sw, r[2], tot[2]); tot[3] = fmaf(sw, r[3], tot[3]);
             off[0] = fmaf(ow, sv.x, off[0]); off[1] = fmaf(ow, sv.y, off[1]);
@@ -140,7 +152,7 @@ __device__ __forceinline__ void qb_chunk(const QbW<T> &W, const uint8_t *img, in
     } else if constexpr (T == FH_Q6_K) {
         const float d = fh_h2f((uint16_t)W.d);
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
+        for (int t = S0; t < S1; t++) {
             const uint4 lq = (t & 4) ? W.l1 : W.l0;
             const uint32_t lw = (t & 3) == 0 ? lq.x : (t & 3) == 1 ? lq.y : (t & 3) == 2 ? lq.z : lq.w;
             const uint32_t hw = (t >> 1) == 0 ? W.hh.x : (t >> 1) == 1 ? W.hh.y : (t >> 1) == 2 ? W.hh.z : W.hh.w;
@@ -162,12 +174,12 @@ __device__ __forceinline__ void qb_chunk(const QbW<T> &W, const uint8_t *img, in
                 ob[p] = sw2[1];
             }
             const half8 ba = qb_h8(oa[0], oa[1], oa[2], oa[3]), bb = qb_h8(ob[0], ob[1], ob[2], ob[3]);
-            const half8 a0 = *(const half8 *)(xa + 64 * t), a1 = *(const half8 *)(xa + 64 * t + 32);
+            const half8 a0 = src.opnd(64 * t), a1 = src.opnd(64 * t + 32);
             const floatx4 r0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, ba, zero, 0, 0, 0);
             const floatx4 r1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bb, zero, 0, 0, 0);
             const uint32_t scw = W.sc[t & 3] >> (16 * (t >> 2));
             const float s0 = d * (float)(int)(int8_t)(scw & 0xFFu), s1 = d * (float)(int)(int8_t)((scw >> 8) & 0xFFu);
-            const float4 v0 = *(const float4 *)(S + 32 * t), v1 = *(const float4 *)(S + 32 * t + 16);
+            const float4 v0 = src.sum(32 * t), v1 = src.sum(32 * t + 16);
             tot[0] = fmaf(s0, r0[0], tot[0]); tot[1] = fmaf(s0, r0[1], tot[1]);
             tot[2] = fmaf(s0, r0[2], tot[2]); tot[3] = fmaf(s0, r0[3], tot[3]);
             tot[0] = fmaf(s1, r1[0], tot[0]); tot[1] = fmaf(s1, r1[1], tot[1]);
@@ -180,7 +192,7 @@ __device__ __forceinline__ void qb_chunk(const QbW<T> &W, const uint8_t *img, in
         }
     } else {
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
+        for (int s = S0; s < S1; s++) {
             half8 bv;
             float sw, ow;
             if constexpr (T == FH_Q8_0) {
@@ -200,17 +212,25 @@ __device__ __forceinline__ void qb_chunk(const QbW<T> &W, const uint8_t *img, in
                 sw = fh_h2f((uint16_t)((s & 1) ? (dw >> 16) : (dw & 0xFFFF)));
                 ow = 8.f * sw;
             }
-            const half8 ah = *(const half8 *)(xa + 32 * s), al = *(const half8 *)(xa + L::PLANE + 32 * s);
+            const half8 ah = src.opnd(32 * s), al = src.opnd(L::PLANE + 32 * s);
             floatx4 r = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bv, zero, 0, 0, 0);
             r = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, bv, r, 0, 0, 0);
-            const float4 sv = *(const float4 *)(S + 16 * s);
+            const float4 sv = src.sum(16 * s);
             tot[0] = fmaf(sw, r[0], tot[0]); tot[1] = fmaf(sw, r[1], tot[1]);
             tot[2] = fmaf(sw, r[2], tot[2]); tot[3] = fmaf(sw, r[3], tot[3]);
             off[0] = fmaf(ow, sv.x, off[0]); off[1] = fmaf(ow, sv.y, off[1]);
             off[2] = fmaf(ow, sv.z, off[2]); off[3] = fmaf(ow, sv.w, off[3]);
         }
     }
-    const float4 fv = *(const float4 *)((const float *)(img + L::F_OFF) + 4 * g);
+}
+
+// yacc[i] += factor[m] * sum_blocks scale * (codes . x_scaled) - sum_blocks offset * sum(x), m = 4g + i.
+template <int T, int MR>
+__device__ __forceinline__ void qb_chunk(const QbW<T> &W, const uint8_t *img, int lane, float *yacc) {
+    const QbLdsSrc<T, MR> src(img, lane);
+    float tot[4] = {0.f, 0.f, 0.f, 0.f}, off[4] = {0.f, 0.f, 0.f, 0.f};
+    qb_steps<T, MR, 0, 8>(W, src, tot, off);
+    const float4 fv = src.fac();
     yacc[0] += fv.x * tot[0] - off[0];
     yacc[1] += fv.y * tot[1] - off[1];
     yacc[2] += fv.z * tot[2] - off[2];
@@ -220,9 +240,24 @@ __device__ __forceinline__ void qb_chunk(const QbW<T> &W, const uint8_t *img, in
 // ------------------------------------------------------------------------------ staging of one activation row chunk
 // The wavefront holds row m of the chunk, lane c elements 4c .. 4c+3.  Positions inside the LDS row follow the
 // order in which the format's code masks deliver the weights of a lane (see qb_chunk).
-template <int T, int MR>
+// Image of one chunk for the kernel that reads its operands straight from memory: the sixteen A operands of a
+// chunk in the order the multiply asks for them (32-group s: hi 2s, lo 2s+1; Q6_K: 16-group G: hi | lo in operand G),
+// each as the 64 lanes' 16 bytes back to back (one fully used 1 KB request per operand), then sums and factors.
+template <int T>
+struct QdImg {
+    static constexpr int NG = T == FH_Q6_K ? 16 : 8;
+    static constexpr int S_OFF = 16 * 1024, F_OFF = S_OFF + NG * 16 * 4, BYTES = F_OFF + 64;
+    // byte offset of half `pos` (a multiple of 4) of plane `plane` of row m
+    __device__ static __forceinline__ int at(int pos, int plane, int m) {
+        const int opnd = T == FH_Q6_K ? pos / 32 : 2 * (pos / 32) + plane;
+        return (opnd * 64 + ((pos % 32) / 8) * 16 + m) * 16 + (pos % 8) * 2;
+    }
+};
+
+template <int T, int MR, bool FRAG = false>
 __device__ __forceinline__ void qb_stage(uint8_t *img, int m, int lane, float4 v) {
     typedef QbLds<T, MR> L;
+    constexpr int S_OFF = FRAG ? QdImg<T>::S_OFF : L::S_OFF, F_OFF = FRAG ? QdImg<T>::F_OFF : L::F_OFF;
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     amax = fmaxf(amax, qb_dpp<QB_DPP_XOR1>(amax));
     amax = fmaxf(amax, qb_dpp<QB_DPP_XOR2>(amax));
@@ -250,11 +285,16 @@ __device__ __forceinline__ void qb_stage(uint8_t *img, int m, int lane, float4 v
     float s4 = (v.x + v.y) + (v.z + v.w);
     s4 += qb_dpp<QB_DPP_XOR1>(s4);
     s4 += qb_dpp<QB_DPP_XOR2>(s4);
-    float *S = (float *)(img + L::S_OFF);
+    float *S = (float *)(img + S_OFF);
     if (T == FH_Q6_K) {
         const int G = lane >> 2, e0 = 4 * (lane & 3);
-        *(uint2 *)(row + 32 * G + e0) = ph;
-        *(uint2 *)(row + 32 * G + 16 + e0) = pl;
+        if constexpr (FRAG) {
+            *(uint2 *)(img + QdImg<T>::at(32 * G + e0, 0, m)) = ph;
+            *(uint2 *)(img + QdImg<T>::at(32 * G + 16 + e0, 0, m)) = pl;
+        } else {
+            *(uint2 *)(row + 32 * G + e0) = ph;
+            *(uint2 *)(row + 32 * G + 16 + e0) = pl;
+        }
         if ((lane & 3) == 0) S[G * 16 + m] = s4;
     } else {
         int pos = 4 * lane;
@@ -262,25 +302,30 @@ __device__ __forceinline__ void qb_stage(uint8_t *img, int m, int lane, float4 v
             const int c = lane & 7;
             pos = 32 * (lane >> 3) + (c < 4 ? 8 * c : 8 * (c - 4) + 4);
         }
-        *(uint2 *)(row + pos) = ph;
-        *(uint2 *)(row + L::PLANE + pos) = pl;
+        if constexpr (FRAG) {
+            *(uint2 *)(img + QdImg<T>::at(pos, 0, m)) = ph;
+            *(uint2 *)(img + QdImg<T>::at(pos, 1, m)) = pl;
+        } else {
+            *(uint2 *)(row + pos) = ph;
+            *(uint2 *)(row + L::PLANE + pos) = pl;
+        }
         s4 += qb_dpp<QB_DPP_HALF_MIRROR>(s4);
         if ((lane & 7) == 0) S[(lane >> 3) * 16 + m] = s4;
     }
-    if (lane == 0) ((float *)(img + L::F_OFF))[m] = __uint_as_float((uint32_t)(24 - e + 127) << 23);
+    if (lane == 0) ((float *)(img + F_OFF))[m] = __uint_as_float((uint32_t)(24 - e + 127) << 23);
 }
 
 // ------------------------------------------------------------------------------ kernel
 // MR: activation rows held per image (4 or 16, m <= MR); TW x TS = 8 wavefronts; D weight chunks in flight.
 // One wavefront per (chunk, row): the LDS image of every chunk, written to global memory [chunk][image bytes].
-template <int T, int MR>
+template <int T, int MR, bool FRAG = false>
 __global__ __launch_bounds__(256) void k_qb_prep(const float *__restrict__ x, int M, int64_t K, uint8_t *__restrict__ out) {
     typedef QbLds<T, MR> L;
-    constexpr int IMG = (L::BYTES + 15) & ~15;
+    constexpr int IMG = FRAG ? QdImg<T>::BYTES : (L::BYTES + 15) & ~15;
     const int lane = threadIdx.x & 63, m = blockIdx.y * 4 + (threadIdx.x >> 6), c = blockIdx.x;
     if (m >= M) return;
     const float4 v = *(const float4 *)(x + (int64_t)m * K + (int64_t)c * 256 + lane * 4);
-    qb_stage<T, MR>(out + (int64_t)c * IMG, m, lane, v);
+    qb_stage<T, MR, FRAG>(out + (int64_t)c * IMG, m, lane, v);
 }
 
 template <int T, int MR, int TW, int TS, int EPI, bool PRE>
@@ -427,19 +472,196 @@ static fh_status qb_launch(const fh_qmatrix *q, const float *x, int m, float *y,
     return FH_OK;
 }
 
+// ------------------------------------------------------------------------------ images read straight from memory
+// A second kernel for the same product: one wavefront per (row tile(s), chunk), no staging.  The wavefront reads
+// the activation operands of its chunk from the image k_qb_prep wrote (16 rows; it stays in the L2) half a chunk
+// at a time into registers, requests its weights once, and multiplies.  Nothing waits for another wavefront until
+// the slices are added, so a chunk costs one memory round trip instead of a staged round with a barrier.  Long k
+// is cut into gridDim.y parts whose partial sums a second launch adds in a fixed order.
+template <int T>
+struct QdRegs {
+    typedef QbLds<T, 16> L;
+    static constexpr int NS = T == FH_Q6_K ? 8 : 4;
+    half8 a[8];
+    float4 s[NS];
+    template <int H>
+    __device__ __forceinline__ void load(const uint8_t *img, int lane) {
+        const uint8_t *A = img + lane * 16;
+        const float *S = (const float *)(img + QdImg<T>::S_OFF) + 4 * (lane >> 4);
+        if constexpr (T == FH_Q6_K) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) a[i] = *(const half8 *)(A + (8 * H + i) * 1024);
+#pragma unroll
+            for (int i = 0; i < 8; i++) s[i] = *(const float4 *)(S + 16 * (8 * H + i));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                a[i] = *(const half8 *)(A + (2 * (4 * H + i)) * 1024);
+                a[4 + i] = *(const half8 *)(A + (2 * (4 * H + i) + 1) * 1024);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) s[i] = *(const float4 *)(S + 16 * (4 * H + i));
+        }
+    }
+    // the offsets qb_steps asks for, folded to register indices (its loops are unrolled: `off` is a constant)
+    __device__ __forceinline__ half8 opnd(int off) const {
+        if constexpr (T == FH_Q6_K) return a[(off / 32) & 7];
+        else return off >= L::PLANE ? a[4 + (((off - L::PLANE) / 32) & 3)] : a[(off / 32) & 3];
+    }
+    __device__ __forceinline__ float4 sum(int off) const { return s[(off / 16) & (NS - 1)]; }
+};
+
+template <int T, int TPW, int EPI>
+__global__ __launch_bounds__(1024) void k_qmv_direct(QView q, const uint8_t *__restrict__ ximg, int M, int cps,
+                                                     float *__restrict__ y, float *__restrict__ part,
+                                                     const float *__restrict__ ea, const float *__restrict__ eb) {
+    constexpr int IMG = QdImg<T>::BYTES;
+    constexpr int NT = EPI == FH_EPI_SWIGLU ? 2 : 1, TOUT = TPW / NT;
+    extern __shared__ float qd_o[]; // [wavefront][TPW][16 rows][17]
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int j = lane & 15, g = lane >> 4, SW = blockDim.x >> 6;
+    const int C = (int)(q.k >> 8);
+    const int64_t nout = NT == 2 ? q.n / 2 : q.n, tiles_out = (nout + 15) / 16;
+    const int c = blockIdx.y * cps + wave;
+    float yacc[TPW][4];
+#pragma unroll
+    for (int tp = 0; tp < TPW; tp++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) yacc[tp][i] = 0.f;
+    if (wave < cps && c < C) { // uniform per wavefront
+        const uint8_t *img = ximg + (size_t)c * IMG;
+        QdRegs<T> a;
+        a.template load<0>(img, lane);
+        __builtin_amdgcn_sched_barrier(0); // activations (L2) are requested ahead of the weights (HBM)
+        QbW<T> w[TPW];
+#pragma unroll
+        for (int tp = 0; tp < TPW; tp++) {
+            int64_t to = (int64_t)blockIdx.x * TOUT + (tp % TOUT);
+            if (to >= tiles_out) to = tiles_out - 1; // a tile past the end re-reads the last one; never stored
+            w[tp].load(q, to + (int64_t)(tp / TOUT) * (nout / 16), c, lane);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        float tot[TPW][4], off[TPW][4];
+#pragma unroll
+        for (int tp = 0; tp < TPW; tp++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) tot[tp][i] = off[tp][i] = 0.f;
+#pragma unroll
+        for (int tp = 0; tp < TPW; tp++) qb_steps<T, 16, 0, 4>(w[tp], a, tot[tp], off[tp]);
+        __builtin_amdgcn_sched_barrier(0);
+        a.template load<1>(img, lane);
+        const float4 fv = *(const float4 *)((const float *)(img + QdImg<T>::F_OFF) + 4 * g);
+#pragma unroll
+        for (int tp = 0; tp < TPW; tp++) {
+            qb_steps<T, 16, 4, 8>(w[tp], a, tot[tp], off[tp]);
+            yacc[tp][0] = fv.x * tot[tp][0] - off[tp][0];
+            yacc[tp][1] = fv.y * tot[tp][1] - off[tp][1];
+            yacc[tp][2] = fv.z * tot[tp][2] - off[tp][2];
+            yacc[tp][3] = fv.w * tot[tp][3] - off[tp][3];
+        }
+    }
+#pragma unroll
+    for (int tp = 0; tp < TPW; tp++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) qd_o[((wave * TPW + tp) * 16 + 4 * g + i) * 17 + j] = yacc[tp][i];
+    __syncthreads();
+    auto total = [&](int tp, int m, int jn) { // slices in wavefront order
+        float s = 0.f;
+        for (int w2 = 0; w2 < SW; w2++) s += qd_o[((w2 * TPW + tp) * 16 + m) * 17 + jn];
+        return s;
+    };
+    if (part) { // partial sums of this k part, one row of `part` per (part, activation row): [gridDim.y][16][q.n]
+        for (int e = tid; e < TPW * 256; e += blockDim.x) {
+            const int tp = e >> 8, m = (e >> 4) & 15, jn = e & 15;
+            const int64_t to = (int64_t)blockIdx.x * TOUT + (tp % TOUT);
+            const int64_t row = (to + (int64_t)(tp / TOUT) * (nout / 16)) * 16 + jn;
+            if (m < M && to < tiles_out && row < q.n) part[((int64_t)blockIdx.y * 16 + m) * q.n + row] = total(tp, m, jn);
+        }
+        return;
+    }
+    for (int e = tid; e < TOUT * 256; e += blockDim.x) {
+        const int t2 = e >> 8, m = (e >> 4) & 15, jn = e & 15;
+        const int64_t n = ((int64_t)blockIdx.x * TOUT + t2) * 16 + jn;
+        if (m < M && n < nout) {
+            float rr = total(t2, m, jn);
+            const int64_t at = (int64_t)m * nout + n;
+            if (EPI == FH_EPI_ADD2) rr = (rr + ea[at]) + eb[at];
+            if (EPI == FH_EPI_SWIGLU) rr = (rr / (__expf(-rr) + 1.0f)) * total(t2 + TOUT, m, jn);
+            y[at] = rr;
+        }
+    }
+}
+
+// y = epilogue(sum over the k parts), parts added in order.
+template <int EPI>
+__global__ __launch_bounds__(256) void k_qd_reduce(const float *__restrict__ part, int parts, int M, int64_t nfull,
+                                                   int64_t nout, float *__restrict__ y, const float *__restrict__ ea,
+                                                   const float *__restrict__ eb) {
+    const int64_t at = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (at >= (int64_t)M * nout) return;
+    const int m = (int)(at / nout);
+    const int64_t n = at % nout;
+    float rr = 0.f, up = 0.f;
+    for (int p = 0; p < parts; p++) {
+        rr += part[((int64_t)p * 16 + m) * nfull + n];
+        if (EPI == FH_EPI_SWIGLU) up += part[((int64_t)p * 16 + m) * nfull + nout + n];
+    }
+    if (EPI == FH_EPI_ADD2) rr = (rr + ea[at]) + eb[at];
+    if (EPI == FH_EPI_SWIGLU) rr = (rr / (__expf(-rr) + 1.0f)) * up;
+    y[at] = rr;
+}
+
+template <int T, int EPI>
+static fh_status qd_launch(const fh_qmatrix *q, const float *x, int m, float *y, const float *a, const float *b) {
+    fh_device *dev = q->dev;
+    constexpr int IMG = QdImg<T>::BYTES;
+    const int C = (int)(q->k / 256);
+    const int parts = (C + 15) / 16, cps = (C + parts - 1) / parts; // at most 16 wavefronts (chunks) per workgroup
+    const int64_t nout = EPI == FH_EPI_SWIGLU ? q->n / 2 : q->n, tiles = (nout + 15) / 16;
+    // two tiles per wavefront share the activation operands once the device is covered more than twice
+    const int64_t force = dev->opt_matvec_tiles;
+    const bool two = EPI == FH_EPI_SWIGLU || force == 2 || (force == 0 && tiles * parts > 2 * (int64_t)dev->compute_units);
+    const int64_t groups = EPI == FH_EPI_SWIGLU ? tiles : (two ? (tiles + 1) / 2 : tiles);
+    FH_REQUIRE(groups <= 0x7FFFFFFF, "matrix too large for one launch");
+    FH_TRY(fh_dev_scratch(dev, &dev->act_buf, &dev->act_cap, (size_t)C * IMG));
+    float *part = nullptr;
+    if (parts > 1) {
+        FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, (size_t)parts * 16 * q->n * 4));
+        part = (float *)dev->ksplit_buf;
+    }
+    k_qb_prep<T, 16, true><<<dim3((unsigned)C, (unsigned)((m + 3) / 4)), dim3(256), 0, dev->stream>>>(
+        x, m, q->k, (uint8_t *)dev->act_buf);
+    const dim3 grid((unsigned)groups, (unsigned)parts), block(64 * cps);
+    const size_t lds = (size_t)cps * (two ? 2 : 1) * 16 * 17 * 4;
+    if (two)
+        k_qmv_direct<T, 2, EPI><<<grid, block, lds, dev->stream>>>(fh_view(q), (const uint8_t *)dev->act_buf, m, cps, y,
+                                                                  part, a, b);
+    else if constexpr (EPI != FH_EPI_SWIGLU)
+        k_qmv_direct<T, 1, EPI><<<grid, block, lds, dev->stream>>>(fh_view(q), (const uint8_t *)dev->act_buf, m, cps, y,
+                                                                  part, a, b);
+    if (part) {
+        const int64_t total = (int64_t)m * nout;
+        k_qd_reduce<EPI><<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream>>>(part, parts, m, q->n, nout, y,
+                                                                                              a, b);
+    }
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
 // m <= 4: one tile (SwiGLU: gate + up tile) per workgroup, k over 8 (4) slices.  m <= 16: four tiles, two slices:
 // the staged activations (4 bytes per element and row) are then shared by enough weight rows.
 template <int T, int EPI>
 static fh_status qb_shape(const fh_qmatrix *q, const float *x, int m, float *y, const float *a, const float *b) {
     const int64_t tiles = (q->n + 15) / 16;
     const int64_t force = q->dev->opt_matvec_tiles; // 0 auto, else tiles per workgroup
-    if (m <= 4) {
+    if (m <= 4 && q->dev->opt_matvec_direct != 2) {
         if constexpr (EPI == FH_EPI_SWIGLU) return qb_launch<T, 4, 2, 4, EPI>(q, x, m, y, a, b);
         else {
             if (force == 2 || (force == 0 && tiles >= 512)) return qb_launch<T, 4, 2, 4, EPI>(q, x, m, y, a, b);
             return qb_launch<T, 4, 1, 8, EPI>(q, x, m, y, a, b);
         }
     }
+    if (q->dev->opt_matvec_direct != 1) return qd_launch<T, EPI>(q, x, m, y, a, b);
     if (force == 2 || (force == 0 && tiles <= 512)) return qb_launch<T, 16, 2, 4, EPI>(q, x, m, y, a, b);
     return qb_launch<T, 16, 4, 2, EPI>(q, x, m, y, a, b);
 }
