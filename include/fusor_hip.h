@@ -48,8 +48,10 @@ enum {
     FH_ERR_NOT_FOUND = -7    /* Error::VarBuilder "Key ... not found" (fusor-ml/fusor/src/varbuilder.rs:81-83) */
 };
 
-/* GgmlType ids, fusor-ml/gguf/src/lib.rs:35-50 */
-enum { FH_Q4_0 = 2, FH_Q8_0 = 8, FH_Q4_K = 12, FH_Q6_K = 14 };
+/* GgmlType ids, fusor-ml/gguf/src/lib.rs:35-50.  Q4_0, Q8_0, Q4_K and Q6_K weights are re-laid-out for the
+ * matrix-core kernels; Q5_0, Q5_K and dense F32 (0) / F16 (1) weights keep the file's layout and run through
+ * the per-element kernels (every fh_qmatrix_* call, fh_embed_rows, fh_qmatmul, fh_qmatmul_add2 / _swiglu). */
+enum { FH_Q4_0 = 2, FH_Q5_0 = 6, FH_Q8_0 = 8, FH_Q4_K = 12, FH_Q5_K = 13, FH_Q6_K = 14 };
 
 /* MaskKind, fusor-ml/fusor/src/composite/flash_attention.rs:12-24 */
 enum { FH_MASK_NONE = 0, FH_MASK_CAUSAL = 1, FH_MASK_ADDITIVE = 2 };

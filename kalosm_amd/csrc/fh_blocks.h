@@ -125,8 +125,48 @@ __device__ __forceinline__ float deq_elem_q6_k(const QView &q, int64_t row, int6
     return ds * (float)v;
 }
 
+// ---- formats kept in the file's block order: block b of row `row` starts at (row * kb + b) * block bytes
+// BlockQ5_0::dequantize, gguf/src/lib.rs:1046-1073: f16 d | 32 high bits | 16 bytes of nibbles;
+// element i < 16: low nibble of byte i with bit i, element i + 16: high nibble with bit i + 16; (code - 16) * d
+__device__ __forceinline__ float deq_elem_q5_0(const QView &q, int64_t row, int64_t k) {
+    const uint8_t *blk = q.data + (row * q.kb + (k >> 5)) * 22;
+    const int e = (int)(k & 31);
+    const float d = fh_h2f(fh_ld16(blk));
+    const uint32_t qh = (uint32_t)fh_ld16(blk + 2) | ((uint32_t)fh_ld16(blk + 4) << 16);
+    const uint8_t byte = blk[6 + (e & 15)];
+    const int nib = e < 16 ? (byte & 0x0F) : (byte >> 4);
+    const int v = (nib | (int)(((qh >> e) & 1u) << 4)) - 16;
+    return (float)v * d;
+}
+// BlockQ5K::dequantize, gguf/src/lib.rs:1819-1861: f16 d | f16 dmin | 12 scale bytes | qh[32] | qs[128];
+// sub-block s (32 elements): nibble of qs[32 (s / 2) + l] (low for even s) + 16 * bit s of qh[l];
+// (sc * d) * code - mn * dmin
+__device__ __forceinline__ float deq_elem_q5_k(const QView &q, int64_t row, int64_t k) {
+    const uint8_t *blk = q.data + (row * q.kb + (k >> 8)) * 176;
+    const int e = (int)(k & 255), s = e >> 5, l = e & 31;
+    const float d = fh_h2f(fh_ld16(blk)), dmin = fh_h2f(fh_ld16(blk + 2));
+    int sc, mn;
+    q4k_scale_min(blk + 4, s, sc, mn);
+    const uint8_t ql = blk[48 + 32 * (s >> 1) + l], qh = blk[16 + l];
+    const int v = ((s & 1) ? (ql >> 4) : (ql & 0x0F)) + (((qh >> s) & 1) ? 16 : 0);
+    const float scale = (float)sc * d;
+    const float off = (float)mn * dmin;
+    const float prod = scale * (float)v;
+    return prod - off;
+}
+__device__ __forceinline__ float deq_elem_f16(const QView &q, int64_t row, int64_t k) {
+    return fh_h2f(((const uint16_t *)q.data)[row * q.k + k]);
+}
+__device__ __forceinline__ float deq_elem_f32(const QView &q, int64_t row, int64_t k) {
+    return ((const float *)q.data)[row * q.k + k];
+}
+
 template <int T>
 __device__ __forceinline__ float deq_elem(const QView &q, int64_t row, int64_t k) {
+    if (T == FH_Q5_0) return deq_elem_q5_0(q, row, k);
+    if (T == FH_Q5_K) return deq_elem_q5_k(q, row, k);
+    if (T == 0) return deq_elem_f32(q, row, k);
+    if (T == 1) return deq_elem_f16(q, row, k);
     if (T == FH_Q4_0) return deq_elem_q4_0(q, row, k);
     if (T == FH_Q8_0) return deq_elem_q8_0(q, row, k);
     if (T == FH_Q4_K) return deq_elem_q4_k(q, row, k);

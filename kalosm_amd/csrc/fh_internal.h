@@ -111,18 +111,27 @@ struct fh_qmatrix {
     size_t bytes = 0;
 };
 
+// Weight types kept in the file's own row-major block order (no tiled re-layout): dense f32 / f16 rows and the
+// 5-bit formats.  They run through the per-element kernels only.
+enum { FH_W_F32 = 0, FH_W_F16 = 1 };
+static inline bool fh_is_plain(uint32_t t) { return t == FH_W_F32 || t == FH_W_F16 || t == FH_Q5_0 || t == FH_Q5_K; }
 static inline int fh_block_elems(uint32_t t) {
     switch (t) {
-    case FH_Q4_0: case FH_Q8_0: return 32;
-    case FH_Q4_K: case FH_Q6_K: return 256;
+    case FH_W_F32: case FH_W_F16: return 1;
+    case FH_Q4_0: case FH_Q8_0: case FH_Q5_0: return 32;
+    case FH_Q4_K: case FH_Q6_K: case FH_Q5_K: return 256;
     default: return 0;
     }
 }
-static inline int fh_block_bytes(uint32_t t) {
+static inline int fh_block_bytes(uint32_t t) { // gguf/src/lib.rs:109-121
     switch (t) {
+    case FH_W_F32: return 4;
+    case FH_W_F16: return 2;
     case FH_Q4_0: return 18;
+    case FH_Q5_0: return 22;
     case FH_Q8_0: return 34;
     case FH_Q4_K: return 144;
+    case FH_Q5_K: return 176;
     case FH_Q6_K: return 210;
     default: return 0;
     }

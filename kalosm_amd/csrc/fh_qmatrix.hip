@@ -76,7 +76,9 @@ __global__ void k_repack_q4_0(const uint8_t *__restrict__ src, uint8_t *__restri
 
 static fh_status qm_alloc(fh_device *dev, uint32_t type, int64_t n, int64_t k, fh_qmatrix **out) {
     int e = fh_block_elems(type);
-    if (!e) FH_FAIL(FH_ERR_UNSUPPORTED, "unsupported ggml type %u (supported: Q4_0=2, Q8_0=8, Q4_K=12, Q6_K=14)", type);
+    if (!e)
+        FH_FAIL(FH_ERR_UNSUPPORTED, "unsupported ggml type %u (supported: F32=0, F16=1, Q4_0=2, Q5_0=6, Q8_0=8, Q4_K=12, "
+                                    "Q5_K=13, Q6_K=14)", type);
     FH_REQUIRE(n > 0 && k > 0, "empty weight [%lld, %lld]", (long long)n, (long long)k);
     FH_REQUIRE(k % e == 0, "k=%lld is not a multiple of the block size %d", (long long)k, e);
     FH_REQUIRE(n < (1ll << 31) && k < (1ll << 31), "weight too large");
@@ -91,6 +93,11 @@ static fh_status qm_alloc(fh_device *dev, uint32_t type, int64_t n, int64_t k, f
     q->recs = (q->kb + rb - 1) / rb;
     q->rec_bytes = fh_rec_bytes(type);
     q->bytes = (size_t)(q->n_pad / 16) * (size_t)q->recs * (size_t)q->rec_bytes;
+    if (fh_is_plain(type)) { // the file's own layout: rows of kb blocks
+        q->recs = 0;
+        q->rec_bytes = fh_block_bytes(type);
+        q->bytes = (size_t)n * (size_t)q->kb * (size_t)fh_block_bytes(type);
+    }
     hipError_t err = hipMalloc((void **)&q->data, q->bytes + 256); // slack: kernels may prefetch one record ahead
     if (err != hipSuccess) {
         delete q;
@@ -113,6 +120,17 @@ extern "C" fh_status fh_qmatrix_from_gguf_bytes(fh_device *dev, uint32_t ggml_ty
         fh_qmatrix_free(q);
         FH_FAIL(FH_ERR_INVALID, "byte length %zu does not match [%lld, %lld] of type %u (%zu expected)", len,
                 (long long)n, (long long)k, ggml_type, want);
+    }
+    if (fh_is_plain(ggml_type)) {
+        hipError_t e = hipMemcpyAsync(q->data, bytes, len, hipMemcpyHostToDevice, dev->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(dev->stream);
+        if (e != hipSuccess) {
+            fh_qmatrix_free(q);
+            FH_FAIL(FH_ERR_HIP, "upload of a [%lld, %lld] type-%u weight failed: %s", (long long)n, (long long)k, ggml_type,
+                    hipGetErrorString(e));
+        }
+        *out = q;
+        return FH_OK;
     }
     uint8_t *staging = nullptr;
     hipError_t err = hipMalloc((void **)&staging, len);
@@ -175,7 +193,7 @@ extern "C" fh_status fh_qmatrix_concat_rows(fh_device *dev, const fh_qmatrix *co
         // Option::None in the reference (fusor-ml/core/src/quantized/mod.rs:329-337)
         if (parts[i]->type != parts[0]->type || parts[i]->k != parts[0]->k)
             FH_FAIL(FH_ERR_UNSUPPORTED, "concat_rows needs one type and one k (part %d differs)", i);
-        if (i + 1 < count && parts[i]->n % 16 != 0)
+        if (i + 1 < count && parts[i]->n % 16 != 0 && !fh_is_plain(parts[0]->type))
             FH_FAIL(FH_ERR_UNSUPPORTED, "concat_rows: part %d has %lld rows, not a multiple of 16", i,
                     (long long)parts[i]->n);
         n += parts[i]->n;
@@ -217,6 +235,10 @@ extern "C" fh_status fh_qmatrix_dequantize(const fh_qmatrix *q, float *out_dev) 
     case FH_Q8_0: k_dequantize<FH_Q8_0><<<grid, block, 0, s>>>(v, out_dev); break;
     case FH_Q4_K: k_dequantize<FH_Q4_K><<<grid, block, 0, s>>>(v, out_dev); break;
     case FH_Q6_K: k_dequantize<FH_Q6_K><<<grid, block, 0, s>>>(v, out_dev); break;
+    case FH_Q5_0: k_dequantize<FH_Q5_0><<<grid, block, 0, s>>>(v, out_dev); break;
+    case FH_Q5_K: k_dequantize<FH_Q5_K><<<grid, block, 0, s>>>(v, out_dev); break;
+    case FH_W_F32: k_dequantize<FH_W_F32><<<grid, block, 0, s>>>(v, out_dev); break;
+    case FH_W_F16: k_dequantize<FH_W_F16><<<grid, block, 0, s>>>(v, out_dev); break;
     }
     FH_HIP(hipGetLastError());
     return FH_OK;
@@ -251,6 +273,10 @@ extern "C" fh_status fh_embed_rows(const fh_qmatrix *q, const uint32_t *ids_dev,
     case FH_Q8_0: k_embed_rows<FH_Q8_0><<<grid, block, 0, s>>>(v, ids_dev, count, out_dev); break;
     case FH_Q4_K: k_embed_rows<FH_Q4_K><<<grid, block, 0, s>>>(v, ids_dev, count, out_dev); break;
     case FH_Q6_K: k_embed_rows<FH_Q6_K><<<grid, block, 0, s>>>(v, ids_dev, count, out_dev); break;
+    case FH_Q5_0: k_embed_rows<FH_Q5_0><<<grid, block, 0, s>>>(v, ids_dev, count, out_dev); break;
+    case FH_Q5_K: k_embed_rows<FH_Q5_K><<<grid, block, 0, s>>>(v, ids_dev, count, out_dev); break;
+    case FH_W_F32: k_embed_rows<FH_W_F32><<<grid, block, 0, s>>>(v, ids_dev, count, out_dev); break;
+    case FH_W_F16: k_embed_rows<FH_W_F16><<<grid, block, 0, s>>>(v, ids_dev, count, out_dev); break;
     }
     FH_HIP(hipGetLastError());
     return FH_OK;

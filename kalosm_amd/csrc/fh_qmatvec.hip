@@ -360,7 +360,7 @@ fh_status fh_launch_qmatvec(const fh_qmatrix *q, const float *x, int m, float *y
         fh_status st = fh_launch_q4k_m1(q, x, y, epi, a, b);
         if (st != FH_ERR_UNSUPPORTED) return st;
     }
-    if (kernel == 0 && q->type != FH_Q6_K && m >= 2 && m <= 4 && dev->opt_matvec_rows != 1) {
+    if (kernel == 0 && q->type != FH_Q6_K && !fh_is_plain(q->type) && m >= 2 && m <= 4 && dev->opt_matvec_rows != 1) {
         fh_status st = fh_launch_q4k_rows(q, x, m, y, epi, a, b);
         if (st != FH_ERR_UNSUPPORTED) return st;
     }
@@ -378,6 +378,10 @@ fh_status fh_launch_qmatvec(const fh_qmatrix *q, const float *x, int m, float *y
     case FH_Q8_0: return launch_generic<FH_Q8_0>(q, x, m, y, epi, a, b);
     case FH_Q4_K: return launch_generic<FH_Q4_K>(q, x, m, y, epi, a, b);
     case FH_Q6_K: return launch_generic<FH_Q6_K>(q, x, m, y, epi, a, b);
+    case FH_Q5_0: return launch_generic<FH_Q5_0>(q, x, m, y, epi, a, b);
+    case FH_Q5_K: return launch_generic<FH_Q5_K>(q, x, m, y, epi, a, b);
+    case FH_W_F32: return launch_generic<FH_W_F32>(q, x, m, y, epi, a, b);
+    case FH_W_F16: return launch_generic<FH_W_F16>(q, x, m, y, epi, a, b);
     }
     FH_FAIL(FH_ERR_UNSUPPORTED, "unsupported type %u", q->type);
 }
@@ -391,7 +395,7 @@ static fh_status qmm_check(const fh_qmatrix *q, const void *x, int m, const void
 extern "C" fh_status fh_qmatmul(const fh_qmatrix *q, const float *x_dev, int32_t m, float *y_dev) {
     FH_TRY(qmm_check(q, x_dev, m, y_dev));
     const int64_t mk = q->dev->opt_matmul_kernel;
-    if ((m > 16 && mk != 1) || mk >= 2) return fh_launch_qmatmul_tile(q, x_dev, 0, m, y_dev);
+    if (((m > 16 && mk != 1) || mk >= 2) && !fh_is_plain(q->type)) return fh_launch_qmatmul_tile(q, x_dev, 0, m, y_dev);
     return fh_launch_qmatvec(q, x_dev, m, y_dev, FH_EPI_NONE, nullptr, nullptr);
 }
 

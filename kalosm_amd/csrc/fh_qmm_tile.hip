@@ -574,6 +574,8 @@ static fh_status qmm_launch_t(const fh_qmatrix *q, const _Float16 *xh, const _Fl
 fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y) {
     fh_device *dev = q->dev;
     const int64_t K = q->k;
+    if (fh_is_plain(q->type))
+        FH_FAIL(FH_ERR_UNSUPPORTED, "type %u has no matrix-core matmul (f32 activations run through fh_qmatmul)", q->type);
     FH_REQUIRE((m + 127) / 128 <= 65535, "m = %d too large for one launch", m);
     // planes: xh | xl | rs
     const size_t plane = ((size_t)m * K * 2 + 255) & ~(size_t)255;

@@ -10,9 +10,11 @@ from __future__ import annotations
 import numpy as np
 
 Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
-BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256}
-BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210}
-TYPE_NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
+W_F32, W_F16, Q5_0, Q5_K = 0, 1, 6, 13  # kept in the file's layout by the library (per-element kernels)
+BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, W_F32: 1, W_F16: 1, Q5_0: 32, Q5_K: 256}
+BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, W_F32: 4, W_F16: 2, Q5_0: 22, Q5_K: 176}
+TYPE_NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", W_F32: "F32", W_F16: "F16", Q5_0: "Q5_0",
+              Q5_K: "Q5_K"}
 
 
 def f16_bytes(x: np.ndarray) -> np.ndarray:
@@ -52,6 +54,20 @@ def random_blocks(ggml_type: int, nblocks: int, rng: np.random.Generator, sigma:
         out[:, 0:192] = rng.integers(0, 256, (nblocks, 192), dtype=np.uint8)
         out[:, 192:208] = rng.integers(-128, 128, (nblocks, 16), dtype=np.int8).view(np.uint8)
         out[:, 208:210] = f16_bytes(rng.normal(0.0, sigma, nblocks))
+    elif ggml_type == Q5_0:
+        out[:, 0:2] = f16_bytes(rng.normal(0.0, sigma, nblocks))
+        out[:, 2:22] = rng.integers(0, 256, (nblocks, 20), dtype=np.uint8)
+    elif ggml_type == Q5_K:
+        out[:, 0:2] = f16_bytes(rng.normal(0.0, sigma, nblocks))
+        out[:, 2:4] = f16_bytes(rng.normal(0.0, sigma, nblocks))
+        sc = rng.integers(0, 64, (nblocks, 8), dtype=np.uint8)
+        mn = rng.integers(0, 64, (nblocks, 8), dtype=np.uint8)
+        out[:, 4:16] = pack_k4_scales(sc, mn)
+        out[:, 16:176] = rng.integers(0, 256, (nblocks, 160), dtype=np.uint8)
+    elif ggml_type == W_F16:
+        out[:, 0:2] = f16_bytes(rng.normal(0.0, sigma * 100.0, nblocks))
+    elif ggml_type == W_F32:
+        out[:] = rng.normal(0.0, sigma * 100.0, nblocks).astype(np.float32).view(np.uint8).reshape(nblocks, 4)
     else:
         raise ValueError(f"unsupported type {ggml_type}")
     return out.reshape(-1)

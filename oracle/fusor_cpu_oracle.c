@@ -38,9 +38,13 @@
 #include <stdlib.h>
 #include <string.h>
 
+#define FO_F32 0
+#define FO_F16 1
 #define FO_Q4_0 2
+#define FO_Q5_0 6
 #define FO_Q8_0 8
 #define FO_Q4_K 12
+#define FO_Q5_K 13
 #define FO_Q6_K 14
 
 /* ---------------------------------------------------------------- f16 <-> f32
@@ -116,16 +120,21 @@ void fo_f32_to_f16_array(const float *f, uint16_t *h, size_t n) {
  * :1425-1432 (Q4_K, 144 B), :1933-1944 (Q6_K, 210 B; the f16 scale is LAST). */
 int fo_block_elems(int t) {
     switch (t) {
-    case FO_Q4_0: case FO_Q8_0: return 32;
-    case FO_Q4_K: case FO_Q6_K: return 256;
+    case FO_F32: case FO_F16: return 1;
+    case FO_Q4_0: case FO_Q8_0: case FO_Q5_0: return 32;
+    case FO_Q4_K: case FO_Q6_K: case FO_Q5_K: return 256;
     default: return 0;
     }
 }
 int fo_block_bytes(int t) {
     switch (t) {
+    case FO_F32: return 4;
+    case FO_F16: return 2;
     case FO_Q4_0: return 18;
+    case FO_Q5_0: return 22;  /* gguf/src/lib.rs:958-966 */
     case FO_Q8_0: return 34;
     case FO_Q4_K: return 144;
+    case FO_Q5_K: return 176; /* gguf/src/lib.rs:1703-1711 */
     case FO_Q6_K: return 210;
     default: return 0;
     }
@@ -206,8 +215,54 @@ static void deq_q6_k(const uint8_t *b, float *out) {
     }
 }
 
+/* gguf/src/lib.rs:1046-1073 (BlockQ5_0): f16 scale, 32 high bits (little-endian u32), 16 nibble bytes.
+ * element i takes bit i, element i + 16 bit i + 16; codes are centred at 16. */
+static void deq_q5_0(const uint8_t *b, float *out) {
+    float d = fo_f16_to_f32(rd16(b));
+    uint32_t hb = (uint32_t)b[2] | ((uint32_t)b[3] << 8) | ((uint32_t)b[4] << 16) | ((uint32_t)b[5] << 24);
+    for (int i = 0; i < 16; i++) {
+        uint8_t byte = b[6 + i];
+        uint8_t low = byte & 0x0F, high = byte >> 4;
+        uint8_t low_bit = (uint8_t)(((hb >> i) << 4) & 0x10);
+        uint8_t high_bit = (uint8_t)((hb >> (i + 12)) & 0x10);
+        int8_t lo = (int8_t)((low | low_bit) - 16), hi = (int8_t)((high | high_bit) - 16);
+        out[i] = (float)lo * d;
+        out[i + 16] = (float)hi * d;
+    }
+}
+
+/* gguf/src/lib.rs:1819-1861 (BlockQ5K): d, dmin, 12 packed scale bytes (the Q4_K packing), qh[32], qs[128].
+ * chunk c: d1 = sc[2c] * d, m1 = mn[2c] * dmin; low nibbles + 16 * bit 2c of qh[l], then high nibbles + bit 2c+1. */
+static void deq_q5_k(const uint8_t *b, float *out) {
+    float d = fo_f16_to_f32(rd16(b)), dmin = fo_f16_to_f32(rd16(b + 2));
+    uint8_t sc[8], mn[8];
+    fo_unpack_k4_scales(b + 4, sc, mn);
+    const uint8_t *qh = b + 16, *qs = b + 48;
+    uint8_t u1 = 1, u2 = 2;
+    for (int c = 0; c < 4; c++) {
+        float d1 = (float)sc[2 * c] * d, m1 = (float)mn[2 * c] * dmin;
+        float d2 = (float)sc[2 * c + 1] * d, m2 = (float)mn[2 * c + 1] * dmin;
+        for (int l = 0; l < 32; l++) {
+            uint8_t q = (uint8_t)((qs[32 * c + l] & 0xF) + ((qh[l] & u1) ? 16 : 0));
+            float p = d1 * (float)q;
+            out[64 * c + l] = p - m1;
+        }
+        for (int l = 0; l < 32; l++) {
+            uint8_t q = (uint8_t)((qs[32 * c + l] >> 4) + ((qh[l] & u2) ? 16 : 0));
+            float p = d2 * (float)q;
+            out[64 * c + 32 + l] = p - m2;
+        }
+        u1 = (uint8_t)(u1 << 2);
+        u2 = (uint8_t)(u2 << 2);
+    }
+}
+
 static void deq_block(int t, const uint8_t *b, float *out) {
     switch (t) {
+    case FO_F32: memcpy(out, b, 4); break;
+    case FO_F16: out[0] = fo_f16_to_f32(rd16(b)); break;
+    case FO_Q5_0: deq_q5_0(b, out); break;
+    case FO_Q5_K: deq_q5_k(b, out); break;
     case FO_Q4_0: deq_q4_0(b, out); break;
     case FO_Q8_0: deq_q8_0(b, out); break;
     case FO_Q4_K: deq_q4_k(b, out); break;
@@ -237,6 +292,23 @@ static float dot_row(int t, const float *x, const uint8_t *wrow, int blocks, int
     float acc[FO_MAX_LANES];
     float deq[256];
     for (int l = 0; l < lanes; l++) acc[l] = 0.0f;
+    if (e == 1) {
+        /* dense f32 / f16 rows: the reference multiplies them with its dense matmul (fusor/src/lib.rs:1183-1215 ->
+         * gemm crate, accumulation order not pinned); here the same lane fold over the row with a scalar tail */
+        int i = 0;
+        for (; i + lanes <= blocks; i += lanes)
+            for (int l = 0; l < lanes; l++) {
+                deq_block(t, wrow + (size_t)(i + l) * bb, deq);
+                acc[l] = fmaf(x[i + l], deq[0], acc[l]);
+            }
+        float s1 = 0.0f;
+        for (int l = 0; l < lanes; l++) s1 = s1 + acc[l];
+        for (; i < blocks; i++) {
+            deq_block(t, wrow + (size_t)i * bb, deq);
+            s1 = fmaf(x[i], deq[0], s1);
+        }
+        return s1;
+    }
     for (int b = 0; b < blocks; b++) {
         deq_block(t, wrow + (size_t)b * bb, deq);
         const float *xb = x + (size_t)b * e;
@@ -346,16 +418,19 @@ static void *qmm_fast_worker(void *arg) {
             const float *xr = j->x + (size_t)r * j->k;
             float acc[FO_MAX_LANES];
             for (int l = 0; l < L; l++) acc[l] = 0.0f;
+            int i = 0;
             if (L == 8) {
-                for (int i = 0; i < j->k; i += 8)
+                for (; i + 8 <= j->k; i += 8)
                     for (int l = 0; l < 8; l++) acc[l] = fmaf(xr[i + l], deq[i + l], acc[l]);
             } else {
-                for (int i = 0; i < j->k; i += L)
+                for (; i + L <= j->k; i += L)
                     for (int l = 0; l < L; l++) acc[l] = fmaf(xr[i + l], deq[i + l], acc[l]);
             }
             float s = 0.0f;
             for (int l = 0; l < L; l++) s = s + acc[l];
-            j->y[(size_t)r * j->n + c] = s + 0.0f;
+            s = s + 0.0f;
+            for (; i < j->k; i++) s = fmaf(xr[i], deq[i], s); /* dense rows whose length is no multiple of L */
+            j->y[(size_t)r * j->n + c] = s;
         }
     }
     free(deq);

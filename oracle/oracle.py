@@ -15,8 +15,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libfusor_cpu_oracle.so")
 
 Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
-BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256}
-BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210}
+BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, 0: 1, 1: 1, 6: 32, 13: 256}   # 0 f32, 1 f16, 6 Q5_0, 13 Q5_K
+BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, 0: 4, 1: 2, 6: 22, 13: 176}
 
 
 def build(force: bool = False) -> str:

@@ -231,7 +231,7 @@ def test_errors():
     assert e.value.status == _lib.FH_ERR_IO
 
 
-def llama_file(cfg, seed=0, arch="llama", extra_md=None, extra_tensors=(), rope_freqs=True, mixed=True):
+def llama_file(cfg, seed=0, arch="llama", extra_md=None, extra_tensors=(), rope_freqs=True, mixed=True, five_bit=False):
     """A small random-init decoder file in the tensor naming of models/kalosm-llama/src/raw/mod.rs:473-604."""
     from kalosm_amd import synth
     rng = np.random.default_rng(seed)
@@ -254,20 +254,24 @@ def llama_file(cfg, seed=0, arch="llama", extra_md=None, extra_tensors=(), rope_
             tensors.append((name, 0, (n,), v.view(np.uint8)))
             weights[name] = v
 
-    q("token_embd.weight", 12, V, D, 1)
+    if five_bit:  # the 5-bit formats and dense f16 rows, as Q5_K_M / Q5_0 files and f16 output heads hold them
+        t_embd, t_o, t_down, t_out = 6, 13, 6, 1
+    else:
+        t_embd, t_o, t_down, t_out = 12, 12, None, 14
+    q("token_embd.weight", t_embd, V, D, 1)
     for l in range(cfg["n_layers"]):
         p = f"blk.{l}."
         f(p + "attn_norm.weight", D)
         q(p + "attn_q.weight", 12, QD, D, 10 * l + 2)
         q(p + "attn_k.weight", 12, KD, D, 10 * l + 3)
         q(p + "attn_v.weight", 14 if mixed and l % 2 == 0 else 12, KD, D, 10 * l + 4)   # as Q4_K_M files do
-        q(p + "attn_output.weight", 12, D, QD, 10 * l + 5)
+        q(p + "attn_output.weight", t_o, D, QD, 10 * l + 5)
         f(p + "ffn_norm.weight", D, f16=(l == 1))
         q(p + "ffn_gate.weight", 12, F, D, 10 * l + 6)
         q(p + "ffn_up.weight", 8 if mixed and l == 1 else 12, F, D, 10 * l + 7)
-        q(p + "ffn_down.weight", 14 if l % 2 == 0 else 12, D, F, 10 * l + 8)
+        q(p + "ffn_down.weight", t_down or (14 if l % 2 == 0 else 12), D, F, 10 * l + 8)
     f("output_norm.weight", D)
-    q("output.weight", 14, V, D, 9)
+    q("output.weight", t_out, V, D, 9)
     if rope_freqs:
         w = np.linspace(1.0, 0.125, cfg["head_dim"] // 2).astype(np.float32)
         tensors.append(("rope_freqs.weight", 0, (cfg["head_dim"] // 2,), w.view(np.uint8)))

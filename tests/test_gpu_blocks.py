@@ -209,7 +209,7 @@ def test_errors_are_status_codes(dev):
         QMatrix.from_raw_bytes(dev, (16, 256), raw[:-1], Q4_K)
     assert e.value.status == -1
     with pytest.raises(FusorHipError) as e:
-        QMatrix.from_raw_bytes(dev, (16, 256), raw, 13)  # Q5_K: outside this library's scope
+        QMatrix.from_raw_bytes(dev, (16, 256), raw, 10)  # Q2K: GgufReadError::UnsupportedDType
     assert e.value.status == -3
     q = QMatrix.from_raw_bytes(dev, (16, 256), raw, Q4_K)
     with pytest.raises(FusorHipError, match="dimension mismatch"):
@@ -255,3 +255,61 @@ def test_q8_activation_path(dev, oracle, ty):
                     acc = np.float32(acc + np.float32(oracle.vec_dot_q4_0_q8_0(wb[c, b], aqb[r, b])))
                 want[r, c] = acc
         assert_close(y.as_slice(), want, abs_tol=1e-3, rel_tol=1e-5, what="Q4_0 x Q8")
+
+
+# ------------------------------------------------------------------ Q5_0, Q5_K, dense f16 / f32 weights
+PLAIN = [synth.Q5_0, synth.Q5_K, synth.W_F16, synth.W_F32]
+
+
+@pytest.mark.parametrize("ty", PLAIN, ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("n,k", [(1, 256), (37, 1024), (130, 768)])
+def test_plain_types_dequantize_bit_exact(dev, oracle, ty, n, k):
+    """GgufBlock::dequantize of BlockQ5_0 / BlockQ5K (gguf/src/lib.rs:1046-1073, :1819-1861) and dense weights."""
+    raw = synth.random_weight(ty, n, k, seed=300 + ty)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    assert q.shape() == (n, k) and q.ggml_type == ty
+    got = q.dequantize().as_slice()
+    want = oracle.dequantize(ty, raw).reshape(n, k)
+    assert np.array_equal(bits(got), bits(want))
+
+
+def test_plain_types_known_answers(dev):
+    """core/src/quantized/matmul/tests.rs:1305-1335 (Q5_0: +528 / -528) and :1399-1423 (Q5K: 32896)."""
+    blk = lambda hb, lo: np.concatenate([h16(1.0), np.uint8(hb), np.full(16, lo, np.uint8)])
+    raw = np.concatenate([blk([0xFF] * 4, 0x11), blk([0] * 4, 0xFF)])
+    x = Tensor.from_slice(dev, np.arange(1, 33, dtype=np.float32)[None, :])
+    y = x.q_mat_mul(QMatrix.from_raw_bytes(dev, (2, 32), raw, synth.Q5_0)).as_slice()
+    assert y.shape == (1, 2) and y[0, 0] == 528.0 and y[0, 1] == -528.0
+    raw = np.concatenate([h16(1.0), h16(0.0), np.uint8([1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1]), np.zeros(32, np.uint8),
+                          np.full(128, 0x11, np.uint8)])
+    x = Tensor.from_slice(dev, np.arange(1, 257, dtype=np.float32)[None, :])
+    y = x.q_mat_mul(QMatrix.from_raw_bytes(dev, (1, 256), raw, synth.Q5_K)).as_slice()
+    assert y[0, 0] == 32896.0
+
+
+@pytest.mark.parametrize("ty", PLAIN, ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("m", [1, 4, 33])
+def test_plain_types_matmul_and_glue(dev, oracle, ty, m):
+    """q_mat_mul, the SwiGLU / add2 epilogues, concat_rows (any row counts) and the embedding gather."""
+    n, k = 72, 1024
+    raw_g = synth.random_weight(ty, n, k, seed=310 + ty, sigma=2e-3)
+    raw_u = synth.random_weight(ty, n, k, seed=311 + ty, sigma=2e-3)
+    x = synth.random_activation(m, k, seed=312 + m)
+    g, u = QMatrix.from_raw_bytes(dev, (n, k), raw_g, ty), QMatrix.from_raw_bytes(dev, (n, k), raw_u, ty)
+    xt = Tensor.from_slice(dev, x)
+    yg, yu = oracle.q_mat_mul(ty, x, raw_g, n), oracle.q_mat_mul(ty, x, raw_u, n)
+    out = Tensor.filled_bytes(dev, (m, n), 0xFF)
+    assert_close(xt.q_mat_mul(g, out=out).as_slice(), yg, what=f"{NAMES[ty]} m={m}")
+    gu = QMatrix.concat_rows([g, u])
+    assert gu.shape() == (2 * n, k)
+    assert np.array_equal(bits(gu.dequantize().as_slice()),
+                          bits(oracle.dequantize(ty, np.concatenate([raw_g, raw_u])).reshape(2 * n, k)))
+    if (2 * n) % 32 == 0:
+        assert_close(xt.q_mat_mul_swiglu(gu).as_slice(), oracle.swiglu(yg, yu), what="swiglu")
+    a, b = synth.random_activation(m, n, seed=313), synth.random_activation(m, n, seed=314)
+    got = xt.q_mat_mul_add2(g, Tensor.from_slice(dev, a), Tensor.from_slice(dev, b)).as_slice()
+    assert_close(got, oracle.add3(yg, a, b), what="add2")
+    ids = np.array([0, n - 1, 5, 5], np.uint32)
+    assert np.array_equal(bits(g.embed(ids).as_slice()), bits(oracle.embed_rows(ty, raw_g, n, k, ids)))
+    assert QMatrix.concat_rows([g, QMatrix.from_raw_bytes(dev, (n, k), synth.random_weight(synth.Q4_K, n, k, seed=1),
+                                                         synth.Q4_K)]) is None

@@ -108,8 +108,8 @@ def test_decode_step_kernel_variants(dev, oracle, heads, kv_heads, opts):
             dev.set_option(k, 0)
 
 
-@pytest.mark.parametrize("variant", [dict(), dict(fuse_qkv=False, fuse_gate_up=False, use_graph=False)],
-                         ids=["fused+graph", "separate+eager"])
+@pytest.mark.parametrize("variant", [dict(), dict(fuse_qkv=False, fuse_gate_up=False, use_graph=False), dict(five_bit=True)],
+                         ids=["fused+graph", "separate+eager", "q5_0+q5_k+f16"])
 def test_decoder_from_gguf_file(dev, oracle, variant, tmp_path):
     """Model::from_gguf (raw/mod.rs:284-648) on a small random-init file with what model files really hold:
     block types that change from layer to layer (so q|k|v and gate|up cannot always be fused), f32 and f16 norm
@@ -117,7 +117,8 @@ def test_decoder_from_gguf_file(dev, oracle, variant, tmp_path):
     from the same file through the plain-Python reader."""
     from test_gguf_reader import TINY, llama_file
     from oracle import gguf_ref
-    data, weights, types = llama_file(TINY, seed=5)
+    variant = dict(variant)
+    data, weights, types = llama_file(TINY, seed=5, five_bit=variant.pop("five_bit", False))
     path = tmp_path / "tiny.gguf"
     path.write_bytes(data)
     m = Model.from_gguf(dev, str(path), ctx=80, **variant)
@@ -126,13 +127,14 @@ def test_decoder_from_gguf_file(dev, oracle, variant, tmp_path):
     rw = {}
     for name, (ty, shape, off) in r.tensors.items():
         raw = r.tensor_bytes(name)
-        if ty == 0:
+        if ty == 0 and len(shape) == 1:
             raw = raw.view(np.float32)
-        elif ty == 1:
+        elif ty == 1 and len(shape) == 1:  # vectors are widened at load (norm weights); matrices stay f16 rows
             raw = raw.view(np.float16).astype(np.float32)
         rw[name.decode()] = raw
-    ocfg = dict(m.cfg, type_attn=synth.Q4_K, type_ffn_gate_up=synth.Q4_K, type_ffn_down=synth.Q6_K, type_embd=synth.Q4_K,
-                type_output=synth.Q6_K, tensor_types={n.decode(): t for n, (t, _, _) in r.tensors.items()})
+    ocfg = dict(m.cfg, type_attn=synth.Q4_K, type_ffn_gate_up=synth.Q4_K, type_ffn_down=synth.Q6_K,
+                type_embd=types["token_embd.weight"], type_output=types["output.weight"],
+                tensor_types={n.decode(): t for n, (t, _, _) in r.tensors.items()})
     ref = oracle.Llama(ocfg, rw)
     rng = np.random.default_rng(2)
     prompt = rng.integers(0, TINY["vocab"], 11)

@@ -281,3 +281,109 @@ def test_vec_dot_exact(oracle):
     wq = raw.reshape(8, 8, 34)
     ref = np.einsum("rbi,cbi->rcb", aq[:, :, 2:].view(np.int8).astype(np.int64), wq[:, :, 2:].view(np.int8).astype(np.int64))
     assert np.array_equal(isums, ref.astype(np.int32))
+
+
+# ------------------------------------------------------------------ Q5_0, Q5_K, dense f16 / f32 weights
+Q5_0, Q5_K, W_F32, W_F16 = 6, 13, 0, 1
+
+
+def q5_0_block(scale, high_bits, low_bits):
+    # the block builder of core/src/quantized/matmul/tests.rs:1312-1319
+    return np.concatenate([h16(scale), np.uint8(high_bits), np.full(16, low_bits, np.uint8)])
+
+
+def test_q5_block_sizes(oracle):
+    # gguf/src/lib.rs:958-966 (22 bytes), :1703-1711 (176 bytes)
+    assert [oracle.lib().fo_block_bytes(t) for t in (Q5_0, Q5_K, W_F32, W_F16)] == [22, 176, 4, 2]
+    assert [oracle.lib().fo_block_elems(t) for t in (Q5_0, Q5_K, W_F32, W_F16)] == [32, 256, 1, 1]
+
+
+def test_q5_0_known_answer_528(oracle):
+    """core/src/quantized/matmul/tests.rs:1305-1335: all high bits set with nibbles 0x11 -> weights +1,
+    no high bits with nibbles 0xff -> weights -1; x = 1..32 -> +528 / -528."""
+    raw = np.concatenate([q5_0_block(1.0, [0xFF] * 4, 0x11), q5_0_block(1.0, [0] * 4, 0xFF)])
+    assert np.array_equal(oracle.dequantize(Q5_0, raw), np.repeat(np.float32([1, -1]), 32))
+    x = np.arange(1, 33, dtype=np.float32)[None, :]
+    y = oracle.q_mat_mul(Q5_0, x, raw, 2)
+    assert y[0, 0] == 528.0 and y[0, 1] == -528.0
+
+
+def test_q5_k_reference_cases(oracle):
+    """tests.rs:1399-1423 (32896) and gguf/src/lib.rs:2376-2433 (nibble identity without high bits; all high bits
+    set over zero nibbles -> 16)."""
+    unit = np.uint8([1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1])
+    raw = np.concatenate([h16(1.0), h16(0.0), unit, np.zeros(32, np.uint8), np.full(128, 0x11, np.uint8)])
+    assert raw.size == 176
+    assert np.array_equal(oracle.dequantize(Q5_K, raw), np.ones(256, np.float32))
+    x = np.arange(1, 257, dtype=np.float32)[None, :]
+    assert oracle.q_mat_mul(Q5_K, x, raw, 1)[0, 0] == 32896.0
+    qs = np.uint8([(i % 16) | (((i + 1) % 16) << 4) for i in range(128)])
+    raw = np.concatenate([h16(1.0), h16(0.0), np.ones(12, np.uint8), np.zeros(32, np.uint8), qs])
+    d = oracle.dequantize(Q5_K, raw)
+    assert d[:16].tolist() == list(range(16))
+    raw = np.concatenate([h16(1.0), h16(0.0), np.ones(12, np.uint8), np.full(32, 0xFF, np.uint8), np.zeros(128, np.uint8)])
+    d = oracle.dequantize(Q5_K, raw)
+    assert np.array_equal(d[:32], np.full(32, 16.0, np.float32))
+
+
+def test_q5_k_without_high_bits_is_q4_k(oracle):
+    """With qh = 0 a Q5_K block decodes exactly like the Q4_K block of the same d, dmin, scales and nibbles
+    (same scale packing, same operation order): a special case that reduces to an already pinned routine."""
+    from kalosm_amd import synth
+    q4 = synth.random_weight(Q4_K, 3, 512, seed=91).reshape(-1, 144)
+    q5 = np.concatenate([q4[:, :16], np.zeros((q4.shape[0], 32), np.uint8), q4[:, 16:]], axis=1).reshape(-1)
+    assert np.array_equal(oracle.dequantize(Q5_K, q5).view(np.uint32), oracle.dequantize(Q4_K, q4.reshape(-1)).view(np.uint32))
+
+
+def np_deq_q5_0(raw):
+    b = raw.reshape(-1, 22)
+    d = b[:, 0:2].copy().view(np.float16).astype(np.float32)           # [nb, 1]
+    hb = b[:, 2:6].copy().view(np.uint32)                               # [nb, 1]
+    i = np.arange(16, dtype=np.uint32)[None, :]
+    lo = (b[:, 6:] & 0xF).astype(np.int32) | ((((hb >> i) & 1) << 4).astype(np.int32))
+    hi = (b[:, 6:] >> 4).astype(np.int32) | ((((hb >> (i + 16)) & 1) << 4).astype(np.int32))
+    codes = np.concatenate([lo, hi], axis=1) - 16
+    return (codes.astype(np.float32) * d).reshape(-1)
+
+
+def np_deq_q5_k(raw, oracle):
+    b = raw.reshape(-1, 176)
+    out = np.empty((b.shape[0], 256), np.float32)
+    for n, blk in enumerate(b):
+        d = blk[0:2].copy().view(np.float16).astype(np.float32)[0]
+        dmin = blk[2:4].copy().view(np.float16).astype(np.float32)[0]
+        sc, mn = oracle.unpack_k4_scales(blk[4:16])                    # pinned by the brute-force test above
+        qh, qs = blk[16:48], blk[48:176]
+        for s in range(8):
+            ql = qs[32 * (s // 2):32 * (s // 2) + 32]
+            code = ((ql >> 4) if s % 2 else (ql & 0xF)).astype(np.float32) + 16 * ((qh >> s) & 1).astype(np.float32)
+            out[n, 32 * s:32 * s + 32] = (np.float32(sc[s]) * d) * code - np.float32(mn[s]) * dmin
+    return out.reshape(-1)
+
+
+def test_q5_dequantize_matches_independent_numpy(oracle):
+    from kalosm_amd import synth
+    raw = synth.random_weight(Q5_0, 5, 256, seed=92)
+    assert np.array_equal(oracle.dequantize(Q5_0, raw).view(np.uint32), np_deq_q5_0(raw).view(np.uint32))
+    raw = synth.random_weight(Q5_K, 3, 768, seed=93)
+    assert np.array_equal(oracle.dequantize(Q5_K, raw).view(np.uint32), np_deq_q5_k(raw, oracle).view(np.uint32))
+    # dense weights: the stored values themselves
+    v = np.random.default_rng(94).standard_normal(64).astype(np.float32)
+    assert np.array_equal(oracle.dequantize(W_F32, v.view(np.uint8)), v)
+    h = v.astype(np.float16)
+    assert np.array_equal(oracle.dequantize(W_F16, h.view(np.uint8)), h.astype(np.float32))
+
+
+@pytest.mark.parametrize("ty", [Q5_0, Q5_K, W_F16, W_F32])
+def test_q5_qmatmul_is_x_times_dequantized(oracle, ty):
+    """q_mat_mul(X, W) ~ X . deq(W)^T in float64, the reference's own host check (fusor/src/quantized.rs:147-157)."""
+    from kalosm_amd import synth
+    n, k = 24, 512
+    raw = synth.random_weight(ty, n, k, seed=95 + ty)
+    w = oracle.dequantize(ty, raw).reshape(n, k).astype(np.float64)
+    for m in (1, 3, 5):
+        x = synth.random_activation(m, k, seed=96 + m)
+        want = x.astype(np.float64) @ w.T
+        for fast in (False, True):
+            got = oracle.q_mat_mul(ty, x, raw, n, fast=fast)
+            assert np.allclose(got, want, rtol=1e-4, atol=1e-4 * np.abs(want).max()), (m, fast)
