@@ -61,3 +61,24 @@ def test_product_package_does_not_touch_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 src = open(os.path.join(dirpath, f), errors="replace").read()
                 assert "fusor_cpu_oracle" not in src and "from oracle" not in src and "import oracle" not in src, f
+
+
+def test_rust_declarations_cover_the_header():
+    """include/fusor_hip_sys.rs declares every function of the header with the same number of parameters."""
+    text = open(os.path.join(ROOT, "include", "fusor_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    c = {}
+    for name, args in re.findall(r"\b(fh_[a-z0-9_]+)\s*\(([^;{}]*?)\)\s*;", text, flags=re.S):
+        args = " ".join(args.split())
+        c[name] = 0 if args == "void" else args.count(",") + 1
+    rs = open(os.path.join(ROOT, "include", "fusor_hip_sys.rs")).read()
+    r = {}
+    for name, args in re.findall(r"pub fn (fh_[a-z0-9_]+)\(([^)]*)\)", rs):
+        r[name] = 0 if not args.strip() else args.count(",") + 1
+    assert set(c) == set(declared_symbols())
+    assert c == r, {k: (c.get(k), r.get(k)) for k in set(c) | set(r) if c.get(k) != r.get(k)}
+    # the two structs passed by pointer have the header's field order
+    cfg = re.search(r"typedef struct \{([^{}]*)\} fh_llama_config;", text).group(1)
+    c_fields = re.findall(r"\b([a-z_0-9]+)\s*[,;]", cfg)
+    rs_cfg = re.search(r"pub struct FhLlamaConfig \{([^{}]*)\}", rs).group(1)
+    assert c_fields == re.findall(r"pub ([a-z_0-9]+):", rs_cfg)
