@@ -177,6 +177,15 @@ fh_status fh_rope_tables(fh_device *dev, int32_t head_dim, int32_t ctx, float th
  * inverse frequency i is multiplied by freq_weight_host[i] (head_dim/2 host floats; NULL: no weights). */
 fh_status fh_rope_tables_weighted(fh_device *dev, int32_t head_dim, int32_t ctx, float theta,
                                   const float *freq_weight_host, float *cos_dev, float *sin_dev);
+/* RopeScalingConfig, models/kalosm-llama/src/raw/mod.rs:163-169, applied as create_inverse_frequency does
+ * (raw/rope.rs:20-38) before the weights; scaling and freq_weight_host may each be NULL. */
+typedef struct {
+    float factor, high_freq_factor, low_freq_factor;
+    int32_t original_max_position_embeddings;
+} fh_rope_scaling;
+fh_status fh_rope_tables_scaled(fh_device *dev, int32_t head_dim, int32_t ctx, float theta,
+                                const fh_rope_scaling *scaling, const float *freq_weight_host,
+                                float *cos_dev, float *sin_dev);
 /* RopeCache::forward{,_interleaved}(&q, &k, start_pos), rope.rs:284-329.  q is [b, hq, s, d] and
  * k is [b, hk, s, d] as VIEWS: element (b, h, t, c) of q lives at q_dev[b*q_sb + h*q_sh + t*q_st + c]
  * (strides in elements), likewise k.  Outputs are contiguous [b, h, s, d].  One launch rotates both. */

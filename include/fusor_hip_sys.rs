@@ -88,6 +88,16 @@ pub struct FhLlamaConfig {
     pub use_graph: i32,
 }
 
+/// `fh_rope_scaling` (`RopeScalingConfig`, models/kalosm-llama/src/raw/mod.rs:163-169)
+#[repr(C)]
+#[derive(Clone, Copy, Debug)]
+pub struct FhRopeScaling {
+    pub factor: f32,
+    pub high_freq_factor: f32,
+    pub low_freq_factor: f32,
+    pub original_max_position_embeddings: i32,
+}
+
 /// `fh_gguf_tensor`: `name` is owned by the `FhGguf` handle
 #[repr(C)]
 #[derive(Clone, Copy, Debug)]
@@ -135,6 +145,7 @@ extern "C" {
     pub fn fh_rms_norm(dev: *mut FhDevice, x_dev: *const f32, residual_dev: *const f32, w_dev: *const f32, bias_dev: *const f32, eps: f32, rows: i32, cols: i32, y_dev: *mut f32) -> FhStatus;
     pub fn fh_rope_tables(dev: *mut FhDevice, head_dim: i32, ctx: i32, theta: f32, cos_dev: *mut f32, sin_dev: *mut f32) -> FhStatus;
     pub fn fh_rope_tables_weighted(dev: *mut FhDevice, head_dim: i32, ctx: i32, theta: f32, freq_weight_host: *const f32, cos_dev: *mut f32, sin_dev: *mut f32) -> FhStatus;
+    pub fn fh_rope_tables_scaled(dev: *mut FhDevice, head_dim: i32, ctx: i32, theta: f32, scaling: *const FhRopeScaling, freq_weight_host: *const f32, cos_dev: *mut f32, sin_dev: *mut f32) -> FhStatus;
     pub fn fh_rope_pair(dev: *mut FhDevice, q_dev: *const f32, q_sb: i64, q_sh: i64, q_st: i64, k_dev: *const f32, k_sb: i64, k_sh: i64, k_st: i64, b: i32, hq: i32, hk: i32, s: i32, d: i32, cos_dev: *const f32, sin_dev: *const f32, table_rows: i32, start_pos: i32, interleaved: i32, q_out_dev: *mut f32, k_out_dev: *mut f32) -> FhStatus;
     pub fn fh_kvcache_create(dev: *mut FhDevice, layers: i32, kv_heads: i32, head_dim: i32, max_len: i32, dtype: i32, out: *mut *mut FhKvCache) -> FhStatus;
     pub fn fh_kvcache_destroy(c: *mut FhKvCache) -> FhStatus;

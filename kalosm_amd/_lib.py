@@ -29,6 +29,11 @@ class LlamaConfig(C.Structure):
                [(n, C.c_int32) for n in ("kv_dtype", "fuse_qkv", "fuse_gate_up", "use_graph")]
 
 
+class RopeScaling(C.Structure):
+    _fields_ = [("factor", C.c_float), ("high_freq_factor", C.c_float), ("low_freq_factor", C.c_float),
+                ("original_max_position_embeddings", C.c_int32)]
+
+
 class GgufTensor(C.Structure):
     _fields_ = [("name", C.c_char_p), ("ggml_type", C.c_uint32), ("rank", C.c_int32), ("shape", C.c_int64 * 8),
                 ("offset", C.c_uint64)]
@@ -101,6 +106,7 @@ SIGNATURES = {
     "fh_llama_config_from_gguf": [_p, C.POINTER(LlamaConfig)],
     "fh_llama_load_gguf": [_p, _p],
     "fh_rope_tables_weighted": [_p, _i32, _i32, _f32, _p, _p, _p],
+    "fh_rope_tables_scaled": [_p, _i32, _i32, _f32, C.POINTER(RopeScaling), _p, _p, _p],
     "fh_gguf_open": [C.c_char_p, _pp],
     "fh_gguf_open_memory": [_p, _sz, _pp],
     "fh_gguf_close": [_p],

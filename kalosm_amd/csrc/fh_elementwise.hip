@@ -110,14 +110,32 @@ extern "C" fh_status fh_rms_norm(fh_device *dev, const float *x_dev, const float
 // Tables: fusor-ml/fusor/src/composite/rope.rs:241-246 + models/kalosm-llama/src/raw/rope.rs:63-85.
 // Built on the host in f32 with the C library (the reference builds them with Rust's f32
 // powf/sin/cos, i.e. the platform libm).
-extern "C" fh_status fh_rope_tables_weighted(fh_device *dev, int32_t head_dim, int32_t ctx, float theta,
-                                             const float *freq_weight_host, float *cos_dev, float *sin_dev) {
+// create_inverse_frequency, models/kalosm-llama/src/raw/rope.rs:9-50: base frequencies, then the optional
+// long-context scaling (frequencies whose wavelength exceeds original_max / low_freq_factor are divided by `factor`;
+// the smooth branch is taken only where the wavelength EQUALS original_max / high_freq_factor, as the reference
+// writes it at :32), then the optional per-frequency weights of the file.
+extern "C" fh_status fh_rope_tables_scaled(fh_device *dev, int32_t head_dim, int32_t ctx, float theta,
+                                           const fh_rope_scaling *scaling, const float *freq_weight_host, float *cos_dev,
+                                           float *sin_dev) {
     FH_REQUIRE(dev && cos_dev && sin_dev, "NULL argument");
     FH_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && ctx > 0, "bad head_dim %d / ctx %d", head_dim, ctx);
     int half = head_dim / 2;
     std::vector<float> inv(half), c((size_t)ctx * half), s((size_t)ctx * half);
     for (int i = 0; i < head_dim; i += 2) inv[i / 2] = 1.0f / powf(theta, (float)i / (float)head_dim);
-    // models/kalosm-llama/src/raw/rope.rs:41-48: the inverse frequencies TIMES the file's rope_freqs.weight
+    if (scaling) {
+        const float orig = (float)scaling->original_max_position_embeddings;
+        const float low_wavelen = orig / scaling->low_freq_factor, high_wavelen = orig / scaling->high_freq_factor;
+        const float two_pi = 2.0f * 3.14159265358979323846f;
+        for (int i = 0; i < half; i++) {
+            const float wavelen = two_pi / inv[i];
+            if (wavelen > low_wavelen) inv[i] = inv[i] / scaling->factor;
+            else if (wavelen == high_wavelen) {
+                const float smooth = (orig / wavelen - scaling->low_freq_factor) /
+                                     (scaling->high_freq_factor - scaling->low_freq_factor);
+                inv[i] = (1.0f - smooth) * inv[i] / scaling->factor + smooth * inv[i];
+            }
+        }
+    }
     if (freq_weight_host)
         for (int i = 0; i < half; i++) inv[i] = inv[i] * freq_weight_host[i];
     for (int p = 0; p < ctx; p++)
@@ -129,6 +147,11 @@ extern "C" fh_status fh_rope_tables_weighted(fh_device *dev, int32_t head_dim, i
     FH_TRY(fh_upload(dev, cos_dev, c.data(), c.size() * 4));
     FH_TRY(fh_upload(dev, sin_dev, s.data(), s.size() * 4));
     return FH_OK;
+}
+
+extern "C" fh_status fh_rope_tables_weighted(fh_device *dev, int32_t head_dim, int32_t ctx, float theta,
+                                             const float *freq_weight_host, float *cos_dev, float *sin_dev) {
+    return fh_rope_tables_scaled(dev, head_dim, ctx, theta, nullptr, freq_weight_host, cos_dev, sin_dev);
 }
 
 extern "C" fh_status fh_rope_tables(fh_device *dev, int32_t head_dim, int32_t ctx, float theta, float *cos_dev,

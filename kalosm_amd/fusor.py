@@ -379,6 +379,23 @@ class RopeCache:
         return RopeCache(device, cos, sin)
 
     @staticmethod
+    def scaled(head_dim: int, context_length: int, rope_theta: float, device: Device, scaling=None,
+               freq_weight=None) -> "RopeCache":
+        """RopeImplementation::new (models/kalosm-llama/src/raw/rope.rs:63-85) with create_inverse_frequency's
+        options (:9-50): `scaling` = (factor, high_freq_factor, low_freq_factor, original_max_position_embeddings),
+        `freq_weight` = the file's rope_freqs.weight values."""
+        cos = Tensor(device, (context_length, head_dim // 2), "f32")
+        sin = Tensor(device, (context_length, head_dim // 2), "f32")
+        sc = None if scaling is None else _lib.RopeScaling(float(scaling[0]), float(scaling[1]), float(scaling[2]),
+                                                           int(scaling[3]))
+        w = None if freq_weight is None else np.ascontiguousarray(freq_weight, np.float32)
+        check(device._lib.fh_rope_tables_scaled(device._h, head_dim, context_length, rope_theta,
+                                                None if sc is None else C.byref(sc),
+                                                None if w is None else w.ctypes.data_as(C.c_void_p),
+                                                C.c_void_p(cos.ptr), C.c_void_p(sin.ptr)))
+        return RopeCache(device, cos, sin)
+
+    @staticmethod
     def from_parts(cos: Tensor, sin: Tensor) -> "RopeCache":
         return RopeCache(cos.device, cos, sin)
 

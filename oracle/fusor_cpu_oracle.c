@@ -677,10 +677,31 @@ void fo_rope_inverse_frequency(int dim, float theta, float *inv) {
 }
 /* freq_weight (optional, dim/2 values): the `rope_freqs.weight` tensor of a model file; the inverse
  * frequencies are MULTIPLIED by it (models/kalosm-llama/src/raw/rope.rs:41-48). */
+/* scaling (optional): {factor, high_freq_factor, low_freq_factor, original_max_position_embeddings as float},
+ * models/kalosm-llama/src/raw/rope.rs:20-38.  Note the `==` of the smooth branch (:32), kept as written. */
+void fo_rope_scale_inverse_frequency(float *inv, int half, const float *scaling) {
+    float factor = scaling[0], high = scaling[1], low = scaling[2], orig = scaling[3];
+    float low_wavelen = orig / low, high_wavelen = orig / high;
+    for (int i = 0; i < half; i++) {
+        float wavelen = 2.0f * 3.14159265358979323846f / inv[i];
+        if (wavelen > low_wavelen) inv[i] = inv[i] / factor;
+        else if (wavelen == high_wavelen) {
+            float smooth = (orig / wavelen - low) / (high - low);
+            inv[i] = (1.0f - smooth) * inv[i] / factor + smooth * inv[i];
+        }
+    }
+}
+void fo_rope_tables_scaled(int dim, int ctx, float theta, const float *scaling, const float *freq_weight, float *cosv,
+                           float *sinv);
 void fo_rope_tables_weighted(int dim, int ctx, float theta, const float *freq_weight, float *cosv, float *sinv) {
+    fo_rope_tables_scaled(dim, ctx, theta, NULL, freq_weight, cosv, sinv);
+}
+void fo_rope_tables_scaled(int dim, int ctx, float theta, const float *scaling, const float *freq_weight, float *cosv,
+                           float *sinv) {
     int half = dim / 2;
     float *inv = (float *)malloc((size_t)half * sizeof(float));
     fo_rope_inverse_frequency(dim, theta, inv);
+    if (scaling) fo_rope_scale_inverse_frequency(inv, half, scaling);
     if (freq_weight)
         for (int i = 0; i < half; i++) inv[i] = inv[i] * freq_weight[i];
     for (int p = 0; p < ctx; p++)

@@ -72,6 +72,7 @@ def lib() -> C.CDLL:
         L.fo_llama_set_layer_types.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int)]
         L.fo_llama_set_rope_freq_weight.argtypes = [C.c_void_p, fp]
         L.fo_rope_tables_weighted.argtypes = [C.c_int, C.c_int, C.c_float, fp, fp, fp]
+        L.fo_rope_tables_scaled.argtypes = [C.c_int, C.c_int, C.c_float, fp, fp, fp, fp]
         L.fo_llama_reset.argtypes = [C.c_void_p]
         L.fo_llama_destroy.argtypes = [C.c_void_p]
         L.fo_llama_forward.argtypes = [C.c_void_p, u32p, C.c_int, fp, fp]
@@ -222,6 +223,17 @@ def rope_inverse_frequency(dim: int, theta: float) -> np.ndarray:
     inv = np.empty(dim // 2, np.float32)
     lib().fo_rope_inverse_frequency(dim, theta, _p(inv, C.c_float))
     return inv
+
+
+def rope_tables_scaled(dim: int, ctx: int, theta: float, scaling, freq_weight=None):
+    """scaling = (factor, high_freq_factor, low_freq_factor, original_max_position_embeddings) or None."""
+    cos = np.empty((ctx, dim // 2), np.float32)
+    sin = np.empty((ctx, dim // 2), np.float32)
+    sc = None if scaling is None else _f32(np.asarray(scaling, np.float32))
+    w = None if freq_weight is None else _f32(freq_weight)
+    lib().fo_rope_tables_scaled(dim, ctx, theta, None if sc is None else _p(sc, C.c_float),
+                                None if w is None else _p(w, C.c_float), _p(cos, C.c_float), _p(sin, C.c_float))
+    return cos, sin
 
 
 def rope_tables_weighted(dim: int, ctx: int, theta: float, freq_weight):

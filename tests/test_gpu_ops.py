@@ -55,6 +55,17 @@ def test_rope_tables_golden(dev, oracle):
     assert np.array_equal(bits(rc.cos.as_slice()), bits(oc)) and np.array_equal(bits(rc.sin.as_slice()), bits(os_))
 
 
+def test_rope_tables_scaled(dev, oracle):
+    """Long-context scaling and rope_freqs.weight factors (models/kalosm-llama/src/raw/rope.rs:9-50)."""
+    w = np.linspace(1.0, 0.5, 64).astype(np.float32)
+    for scaling, fw in [((8.0, 4.0, 1.0, 8192), None), (None, w), ((8.0, 4.0, 1.0, 8192), w), ((32.0, 4.0, 1.0, 8192), None)]:
+        rc = RopeCache.scaled(128, 300, 500000.0, dev, scaling=scaling, freq_weight=fw)
+        oc, os_ = oracle.rope_tables_scaled(128, 300, 500000.0, scaling, fw)
+        assert np.array_equal(bits(rc.cos.as_slice()), bits(oc)) and np.array_equal(bits(rc.sin.as_slice()), bits(os_))
+    plain = RopeCache.new(128, 300, 500000.0, dev).cos.as_slice()
+    assert not np.array_equal(plain, oc)
+
+
 @pytest.mark.parametrize("interleaved", [True, False])
 @pytest.mark.parametrize("start_pos", [0, 5])
 def test_rope_pair(dev, oracle, interleaved, start_pos):

@@ -387,3 +387,23 @@ def test_q5_qmatmul_is_x_times_dequantized(oracle, ty):
         for fast in (False, True):
             got = oracle.q_mat_mul(ty, x, raw, n, fast=fast)
             assert np.allclose(got, want, rtol=1e-4, atol=1e-4 * np.abs(want).max()), (m, fast)
+
+
+def test_rope_scaling_closed_form(oracle):
+    """create_inverse_frequency (models/kalosm-llama/src/raw/rope.rs:9-50) against numpy: frequencies whose
+    wavelength exceeds original_max / low_freq_factor are divided by the factor, all others stay (the smooth branch
+    needs an exact float equality and does not fire for these parameters), then the file's weights multiply."""
+    dim, ctx, theta = 128, 64, 500000.0
+    scaling = (8.0, 4.0, 1.0, 8192)       # Llama 3.1's published values
+    inv = oracle.rope_inverse_frequency(dim, theta)
+    assert inv[0] == 1.0 and abs(inv[1] - theta ** (-2.0 / dim)) < 1e-7
+    wavelen = np.float32(2.0) * np.float32(np.pi) / inv
+    want = np.where(wavelen > np.float32(8192.0 / 1.0), inv / np.float32(8.0), inv).astype(np.float32)
+    assert (want != inv).sum() == (wavelen > 8192).sum() > 10           # the long wavelengths are really scaled
+    w = np.linspace(1.0, 0.5, dim // 2).astype(np.float32)
+    cos, sin = oracle.rope_tables_scaled(dim, ctx, theta, scaling, w)
+    ang = np.arange(ctx, dtype=np.float32)[:, None] * (want * w)[None, :]
+    assert np.abs(cos - np.cos(ang.astype(np.float64))).max() < 1e-6 and np.abs(sin - np.sin(ang.astype(np.float64))).max() < 1e-6
+    c0, s0 = oracle.rope_tables_scaled(dim, ctx, theta, None, None)
+    c1, s1 = oracle.rope_tables(dim, ctx, theta)
+    assert np.array_equal(c0, c1) and np.array_equal(s0, s1)
