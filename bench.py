@@ -39,7 +39,7 @@ def prefill_legs(dev) -> dict:
     from kalosm_amd import synth
     from kalosm_amd.fusor import MaskKind, QMatrix, Tensor
 
-    res = {"matmul": [], "attention": []}
+    res = {"matmul": [], "attention": [], "attention_decode": []}
     n, k = 14336, 4096
     for ty, name in ((synth.Q6_K, "Q6_K"), (synth.Q8_0, "Q8_0")):
         q = QMatrix.from_raw_bytes(dev, (n, k), synth.random_weight(ty, n, k, seed=7), ty)
@@ -102,6 +102,33 @@ def prefill_legs(dev) -> dict:
         tf = 4.0 * s * s * d * h / 2 / ms / 1e9
         res["attention"].append({"seq": s, "us": round(ms * 1e3, 1), "TFLOPs": round(tf, 1),
                                  "frac_mfma_peak": round(tf / 2500.0, 4)})
+    # configs[3], decode variant: one query per head against a cache of L keys (f16 K / V), HBM bound:
+    # bytes = K and V once (2 * hkv * L * d * 2) + the query and the output (2 * h * d * 2); caches rotate over
+    # more than the Infinity Cache
+    for L in (1024, 4096, 16384):
+        rng = np.random.default_rng(L)
+        kv_bytes = 2 * hkv * L * d * 2
+        copies = max(2, -(-(640 << 20) // kv_bytes))
+        kvs = []
+        base_k = rng.standard_normal((1, hkv, L, d)).astype(np.float16)
+        base_v = rng.standard_normal((1, hkv, L, d)).astype(np.float16)
+        for c in range(min(copies, 160)):
+            kvs.append((Tensor.from_slice(dev, base_k, "f16"), Tensor.from_slice(dev, base_v, "f16")))
+        qt = Tensor.from_slice(dev, rng.standard_normal((1, h, 1, d)).astype(np.float16), "f16")
+        ot = Tensor(dev, (1, h, 1, d), "f16")
+        reps = 200
+        for i in range(20):
+            qt.flash_attention(*kvs[i % len(kvs)], 1 / np.sqrt(d), None, out=ot)
+        dev.sync()
+        dev.timer_start()
+        for i in range(reps):
+            qt.flash_attention(*kvs[i % len(kvs)], 1 / np.sqrt(d), None, out=ot)
+        ms = dev.timer_stop() / reps
+        nbytes = kv_bytes + 2 * h * d * 2
+        res["attention_decode"].append({"kv_len": L, "us": round(ms * 1e3, 2), "bytes": nbytes,
+                                        "GBps": round(nbytes / ms / 1e6, 1), "frac_hbm_peak": round(nbytes / ms / 1e6 / 8000.0, 4),
+                                        "cache_copies_rotated": len(kvs)})
+        del kvs
     return res
 
 

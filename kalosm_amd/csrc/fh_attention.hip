@@ -8,6 +8,8 @@
 //                                    KV in 256-key tiles with an online softmax (fallback / cross-check)
 #include "fh_internal.h"
 
+#include <type_traits>
+
 typedef _Float16 fh_half;
 
 template <typename T>
@@ -302,6 +304,19 @@ static fh_status attn_typed(fh_device *dev, const void *q, int64_t q_sb, int64_t
                             int skv, int d, float scale, int mask_kind, const float *mask, void *out) {
     const int G = hq / hkv;
     const bool aligned = (kv_st % 8 == 0) && (kv_sh % 8 == 0) && (kv_sb % 8 == 0);
+    // one batch entry, head_dim 128, contiguous query heads, no additive mask: the decode-step kernel (an f16
+    // query is widened into the device's small buffer first)
+    if (sq == 1 && b == 1 && d == 128 && aligned && q_sh == d && mask_kind != FH_MASK_ADDITIVE && hq <= 64 &&
+        dev->opt_attn_kernel != 1) {
+        const float *q32 = (const float *)q;
+        if constexpr (!std::is_same<TQ, float>::value) {
+            FH_TRY(fh_cast_f16_f32(dev, q, (float *)dev->small_buf, (int64_t)hq * d));
+            q32 = (const float *)dev->small_buf;
+        }
+        fh_status st = fh_attention_decode_hostlen(dev, std::is_same<TKV, float>::value ? FH_F32 : FH_F16, q32, k, v, kv_sh,
+                                                   kv_st, hq, hkv, d, scale, skv, out, !std::is_same<TQ, float>::value);
+        if (st != FH_ERR_UNSUPPORTED) return st;
+    }
     if (sq == 1 && aligned && (d == 128 || d == 64) && (G == 1 || G == 2 || G == 4 || G == 8)) {
         const float *mrow = mask_kind == FH_MASK_ADDITIVE ? mask : nullptr;
         fh_status st = d == 128 ? decode_dispatch_g<TQ, TKV, 128>(dev, G, q, q_sb, q_sh, k, v, kv_sb, kv_sh, kv_st, b, hq,

@@ -65,8 +65,8 @@ __device__ __forceinline__ float ad_rows_sum(float a) {
 template <typename TKV, int D, int G, int NWV>
 __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__restrict__ q, const TKV *__restrict__ k,
                                                               const TKV *__restrict__ v, int64_t kv_sh, int64_t kv_st,
-                                                              const int *__restrict__ len_dev, float scale,
-                                                              int chunk_max, int cap, int gtot,
+                                                              const int *__restrict__ len_dev, int len_host,
+                                                              float scale, int chunk_max, int cap, int gtot,
                                                               float *__restrict__ part) {
     constexpr int LP = D / 8, RPW = 64 / LP, RW = NWV * RPW, U = 4;
     static_assert(NWV >= G, "one wavefront per query head for the softmax statistics");
@@ -97,7 +97,8 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
         ad_load8<TKV>(vb + (int64_t)(t < cap ? t : 0) * kv_st, vpre[u]);
     }
     __builtin_amdgcn_sched_barrier(0); // the requests above do not wait for the length
-    const int skv = *len_dev + 1;      // the step's own key is already appended at index len
+    // the step's own key is already appended at index len; a caller that knows the length passes it by value
+    const int skv = (len_dev ? *len_dev : len_host) + 1;
     // local rows of this split: 16 per whole granule it owns, plus the tail if the last, partial granule is its own
     const int gfull = skv >> 4;
     int nk = gfull > split ? ((gfull - split + S - 1) / S) * 16 : 0;
@@ -251,8 +252,8 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
     }
 }
 
-template <int D>
-__global__ __launch_bounds__(D) void k_attn_combine_dl(const float *__restrict__ part, int splits, float *__restrict__ out) {
+template <int D, typename TO = float>
+__global__ __launch_bounds__(D) void k_attn_combine_dl(const float *__restrict__ part, int splits, TO *__restrict__ out) {
     const int64_t h = blockIdx.x;
     const float *pp = part + h * splits * (D + 4);
     float mx = -INFINITY;
@@ -264,18 +265,20 @@ __global__ __launch_bounds__(D) void k_attn_combine_dl(const float *__restrict__
         num = fmaf(pp[s * (D + 4) + threadIdx.x], w, num);
         den = fmaf(pp[s * (D + 4) + D + 1], w, den);
     }
-    out[h * D + threadIdx.x] = num / den;
+    out[h * D + threadIdx.x] = (TO)(num / den);
 }
 
 template <typename TKV, int G, int NWV>
 static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const void *v, int64_t kv_sh, int64_t kv_st,
                            int hq, int hkv, float scale, const int *len_dev, int max_len, float *out, int *splits_out,
-                           int gtot) {
+                           int gtot, int len_host = 0, int splits_req = 0, bool out_f16 = false) {
     constexpr int D = 128;
     // splits: 8 measured best from a few hundred to a few thousand keys (MI355X); it is also the most the output
-    // projection merges while staging its input.  The option allows 4 .. 16.
+    // projection merges while staging its input.  The option allows 4 .. 16; a caller with a long cache and its
+    // own merge asks for more.
     int S = dev->opt_attn_splits > 0 ? (int)dev->opt_attn_splits : 8;
     S = S < 4 ? 4 : (S > 16 ? 16 : S);
+    if (splits_req > 0) S = splits_req;
     const int chunk_max = (((max_len + 15) / 16 + S - 1) / S) * 16; // most local rows of a split
     const size_t lds = ((size_t)G * chunk_max + (size_t)NWV * G * D) * 4;
     FH_REQUIRE(lds <= 150 * 1024, "KV capacity %d too large for the decode attention kernel", max_len);
@@ -287,11 +290,13 @@ static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const 
         attr_done = true;
     }
     k_attn_decode_dl<TKV, D, G, NWV><<<dim3((unsigned)S, (unsigned)hkv, (unsigned)(gtot / G)), dim3(64 * NWV), lds, dev->stream>>>(
-        q, (const TKV *)k, (const TKV *)v, kv_sh, kv_st, len_dev, scale, chunk_max, max_len, gtot, dev->part_buf);
+        q, (const TKV *)k, (const TKV *)v, kv_sh, kv_st, len_dev, len_host, scale, chunk_max, max_len, gtot, dev->part_buf);
     FH_HIP(hipGetLastError());
     if (splits_out) *splits_out = S;
     if (out) {
-        k_attn_combine_dl<D><<<dim3((unsigned)hq), dim3(D), 0, dev->stream>>>(dev->part_buf, S, out);
+        if (out_f16)
+            k_attn_combine_dl<D, fh_half><<<dim3((unsigned)hq), dim3(D), 0, dev->stream>>>(dev->part_buf, S, (fh_half *)out);
+        else k_attn_combine_dl<D><<<dim3((unsigned)hq), dim3(D), 0, dev->stream>>>(dev->part_buf, S, out);
         FH_HIP(hipGetLastError());
     }
     return FH_OK;
@@ -306,18 +311,43 @@ fh_status fh_attention_combine_dl(fh_device *dev, int hq, int splits, float *out
 
 // out != NULL: the attention output [hq, d].  out == NULL: the partials stay in the device's scratch
 // ([hq][*splits_out][d + 4]) for a consumer that merges them itself.
+static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v, int64_t kv_sh,
+                        int64_t kv_st, int hq, int hkv, int d, float scale, const int *len_dev, int max_len, float *out,
+                        int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req = 0);
+
 fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
                                      int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale,
                                      const int *len_dev, int max_len, float *out, int *splits_out) {
+    return ad_any(dev, kv_dtype, q, k, v, kv_sh, kv_st, hq, hkv, d, scale, len_dev, max_len, out, splits_out, 0, 0, false);
+}
+
+// One f32 query per head against `skv` cached keys known on the host; `out` is f32 or f16 [hq, d].  The key
+// range is cut into more parts the longer it is (every part is a workgroup per KV head and query-head group).
+fh_status fh_attention_decode_hostlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
+                                      int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale, int skv,
+                                      void *out, bool out_f16) {
+    int splits = skv <= 2048 ? 8 : (skv <= 8192 ? 16 : 32);
+    if (dev->opt_attn_splits > 0) splits = dev->opt_attn_splits > 128 ? 128 : (int)dev->opt_attn_splits;
+    // long caches are bandwidth bound: all query heads of a KV head in one workgroup, so K and V are read once
+    // (measured on MI355X, 32 / 8 heads, f16 cache: 1 head x 8 parts at 1024 keys, 2 x 16 at 4096, 4 x 32 at 16384)
+    const int heads = dev->opt_attn_heads > 0 ? (int)dev->opt_attn_heads : (skv <= 2048 ? 1 : (skv <= 8192 ? 2 : 4));
+    return ad_any(dev, kv_dtype, q, k, v, kv_sh, kv_st, hq, hkv, d, scale, nullptr, skv, (float *)out, nullptr, skv - 1,
+                  splits, out_f16, heads);
+}
+
+static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v, int64_t kv_sh,
+                        int64_t kv_st, int hq, int hkv, int d, float scale, const int *len_dev, int max_len, float *out,
+                        int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req) {
     const int gtot = hq / hkv;
     if (d != 128 || (gtot != 1 && gtot != 2 && gtot != 4 && gtot != 8) || kv_st % 8 || kv_sh % 8) return FH_ERR_UNSUPPORTED;
     // query heads per workgroup: the arithmetic of a workgroup grows with them, the K and V reads do not; one
     // (the workgroups of a KV head then share the rows through the L2) measured best on MI355X for 4 heads per KV
     // head at contexts of some hundred keys: 256 workgroups instead of 64
     int G = dev->opt_attn_heads > 0 ? (int)dev->opt_attn_heads : 1;
+    if (heads_req > 0) G = heads_req > gtot ? gtot : heads_req;
     while (G > 1 && (gtot % G || (G != 2 && G != 4 && G != 8))) G /= 2;
     const bool w8 = dev->opt_attn_waves == 8 && G <= 8; // 8 wavefronts per workgroup instead of 16
-#define AD_ARGS dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out, gtot
+#define AD_ARGS dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out, gtot, len_host, splits_req, out_f16
 #define AD_GO(TKV_)                                                                       \
     switch (G) {                                                                          \
     case 1: return w8 ? ad_launch<TKV_, 1, 8>(AD_ARGS) : ad_launch<TKV_, 1, 16>(AD_ARGS); \
