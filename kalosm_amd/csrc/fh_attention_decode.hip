@@ -252,20 +252,45 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
     }
 }
 
+// Merge of the parts of one head: thread t fetches the statistics of part t (all parts at once instead of one
+// dependent load per loop trip), the weights go through LDS, and the weighted rows are summed eight loads at a time.
 template <int D, typename TO = float>
 __global__ __launch_bounds__(D) void k_attn_combine_dl(const float *__restrict__ part, int splits, TO *__restrict__ out) {
+    static_assert(D >= 128, "one thread per part: up to 128 parts");
+    __shared__ float s_m[D], s_w[D];
     const int64_t h = blockIdx.x;
+    const int t = threadIdx.x;
     const float *pp = part + h * splits * (D + 4);
-    float mx = -INFINITY;
-    for (int s = 0; s < splits; s++) mx = fmaxf(mx, pp[s * (D + 4) + D]);
-    float num = 0.f, den = 0.f;
-    for (int s = 0; s < splits; s++) {
-        const float m = pp[s * (D + 4) + D];
-        const float w = (m == -INFINITY) ? 0.f : __expf(m - mx);
-        num = fmaf(pp[s * (D + 4) + threadIdx.x], w, num);
-        den = fmaf(pp[s * (D + 4) + D + 1], w, den);
+    float m = -INFINITY, l = 0.f;
+    if (t < splits) {
+        m = pp[t * (D + 4) + D];
+        l = pp[t * (D + 4) + D + 1];
     }
-    out[h * D + threadIdx.x] = (TO)(num / den);
+    s_m[t] = m;
+    __syncthreads();
+    float mx = -INFINITY;
+    for (int s = 0; s < splits; s++) mx = fmaxf(mx, s_m[s]);
+    const float w = (m == -INFINITY) ? 0.f : __expf(m - mx);
+    s_w[t] = w;
+    s_m[t] = l * w; // reuse: weighted denominators
+    __syncthreads();
+    float num = 0.f, den = 0.f;
+    int s = 0;
+    for (; s + 8 <= splits; s += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = pp[(s + u) * (D + 4) + t];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            num = fmaf(v[u], s_w[s + u], num);
+            den += s_m[s + u];
+        }
+    }
+    for (; s < splits; s++) {
+        num = fmaf(pp[s * (D + 4) + t], s_w[s], num);
+        den += s_m[s];
+    }
+    out[h * D + t] = (TO)(num / den);
 }
 
 template <typename TKV, int G, int NWV>
