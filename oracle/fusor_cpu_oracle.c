@@ -19,11 +19,17 @@
  *   f16 conversion ........ exhaustive 65536-value round trip vs numpy.float16
  *   dequantize (4 formats)  reference known answers (+528/-528, nibble identity),
  *                           an independent numpy restatement, brute-force scale unpack
+ *   dequantize Q5_0 / Q5_K  reference known answers (+528/-528, 32896, nibble identity, all high
+ *                           bits -> 16), an independent numpy restatement, and the special case
+ *                           qh = 0 where a Q5_K block must equal the Q4_K block bit for bit
+ *   dense f16 / f32 rows .. the stored values; their product goes through the reference's dense
+ *                           matmul (gemm crate): accumulation order UNPINNED, tolerance only
  *   q_mat_mul ............. one-hot / zero / linearity invariants, float64 dense product
  *   q8_0 quantize/vec_dot . closed form, exact integer sums, round trip < 0.02
  *   attention ............. torch CPU scaled_dot_product_attention, softmax invariants
  *   rms_norm / rope / silu  numpy formulas from the reference's conformance host
- *                           references; RoPE golden sextets; inverse-frequency closed form
+ *                           references; RoPE golden sextets; inverse-frequency closed form;
+ *                           long-context scaling and rope_freqs weights against numpy
  *   argmax ................ tie and non-finite cases from the reference's rule
  *   decoder ............... PARITY UNPINNED in the reference (no stored logits);
  *                           pinned here only by composition of the pinned ops and an
