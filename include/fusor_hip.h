@@ -254,6 +254,11 @@ fh_status fh_cast_f32_bf16(fh_device *dev, const float *x_dev, void *y_bf16_dev,
 /* Tensor::top_k_pairs(1), fusor-ml/fusor/src/lib.rs:416-447: largest finite value, ties to the
  * larger index, non-finite skipped; *id_dev = 0xFFFFFFFF when nothing is finite. */
 fh_status fh_argmax(fh_device *dev, const float *x_dev, int64_t count, uint32_t *id_dev);
+/* Tensor::top_k_pairs(k), fusor-ml/fusor/src/lib.rs:416-447, 1 <= k <= 256: ids_dev[k] / values_dev[k] in
+ * descending order of the value, ties to the larger index, non-finite values skipped; *found_dev
+ * (optional) = number of pairs found, the rest is filled with id 0xFFFFFFFF / NaN. */
+fh_status fh_top_k(fh_device *dev, const float *x_dev, int64_t count, int32_t k, uint32_t *ids_dev,
+                   float *values_dev, uint32_t *found_dev);
 
 /* -------------------------------------------------------------- GGUF files
  * GgufMetadata::read, fusor-ml/gguf/src/lib.rs:559-613: versions 1 .. 3, metadata key/values, tensor

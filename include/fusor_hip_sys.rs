@@ -161,6 +161,7 @@ extern "C" {
     pub fn fh_cast_f16_f32(dev: *mut FhDevice, x_f16_dev: *const c_void, y_dev: *mut f32, count: i64) -> FhStatus;
     pub fn fh_cast_f32_bf16(dev: *mut FhDevice, x_dev: *const f32, y_bf16_dev: *mut c_void, count: i64) -> FhStatus;
     pub fn fh_argmax(dev: *mut FhDevice, x_dev: *const f32, count: i64, id_dev: *mut u32) -> FhStatus;
+    pub fn fh_top_k(dev: *mut FhDevice, x_dev: *const f32, count: i64, k: i32, ids_dev: *mut u32, values_dev: *mut f32, found_dev: *mut u32) -> FhStatus;
     pub fn fh_gguf_open(path: *const c_char, out: *mut *mut FhGguf) -> FhStatus;
     pub fn fh_gguf_open_memory(bytes: *const c_void, len: usize, out: *mut *mut FhGguf) -> FhStatus;
     pub fn fh_gguf_close(g: *mut FhGguf) -> FhStatus;

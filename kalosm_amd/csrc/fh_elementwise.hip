@@ -393,6 +393,94 @@ extern "C" fh_status fh_argmax(fh_device *dev, const float *x_dev, int64_t count
     return FH_OK;
 }
 
+// ------------------------------------------------------------------------------ top-k
+// Tensor::top_k_pairs(k), fusor-ml/fusor/src/lib.rs:416-447: the k largest FINITE logits in descending order, ties
+// to the larger token id.  (value, id) becomes one 64-bit key whose unsigned order is that order (-0.0 ranks with
+// +0.0, as the reference's float compare does); every workgroup sorts 1024 keys in LDS (bitonic, descending) and
+// keeps its first k; passes repeat over the survivors until one workgroup is left.
+__device__ __forceinline__ uint64_t topk_key(float v, uint32_t id) {
+    uint32_t b = __float_as_uint(v);
+    if ((b & 0x7F800000u) == 0x7F800000u) return 0; // infinities and NaNs are skipped
+    if (b == 0x80000000u) b = 0;
+    const uint32_t o = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+    return ((uint64_t)o << 32) | id;
+}
+
+template <bool FIRST>
+__global__ __launch_bounds__(512) void k_topk_pass(const float *__restrict__ x, const uint64_t *__restrict__ keys_in,
+                                                   int64_t n_in, int k, int last, uint64_t *__restrict__ keys_out,
+                                                   uint32_t *__restrict__ ids_out, float *__restrict__ vals_out,
+                                                   uint32_t *__restrict__ found_out) {
+    __shared__ uint64_t s[1024];
+    const int tid = threadIdx.x;
+    const int64_t base = (int64_t)blockIdx.x * 1024;
+    for (int i = tid; i < 1024; i += 512) {
+        const int64_t idx = base + i;
+        s[i] = idx < n_in ? (FIRST ? topk_key(x[idx], (uint32_t)idx) : keys_in[idx]) : 0ull;
+    }
+    __syncthreads();
+    for (int size = 2; size <= 1024; size <<= 1)
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            const int a = 2 * tid - (tid & (stride - 1)), b = a + stride;
+            const uint64_t va = s[a], vb = s[b];
+            const bool down = (a & size) == 0; // this run is sorted descending
+            if ((va < vb) == down) {
+                s[a] = vb;
+                s[b] = va;
+            }
+            __syncthreads();
+        }
+    if (!last) {
+        for (int i = tid; i < k; i += 512) keys_out[(int64_t)blockIdx.x * k + i] = s[i];
+        return;
+    }
+    for (int i = tid; i < k; i += 512) {
+        const uint64_t key = s[i];
+        ids_out[i] = key ? (uint32_t)key : 0xFFFFFFFFu;
+        vals_out[i] = key ? x[(uint32_t)key] : __uint_as_float(0x7FC00000u);
+    }
+    if (tid == 0 && found_out) {
+        int c = 0;
+        while (c < k && s[c]) c++;
+        *found_out = (uint32_t)c;
+    }
+}
+
+extern "C" fh_status fh_top_k(fh_device *dev, const float *x_dev, int64_t count, int32_t k, uint32_t *ids_dev,
+                              float *values_dev, uint32_t *found_dev) {
+    FH_REQUIRE(dev && x_dev && ids_dev && values_dev, "NULL argument");
+    FH_REQUIRE(count > 0 && count < 0xFFFFFFFFll, "count %lld out of range", (long long)count);
+    FH_REQUIRE(k >= 1 && k <= 256, "k = %d out of range (1 .. 256)", k);
+    int64_t n = count, blocks = (n + 1023) / 1024;
+    uint64_t *buf[2] = {nullptr, nullptr};
+    if (blocks > 1) {
+        const size_t half = ((size_t)blocks * k * 8 + 255) & ~(size_t)255;
+        FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, 2 * half));
+        buf[0] = (uint64_t *)dev->ksplit_buf;
+        buf[1] = (uint64_t *)((uint8_t *)dev->ksplit_buf + half);
+    }
+    const uint64_t *in = nullptr;
+    bool first = true;
+    int turn = 0;
+    for (;;) {
+        const int last = blocks == 1;
+        if (first)
+            k_topk_pass<true><<<dim3((unsigned)blocks), dim3(512), 0, dev->stream>>>(x_dev, nullptr, n, k, last, buf[turn],
+                                                                                    ids_dev, values_dev, found_dev);
+        else
+            k_topk_pass<false><<<dim3((unsigned)blocks), dim3(512), 0, dev->stream>>>(x_dev, in, n, k, last, buf[turn],
+                                                                                     ids_dev, values_dev, found_dev);
+        FH_HIP(hipGetLastError());
+        if (last) break;
+        in = buf[turn];
+        turn ^= 1;
+        n = blocks * k;
+        blocks = (n + 1023) / 1024;
+        first = false;
+    }
+    return FH_OK;
+}
+
 // ------------------------------------------------------------------------------ KV cache
 // fusor-ml/fusor/src/cache/tensor_cache.rs:70-114 (in-place slice write into a grown backing buffer),
 // :304-312 (power-of-two growth, minimum 256, capped at max_len).

@@ -294,6 +294,16 @@ class Tensor:
         check(self.device._lib.fh_transpose_shd(self.device._h, C.c_void_p(self.ptr), s, h, d, C.c_void_p(out.ptr)))
         return out
 
+    def top_k_pairs(self, k: int):
+        """Tensor::top_k_pairs(k) (fusor-ml/fusor/src/lib.rs:416-447): [(token id, logit)] in descending order."""
+        if k == 0:
+            return []
+        ids, vals, found = Tensor(self.device, (k,), "u32"), Tensor(self.device, (k,), "f32"), Tensor(self.device, (1,), "u32")
+        check(self.device._lib.fh_top_k(self.device._h, C.c_void_p(self.ptr), int(np.prod(self.shape)), k,
+                                        C.c_void_p(ids.ptr), C.c_void_p(vals.ptr), C.c_void_p(found.ptr)))
+        n = int(found.as_slice()[0])
+        return list(zip(ids.as_slice()[:n].tolist(), vals.as_slice()[:n].tolist()))
+
     def top_k_pairs_1(self) -> int:
         """Tensor::top_k_pairs(1) (fusor-ml/fusor/src/lib.rs:416-447): the greedy token id, or -1."""
         out = Tensor(self.device, (1,), "u32")

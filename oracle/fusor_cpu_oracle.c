@@ -783,6 +783,30 @@ int64_t fo_argmax(const float *x, size_t n) {
     return best;
 }
 
+/* fusor/src/lib.rs:416-447 for any k: the insertion loop as written (a sorted list of at most k pairs; a new
+ * finite logit replaces the last one when it is larger, or equal with a larger token id).  Returns the count. */
+int fo_top_k(const float *x, size_t n, int k, uint32_t *ids, float *vals) {
+    int len = 0;
+    if (k <= 0) return 0;
+    for (size_t t = 0; t < n; t++) {
+        float v = x[t];
+        if (!isfinite(v)) continue;
+        if (len == k) {
+            float lv = vals[len - 1];
+            uint32_t li = ids[len - 1];
+            if (v > lv || (v == lv && (uint32_t)t > li)) len = k - 1;
+            else continue;
+        }
+        int at = 0; /* partition point: entries that stay in front of the new one */
+        while (at < len && (vals[at] > v || (vals[at] == v && ids[at] > (uint32_t)t))) at++;
+        for (int i = len; i > at; i--) { vals[i] = vals[i - 1]; ids[i] = ids[i - 1]; }
+        vals[at] = v;
+        ids[at] = (uint32_t)t;
+        len++;
+    }
+    return len;
+}
+
 /* fusor/src/layers/embedding.rs:43-89: out[t,:] = dequantize(W)[id[t],:] */
 int fo_embed_rows(int t, const uint8_t *w, int n, int k, const uint32_t *ids, int count, float *out) {
     int e = fo_block_elems(t), bb = fo_block_bytes(t);

@@ -282,6 +282,16 @@ def add3(a, b, c) -> np.ndarray:
     return y
 
 
+def top_k(x, k: int):
+    """[(id, value)] as Tensor::top_k_pairs(k) returns them."""
+    x = _f32(x).reshape(-1)
+    ids, vals = np.empty(max(k, 1), np.uint32), np.empty(max(k, 1), np.float32)
+    L = lib()
+    L.fo_top_k.argtypes = [C.POINTER(C.c_float), C.c_size_t, C.c_int, C.POINTER(C.c_uint32), C.POINTER(C.c_float)]
+    n = L.fo_top_k(_p(x, C.c_float), x.size, k, _p(ids, C.c_uint32), _p(vals, C.c_float))
+    return list(zip(ids[:n].tolist(), vals[:n].tolist()))
+
+
 def argmax(x) -> int:
     x = _f32(x).reshape(-1)
     return int(lib().fo_argmax(_p(x, C.c_float), x.size))

@@ -313,3 +313,30 @@ def test_attention_prefill_f32_on_request(dev, oracle):
         assert_close(got, np.full_like(got, 0.75), abs_tol=1e-3, rel_tol=1e-3, what="constant V")
     finally:
         dev.set_option("attn_kernel", 0)
+
+
+@pytest.mark.parametrize("n", [5, 1000, 1024, 1025, 128256])
+def test_top_k_pairs(dev, oracle, n):
+    """Tensor::top_k_pairs(k) (fusor/src/lib.rs:416-447) at vocabulary size and at the pass boundaries: bit-equal
+    pairs in the reference's order (descending logit, ties to the larger id, non-finite skipped)."""
+    rng = np.random.default_rng(n)
+    for variant in range(3):
+        if variant == 0:
+            x = rng.standard_normal(n).astype(np.float32)
+        elif variant == 1:
+            x = rng.integers(-3, 4, n).astype(np.float32)      # almost everything ties
+            x[rng.integers(0, n, max(1, n // 50))] = np.nan
+            x[rng.integers(0, n, 2)] = [np.inf, -np.inf]
+            x[rng.integers(0, n, 2)] = [0.0, -0.0]
+        else:
+            x = np.full(n, np.nan, np.float32)                 # fewer finite values than k
+            x[rng.integers(0, n, 3)] = [1.5, -2.0, 1.5]
+        t = Tensor.from_slice(dev, x)
+        for k in (1, 5, 64, 256):
+            got = t.top_k_pairs(k)
+            want = oracle.top_k(x, k)
+            assert [g[0] for g in got] == [w[0] for w in want], (n, variant, k)
+            assert np.array_equal(np.float32([g[1] for g in got]).view(np.uint32), np.float32([w[1] for w in want]).view(np.uint32))
+    assert t.top_k_pairs(0) == []
+    with pytest.raises(Exception):
+        t.top_k_pairs(257)

@@ -407,3 +407,23 @@ def test_rope_scaling_closed_form(oracle):
     c0, s0 = oracle.rope_tables_scaled(dim, ctx, theta, None, None)
     c1, s1 = oracle.rope_tables(dim, ctx, theta)
     assert np.array_equal(c0, c1) and np.array_equal(s0, s1)
+
+
+def np_top_k(x, k):
+    """Brute force: finite entries sorted by (value descending, id descending)."""
+    idx = [i for i in range(len(x)) if np.isfinite(x[i])]
+    idx.sort(key=lambda i: (-float(x[i]), -i))
+    return [(i, float(x[i])) for i in idx[:k]]
+
+
+def test_top_k_matches_brute_force(oracle):
+    """fusor/src/lib.rs:416-447: descending logits, ties to the larger id, non-finite skipped, fewer than k allowed."""
+    rng = np.random.default_rng(5)
+    x = rng.integers(-5, 6, 200).astype(np.float32)          # many ties
+    x[[3, 50, 199]] = np.nan
+    x[[7, 8]] = [np.inf, -np.inf]
+    x[[20, 21]] = [0.0, -0.0]
+    for k in (1, 2, 7, 64, 195, 300):
+        assert oracle.top_k(x, k) == np_top_k(x, k)
+    assert oracle.top_k(x, 1)[0][0] == oracle.argmax(x)
+    assert oracle.top_k(np.float32([np.nan, np.inf]), 3) == [] and oracle.top_k(x, 0) == []
