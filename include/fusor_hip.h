@@ -200,11 +200,15 @@ fh_status fh_rope_pair(fh_device *dev, const float *q_dev, int64_t q_sb, int64_t
  * tensor_cache.rs:70-114, :304-312.  One object holds all layers.  Storage is
  * [layer][kv_head][capacity][head_dim] per K and V, f32 (the reference's cache type,
  * models/kalosm-llama/src/raw/cache.rs:18) or f16.  Capacity grows to the next power of two
- * (minimum 256, capped at max_len) preserving contents; exceeding max_len is FH_ERR_INVALID
- * (sliding-window eviction is outside this library's scope). */
+ * (minimum 256, capped at max_len) preserving contents; exceeding max_len is FH_ERR_INVALID unless
+ * the cache was switched to a sliding window (fh_kvcache_set_sliding). */
 fh_status fh_kvcache_create(fh_device *dev, int32_t layers, int32_t kv_heads, int32_t head_dim,
                             int32_t max_len, int32_t dtype, fh_kvcache **out);
 fh_status fh_kvcache_destroy(fh_kvcache *c);
+/* Sliding-window caches (KvCache with a window, fusor-ml/fusor/src/cache/tensor_cache.rs:175-202):
+ * once an append would exceed max_len the cache keeps the last max_len positions of [cached | new].
+ * Applies to fh_kvcache_append; the decoder driver's captured steps do not evict. */
+fh_status fh_kvcache_set_sliding(fh_kvcache *c, int32_t on);
 fh_status fh_kvcache_reset(fh_kvcache *c);
 /* Append s positions to `layer`.  k and v are [kv_heads, s, head_dim] f32 views with head stride
  * `sh` and position stride `st` (elements).  The cache length advances when the LAST layer is

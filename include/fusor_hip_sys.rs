@@ -149,6 +149,7 @@ extern "C" {
     pub fn fh_rope_pair(dev: *mut FhDevice, q_dev: *const f32, q_sb: i64, q_sh: i64, q_st: i64, k_dev: *const f32, k_sb: i64, k_sh: i64, k_st: i64, b: i32, hq: i32, hk: i32, s: i32, d: i32, cos_dev: *const f32, sin_dev: *const f32, table_rows: i32, start_pos: i32, interleaved: i32, q_out_dev: *mut f32, k_out_dev: *mut f32) -> FhStatus;
     pub fn fh_kvcache_create(dev: *mut FhDevice, layers: i32, kv_heads: i32, head_dim: i32, max_len: i32, dtype: i32, out: *mut *mut FhKvCache) -> FhStatus;
     pub fn fh_kvcache_destroy(c: *mut FhKvCache) -> FhStatus;
+    pub fn fh_kvcache_set_sliding(c: *mut FhKvCache, on: i32) -> FhStatus;
     pub fn fh_kvcache_reset(c: *mut FhKvCache) -> FhStatus;
     pub fn fh_kvcache_append(c: *mut FhKvCache, layer: i32, k_dev: *const f32, v_dev: *const f32, sh: i64, st: i64, s: i32) -> FhStatus;
     pub fn fh_kvcache_view(c: *const FhKvCache, layer: i32, len: *mut i32, capacity: *mut i32, k_dev: *mut *const c_void, v_dev: *mut *const c_void) -> FhStatus;

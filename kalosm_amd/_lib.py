@@ -95,6 +95,7 @@ SIGNATURES = {
     "fh_cast_f16_f32": [_p, _p, _p, _i64],
     "fh_cast_f32_bf16": [_p, _p, _p, _i64],
     "fh_argmax": [_p, _p, _i64, _p],
+    "fh_kvcache_set_sliding": [_p, _i32],
     "fh_top_k": [_p, _p, _i64, _i32, _p, _p, _p],
     "fh_llama_create": [_p, C.POINTER(LlamaConfig), _pp],
     "fh_llama_destroy": [_p],

@@ -627,10 +627,45 @@ fh_status fh_kvcache_set_len_dev(fh_kvcache *c, int len) {
     return FH_OK;
 }
 
+extern "C" fh_status fh_kvcache_set_sliding(fh_kvcache *c, int32_t on) {
+    FH_REQUIRE(c, "NULL argument");
+    c->sliding = on != 0;
+    return FH_OK;
+}
+
 extern "C" fh_status fh_kvcache_append(fh_kvcache *c, int32_t layer, const float *k_dev, const float *v_dev, int64_t sh,
                                        int64_t st, int32_t s) {
     FH_REQUIRE(c && k_dev && v_dev, "NULL argument");
     FH_REQUIRE(layer >= 0 && layer < c->layers && s > 0, "bad layer %d / s %d", layer, s);
+    if (c->sliding && c->len + s > c->max_len) {
+        // TensorCache::append_gpu_evict, fusor-ml/fusor/src/cache/tensor_cache.rs:175-202: the cache becomes the
+        // last max_len positions of [cached | new]
+        const int max = c->max_len, evict = c->len + s - max;
+        const int keep = c->len > evict ? c->len - evict : 0; // cached rows that survive, moved to the front
+        const int skip = s > max ? s - max : 0;               // new rows that fall out at once
+        FH_TRY(fh_kvcache_reserve(c, max));
+        if (keep > 0) {
+            const size_t es = fh_dtype_size(c->dtype), row = (size_t)c->head_dim * es;
+            const size_t pitch = (size_t)c->capacity * row, width = (size_t)keep * row;
+            const size_t plane = (size_t)c->kv_heads * pitch;
+            FH_TRY(fh_dev_scratch(c->dev, &c->dev->act_buf, &c->dev->act_cap, (size_t)c->kv_heads * width));
+            for (void *base : {c->k, c->v}) { // through a scratch copy: the ranges overlap
+                uint8_t *lp = (uint8_t *)base + (size_t)layer * plane;
+                FH_HIP(hipMemcpy2DAsync(c->dev->act_buf, width, lp + (size_t)evict * row, pitch, width, c->kv_heads,
+                                        hipMemcpyDeviceToDevice, c->dev->stream));
+                FH_HIP(hipMemcpy2DAsync(lp, pitch, c->dev->act_buf, width, width, c->kv_heads, hipMemcpyDeviceToDevice,
+                                        c->dev->stream));
+            }
+        }
+        FH_TRY(kv_append_launch(c, layer, k_dev + (int64_t)skip * st, sh, st, v_dev + (int64_t)skip * st, sh, st, s - skip,
+                                keep, nullptr));
+        if (layer == c->layers - 1) {
+            c->len = max;
+            k_set_int<<<1, 1, 0, c->dev->stream>>>(c->len_dev, c->len);
+            FH_HIP(hipGetLastError());
+        }
+        return FH_OK;
+    }
     FH_TRY(fh_kvcache_reserve(c, c->len + s));
     FH_TRY(kv_append_launch(c, layer, k_dev, sh, st, v_dev, sh, st, s, c->len, nullptr));
     if (layer == c->layers - 1) {

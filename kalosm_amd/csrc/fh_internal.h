@@ -186,6 +186,7 @@ struct fh_kvcache {
     fh_device *dev = nullptr;
     int layers = 0, kv_heads = 0, head_dim = 0, max_len = 0, dtype = FH_F32;
     int len = 0, capacity = 0;
+    bool sliding = false;            // past max_len: keep the last max_len positions instead of failing
     void *k = nullptr, *v = nullptr; // [layers][kv_heads][capacity][head_dim]
     int *len_dev = nullptr;          // device copy of len (for graph-replayed decode steps)
 };

@@ -431,12 +431,15 @@ class RopeCache:
 class KvCache:
     """fusor::KvCache (fusor-ml/fusor/src/cache/kv_cache.rs:24-63) for `layers` layers at once."""
 
-    def __init__(self, device: Device, layers: int, kv_heads: int, head_dim: int, max_len: int, dtype: str = "f32"):
+    def __init__(self, device: Device, layers: int, kv_heads: int, head_dim: int, max_len: int, dtype: str = "f32",
+                 sliding_window: bool = False):
         self.device, self.layers, self.kv_heads, self.head_dim, self.dtype = device, layers, kv_heads, head_dim, dtype
         h = C.c_void_p()
         check(device._lib.fh_kvcache_create(device._h, layers, kv_heads, head_dim, max_len, F16 if dtype == "f16" else F32,
                                             C.byref(h)))
         self._h = h
+        if sliding_window:  # keep the last max_len positions (tensor_cache.rs:175-202) instead of failing when full
+            check(device._lib.fh_kvcache_set_sliding(h, 1))
 
     def append(self, layer: int, k: Tensor, v: Tensor) -> None:
         """k, v: [kv_heads, s, head_dim] f32 contiguous."""

@@ -248,6 +248,29 @@ def test_kv_cache_growth_append_reset(dev, dtype):
     assert c.view(0)[0] == 0
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_kv_cache_sliding_window(dev, dtype):
+    """TensorCache sliding window (tensor_cache.rs:175-202): past max_len the cache is the last max_len positions of
+    [cached | new], also when one append is longer than the window."""
+    layers, hk, d, window = 2, 2, 64, 300
+    c = KvCache(dev, layers, hk, d, max_len=window, dtype=dtype, sliding_window=True)
+    rng = np.random.default_rng(12)
+    hist = [[np.zeros((hk, 0, d), np.float32) for _ in range(2)] for _ in range(layers)]
+    for s in (200, 99, 1, 1, 7, 150, 299, 300, 1, 450, 3):
+        for l in range(layers):
+            k = rng.standard_normal((hk, s, d)).astype(np.float32)
+            v = rng.standard_normal((hk, s, d)).astype(np.float32)
+            c.append(l, Tensor.from_slice(dev, k), Tensor.from_slice(dev, v))
+            hist[l][0] = np.concatenate([hist[l][0], k], 1)[:, -window:]
+            hist[l][1] = np.concatenate([hist[l][1], v], 1)[:, -window:]
+        for l in range(layers):
+            ln, cap, kt, vt = c.view(l)
+            assert ln == hist[l][0].shape[1] <= window
+            for got, want in ((kt, hist[l][0]), (vt, hist[l][1])):
+                want = want.astype(np.float16).astype(np.float32) if dtype == "f16" else want
+                assert np.array_equal(got.as_slice()[:, :ln].astype(np.float32), want), (s, l)
+
+
 # ----------------------------------------------------------------------------- prefill attention on the matrix cores
 @pytest.mark.parametrize("d", [128, 64])
 @pytest.mark.parametrize("sq,skv,causal", [(128, 128, True), (200, 200, True), (64, 300, True), (160, 97, False),
