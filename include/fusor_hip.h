@@ -54,7 +54,8 @@ enum {
 enum { FH_Q4_0 = 2, FH_Q5_0 = 6, FH_Q8_0 = 8, FH_Q4_K = 12, FH_Q5_K = 13, FH_Q6_K = 14 };
 
 /* MaskKind, fusor-ml/fusor/src/composite/flash_attention.rs:12-24 */
-enum { FH_MASK_NONE = 0, FH_MASK_CAUSAL = 1, FH_MASK_ADDITIVE = 2 };
+enum { FH_MASK_NONE = 0, FH_MASK_CAUSAL = 1, FH_MASK_ADDITIVE = 2 /* QKMask [sq, skv] */,
+       FH_MASK_BATCH_KEY = 3 /* BatchKeyMask [b, skv], added for every head and query of a batch entry */ };
 
 /* element types of attention operands */
 enum { FH_F32 = 0, FH_F16 = 1 };

@@ -42,6 +42,8 @@ pub const FH_Q6_K: u32 = 14;
 pub const FH_MASK_NONE: i32 = 0;
 pub const FH_MASK_CAUSAL: i32 = 1;
 pub const FH_MASK_ADDITIVE: i32 = 2;
+/// `MaskKind::BatchKeyMask`: additive [batch, kv_len] mask
+pub const FH_MASK_BATCH_KEY: i32 = 3;
 
 /// element types of attention operands and of the KV cache
 pub const FH_F32: i32 = 0;

@@ -213,6 +213,7 @@ __global__ __launch_bounds__(256) void k_attn_rows(const TQ *__restrict__ q, int
             for (int c = 0; c < d; c++) a = fmaf(s_q[c], ld1(kr + c), a);
             sc = a * scale;
             if (mask_kind == FH_MASK_ADDITIVE) sc = sc + mask[(int64_t)i * skv + t];
+            if (mask_kind == FH_MASK_BATCH_KEY) sc = sc + mask[(int64_t)bi * skv + t];
         }
         float mx = sc;
 #pragma unroll
@@ -306,7 +307,8 @@ static fh_status attn_typed(fh_device *dev, const void *q, int64_t q_sb, int64_t
     const bool aligned = (kv_st % 8 == 0) && (kv_sh % 8 == 0) && (kv_sb % 8 == 0);
     // one batch entry, head_dim 128, contiguous query heads, no additive mask: the decode-step kernel (an f16
     // query is widened into the device's small buffer first)
-    if (sq == 1 && b == 1 && d == 128 && aligned && q_sh == d && mask_kind != FH_MASK_ADDITIVE && hq <= 64 &&
+    const bool masked = mask_kind == FH_MASK_ADDITIVE || mask_kind == FH_MASK_BATCH_KEY;
+    if (sq == 1 && b == 1 && d == 128 && aligned && q_sh == d && !masked && hq <= 64 &&
         dev->opt_attn_kernel != 1) {
         const float *q32 = (const float *)q;
         if constexpr (!std::is_same<TQ, float>::value) {
@@ -317,7 +319,8 @@ static fh_status attn_typed(fh_device *dev, const void *q, int64_t q_sb, int64_t
                                                    kv_st, hq, hkv, d, scale, skv, out, !std::is_same<TQ, float>::value);
         if (st != FH_ERR_UNSUPPORTED) return st;
     }
-    if (sq == 1 && aligned && (d == 128 || d == 64) && (G == 1 || G == 2 || G == 4 || G == 8)) {
+    if (sq == 1 && aligned && (d == 128 || d == 64) && (G == 1 || G == 2 || G == 4 || G == 8) &&
+        mask_kind != FH_MASK_BATCH_KEY) {
         const float *mrow = mask_kind == FH_MASK_ADDITIVE ? mask : nullptr;
         fh_status st = d == 128 ? decode_dispatch_g<TQ, TKV, 128>(dev, G, q, q_sb, q_sh, k, v, kv_sb, kv_sh, kv_st, b, hq,
                                                                  hkv, skv, nullptr, scale, mrow, out)
@@ -342,14 +345,14 @@ extern "C" fh_status fh_flash_attention_ex(fh_device *dev, int32_t q_dtype, int3
     FH_REQUIRE(dev && q_dev && k_dev && v_dev && out_dev, "NULL argument");
     FH_REQUIRE(b > 0 && hq > 0 && hkv > 0 && sq > 0 && skv > 0 && d > 0, "empty attention operand");
     FH_REQUIRE(hq % hkv == 0, "number of Q heads (%d) must be divisible by number of K/V heads (%d)", hq, hkv);
-    FH_REQUIRE(mask_kind == FH_MASK_NONE || mask_kind == FH_MASK_CAUSAL || mask_kind == FH_MASK_ADDITIVE, "bad mask kind %d", mask_kind);
-    FH_REQUIRE(mask_kind != FH_MASK_ADDITIVE || mask_dev, "additive mask is NULL");
+    FH_REQUIRE(mask_kind >= FH_MASK_NONE && mask_kind <= FH_MASK_BATCH_KEY, "bad mask kind %d", mask_kind);
+    FH_REQUIRE((mask_kind != FH_MASK_ADDITIVE && mask_kind != FH_MASK_BATCH_KEY) || mask_dev, "additive mask is NULL");
     FH_REQUIRE(sq <= 65535 && hq <= 65535 && b <= 65535, "grid dimension too large");
     const bool qh = q_dtype == FH_F16, kh = kv_dtype == FH_F16;
     FH_REQUIRE((qh || q_dtype == FH_F32) && (kh || kv_dtype == FH_F32), "dtype must be FH_F32 or FH_F16");
     // many query rows of head_dim 64 / 128 without an additive mask: the matrix-core kernel (all-f32 inputs go
     // through its split-operand form, which keeps f32 accuracy; attn_kernel = 2 asks for plain f16 rounding)
-    if (sq >= 32 && dev->opt_attn_kernel != 1) {
+    if (sq >= 32 && dev->opt_attn_kernel != 1 && mask_kind != FH_MASK_BATCH_KEY) {
         fh_status st = fh_attention_prefill_mfma(dev, q_dtype, kv_dtype, q_dev, q_sb, q_sh, q_st, k_dev, v_dev, kv_sb, kv_sh,
                                                  kv_st, b, hq, hkv, sq, skv, d, scale, mask_kind, out_dev);
         if (st != FH_ERR_UNSUPPORTED) return st;

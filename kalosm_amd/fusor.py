@@ -26,7 +26,7 @@ class GgmlType:
 
 class MaskKind:
     """fusor-ml/fusor/src/composite/flash_attention.rs:12-24"""
-    QKMask, Causal = MASK_ADDITIVE, MASK_CAUSAL
+    QKMask, Causal, BatchKeyMask = MASK_ADDITIVE, MASK_CAUSAL, 3
 
 
 _NP = {"f32": np.float32, "f16": np.float16, "bf16": np.uint16, "u32": np.uint32, "i32": np.int32, "u8": np.uint8}
@@ -262,6 +262,9 @@ class Tensor:
                 mt, kind = mask
                 if kind == MASK_ADDITIVE:
                     assert mt.shape == (sq, skv), f"QKMask shape {mt.shape} does not match expected [{sq}, {skv}]"
+                    mptr = C.c_void_p(mt.ptr)
+                elif kind == MaskKind.BatchKeyMask:
+                    assert mt.shape == (b, skv), f"BatchKeyMask shape {mt.shape} does not match expected [{b}, {skv}]"
                     mptr = C.c_void_p(mt.ptr)
         qs = q_strides or (hq * sq * d, sq * d, d)
         qdt = F16 if self.dtype == "f16" else F32

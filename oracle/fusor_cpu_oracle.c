@@ -555,7 +555,8 @@ int fo_q8_0_matmul_q8(const float *x, int m, int k, const uint8_t *w, int n, flo
  * sum, divide, . V.  Every step in f32 with libm expf (cpu/src/elementwise.rs:157).
  * mask_kind: 0 none, 1 causal generated here as attention_mask.rs:46-66 with the
  * cache offset of mask_cache.rs:73-88 (query i sees keys j <= i + (skv - sq)),
- * 2 additive [sq, skv] mask supplied by the caller.
+ * 2 additive [sq, skv] mask supplied by the caller (MaskKind::QKMask), 3 additive [b, skv] mask
+ * broadcast over heads and queries (MaskKind::BatchKeyMask, flash_attention.rs:199-213).
  * Layout: q [b,h,sq,d], k/v [b,hkv,skv,d], out [b,h,sq,d], all contiguous.
  * One score row is materialised at a time; the arithmetic per row is that of the
  * reference. */
@@ -589,6 +590,8 @@ static void *att_worker(void *arg) {
                     if (t > i + (j->skv - j->sq)) acc = acc + ninf;
                 } else if (j->mask_kind == 2) {
                     acc = acc + j->mask[(size_t)i * j->skv + t];
+                } else if (j->mask_kind == 3) {
+                    acc = acc + j->mask[(size_t)bi * j->skv + t];
                 }
                 s[t] = acc;
                 mx = acc > mx ? acc : mx;
@@ -615,7 +618,7 @@ int fo_flash_attention(const float *q, const float *k, const float *v, int b, in
                        int sq, int skv, int d, float scale, int mask_kind, const float *mask,
                        float *out, int nthreads) {
     if (hkv <= 0 || h % hkv) return -1; /* flash_attention.rs:131-136 */
-    if (mask_kind == 2 && !mask) return -2;
+    if ((mask_kind == 2 || mask_kind == 3) && !mask) return -2;
     int total = b * h;
     if (nthreads < 1) nthreads = 1;
     if (nthreads > total) nthreads = total;

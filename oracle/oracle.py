@@ -191,7 +191,7 @@ def flash_attention(q, k, v, scale: float, mask_kind: int = MASK_NONE, mask=None
     mp = None
     if mask is not None:
         mask = _f32(mask)
-        assert mask.shape == (sq, skv)
+        assert mask.shape == ((b, skv) if mask_kind == 3 else (sq, skv))
         mp = _p(mask, C.c_float)
     rc = lib().fo_flash_attention(_p(q, C.c_float), _p(k, C.c_float), _p(v, C.c_float), b, h, hkv, sq, skv, d,
                                   scale, mask_kind, mp, _p(out, C.c_float), threads or default_threads())

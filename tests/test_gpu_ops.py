@@ -363,3 +363,27 @@ def test_top_k_pairs(dev, oracle, n):
     assert t.top_k_pairs(0) == []
     with pytest.raises(Exception):
         t.top_k_pairs(257)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_attention_batch_key_mask(dev, oracle, dtype):
+    """MaskKind::BatchKeyMask (flash_attention.rs:12-24, :199-213): an additive [batch, kv_len] mask for every head
+    and query of a batch entry (padding masks); masked keys of entry 1 must not influence its output."""
+    b, h, hkv, sq, skv, d = 3, 4, 2, 37, 50, 64
+    rng = np.random.default_rng(21)
+    npdt = np.float16 if dtype == "f16" else np.float32
+    q = rng.standard_normal((b, h, sq, d)).astype(npdt)
+    k = rng.standard_normal((b, hkv, skv, d)).astype(npdt)
+    v = rng.standard_normal((b, hkv, skv, d)).astype(npdt)
+    mask = np.zeros((b, skv), np.float32)
+    mask[1, 30:] = -np.inf
+    mask[2, ::3] = -0.75
+    got = Tensor.from_slice(dev, q, dtype).flash_attention(Tensor.from_slice(dev, k, dtype), Tensor.from_slice(dev, v, dtype),
+                                                           0.125, (Tensor.from_slice(dev, mask), MaskKind.BatchKeyMask)).as_slice()
+    want = oracle.flash_attention(q.astype(np.float32), k.astype(np.float32), v.astype(np.float32), 0.125, 3, mask)
+    tol = dict(abs_tol=2e-3, rel_tol=2e-3) if dtype == "f16" else dict(abs_tol=1e-4, rel_tol=1e-4)
+    assert_close(got.astype(np.float32), want, what="BatchKeyMask", **tol)
+    k2 = k.copy(); k2[1, :, 30:] = 9.0
+    got2 = Tensor.from_slice(dev, q, dtype).flash_attention(Tensor.from_slice(dev, k2, dtype), Tensor.from_slice(dev, v, dtype),
+                                                            0.125, (Tensor.from_slice(dev, mask), MaskKind.BatchKeyMask)).as_slice()
+    assert np.array_equal(got[1], got2[1])
