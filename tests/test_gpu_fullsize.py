@@ -110,3 +110,35 @@ def test_config4_decoder_full_width(dev, oracle):
         want.append(t)
     assert got.tolist() == want
     assert_close(m.forward([want[-1]]), ref.forward([want[-1]]), what="logits after 12 device-side steps")
+
+
+def test_decoder_from_gguf_file_full_width(dev, oracle, tmp_path):
+    """The model-file path at real tensor sizes: a 1 GB GGUF file (2 layers at Llama-3-8B widths, vocabulary 128256,
+    the per-layer type mix of a Q4_K_M file, rope_freqs.weight) written to disk, mapped and loaded by the library,
+    against the checker's decoder fed from the same bytes."""
+    from test_gguf_reader import llama_file
+    from kalosm_amd.gguf import GgufMetadata
+    cfg = {k: synth.LLAMA3_8B[k] for k in ("d_model", "n_heads", "n_kv_heads", "head_dim", "ffn", "vocab", "eps", "theta")}
+    cfg.update(n_layers=2, ctx=8192)
+    data, weights, types = llama_file(cfg, seed=6)
+    path = tmp_path / "llama_2_layers.gguf"
+    path.write_bytes(data)
+    assert len(data) > 900_000_000
+    del data
+    g = GgufMetadata.read(str(path))
+    assert g.get_value(".context_length") == 8192 and len(g.tensor_infos) == 3 + 1 + 9 * 2
+    m = Model.from_gguf(dev, g, ctx=512)
+    assert m.cfg["vocab"] == 128256 and m.cfg["ffn"] == 14336 and m.cfg["ctx"] == 512
+    ocfg = dict(m.cfg, type_attn=synth.Q4_K, type_ffn_gate_up=synth.Q4_K, type_ffn_down=synth.Q6_K,
+                type_embd=types["token_embd.weight"], type_output=types["output.weight"], tensor_types=types)
+    ref = oracle.Llama(ocfg, weights)
+    prompt = np.random.default_rng(7).integers(0, cfg["vocab"], 24)
+    lg, wl = m.forward(prompt), ref.forward(prompt)
+    assert_close(lg, wl, what="prefill logits from the model file")
+    tok = oracle.argmax(wl)
+    got, _ = m.decode_greedy(tok, 8)
+    want, t = [], tok
+    for _ in range(8):
+        t = oracle.argmax(ref.forward([t]))
+        want.append(t)
+    assert got.tolist() == want
