@@ -8,7 +8,9 @@ HBM before the timed region.  Each shape rotates over enough distinct weight buf
 256 MB last-level cache, so the bytes really come from HBM.
 
 Prints ONE JSON line: whole-path GB/s (algorithmic bytes / device time), the roofline of the dominant
-kernel and the CPU checker timed on the host cores beside it.
+kernel and the CPU checker timed on the host cores beside it.  The same line carries, under "e2e", the second
+half of the metric: tokens/s of the random-init Q4_K_M Llama-3-8B-architecture decoder (512-token prompt, 256
+greedy steps, batch 1; about 10 s including the weight upload; --no-e2e skips it).
 """
 from __future__ import annotations
 
@@ -139,7 +141,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--m", type=int, default=1, help="activation rows (decode batch)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
-    ap.add_argument("--e2e", action="store_true", help="also run the 8B-architecture decoder (tok/s) and report it")
+    ap.add_argument("--e2e", action="store_true", help="(default) also run the 8B-architecture decoder and report tok/s")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the 8B-architecture decoder leg (about 10 s)")
     ap.add_argument("--e2e-eager", action="store_true",
                     help="also run 32 decode steps of the decoder with stream launches (for a kernel tracer)")
     ap.add_argument("--prefill", action="store_true",
@@ -277,7 +280,7 @@ def main() -> int:
             worst = max(worst, float(diff.max()))
         out["parity_max_abs_err"] = worst
 
-    if args.e2e:
+    if not args.no_e2e and not args.e2e_eager:
         from kalosm_amd import e2e
         out["e2e"] = e2e.run(dev)
     if args.e2e_eager:
