@@ -30,6 +30,31 @@ __device__ __forceinline__ void ad_load8<fh_half>(const fh_half *p, float *o) {
     for (int i = 0; i < 8; i++) o[i] = (float)h[i];
 }
 
+// One lane's eight elements of a cache row as they sit in the prefetch ring: f32 rows converted (nothing to do),
+// f16 rows still packed (four registers instead of eight, so the ring can be twice as deep).
+template <typename T>
+struct AdRow;
+template <>
+struct AdRow<float> {
+    float v[8];
+    __device__ __forceinline__ void load(const float *p) { ad_load8<float>(p, v); }
+    __device__ __forceinline__ void get(float *o) const {
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[i] = v[i];
+    }
+};
+template <>
+struct AdRow<fh_half> {
+    uint4 raw;
+    __device__ __forceinline__ void load(const fh_half *p) { raw = *(const uint4 *)p; }
+    __device__ __forceinline__ void get(float *o) const {
+        fh_half h[8];
+        __builtin_memcpy(h, &raw, 16);
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[i] = (float)h[i];
+    }
+};
+
 template <int CTRL>
 __device__ __forceinline__ float ad_dpp(float v) {
     return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
@@ -68,7 +93,9 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
                                                               const int *__restrict__ len_dev, int len_host,
                                                               float scale, int chunk_max, int cap, int gtot,
                                                               float *__restrict__ part) {
-    constexpr int LP = D / 8, RPW = 64 / LP, RW = NWV * RPW, U = 4;
+    // ring depth: rows in flight per lane group (every refill costs a full memory round trip, so long parts
+    // want all their iterations in the ring; packed f16 rows make eight slots as cheap as four f32 ones)
+    constexpr int LP = D / 8, RPW = 64 / LP, RW = NWV * RPW, U = sizeof(TKV) == 2 ? 8 : 4;
     static_assert(NWV >= G, "one wavefront per query head for the softmax statistics");
     extern __shared__ float sm[];
     float *s_sc = sm;                  // [G][chunk_max]
@@ -85,16 +112,16 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
     // the first U0 rows of every lane group are requested blind (U0 * RW = 128 local rows = 1024 keys with 8 splits); the
     // other prefetched rows wait for the length, so that a short context does not pay for requests it drops
     constexpr int U0 = 32 / NWV < U ? 32 / NWV : U;
-    float kpre[U][8], vpre[U][8];
+    AdRow<TKV> kpre[U], vpre[U];
 #pragma unroll
     for (int u = 0; u < U0; u++) {
         const int t = cache_row(u * RW + trow);
-        ad_load8<TKV>(kb + (int64_t)(t < cap ? t : 0) * kv_st, kpre[u]);
+        kpre[u].load(kb + (int64_t)(t < cap ? t : 0) * kv_st);
     }
 #pragma unroll
     for (int u = 0; u < U0; u++) {
         const int t = cache_row(u * RW + trow);
-        ad_load8<TKV>(vb + (int64_t)(t < cap ? t : 0) * kv_st, vpre[u]);
+        vpre[u].load(vb + (int64_t)(t < cap ? t : 0) * kv_st);
     }
     __builtin_amdgcn_sched_barrier(0); // the requests above do not wait for the length
     // the step's own key is already appended at index len; a caller that knows the length passes it by value
@@ -108,8 +135,8 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
     for (int u = U0; u < U; u++) {
         const int lr = u * RW + trow;
         if (u * RW < nk) {
-            ad_load8<TKV>(kb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st, kpre[u]);
-            ad_load8<TKV>(vb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st, vpre[u]);
+            kpre[u].load(kb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st);
+            vpre[u].load(vb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st);
         }
     }
     // (rows past nk hold whatever the cache allocation held: every use below is guarded by the row index)
@@ -123,7 +150,9 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
         qr[h][4] = b.x; qr[h][5] = b.y; qr[h][6] = b.z; qr[h][7] = b.w;
     }
     // ---- scores
-    auto score = [&](const float *kv8, int t) {
+    auto score = [&](const AdRow<TKV> &row, int t) {
+        float kv8[8];
+        row.get(kv8);
 #pragma unroll
         for (int h = 0; h < G; h++) {
             float a = 0.f;
@@ -142,7 +171,7 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
                 score(kpre[u], it * RW + trow);
                 if ((it + U) * RW < nk) {
                     const int lr = (it + U) * RW + trow;
-                    ad_load8<TKV>(kb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st, kpre[u]);
+                    kpre[u].load(kb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st);
                 }
             }
         }
@@ -175,8 +204,10 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
     for (int h = 0; h < G; h++)
 #pragma unroll
         for (int i = 0; i < 8; i++) o[h][i] = 0.f;
-    auto accum = [&](const float *v8, int t) {
+    auto accum = [&](const AdRow<TKV> &row, int t) {
         if (t < nk) {
+            float v8[8];
+            row.get(v8);
 #pragma unroll
             for (int h = 0; h < G; h++) {
                 const float p = s_sc[h * chunk_max + t];
@@ -193,7 +224,7 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
                 accum(vpre[u], it * RW + trow);
                 if ((it + U) * RW < nk) {
                     const int lr = (it + U) * RW + trow;
-                    ad_load8<TKV>(vb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st, vpre[u]);
+                    vpre[u].load(vb + (int64_t)cache_row(lr < nk ? lr : 0) * kv_st);
                 }
             }
         }
