@@ -283,6 +283,154 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_dl(const float *__rest
     }
 }
 
+// max over the four rows of 16 lanes of a wavefront (lane i of every row gets it)
+__device__ __forceinline__ float ad_rows_max(float a) {
+    const uint32_t u = __float_as_uint(a);
+    auto s16 = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    a = fmaxf(__uint_as_float(s16[0]), __uint_as_float(s16[1]));
+    const uint32_t w = __float_as_uint(a);
+    auto s32 = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    return fmaxf(__uint_as_float(s32[0]), __uint_as_float(s32[1]));
+}
+
+// ------------------------------------------------------------------------------ one pass over long caches
+// The same part of the same grid as k_attn_decode_dl, for parts of many keys: a lane group (16 lanes, 8 dims each)
+// takes C rows at a time, K and V row of a key together, and keeps a running maximum, denominator and weighted V sum
+// per query head (online softmax); nothing is staged in LDS and no barrier separates scores from P.V, so the
+// arithmetic of one wavefront runs under the transfers of the others.  Lane groups and wavefronts are merged at
+// the end.  Partials as k_attn_decode_dl writes them: [head][part][D weighted sums | max | denominator | 2 unused].
+template <typename TKV, int G, int NWV>
+__global__ __launch_bounds__(64 * NWV) void k_attn_decode_1p(const float *__restrict__ q, const TKV *__restrict__ k,
+                                                              const TKV *__restrict__ v, int64_t kv_sh, int64_t kv_st,
+                                                              const int *__restrict__ len_dev, int len_host, float scale,
+                                                              int cap, int gtot, float *__restrict__ part) {
+    constexpr int D = 128, LP = D / 8, RPW = 64 / LP, RW = NWV * RPW;
+    constexpr int C = sizeof(TKV) == 2 ? 4 : 2; // rows of a chunk per lane group: 2 KB of K and V per lane group
+    __shared__ float s_red[NWV * G * D];
+    __shared__ float s_st[NWV * G * 2];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, grp = lane / LP, c = lane % LP;
+    const int split = blockIdx.x, S = gridDim.x, kh = blockIdx.y, h0 = kh * gtot + (int)blockIdx.z * G;
+    const TKV *kb = k + kh * kv_sh + 8 * c, *vb = v + kh * kv_sh + 8 * c;
+    const int trow = wave * RPW + grp;
+    const int skv = (len_dev ? *len_dev : len_host) + 1;
+    const int gfull = skv >> 4;
+    int nk = gfull > split ? ((gfull - split + S - 1) / S) * 16 : 0;
+    if (gfull % S == split) nk += skv & 15;
+    const int niter = (nk + RW - 1) / RW;
+    float qr[G][8];
+#pragma unroll
+    for (int h = 0; h < G; h++) {
+        const float4 a = *(const float4 *)(q + (int64_t)(h0 + h) * D + 8 * c);
+        const float4 b = *(const float4 *)(q + (int64_t)(h0 + h) * D + 8 * c + 4);
+        qr[h][0] = a.x * scale; qr[h][1] = a.y * scale; qr[h][2] = a.z * scale; qr[h][3] = a.w * scale;
+        qr[h][4] = b.x * scale; qr[h][5] = b.y * scale; qr[h][6] = b.z * scale; qr[h][7] = b.w * scale;
+    }
+    float m[G], l[G], o[G][8];
+#pragma unroll
+    for (int h = 0; h < G; h++) {
+        m[h] = -INFINITY;
+        l[h] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[h][i] = 0.f;
+    }
+    for (int it0 = 0; it0 < niter; it0 += C) {
+        AdRow<TKV> kr[C], vr[C];
+        bool ok[C];
+#pragma unroll
+        for (int j = 0; j < C; j++) {
+            const int lr = (it0 + j) * RW + trow; // local row -> granule (lr / 16) * S + split of the head's rows
+            ok[j] = lr < nk;
+            int row = (((ok[j] ? lr : 0) >> 4) * S + split) * 16 + ((ok[j] ? lr : 0) & 15);
+            row = row < cap ? row : 0; // rows past the live ones are read from a valid address and never used
+            kr[j].load(kb + (int64_t)row * kv_st);
+            vr[j].load(vb + (int64_t)row * kv_st);
+        }
+        float sc[C][G];
+#pragma unroll
+        for (int j = 0; j < C; j++) {
+            float k8[8];
+            kr[j].get(k8);
+#pragma unroll
+            for (int h = 0; h < G; h++) {
+                float a = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) a = fmaf(qr[h][i], k8[i], a);
+                a = ad_row16_sum(a);
+                sc[j][h] = ok[j] ? a : -INFINITY;
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < G; h++) {
+            float cm = sc[0][h];
+#pragma unroll
+            for (int j = 1; j < C; j++) cm = fmaxf(cm, sc[j][h]);
+            const float mn = fmaxf(m[h], cm);
+            const float ref = mn == -INFINITY ? 0.f : mn; // nothing live yet: every weight below becomes exp(-inf) = 0
+            const float alpha = __expf(m[h] - ref);
+            l[h] *= alpha;
+#pragma unroll
+            for (int i = 0; i < 8; i++) o[h][i] *= alpha;
+#pragma unroll
+            for (int j = 0; j < C; j++) {
+                const float p = __expf(sc[j][h] - ref);
+                sc[j][h] = p;
+                l[h] += p;
+            }
+            m[h] = mn;
+        }
+#pragma unroll
+        for (int j = 0; j < C; j++) {
+            float v8[8];
+            vr[j].get(v8);
+#pragma unroll
+            for (int h = 0; h < G; h++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) o[h][i] = fmaf(sc[j][h], v8[i], o[h][i]);
+        }
+    }
+    // ---- the four lane groups of the wavefront, then the wavefronts
+#pragma unroll
+    for (int h = 0; h < G; h++) {
+        const float ma = ad_rows_max(m[h]);
+        const float ref = ma == -INFINITY ? 0.f : ma;
+        const float f = __expf(m[h] - ref);
+        const float la = ad_rows_sum(l[h] * f);
+        float oa[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) oa[i] = ad_rows_sum(o[h][i] * f);
+        if (grp == 0) {
+            float *dst = s_red + (wave * G + h) * D + 8 * c;
+            *(float4 *)dst = make_float4(oa[0], oa[1], oa[2], oa[3]);
+            *(float4 *)(dst + 4) = make_float4(oa[4], oa[5], oa[6], oa[7]);
+            if (c == 0) {
+                s_st[(wave * G + h) * 2] = ma;
+                s_st[(wave * G + h) * 2 + 1] = la;
+            }
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < G * D; idx += 64 * NWV) {
+        const int h = idx / D, dd = idx % D;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < NWV; w++) mx = fmaxf(mx, s_st[(w * G + h) * 2]);
+        const float ref = mx == -INFINITY ? 0.f : mx;
+        float a = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < NWV; w++) {
+            const float f = __expf(s_st[(w * G + h) * 2] - ref);
+            a = fmaf(s_red[(w * G + h) * D + dd], f, a);
+            den = fmaf(s_st[(w * G + h) * 2 + 1], f, den);
+        }
+        float *pp = part + ((int64_t)(h0 + h) * S + split) * (D + 4);
+        pp[dd] = a;
+        if (dd == 0) {
+            pp[D] = mx;
+            pp[D + 1] = den;
+        }
+    }
+}
+
 // Merge of the parts of one head: thread t fetches the statistics of part t (all parts at once instead of one
 // dependent load per loop trip), the weights go through LDS, and the weighted rows are summed eight loads at a time.
 template <int D, typename TO = float>
@@ -327,7 +475,7 @@ __global__ __launch_bounds__(D) void k_attn_combine_dl(const float *__restrict__
 template <typename TKV, int G, int NWV>
 static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const void *v, int64_t kv_sh, int64_t kv_st,
                            int hq, int hkv, float scale, const int *len_dev, int max_len, float *out, int *splits_out,
-                           int gtot, int len_host = 0, int splits_req = 0, bool out_f16 = false) {
+                           int gtot, int len_host = 0, int splits_req = 0, bool out_f16 = false, bool one_pass = false) {
     constexpr int D = 128;
     // splits: 8 measured best from a few hundred to a few thousand keys (MI355X); it is also the most the output
     // projection merges while staging its input.  The option allows 4 .. 16; a caller with a long cache and its
@@ -335,6 +483,21 @@ static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const 
     int S = dev->opt_attn_splits > 0 ? (int)dev->opt_attn_splits : 8;
     S = S < 4 ? 4 : (S > 16 ? 16 : S);
     if (splits_req > 0) S = splits_req;
+    if (one_pass && G <= 4) {
+        FH_TRY(fh_dev_scratch(dev, (void **)&dev->part_buf, &dev->part_cap, (size_t)hq * S * (D + 4) * 4));
+        k_attn_decode_1p<TKV, (G <= 4 ? G : 4), NWV><<<dim3((unsigned)S, (unsigned)hkv, (unsigned)(gtot / G)), dim3(64 * NWV), 0,
+                                                       dev->stream>>>(q, (const TKV *)k, (const TKV *)v, kv_sh, kv_st, len_dev,
+                                                                      len_host, scale, max_len, gtot, dev->part_buf);
+        FH_HIP(hipGetLastError());
+        if (splits_out) *splits_out = S;
+        if (out) {
+            if (out_f16)
+                k_attn_combine_dl<D, fh_half><<<dim3((unsigned)hq), dim3(D), 0, dev->stream>>>(dev->part_buf, S, (fh_half *)out);
+            else k_attn_combine_dl<D><<<dim3((unsigned)hq), dim3(D), 0, dev->stream>>>(dev->part_buf, S, out);
+            FH_HIP(hipGetLastError());
+        }
+        return FH_OK;
+    }
     const int chunk_max = (((max_len + 15) / 16 + S - 1) / S) * 16; // most local rows of a split
     const size_t lds = ((size_t)G * chunk_max + (size_t)NWV * G * D) * 4;
     FH_REQUIRE(lds <= 150 * 1024, "KV capacity %d too large for the decode attention kernel", max_len);
@@ -382,11 +545,11 @@ fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *
 fh_status fh_attention_decode_hostlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
                                       int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale, int skv,
                                       void *out, bool out_f16) {
-    int splits = skv <= 2048 ? 8 : (skv <= 8192 ? 16 : 32);
+    int splits = skv <= 4096 ? 8 : (skv <= 8192 ? 16 : 32);
     if (dev->opt_attn_splits > 0) splits = dev->opt_attn_splits > 128 ? 128 : (int)dev->opt_attn_splits;
     // long caches are bandwidth bound: all query heads of a KV head in one workgroup, so K and V are read once
-    // (measured on MI355X, 32 / 8 heads, f16 cache: 1 head x 8 parts at 1024 keys, 2 x 16 at 4096, 4 x 32 at 16384)
-    const int heads = dev->opt_attn_heads > 0 ? (int)dev->opt_attn_heads : (skv <= 2048 ? 1 : (skv <= 8192 ? 2 : 4));
+    // (measured on MI355X, 32 / 8 heads, f16 cache: 1 head x 8 parts at 1024 and 4096 keys, 4 x 32 at 16384)
+    const int heads = dev->opt_attn_heads > 0 ? (int)dev->opt_attn_heads : (skv <= 8192 ? 1 : 4);
     return ad_any(dev, kv_dtype, q, k, v, kv_sh, kv_st, hq, hkv, d, scale, nullptr, skv, (float *)out, nullptr, skv - 1,
                   splits, out_f16, heads);
 }
@@ -403,7 +566,9 @@ static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void
     if (heads_req > 0) G = heads_req > gtot ? gtot : heads_req;
     while (G > 1 && (gtot % G || (G != 2 && G != 4 && G != 8))) G /= 2;
     const bool w8 = dev->opt_attn_waves == 8 && G <= 8; // 8 wavefronts per workgroup instead of 16
-#define AD_ARGS dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out, gtot, len_host, splits_req, out_f16
+    // the one-pass kernel unless attn_kernel = 4 asks for the two-pass one (or 8 heads per workgroup are wanted)
+    const bool one_pass = dev->opt_attn_kernel != 4;
+#define AD_ARGS dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out, gtot, len_host, splits_req, out_f16, one_pass
 #define AD_GO(TKV_)                                                                       \
     switch (G) {                                                                          \
     case 1: return w8 ? ad_launch<TKV_, 1, 8>(AD_ARGS) : ad_launch<TKV_, 1, 16>(AD_ARGS); \

@@ -80,8 +80,10 @@ def test_decoder_matches_checker(dev, oracle, variant, cfg):
 
 @pytest.mark.parametrize("heads,kv_heads", [(4, 1), (4, 2), (8, 1), (2, 2)], ids=["g4", "g2", "g8", "g1"])
 @pytest.mark.parametrize("opts", [{}, dict(attn_heads=2), dict(attn_heads=4, attn_waves=8), dict(attn_splits=4, wo_tiles=1),
-                                  dict(wo_tiles=2, down_tiles=2, matvec_tiles=2), dict(matvec_per=2, down_tiles=4)],
-                         ids=["default", "heads2", "heads4-waves8", "splits4-wo1", "tiles2", "per2-down4"])
+                                  dict(wo_tiles=2, down_tiles=2, matvec_tiles=2), dict(matvec_per=2, down_tiles=4),
+                                  dict(attn_kernel=4), dict(attn_kernel=4, attn_heads=4, attn_waves=8)],
+                         ids=["default", "heads2", "heads4-waves8", "splits4-wo1", "tiles2", "per2-down4", "twopass",
+                              "twopass-heads4"])
 def test_decode_step_kernel_variants(dev, oracle, heads, kv_heads, opts):
     """The fused decode step (head_dim 128) with other groupings of query heads per KV head and with the kernel
     shapes the options select: 70 greedy steps on the device (five granules of 16 keys, so every attention split
