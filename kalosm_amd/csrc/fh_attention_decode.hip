@@ -333,30 +333,36 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_1p(const float *__rest
 #pragma unroll
         for (int i = 0; i < 8; i++) o[h][i] = 0.f;
     }
-    for (int it0 = 0; it0 < niter; it0 += C) {
-        AdRow<TKV> kr[C], vr[C];
-        bool ok[C];
+    // a chunk: C rows per lane group.  With few query heads per workgroup there are registers for two chunks: the
+    // next one is requested before the current one is multiplied (requests past the end re-read a live row and
+    // are ignored).
+    constexpr bool DB = G <= 2;
+    AdRow<TKV> kr[DB ? 2 : 1][C], vr[DB ? 2 : 1][C];
+    auto issue = [&](int b, int it0) {
 #pragma unroll
         for (int j = 0; j < C; j++) {
             const int lr = (it0 + j) * RW + trow; // local row -> granule (lr / 16) * S + split of the head's rows
-            ok[j] = lr < nk;
-            int row = (((ok[j] ? lr : 0) >> 4) * S + split) * 16 + ((ok[j] ? lr : 0) & 15);
+            const int lv = lr < nk ? lr : 0;
+            int row = ((lv >> 4) * S + split) * 16 + (lv & 15);
             row = row < cap ? row : 0; // rows past the live ones are read from a valid address and never used
-            kr[j].load(kb + (int64_t)row * kv_st);
-            vr[j].load(vb + (int64_t)row * kv_st);
+            kr[b][j].load(kb + (int64_t)row * kv_st);
+            vr[b][j].load(vb + (int64_t)row * kv_st);
         }
+    };
+    auto process = [&](int b, int it0) {
         float sc[C][G];
 #pragma unroll
         for (int j = 0; j < C; j++) {
+            const bool ok = (it0 + j) * RW + trow < nk;
             float k8[8];
-            kr[j].get(k8);
+            kr[b][j].get(k8);
 #pragma unroll
             for (int h = 0; h < G; h++) {
                 float a = 0.f;
 #pragma unroll
                 for (int i = 0; i < 8; i++) a = fmaf(qr[h][i], k8[i], a);
                 a = ad_row16_sum(a);
-                sc[j][h] = ok[j] ? a : -INFINITY;
+                sc[j][h] = ok ? a : -INFINITY;
             }
         }
 #pragma unroll
@@ -381,11 +387,37 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_1p(const float *__rest
 #pragma unroll
         for (int j = 0; j < C; j++) {
             float v8[8];
-            vr[j].get(v8);
+            vr[b][j].get(v8);
 #pragma unroll
             for (int h = 0; h < G; h++)
 #pragma unroll
                 for (int i = 0; i < 8; i++) o[h][i] = fmaf(sc[j][h], v8[i], o[h][i]);
+        }
+    };
+    if constexpr (DB) {
+        issue(0, 0);
+        if (niter <= C) { // a short part (the usual decode step): one chunk, nothing to overlap
+            // (a part without keys multiplies nothing: its clamped rows lie past the live ones and may hold anything,
+            // and a weight of zero does not silence a NaN)
+            if (niter > 0) process(0, 0);
+        } else {
+            // no branches around the requests (a wait after a branch waits for everything in flight): the last trips
+            // re-read a live row and ignore it
+            for (int it0 = 0; it0 < niter; it0 += 2 * C) {
+                issue(1, it0 + C);
+                __builtin_amdgcn_sched_barrier(0); // the requests stay ahead of the arithmetic on the other chunk
+                process(0, it0);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(0, it0 + 2 * C);
+                __builtin_amdgcn_sched_barrier(0);
+                process(1, it0 + C);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    } else {
+        for (int it0 = 0; it0 < niter; it0 += C) {
+            issue(0, it0);
+            process(0, it0);
         }
     }
     // ---- the four lane groups of the wavefront, then the wavefronts
@@ -532,7 +564,7 @@ fh_status fh_attention_combine_dl(fh_device *dev, int hq, int splits, float *out
 // ([hq][*splits_out][d + 4]) for a consumer that merges them itself.
 static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v, int64_t kv_sh,
                         int64_t kv_st, int hq, int hkv, int d, float scale, const int *len_dev, int max_len, float *out,
-                        int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req = 0);
+                        int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req = 0, int waves_req = 0);
 
 fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
                                      int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale,
@@ -545,18 +577,19 @@ fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *
 fh_status fh_attention_decode_hostlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
                                       int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale, int skv,
                                       void *out, bool out_f16) {
-    int splits = skv <= 4096 ? 8 : (skv <= 8192 ? 16 : 32);
+    int splits = skv <= 2048 ? 8 : 16;
     if (dev->opt_attn_splits > 0) splits = dev->opt_attn_splits > 128 ? 128 : (int)dev->opt_attn_splits;
     // long caches are bandwidth bound: all query heads of a KV head in one workgroup, so K and V are read once
-    // (measured on MI355X, 32 / 8 heads, f16 cache: 1 head x 8 parts at 1024 and 4096 keys, 4 x 32 at 16384)
-    const int heads = dev->opt_attn_heads > 0 ? (int)dev->opt_attn_heads : (skv <= 8192 ? 1 : 4);
+    // (measured on MI355X, 32 / 8 heads, f16 cache: 1 head x 8 parts x 16 wavefronts at 1024 keys, 2 x 16 x 8 at
+    // 4096 and 16384)
+    const int heads = dev->opt_attn_heads > 0 ? (int)dev->opt_attn_heads : (skv <= 2048 ? 1 : 2);
     return ad_any(dev, kv_dtype, q, k, v, kv_sh, kv_st, hq, hkv, d, scale, nullptr, skv, (float *)out, nullptr, skv - 1,
-                  splits, out_f16, heads);
+                  splits, out_f16, heads, skv > 2048 ? 8 : 0);
 }
 
 static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v, int64_t kv_sh,
                         int64_t kv_st, int hq, int hkv, int d, float scale, const int *len_dev, int max_len, float *out,
-                        int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req) {
+                        int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req, int waves_req) {
     const int gtot = hq / hkv;
     if (d != 128 || (gtot != 1 && gtot != 2 && gtot != 4 && gtot != 8) || kv_st % 8 || kv_sh % 8) return FH_ERR_UNSUPPORTED;
     // query heads per workgroup: the arithmetic of a workgroup grows with them, the K and V reads do not; one
@@ -565,7 +598,8 @@ static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void
     int G = dev->opt_attn_heads > 0 ? (int)dev->opt_attn_heads : 1;
     if (heads_req > 0) G = heads_req > gtot ? gtot : heads_req;
     while (G > 1 && (gtot % G || (G != 2 && G != 4 && G != 8))) G /= 2;
-    const bool w8 = dev->opt_attn_waves == 8 && G <= 8; // 8 wavefronts per workgroup instead of 16
+    // 8 wavefronts per workgroup instead of 16
+    const bool w8 = (dev->opt_attn_waves == 8 || (dev->opt_attn_waves == 0 && waves_req == 8)) && G <= 8;
     // the one-pass kernel unless attn_kernel = 4 asks for the two-pass one (or 8 heads per workgroup are wanted)
     const bool one_pass = dev->opt_attn_kernel != 4;
 #define AD_ARGS dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out, gtot, len_host, splits_req, out_f16, one_pass

@@ -561,6 +561,10 @@ fh_status fh_kvcache_reserve(fh_kvcache *c, int required) {
         FH_FAIL(FH_ERR_OOM, "hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
     }
     hipStream_t s = c->dev->stream;
+    // New cache memory starts as NaN bit patterns (f32 and f16 alike): a kernel that lets a row past the live length
+    // reach its result then fails in every run, not only when the allocation happens to hold such bytes.
+    FH_HIP(hipMemsetAsync(nk, 0xFF, bytes, s));
+    FH_HIP(hipMemsetAsync(nv, 0xFF, bytes, s));
     if (c->len > 0 && c->k) {
         int wpp = (int)(c->head_dim * es / 4);
         int64_t rows = (int64_t)c->layers * c->kv_heads, total = rows * c->len * wpp;
