@@ -310,13 +310,14 @@ static fh_status attn_typed(fh_device *dev, const void *q, int64_t q_sb, int64_t
     const bool masked = mask_kind == FH_MASK_ADDITIVE || mask_kind == FH_MASK_BATCH_KEY;
     if (sq == 1 && b == 1 && d == 128 && aligned && q_sh == d && !masked && hq <= 64 &&
         dev->opt_attn_kernel != 1) {
-        const float *q32 = (const float *)q;
-        if constexpr (!std::is_same<TQ, float>::value) {
+        constexpr bool QH = !std::is_same<TQ, float>::value;
+        const int kvt = std::is_same<TKV, float>::value ? FH_F32 : FH_F16;
+        fh_status st = fh_attention_decode_hostlen(dev, kvt, q, QH, k, v, kv_sh, kv_st, hq, hkv, d, scale, skv, out, QH);
+        if (st == FH_ERR_UNSUPPORTED && QH) { // the two-pass kernel reads an f32 query: widen it first
             FH_TRY(fh_cast_f16_f32(dev, q, (float *)dev->small_buf, (int64_t)hq * d));
-            q32 = (const float *)dev->small_buf;
+            st = fh_attention_decode_hostlen(dev, kvt, dev->small_buf, false, k, v, kv_sh, kv_st, hq, hkv, d, scale, skv, out,
+                                             QH);
         }
-        fh_status st = fh_attention_decode_hostlen(dev, std::is_same<TKV, float>::value ? FH_F32 : FH_F16, q32, k, v, kv_sh,
-                                                   kv_st, hq, hkv, d, scale, skv, out, !std::is_same<TQ, float>::value);
         if (st != FH_ERR_UNSUPPORTED) return st;
     }
     if (sq == 1 && aligned && (d == 128 || d == 64) && (G == 1 || G == 2 || G == 4 || G == 8) &&

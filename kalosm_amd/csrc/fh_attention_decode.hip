@@ -38,6 +38,7 @@ template <>
 struct AdRow<float> {
     float v[8];
     __device__ __forceinline__ void load(const float *p) { ad_load8<float>(p, v); }
+    __device__ __forceinline__ void load_get(const float *p, float *o) const { ad_load8<float>(p, o); }
     __device__ __forceinline__ void get(float *o) const {
 #pragma unroll
         for (int i = 0; i < 8; i++) o[i] = v[i];
@@ -300,7 +301,7 @@ __device__ __forceinline__ float ad_rows_max(float a) {
 // arithmetic of one wavefront runs under the transfers of the others.  Lane groups and wavefronts are merged at
 // the end.  Partials as k_attn_decode_dl writes them: [head][part][D weighted sums | max | denominator | 2 unused].
 template <typename TKV, int G, int NWV>
-__global__ __launch_bounds__(64 * NWV) void k_attn_decode_1p(const float *__restrict__ q, const TKV *__restrict__ k,
+__global__ __launch_bounds__(64 * NWV) void k_attn_decode_1p(const void *__restrict__ qv, int q_f16, const TKV *__restrict__ k,
                                                               const TKV *__restrict__ v, int64_t kv_sh, int64_t kv_st,
                                                               const int *__restrict__ len_dev, int len_host, float scale,
                                                               int cap, int gtot, float *__restrict__ part) {
@@ -317,13 +318,13 @@ __global__ __launch_bounds__(64 * NWV) void k_attn_decode_1p(const float *__rest
     int nk = gfull > split ? ((gfull - split + S - 1) / S) * 16 : 0;
     if (gfull % S == split) nk += skv & 15;
     const int niter = (nk + RW - 1) / RW;
-    float qr[G][8];
+    float qr[G][8]; // the query may arrive as f16 (a caller's tensor) or f32 (the decoder's own)
 #pragma unroll
     for (int h = 0; h < G; h++) {
-        const float4 a = *(const float4 *)(q + (int64_t)(h0 + h) * D + 8 * c);
-        const float4 b = *(const float4 *)(q + (int64_t)(h0 + h) * D + 8 * c + 4);
-        qr[h][0] = a.x * scale; qr[h][1] = a.y * scale; qr[h][2] = a.z * scale; qr[h][3] = a.w * scale;
-        qr[h][4] = b.x * scale; qr[h][5] = b.y * scale; qr[h][6] = b.z * scale; qr[h][7] = b.w * scale;
+        if (q_f16) AdRow<fh_half>{*(const uint4 *)((const fh_half *)qv + (int64_t)(h0 + h) * D + 8 * c)}.get(qr[h]);
+        else AdRow<float>().load_get((const float *)qv + (int64_t)(h0 + h) * D + 8 * c, qr[h]);
+#pragma unroll
+        for (int i = 0; i < 8; i++) qr[h][i] *= scale;
     }
     float m[G], l[G], o[G][8];
 #pragma unroll
@@ -507,7 +508,8 @@ __global__ __launch_bounds__(D) void k_attn_combine_dl(const float *__restrict__
 template <typename TKV, int G, int NWV>
 static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const void *v, int64_t kv_sh, int64_t kv_st,
                            int hq, int hkv, float scale, const int *len_dev, int max_len, float *out, int *splits_out,
-                           int gtot, int len_host = 0, int splits_req = 0, bool out_f16 = false, bool one_pass = false) {
+                           int gtot, int len_host = 0, int splits_req = 0, bool out_f16 = false, bool one_pass = false,
+                           bool q_f16 = false) {
     constexpr int D = 128;
     // splits: 8 measured best from a few hundred to a few thousand keys (MI355X); it is also the most the output
     // projection merges while staging its input.  The option allows 4 .. 16; a caller with a long cache and its
@@ -515,11 +517,13 @@ static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const 
     int S = dev->opt_attn_splits > 0 ? (int)dev->opt_attn_splits : 8;
     S = S < 4 ? 4 : (S > 16 ? 16 : S);
     if (splits_req > 0) S = splits_req;
+    FH_REQUIRE(!q_f16 || (one_pass && G <= 4), "an f16 query needs the one-pass kernel");
     if (one_pass && G <= 4) {
         FH_TRY(fh_dev_scratch(dev, (void **)&dev->part_buf, &dev->part_cap, (size_t)hq * S * (D + 4) * 4));
         k_attn_decode_1p<TKV, (G <= 4 ? G : 4), NWV><<<dim3((unsigned)S, (unsigned)hkv, (unsigned)(gtot / G)), dim3(64 * NWV), 0,
-                                                       dev->stream>>>(q, (const TKV *)k, (const TKV *)v, kv_sh, kv_st, len_dev,
-                                                                      len_host, scale, max_len, gtot, dev->part_buf);
+                                                       dev->stream>>>(q, q_f16 ? 1 : 0, (const TKV *)k, (const TKV *)v, kv_sh,
+                                                                      kv_st, len_dev, len_host, scale, max_len, gtot,
+                                                                      dev->part_buf);
         FH_HIP(hipGetLastError());
         if (splits_out) *splits_out = S;
         if (out) {
@@ -564,7 +568,8 @@ fh_status fh_attention_combine_dl(fh_device *dev, int hq, int splits, float *out
 // ([hq][*splits_out][d + 4]) for a consumer that merges them itself.
 static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v, int64_t kv_sh,
                         int64_t kv_st, int hq, int hkv, int d, float scale, const int *len_dev, int max_len, float *out,
-                        int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req = 0, int waves_req = 0);
+                        int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req = 0, int waves_req = 0,
+                        bool q_f16 = false);
 
 fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
                                      int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale,
@@ -574,22 +579,24 @@ fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *
 
 // One f32 query per head against `skv` cached keys known on the host; `out` is f32 or f16 [hq, d].  The key
 // range is cut into more parts the longer it is (every part is a workgroup per KV head and query-head group).
-fh_status fh_attention_decode_hostlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
-                                      int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale, int skv,
-                                      void *out, bool out_f16) {
+fh_status fh_attention_decode_hostlen(fh_device *dev, int kv_dtype, const void *q, bool q_f16, const void *k,
+                                      const void *v, int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale,
+                                      int skv, void *out, bool out_f16) {
+    if (q_f16 && (dev->opt_attn_kernel == 4 || (dev->opt_attn_heads > 4))) return FH_ERR_UNSUPPORTED; // caller widens q
     int splits = skv <= 2048 ? 8 : 16;
     if (dev->opt_attn_splits > 0) splits = dev->opt_attn_splits > 128 ? 128 : (int)dev->opt_attn_splits;
     // long caches are bandwidth bound: all query heads of a KV head in one workgroup, so K and V are read once
     // (measured on MI355X, 32 / 8 heads, f16 cache: 1 head x 8 parts x 16 wavefronts at 1024 keys, 2 x 16 x 8 at
     // 4096 and 16384)
     const int heads = dev->opt_attn_heads > 0 ? (int)dev->opt_attn_heads : (skv <= 2048 ? 1 : 2);
-    return ad_any(dev, kv_dtype, q, k, v, kv_sh, kv_st, hq, hkv, d, scale, nullptr, skv, (float *)out, nullptr, skv - 1,
-                  splits, out_f16, heads, skv > 2048 ? 8 : 0);
+    return ad_any(dev, kv_dtype, (const float *)q, k, v, kv_sh, kv_st, hq, hkv, d, scale, nullptr, skv, (float *)out, nullptr,
+                  skv - 1, splits, out_f16, heads, skv > 2048 ? 8 : 0, q_f16);
 }
 
 static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v, int64_t kv_sh,
                         int64_t kv_st, int hq, int hkv, int d, float scale, const int *len_dev, int max_len, float *out,
-                        int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req, int waves_req) {
+                        int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req, int waves_req,
+                        bool q_f16) {
     const int gtot = hq / hkv;
     if (d != 128 || (gtot != 1 && gtot != 2 && gtot != 4 && gtot != 8) || kv_st % 8 || kv_sh % 8) return FH_ERR_UNSUPPORTED;
     // query heads per workgroup: the arithmetic of a workgroup grows with them, the K and V reads do not; one
@@ -602,7 +609,7 @@ static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void
     const bool w8 = (dev->opt_attn_waves == 8 || (dev->opt_attn_waves == 0 && waves_req == 8)) && G <= 8;
     // the one-pass kernel unless attn_kernel = 4 asks for the two-pass one (or 8 heads per workgroup are wanted)
     const bool one_pass = dev->opt_attn_kernel != 4;
-#define AD_ARGS dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out, gtot, len_host, splits_req, out_f16, one_pass
+#define AD_ARGS dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out, gtot, len_host, splits_req, out_f16, one_pass, q_f16
 #define AD_GO(TKV_)                                                                       \
     switch (G) {                                                                          \
     case 1: return w8 ? ad_launch<TKV_, 1, 8>(AD_ARGS) : ad_launch<TKV_, 1, 16>(AD_ARGS); \

@@ -172,9 +172,9 @@ fh_status fh_launch_q4k_m1_norm(const fh_qmatrix *q, const float *x, const float
 fh_status fh_launch_q4k_m1_attn(const fh_qmatrix *q, const float *part, int nsplit, float *y);
 fh_status fh_launch_q4k_m1_attn_acc(const fh_qmatrix *q, const float *part, int nsplit, float *y_inout);
 fh_status fh_attention_combine_dl(fh_device *dev, int hq, int splits, float *out);
-fh_status fh_attention_decode_hostlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
-                                      int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale, int skv,
-                                      void *out, bool out_f16);
+fh_status fh_attention_decode_hostlen(fh_device *dev, int kv_dtype, const void *q, bool q_f16, const void *k,
+                                      const void *v, int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale,
+                                      int skv, void *out, bool out_f16);
 fh_status fh_attention_prefill_mfma(fh_device *dev, int q_dtype, int kv_dtype, const void *q, int64_t q_sb,
                                     int64_t q_sh, int64_t q_st, const void *k, const void *v, int64_t kv_sb,
                                     int64_t kv_sh, int64_t kv_st, int b, int hq, int hkv, int sq, int skv, int d,
