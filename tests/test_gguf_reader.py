@@ -324,3 +324,46 @@ def test_decoder_config_from_metadata():
     g = GgufMetadata.read_bytes(R.write_gguf({"general.architecture": "llama"}, []))
     assert L.fh_llama_config_from_gguf(g._h, C.byref(c)) == _lib.FH_ERR_NOT_FOUND
     assert b".attention.head_count" in L.fh_last_error()
+
+
+def test_corrupted_files_are_rejected_like_the_checker_does():
+    """Random byte damage and truncation of a valid file: the library must answer with a status (never crash), and
+    accept or reject exactly the inputs the plain-Python reader accepts or rejects."""
+    rng = np.random.default_rng(0)
+    _, _, good = random_file(3, 3, None)
+    accepted = 0
+    for it in range(600):
+        data = bytearray(good)
+        mode = it % 3
+        if mode == 0:
+            for _ in range(int(rng.integers(1, 4))):
+                data[int(rng.integers(0, 1400))] = int(rng.integers(0, 256))
+        elif mode == 1:
+            data = data[:int(rng.integers(0, len(data)))]
+        else:
+            p = int(rng.integers(0, 1400))
+            data[p:p + 8] = rng.integers(0, 256, 8, dtype=np.uint8).tobytes()
+        data = bytes(data)
+        try:
+            g = GgufMetadata.read_bytes(data)
+            for k in g.keys():
+                try:
+                    g.get_value(k)
+                except FusorHipError:
+                    pass
+            for name in g.tensor_infos:
+                try:
+                    g.read_tensor_bytes(name)
+                except FusorHipError:
+                    pass
+            lib_ok = True
+        except FusorHipError:
+            lib_ok = False
+        try:
+            R.GgufRef(data)
+            ref_ok = True
+        except Exception:
+            ref_ok = False
+        assert lib_ok == ref_ok, (it, mode)
+        accepted += lib_ok
+    assert 100 < accepted < 500
