@@ -265,6 +265,37 @@ fh_status fh_argmax(fh_device *dev, const float *x_dev, int64_t count, uint32_t 
 fh_status fh_top_k(fh_device *dev, const float *x_dev, int64_t count, int32_t k, uint32_t *ids_dev,
                    float *values_dev, uint32_t *found_dev);
 
+/* Token sampling on the device, fusor-ml/core/src/sampling: logit processors (row_kernels.rs:150-205:
+ * repetition penalty over the previous tokens, then temperature), exact top-k in descending order (ties to
+ * the larger id), then one of two samplers over the sorted candidates: the standard one (row_kernels.rs:799-919:
+ * min_p against exp(value - max), top_p of the filtered weight, weighted pick) or Mirostat 2 (:672-797: cutoff
+ * where the surprise -log2(p) exceeds mu, weighted pick, mu -= eta * (surprise - tau)).  `random` is the caller's
+ * uniform number in [0, 1) (GpuStandardSamplerParams / GpuMirostat2SamplerParams, sampling/mod.rs:96-114).
+ * The reference's retry status (0) never occurs: the top-k here is exact. */
+#define FH_SAMPLER_STANDARD 0u
+#define FH_SAMPLER_MIROSTAT2 1u
+#define FH_SAMPLE_STATUS_SAMPLED 1u /* GPU_SAMPLE_STATUS_SAMPLED, sampling/mod.rs:25 */
+#define FH_SAMPLE_STATUS_INVALID 2u /* no finite logit, sampling/mod.rs:26 */
+#define FH_SAMPLER_PREVIOUS_TOKENS 64 /* GPU_SAMPLER_PREVIOUS_TOKENS, sampling/mod.rs:22 */
+typedef struct fh_sampler_params {
+    uint32_t kind;  /* FH_SAMPLER_* */
+    uint32_t top_k; /* 1 .. 256 */
+    float temperature;        /* 0 leaves the logits as they are */
+    float repetition_penalty; /* applied when above 1 */
+    float top_p, min_p;       /* standard sampler */
+    float tau, eta;           /* Mirostat 2 */
+    float random;
+} fh_sampler_params;
+/* sample_token_pending, sampling/pipeline.rs: result_dev[0] = status, result_dev[1] = token id.  previous_host:
+ * the caller's token history, of which the last 64 are used (63 when previous_tail_dev, one id left in device
+ * memory by an earlier call, is appended: processors.rs:20-81).  mu_dev: the Mirostat state (one float, device),
+ * updated in place; may be NULL for the standard sampler.  ids_dev / values_dev (optional, top_k entries each)
+ * receive the processed candidates in sorted order (a processed -0.0 reads 0.0), id 0xFFFFFFFF / NaN where
+ * fewer were finite. */
+fh_status fh_sample_token(fh_device *dev, const float *logits_dev, int64_t count, const fh_sampler_params *params,
+                          const uint32_t *previous_host, uint32_t n_previous, const uint32_t *previous_tail_dev,
+                          float *mu_dev, uint32_t *result_dev, uint32_t *ids_dev, float *values_dev);
+
 /* -------------------------------------------------------------- GGUF files
  * GgufMetadata::read, fusor-ml/gguf/src/lib.rs:559-613: versions 1 .. 3, metadata key/values, tensor
  * directory (dimensions reversed to row-major order, :583), payload start rounded up to
@@ -356,6 +387,15 @@ fh_status fh_llama_forward(fh_llama *m, const uint32_t *tokens_host, int32_t cou
 fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, int32_t steps,
                                  uint32_t *out_tokens_host, float *elapsed_ms);
 /* Bytes of weights read per decoded token (for roofline reports). */
+/* Sampled decode with the token resident on the device (models/kalosm-llama/src/model/inference.rs:38-173): every
+ * step samples from the logits as fh_sample_token does and feeds the id to the next step without a host round
+ * trip.  randoms_host[steps]: one uniform number per step.  previous_host: the history before first_token (the
+ * last repetition_range <= 64 ids count, first_token and the sampled ids are appended as they come).  *mu: the
+ * Mirostat state, in and out (ignored by the standard sampler, may be NULL then).  A step without a finite
+ * logit stores 0xFFFFFFFF and continues with id 0. */
+fh_status fh_llama_decode_sampled(fh_llama *m, uint32_t first_token, int32_t steps, const fh_sampler_params *params,
+                                  const float *randoms_host, const uint32_t *previous_host, uint32_t n_previous,
+                                  uint32_t repetition_range, float *mu, uint32_t *out_tokens_host, float *elapsed_ms);
 fh_status fh_llama_weight_bytes(const fh_llama *m, uint64_t *bytes);
 /* Model parameters from GGUF metadata, models/kalosm-llama/src/raw/mod.rs:377-416 (architecture
  * `llama` only; kv_dtype f32, fusions and graph replay switched on: adjust before fh_llama_create,

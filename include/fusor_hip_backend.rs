@@ -226,6 +226,26 @@ impl HipTensor<1> {
         let n = hf[0] as usize;
         Ok(hi.into_iter().zip(hv).take(n).collect())
     }
+
+    /// `sample_standard_token` / `sample_mirostat2_token` (fusor-ml/core/src/sampling/pipeline.rs): `params.kind`
+    /// selects the sampler, `mu` is the Mirostat state (a one-element tensor, updated in place).
+    /// `None` when no logit is finite.
+    pub fn sample_token(&self, params: &sys::FhSamplerParams, previous_tokens: &[u32], mu: Option<&HipTensor<1>>) -> Result<Option<u32>> {
+        let dev = self.device();
+        let result = Buffer::new(dev, 8)?;
+        let mut host = [0u32; 2];
+        let _g = dev.lock();
+        unsafe {
+            check(sys::fh_sample_token(
+                dev.raw(), self.ptr(), self.len() as i64, params,
+                if previous_tokens.is_empty() { std::ptr::null() } else { previous_tokens.as_ptr() },
+                previous_tokens.len() as u32, std::ptr::null(),
+                mu.map_or(std::ptr::null_mut(), |t| t.ptr() as *mut f32), result.ptr.cast(), std::ptr::null_mut(), std::ptr::null_mut(),
+            ))?;
+            check(sys::fh_download(dev.raw(), host.as_mut_ptr().cast(), result.ptr, 8))?;
+        }
+        Ok((host[0] == 1).then_some(host[1]))
+    }
 }
 
 impl HipTensor<4> {

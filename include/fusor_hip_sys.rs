@@ -100,6 +100,21 @@ pub struct FhRopeScaling {
     pub original_max_position_embeddings: i32,
 }
 
+/// `fh_sampler_params` (`GpuStandardSamplerParams` / `GpuMirostat2SamplerParams`, fusor-ml/core/src/sampling/mod.rs:96-114)
+#[repr(C)]
+#[derive(Clone, Copy, Debug)]
+pub struct FhSamplerParams {
+    pub kind: u32,
+    pub top_k: u32,
+    pub temperature: f32,
+    pub repetition_penalty: f32,
+    pub top_p: f32,
+    pub min_p: f32,
+    pub tau: f32,
+    pub eta: f32,
+    pub random: f32,
+}
+
 /// `fh_gguf_tensor`: `name` is owned by the `FhGguf` handle
 #[repr(C)]
 #[derive(Clone, Copy, Debug)]
@@ -165,6 +180,7 @@ extern "C" {
     pub fn fh_cast_f32_bf16(dev: *mut FhDevice, x_dev: *const f32, y_bf16_dev: *mut c_void, count: i64) -> FhStatus;
     pub fn fh_argmax(dev: *mut FhDevice, x_dev: *const f32, count: i64, id_dev: *mut u32) -> FhStatus;
     pub fn fh_top_k(dev: *mut FhDevice, x_dev: *const f32, count: i64, k: i32, ids_dev: *mut u32, values_dev: *mut f32, found_dev: *mut u32) -> FhStatus;
+    pub fn fh_sample_token(dev: *mut FhDevice, logits_dev: *const f32, count: i64, params: *const FhSamplerParams, previous_host: *const u32, n_previous: u32, previous_tail_dev: *const u32, mu_dev: *mut f32, result_dev: *mut u32, ids_dev: *mut u32, values_dev: *mut f32) -> FhStatus;
     pub fn fh_gguf_open(path: *const c_char, out: *mut *mut FhGguf) -> FhStatus;
     pub fn fh_gguf_open_memory(bytes: *const c_void, len: usize, out: *mut *mut FhGguf) -> FhStatus;
     pub fn fh_gguf_close(g: *mut FhGguf) -> FhStatus;
@@ -190,6 +206,7 @@ extern "C" {
     pub fn fh_llama_reset(m: *mut FhLlama) -> FhStatus;
     pub fn fh_llama_forward(m: *mut FhLlama, tokens_host: *const u32, count: i32, logits_host: *mut f32, hidden_host: *mut f32) -> FhStatus;
     pub fn fh_llama_decode_greedy(m: *mut FhLlama, first_token: u32, steps: i32, out_tokens_host: *mut u32, elapsed_ms: *mut f32) -> FhStatus;
+    pub fn fh_llama_decode_sampled(m: *mut FhLlama, first_token: u32, steps: i32, params: *const FhSamplerParams, randoms_host: *const f32, previous_host: *const u32, n_previous: u32, repetition_range: u32, mu: *mut f32, out_tokens_host: *mut u32, elapsed_ms: *mut f32) -> FhStatus;
     pub fn fh_llama_weight_bytes(m: *const FhLlama, bytes: *mut u64) -> FhStatus;
     pub fn fh_llama_config_from_gguf(g: *const FhGguf, cfg: *mut FhLlamaConfig) -> FhStatus;
     pub fn fh_llama_load_gguf(m: *mut FhLlama, g: *const FhGguf) -> FhStatus;

@@ -34,6 +34,11 @@ class RopeScaling(C.Structure):
                 ("original_max_position_embeddings", C.c_int32)]
 
 
+class SamplerParams(C.Structure):
+    _fields_ = [("kind", C.c_uint32), ("top_k", C.c_uint32), ("temperature", C.c_float), ("repetition_penalty", C.c_float),
+                ("top_p", C.c_float), ("min_p", C.c_float), ("tau", C.c_float), ("eta", C.c_float), ("random", C.c_float)]
+
+
 class GgufTensor(C.Structure):
     _fields_ = [("name", C.c_char_p), ("ggml_type", C.c_uint32), ("rank", C.c_int32), ("shape", C.c_int64 * 8),
                 ("offset", C.c_uint64)]
@@ -97,6 +102,9 @@ SIGNATURES = {
     "fh_argmax": [_p, _p, _i64, _p],
     "fh_kvcache_set_sliding": [_p, _i32],
     "fh_top_k": [_p, _p, _i64, _i32, _p, _p, _p],
+    "fh_sample_token": [_p, _p, _i64, C.POINTER(SamplerParams), _p, _u32, _p, _p, _p, _p, _p],
+    "fh_llama_decode_sampled": [_p, _u32, _i32, C.POINTER(SamplerParams), _p, _p, _u32, _u32, C.POINTER(_f32), _p,
+                                C.POINTER(_f32)],
     "fh_llama_create": [_p, C.POINTER(LlamaConfig), _pp],
     "fh_llama_destroy": [_p],
     "fh_llama_load_tensor": [_p, C.c_char_p, _u32, _i64, _i64, _p, _sz],

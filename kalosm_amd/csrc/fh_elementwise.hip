@@ -406,17 +406,138 @@ __device__ __forceinline__ uint64_t topk_key(float v, uint32_t id) {
     return ((uint64_t)o << 32) | id;
 }
 
+__device__ __forceinline__ float topk_value(uint64_t key) {
+    const uint32_t o = (uint32_t)(key >> 32);
+    return __uint_as_float((o & 0x80000000u) ? (o & 0x7FFFFFFFu) : ~o);
+}
+
+// Logit processors of the sampling front end (fusor-ml/core/src/sampling/row_kernels.rs:150-205; the host form is
+// process_logit, models/kalosm-llama/src/sampler.rs:275-307): a finite logit whose id is among the previous tokens is
+// multiplied (<= 0) or divided (> 0) by a repetition penalty above 1, then every logit is divided by a non-zero
+// temperature; what is not finite before or after is skipped.  `prev` holds up to 64 ids in device memory (membership
+// only, so the order of the slots does not matter), its length is *prev_len when that pointer is given.
+struct TopkProc {
+    int on;
+    float temperature, penalty;
+    const uint32_t *prev;
+    const uint32_t *prev_len;
+    uint32_t n_prev;
+};
+
+// Sampler that ends the last pass (row_kernels.rs:484-660 helpers, :672-797 Mirostat 2, :799-919 standard):
+// weights exp(value - max) of the sorted candidates, a cutoff, then the first candidate whose running weight reaches
+// random * (sum of the weights before the cutoff).  result = [status, token]: 1 sampled, 2 no finite logit.
+struct TopkSample {
+    int on;
+    uint32_t kind;
+    float top_p, min_p, tau, eta, random;
+    const float *randoms; // device; entry *step (entry 0 without `step`) replaces `random`
+    const int *step;
+    float *mu;            // Mirostat state, device
+    uint32_t *result;
+};
+
+__device__ void topk_sample(const uint64_t *s, float *w, int k, const TopkSample &a) {
+    // called by thread 0 after w[i] = exp(value_i - value_0) (0 for a missing candidate) is in LDS
+    const float eps = 1.0e-20f;
+    if (!s[0]) {
+        a.result[0] = 2u;
+        a.result[1] = 0u;
+        return;
+    }
+    const float random = a.randoms ? a.randoms[a.step ? *a.step : 0] : a.random;
+    int cutoff = k;
+    float cutoff_sum = 0.f, mu = 0.f;
+    if (a.kind == 1u) {
+        float total = 0.f;
+        for (int i = 0; i < k; i++) total += w[i];
+        total = fmaxf(total, eps);
+        mu = *a.mu;
+        for (int i = 0; i < k; i++) {
+            const float p = fmaxf(w[i] / total, eps);
+            if (-log2f(p) > mu) {
+                cutoff = i > 1 ? i : 1;
+                break;
+            }
+        }
+        for (int i = 0; i < cutoff; i++) cutoff_sum += w[i];
+    } else {
+        float filtered = 0.f;
+        for (int i = 0; i < k; i++)
+            if (w[i] >= a.min_p) filtered += w[i];
+        const float target = __fmul_rn(fmaxf(filtered, eps), a.top_p);
+        for (int i = 0; i < k; i++) {
+            if (w[i] >= a.min_p) {
+                cutoff_sum += w[i];
+                if (cutoff_sum >= target) {
+                    cutoff = i + 1;
+                    break;
+                }
+            } else {
+                cutoff = i;
+                break;
+            }
+        }
+        if (cutoff == 0) {
+            cutoff = 1;
+            cutoff_sum = w[0];
+        }
+    }
+    cutoff_sum = fmaxf(cutoff_sum, eps);
+    const float threshold = __fmul_rn(random, cutoff_sum);
+    uint32_t token = (uint32_t)s[0];
+    float prob = w[0] / cutoff_sum, cum = 0.f;
+    for (int i = 0; i < cutoff; i++) {
+        cum += w[i];
+        if (cum >= threshold) {
+            token = s[i] ? (uint32_t)s[i] : 0xFFFFFFFFu;
+            prob = w[i] / cutoff_sum;
+            break;
+        }
+    }
+    if (a.kind == 1u) {
+        const float surprise = -log2f(fmaxf(prob, eps));
+        *a.mu = __fsub_rn(mu, __fmul_rn(a.eta, __fsub_rn(surprise, a.tau)));
+    }
+    a.result[0] = 1u;
+    a.result[1] = token;
+}
+
 template <bool FIRST>
 __global__ __launch_bounds__(512) void k_topk_pass(const float *__restrict__ x, const uint64_t *__restrict__ keys_in,
                                                    int64_t n_in, int k, int last, uint64_t *__restrict__ keys_out,
                                                    uint32_t *__restrict__ ids_out, float *__restrict__ vals_out,
-                                                   uint32_t *__restrict__ found_out) {
+                                                   uint32_t *__restrict__ found_out, TopkProc proc, TopkSample samp) {
     __shared__ uint64_t s[1024];
+    __shared__ uint32_t s_prev[64];
+    __shared__ float s_w[256];
     const int tid = threadIdx.x;
     const int64_t base = (int64_t)blockIdx.x * 1024;
+    uint32_t n_prev = 0;
+    if (FIRST && proc.on && proc.penalty > 1.0f) {
+        n_prev = proc.prev_len ? *proc.prev_len : proc.n_prev;
+        n_prev = n_prev < 64u ? n_prev : 64u;
+        if (tid < 64) s_prev[tid] = (uint32_t)tid < n_prev ? proc.prev[tid] : 0u;
+        __syncthreads();
+    }
     for (int i = tid; i < 1024; i += 512) {
         const int64_t idx = base + i;
-        s[i] = idx < n_in ? (FIRST ? topk_key(x[idx], (uint32_t)idx) : keys_in[idx]) : 0ull;
+        uint64_t key = 0ull;
+        if (idx < n_in) {
+            if (FIRST) {
+                float v = x[idx];
+                if (proc.on && (__float_as_uint(v) & 0x7F800000u) != 0x7F800000u) {
+                    bool repeated = false;
+                    for (uint32_t j = 0; j < n_prev; j++) repeated |= s_prev[j] == (uint32_t)idx;
+                    if (repeated) v = v <= 0.0f ? __fmul_rn(v, proc.penalty) : __fdiv_rn(v, proc.penalty);
+                    if (proc.temperature != 0.0f) v = __fdiv_rn(v, proc.temperature);
+                }
+                key = topk_key(v, (uint32_t)idx);
+            } else {
+                key = keys_in[idx];
+            }
+        }
+        s[i] = key;
     }
     __syncthreads();
     for (int size = 2; size <= 1024; size <<= 1)
@@ -434,23 +555,27 @@ __global__ __launch_bounds__(512) void k_topk_pass(const float *__restrict__ x, 
         for (int i = tid; i < k; i += 512) keys_out[(int64_t)blockIdx.x * k + i] = s[i];
         return;
     }
-    for (int i = tid; i < k; i += 512) {
-        const uint64_t key = s[i];
-        ids_out[i] = key ? (uint32_t)key : 0xFFFFFFFFu;
-        vals_out[i] = key ? x[(uint32_t)key] : __uint_as_float(0x7FC00000u);
-    }
+    if (ids_out)
+        for (int i = tid; i < k; i += 512) {
+            const uint64_t key = s[i];
+            ids_out[i] = key ? (uint32_t)key : 0xFFFFFFFFu;
+            // the processed value is the one the key carries; the plain top-k returns the stored logit (-0.0 kept)
+            vals_out[i] = key ? (proc.on ? topk_value(key) : x[(uint32_t)key]) : __uint_as_float(0x7FC00000u);
+        }
     if (tid == 0 && found_out) {
         int c = 0;
         while (c < k && s[c]) c++;
         *found_out = (uint32_t)c;
     }
+    if (samp.on) {
+        if (tid < k) s_w[tid] = s[tid] ? expf(topk_value(s[tid]) - topk_value(s[0])) : 0.f;
+        __syncthreads();
+        if (tid == 0) topk_sample(s, s_w, k, samp);
+    }
 }
 
-extern "C" fh_status fh_top_k(fh_device *dev, const float *x_dev, int64_t count, int32_t k, uint32_t *ids_dev,
-                              float *values_dev, uint32_t *found_dev) {
-    FH_REQUIRE(dev && x_dev && ids_dev && values_dev, "NULL argument");
-    FH_REQUIRE(count > 0 && count < 0xFFFFFFFFll, "count %lld out of range", (long long)count);
-    FH_REQUIRE(k >= 1 && k <= 256, "k = %d out of range (1 .. 256)", k);
+static fh_status topk_run(fh_device *dev, const float *x_dev, int64_t count, int32_t k, uint32_t *ids_dev,
+                          float *values_dev, uint32_t *found_dev, const TopkProc &proc, const TopkSample &samp) {
     int64_t n = count, blocks = (n + 1023) / 1024;
     uint64_t *buf[2] = {nullptr, nullptr};
     if (blocks > 1) {
@@ -465,11 +590,11 @@ extern "C" fh_status fh_top_k(fh_device *dev, const float *x_dev, int64_t count,
     for (;;) {
         const int last = blocks == 1;
         if (first)
-            k_topk_pass<true><<<dim3((unsigned)blocks), dim3(512), 0, dev->stream>>>(x_dev, nullptr, n, k, last, buf[turn],
-                                                                                    ids_dev, values_dev, found_dev);
+            k_topk_pass<true><<<dim3((unsigned)blocks), dim3(512), 0, dev->stream>>>(
+                x_dev, nullptr, n, k, last, buf[turn], ids_dev, values_dev, found_dev, proc, samp);
         else
-            k_topk_pass<false><<<dim3((unsigned)blocks), dim3(512), 0, dev->stream>>>(x_dev, in, n, k, last, buf[turn],
-                                                                                     ids_dev, values_dev, found_dev);
+            k_topk_pass<false><<<dim3((unsigned)blocks), dim3(512), 0, dev->stream>>>(
+                x_dev, in, n, k, last, buf[turn], ids_dev, values_dev, found_dev, proc, samp);
         FH_HIP(hipGetLastError());
         if (last) break;
         in = buf[turn];
@@ -479,6 +604,49 @@ extern "C" fh_status fh_top_k(fh_device *dev, const float *x_dev, int64_t count,
         first = false;
     }
     return FH_OK;
+}
+
+extern "C" fh_status fh_top_k(fh_device *dev, const float *x_dev, int64_t count, int32_t k, uint32_t *ids_dev,
+                              float *values_dev, uint32_t *found_dev) {
+    FH_REQUIRE(dev && x_dev && ids_dev && values_dev, "NULL argument");
+    FH_REQUIRE(count > 0 && count < 0xFFFFFFFFll, "count %lld out of range", (long long)count);
+    FH_REQUIRE(k >= 1 && k <= 256, "k = %d out of range (1 .. 256)", k);
+    TopkProc proc = {};
+    TopkSample samp = {};
+    return topk_run(dev, x_dev, count, k, ids_dev, values_dev, found_dev, proc, samp);
+}
+
+// Device-side form used by the decoder's sampled decode loop: previous tokens, their count, the random numbers and
+// the step index all live in device memory, so the same launches can be replayed as a graph.
+fh_status fh_sample_token_dev(fh_device *dev, const float *logits_dev, int64_t count, const fh_sampler_params *p,
+                              const uint32_t *prev_dev, const uint32_t *prev_len_dev, uint32_t n_prev,
+                              const float *randoms_dev, const int *step_dev, float *mu_dev, uint32_t *result_dev,
+                              uint32_t *ids_dev, float *values_dev) {
+    FH_REQUIRE(p->kind == FH_SAMPLER_STANDARD || p->kind == FH_SAMPLER_MIROSTAT2, "sampler kind %u unknown", p->kind);
+    FH_REQUIRE(p->top_k >= 1 && p->top_k <= 256, "top_k = %u out of range (1 .. 256)", p->top_k);
+    FH_REQUIRE(p->kind != FH_SAMPLER_MIROSTAT2 || mu_dev, "Mirostat 2 needs its state");
+    FH_REQUIRE((ids_dev == nullptr) == (values_dev == nullptr), "ids and values go together");
+    TopkProc proc = {1, p->temperature, p->repetition_penalty, prev_dev, prev_len_dev, n_prev};
+    TopkSample samp = {1, p->kind, p->top_p, p->min_p, p->tau, p->eta, p->random, randoms_dev, step_dev, mu_dev, result_dev};
+    return topk_run(dev, logits_dev, count, (int32_t)p->top_k, ids_dev, values_dev, nullptr, proc, samp);
+}
+
+extern "C" fh_status fh_sample_token(fh_device *dev, const float *logits_dev, int64_t count, const fh_sampler_params *params,
+                                     const uint32_t *previous_host, uint32_t n_previous, const uint32_t *previous_tail_dev,
+                                     float *mu_dev, uint32_t *result_dev, uint32_t *ids_dev, float *values_dev) {
+    FH_REQUIRE(dev && logits_dev && params && result_dev, "NULL argument");
+    FH_REQUIRE(count > 0 && count < 0xFFFFFFFFll, "count %lld out of range", (long long)count);
+    FH_REQUIRE(n_previous == 0 || previous_host, "previous tokens missing");
+    // fixed_previous_tokens_data{,_with_gpu_tail}, fusor-ml/core/src/sampling/processors.rs:20-81: the last 64 ids,
+    // or the last 63 followed by the id another kernel left in device memory.
+    const uint32_t room = previous_tail_dev ? 63u : 64u;
+    const uint32_t keep = n_previous < room ? n_previous : room;
+    uint32_t *prev = (uint32_t *)((uint8_t *)dev->small_buf + 60 * 1024); // the last 4 KB of the 64 KB buffer: no other user
+    if (keep) FH_TRY(fh_upload(dev, prev, previous_host + (n_previous - keep), (size_t)keep * 4));
+    if (previous_tail_dev)
+        FH_HIP(hipMemcpyAsync(prev + keep, previous_tail_dev, 4, hipMemcpyDeviceToDevice, dev->stream));
+    return fh_sample_token_dev(dev, logits_dev, count, params, prev, nullptr, keep + (previous_tail_dev ? 1u : 0u), nullptr,
+                               nullptr, mu_dev, result_dev, ids_dev, values_dev);
 }
 
 // ------------------------------------------------------------------------------ KV cache

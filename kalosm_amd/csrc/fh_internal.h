@@ -214,3 +214,9 @@ fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *
 fh_status fh_rope_pair_devpos(fh_device *dev, const float *q, const float *k, int hq, int hk, int d,
                               const float *cos_t, const float *sin_t, int table_rows,
                               const int *pos_dev, float *q_out, float *k_out);
+// Sampler with every per-step input in device memory (fh_elementwise.hip); fh_sample_token is its host-input form.
+fh_status fh_sample_token_dev(fh_device *dev, const float *logits_dev, int64_t count, const fh_sampler_params *p,
+                              const uint32_t *prev_dev, const uint32_t *prev_len_dev, uint32_t n_prev,
+                              const float *randoms_dev, const int *step_dev, float *mu_dev, uint32_t *result_dev,
+                              uint32_t *ids_dev, float *values_dev);
+

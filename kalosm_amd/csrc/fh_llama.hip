@@ -40,6 +40,14 @@ struct fh_llama {
     hipGraphExec_t graph_exec = nullptr;
     hipGraph_t graph = nullptr;
     int captured_capacity = -1;
+    // sampled decode state: [0..63] previous ids, [64] their count, [65] next slot, [66] Mirostat mu (f32),
+    // [68..69] status and token of the last step, [128..] one random number per step
+    uint32_t *samp_dev = nullptr;
+    hipGraphExec_t samp_exec = nullptr;
+    hipGraph_t samp_graph = nullptr;
+    int samp_capacity = -1;
+    uint32_t samp_range = 0;
+    fh_sampler_params samp_params = {};
 };
 
 static void free_dev(void *p) {
@@ -69,6 +77,7 @@ static void free_steps(fh_llama *m) {
     m->x = m->xn = m->qkv = m->qrot = m->krot = m->att = m->att_t = m->attn_out = m->gu = m->act = m->ff = nullptr;
     m->cap_s = 0;
     m->captured_capacity = -1; // a captured decode step holds these pointers
+    m->samp_capacity = -1;
 }
 
 extern "C" fh_status fh_llama_destroy(fh_llama *m) {
@@ -85,7 +94,9 @@ extern "C" fh_status fh_llama_destroy(fh_llama *m) {
     fh_qmatrix_free(m->embd);
     if (!m->output_is_embd) fh_qmatrix_free(m->output);
     free_dev(m->out_norm); free_dev(m->cos_t); free_dev(m->sin_t);
-    free_dev(m->logits); free_dev(m->tok_dev); free_dev(m->out_tok_dev); free_dev(m->step_dev);
+    free_dev(m->logits); free_dev(m->tok_dev); free_dev(m->out_tok_dev); free_dev(m->step_dev); free_dev(m->samp_dev);
+    if (m->samp_exec) (void)hipGraphExecDestroy(m->samp_exec);
+    if (m->samp_graph) (void)hipGraphDestroy(m->samp_graph);
     free_steps(m);
     fh_kvcache_destroy(m->cache);
     delete m;
@@ -210,6 +221,7 @@ extern "C" fh_status fh_llama_finalize(fh_llama *m) {
     FH_TRY(fh_malloc(m->dev, 256, (void **)&m->tok_dev));
     FH_TRY(fh_malloc(m->dev, (size_t)c.ctx * 4 + 256, (void **)&m->out_tok_dev));
     FH_TRY(fh_malloc(m->dev, 256, (void **)&m->step_dev));
+    FH_TRY(fh_malloc(m->dev, (size_t)(128 + c.ctx) * 4, (void **)&m->samp_dev));
     FH_TRY(ensure_steps(m, 1));
     m->finalized = true;
     return FH_OK;
@@ -462,5 +474,106 @@ extern "C" fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, i
     m->pos += steps;
     m->cache->len = m->pos;
     FH_TRY(fh_download(dev, out_tokens_host, m->out_tok_dev, (size_t)steps * 4));
+    return FH_OK;
+}
+
+// Sampled decode (models/kalosm-llama/src/model/inference.rs:38-173, forward.rs:346-404): the sampled id stays in
+// device memory and feeds the next step; it also joins the window of previous ids that the repetition penalty
+// looks at (membership only, so the window is a ring).
+__global__ void k_store_sampled(const uint32_t *result, uint32_t *ids, uint32_t *out, int *step, uint32_t *prev,
+                                uint32_t range) {
+    const uint32_t t = result[0] == FH_SAMPLE_STATUS_SAMPLED ? result[1] : 0xFFFFFFFFu;
+    const uint32_t next = t == 0xFFFFFFFFu ? 0u : t;
+    ids[0] = next;
+    out[*step] = t;
+    *step = *step + 1;
+    if (range) {
+        const uint32_t slot = prev[65];
+        prev[slot] = next;
+        prev[65] = slot + 1 == range ? 0u : slot + 1;
+        if (prev[64] < range) prev[64] = prev[64] + 1;
+    }
+}
+
+static fh_status sampled_step_enqueue(fh_llama *m) {
+    FH_TRY(run_layers(m, 1, true));
+    FH_TRY(fh_kvcache_advance_dev(m->cache));
+    uint32_t *sd = m->samp_dev;
+    FH_TRY(fh_sample_token_dev(m->dev, m->logits, m->c.vocab, &m->samp_params, sd, sd + 64, 0, (const float *)(sd + 128),
+                               m->step_dev, (float *)(sd + 66), sd + 68, nullptr, nullptr));
+    k_store_sampled<<<1, 1, 0, m->dev->stream>>>(sd + 68, m->ids, m->out_tok_dev, m->step_dev, sd, m->samp_range);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+extern "C" fh_status fh_llama_decode_sampled(fh_llama *m, uint32_t first_token, int32_t steps,
+                                             const fh_sampler_params *params, const float *randoms_host,
+                                             const uint32_t *previous_host, uint32_t n_previous, uint32_t repetition_range,
+                                             float *mu, uint32_t *out_tokens_host, float *elapsed_ms) {
+    FH_REQUIRE(m && m->finalized && out_tokens_host && params && randoms_host, "decoder not finalized or NULL argument");
+    FH_REQUIRE(steps > 0 && m->pos + steps <= m->c.ctx, "context overflow: %d + %d > %d", m->pos, steps, m->c.ctx);
+    FH_REQUIRE(first_token < (uint32_t)m->c.vocab, "token id %u outside the vocabulary", first_token);
+    FH_REQUIRE(n_previous == 0 || previous_host, "previous tokens missing");
+    FH_REQUIRE(params->kind != FH_SAMPLER_MIROSTAT2 || mu, "Mirostat 2 needs its state");
+    fh_device *dev = m->dev;
+    hipStream_t s = dev->stream;
+    const uint32_t range = repetition_range < FH_SAMPLER_PREVIOUS_TOKENS ? repetition_range : FH_SAMPLER_PREVIOUS_TOKENS;
+    // window = the last `range` ids of (history, first_token)
+    uint32_t head[128] = {0};
+    uint32_t len = 0;
+    if (range) {
+        const uint32_t keep = n_previous < range - 1 ? n_previous : range - 1;
+        for (uint32_t i = 0; i < keep; i++) head[len++] = previous_host[n_previous - keep + i];
+        head[len++] = first_token;
+    }
+    head[64] = len;
+    head[65] = range ? len % range : 0u;
+    const float mu0 = mu ? *mu : 0.f;
+    memcpy(&head[66], &mu0, 4);
+    FH_TRY(fh_upload(dev, m->samp_dev, head, sizeof(head)));
+    FH_TRY(fh_upload(dev, m->samp_dev + 128, randoms_host, (size_t)steps * 4));
+    FH_TRY(fh_kvcache_reserve(m->cache, m->pos + steps));
+    k_set_u32<<<1, 1, 0, s>>>(m->ids, first_token);
+    k_set_u32<<<1, 1, 0, s>>>((uint32_t *)m->step_dev, 0u);
+    FH_HIP(hipGetLastError());
+    int done = 0;
+    if (m->c.use_graph) {
+        // the captured step holds the sampler's parameters and the window size as kernel arguments
+        const bool same = m->samp_exec && m->samp_capacity == m->cache->capacity && m->samp_range == range &&
+                          memcmp(&m->samp_params, params, sizeof(*params)) == 0;
+        m->samp_params = *params;
+        m->samp_range = range;
+        if (!same) {
+            FH_TRY(fh_timer_start(dev));
+            FH_TRY(sampled_step_enqueue(m));
+            done = 1;
+            FH_HIP(hipStreamSynchronize(s));
+            if (m->samp_exec) { (void)hipGraphExecDestroy(m->samp_exec); m->samp_exec = nullptr; }
+            if (m->samp_graph) { (void)hipGraphDestroy(m->samp_graph); m->samp_graph = nullptr; }
+            m->samp_capacity = -1;
+            FH_HIP(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+            fh_status st = sampled_step_enqueue(m);
+            hipError_t e = hipStreamEndCapture(s, &m->samp_graph);
+            if (st != FH_OK) return st;
+            FH_HIP(e);
+            FH_HIP(hipGraphInstantiate(&m->samp_exec, m->samp_graph, nullptr, nullptr, 0));
+            m->samp_capacity = m->cache->capacity;
+        } else {
+            FH_TRY(fh_timer_start(dev));
+        }
+        for (; done < steps; done++) FH_HIP(hipGraphLaunch(m->samp_exec, s));
+    } else {
+        m->samp_params = *params;
+        m->samp_range = range;
+        FH_TRY(fh_timer_start(dev));
+        for (; done < steps; done++) FH_TRY(sampled_step_enqueue(m));
+    }
+    float ms = 0.f;
+    FH_TRY(fh_timer_stop(dev, &ms));
+    if (elapsed_ms) *elapsed_ms = ms;
+    m->pos += steps;
+    m->cache->len = m->pos;
+    FH_TRY(fh_download(dev, out_tokens_host, m->out_tok_dev, (size_t)steps * 4));
+    if (mu) FH_TRY(fh_download(dev, mu, m->samp_dev + 66, 4));
     return FH_OK;
 }

@@ -14,7 +14,45 @@ import numpy as np
 from . import _lib
 from ._lib import (F16, F32, MASK_ADDITIVE, MASK_CAUSAL, MASK_NONE, Q4_0, Q4_K, Q6_K, Q8_0, FusorHipError, check)
 
-__all__ = ["Device", "Tensor", "QMatrix", "RopeCache", "KvCache", "MaskKind", "GgmlType", "FusorHipError"]
+__all__ = ["Device", "Tensor", "QMatrix", "RopeCache", "KvCache", "MaskKind", "GgmlType", "FusorHipError",
+           "GpuStandardSamplerParams", "GpuMirostat2SamplerParams", "GpuMirostat2Sampler"]
+
+
+class GpuStandardSamplerParams:
+    """fusor-ml/core/src/sampling/mod.rs:106-114"""
+
+    def __init__(self, top_k: int, temperature: float, repetition_penalty: float, top_p: float, min_p: float,
+                 random: float):
+        self.top_k, self.temperature, self.repetition_penalty = top_k, temperature, repetition_penalty
+        self.top_p, self.min_p, self.random = top_p, min_p, random
+
+    def to_c(self) -> "_lib.SamplerParams":
+        return _lib.SamplerParams(0, self.top_k, self.temperature, self.repetition_penalty, self.top_p, self.min_p, 0.0,
+                                  0.0, self.random)
+
+
+class GpuMirostat2SamplerParams:
+    """fusor-ml/core/src/sampling/mod.rs:96-104"""
+
+    def __init__(self, top_k: int, temperature: float, repetition_penalty: float, tau: float, eta: float,
+                 random: float):
+        self.top_k, self.temperature, self.repetition_penalty = top_k, temperature, repetition_penalty
+        self.tau, self.eta, self.random = tau, eta, random
+
+    def to_c(self) -> "_lib.SamplerParams":
+        return _lib.SamplerParams(1, self.top_k, self.temperature, self.repetition_penalty, 1.0, 0.0, self.tau,
+                                  self.eta, self.random)
+
+
+class GpuMirostat2Sampler:
+    """GpuMirostat2Sampler::new(device, mu) (sampling/mod.rs:116-125): the state mu in device memory."""
+
+    def __init__(self, device: "Device", mu: float):
+        self.state = Tensor.from_slice(device, np.array([mu], np.float32))
+
+    @property
+    def mu(self) -> float:
+        return float(self.state.as_slice()[0])
 
 
 class GgmlType:
@@ -306,6 +344,36 @@ class Tensor:
                                         C.c_void_p(ids.ptr), C.c_void_p(vals.ptr), C.c_void_p(found.ptr)))
         n = int(found.as_slice()[0])
         return list(zip(ids.as_slice()[:n].tolist(), vals.as_slice()[:n].tolist()))
+
+    def _sample(self, params, previous_tokens, mu_ptr, previous_gpu_token=None, want_candidates=False):
+        prev = np.ascontiguousarray(previous_tokens, np.uint32)
+        res = Tensor(self.device, (2,), "u32")
+        k = params.top_k
+        ids = Tensor(self.device, (k,), "u32") if want_candidates else None
+        vals = Tensor(self.device, (k,), "f32") if want_candidates else None
+        cp = params.to_c()
+        check(self.device._lib.fh_sample_token(
+            self.device._h, C.c_void_p(self.ptr), int(np.prod(self.shape)), C.byref(cp),
+            prev.ctypes.data_as(C.c_void_p) if prev.size else None, int(prev.size),
+            C.c_void_p(previous_gpu_token.ptr) if previous_gpu_token is not None else None,
+            C.c_void_p(mu_ptr) if mu_ptr else None, C.c_void_p(res.ptr),
+            C.c_void_p(ids.ptr) if ids is not None else None, C.c_void_p(vals.ptr) if vals is not None else None))
+        status, token = (int(v) for v in res.as_slice())
+        token = token if status == 1 else None
+        if want_candidates:
+            return token, ids.as_slice(), vals.as_slice()
+        return token
+
+    def sample_standard_token(self, previous_tokens, params: "GpuStandardSamplerParams", previous_gpu_token=None,
+                              want_candidates=False):
+        """Tensor::sample_standard_token (fusor-ml/core/src/sampling/pipeline.rs): the sampled id, or None when no
+        logit is finite.  `want_candidates` also returns the processed top-k ids and values in sorted order."""
+        return self._sample(params, previous_tokens, None, previous_gpu_token, want_candidates)
+
+    def sample_mirostat2_token(self, sampler: "GpuMirostat2Sampler", previous_tokens,
+                               params: "GpuMirostat2SamplerParams", previous_gpu_token=None, want_candidates=False):
+        """Tensor::sample_mirostat2_token (fusor-ml/core/src/sampling/pipeline.rs); updates `sampler`'s mu."""
+        return self._sample(params, previous_tokens, sampler.state.ptr, previous_gpu_token, want_candidates)
 
     def top_k_pairs_1(self) -> int:
         """Tensor::top_k_pairs(1) (fusor-ml/fusor/src/lib.rs:416-447): the greedy token id, or -1."""

@@ -92,6 +92,23 @@ class Model:
                                                       C.byref(ms)))
         return out, ms.value
 
+    def decode_sampled(self, first_token: int, steps: int, params, randoms, previous_tokens=(), repetition_range: int = 64,
+                       mu: Optional[float] = None):
+        """Sampled decode of `steps` tokens with the token resident on the device (models/kalosm-llama/src/model/
+        inference.rs:38-173).  `params`: GpuStandardSamplerParams or GpuMirostat2SamplerParams (its `random` is
+        replaced by `randoms[step]`).  Returns (token ids, device milliseconds, mu after the last step)."""
+        out = np.empty(steps, np.uint32)
+        rnd = np.ascontiguousarray(randoms, np.float32)
+        assert rnd.size >= steps
+        prev = np.ascontiguousarray(previous_tokens, np.uint32)
+        ms, mu_c = C.c_float(), C.c_float(0.0 if mu is None else mu)
+        cp = params.to_c()
+        check(self.device._lib.fh_llama_decode_sampled(
+            self._h, int(first_token), steps, C.byref(cp), rnd.ctypes.data_as(C.c_void_p),
+            prev.ctypes.data_as(C.c_void_p) if prev.size else None, int(prev.size), int(repetition_range),
+            C.byref(mu_c), out.ctypes.data_as(C.c_void_p), C.byref(ms)))
+        return out, ms.value, mu_c.value
+
     def weight_bytes(self) -> int:
         b = C.c_uint64()
         check(self.device._lib.fh_llama_weight_bytes(self._h, C.byref(b)))

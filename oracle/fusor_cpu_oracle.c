@@ -31,6 +31,11 @@
  *                           references; RoPE golden sextets; inverse-frequency closed form;
  *                           long-context scaling and rope_freqs weights against numpy
  *   argmax ................ tie and non-finite cases from the reference's rule
+ *   samplers .............. the reference's stored answers (flat logits: Mirostat 2 with random 0.8 -> id 0, top_p 0.5
+ *                           with random 0.8 -> id 2, min_p 0.1 -> id 3, processed order -> id 0), the processor
+ *                           case of its test (temperature 0.5, penalty 2, previous {0, 3, 9}) worked by hand,
+ *                           sampled frequencies against the softmax probabilities, and the Mirostat update
+ *                           against the closed form on two-candidate cases
  *   decoder ............... PARITY UNPINNED in the reference (no stored logits);
  *                           pinned here only by composition of the pinned ops and an
  *                           independent numpy float64 decoder on a tiny configuration.
@@ -38,6 +43,7 @@
  *   machine/library dependent in the reference itself (pulp lane width, gemm
  *   crate, platform libm) and are held to tolerance, never to bit equality.
  */
+#include <float.h>
 #include <math.h>
 #include <pthread.h>
 #include <stdint.h>
@@ -808,6 +814,108 @@ int fo_top_k(const float *x, size_t n, int k, uint32_t *ids, float *vals) {
         len++;
     }
     return len;
+}
+
+/* Device sampling of fusor-ml/core/src/sampling, restated step by step.
+ * Processors (row_kernels.rs:150-205; host form process_logit, models/kalosm-llama/src/sampler.rs:275-307): a
+ * non-finite logit is dropped; one whose id is among `prev` is multiplied (<= 0) or divided (> 0) by a repetition
+ * penalty above 1; a non-zero temperature divides; a non-finite result is dropped.
+ * Top-k: descending, ties to the larger id (better_candidate, row_kernels.rs:85-87); slots past the finite
+ * candidates read as value -FLT_MAX / id 0xFFFFFFFF (sampler_top_value / sampler_top_id, :484-497).
+ * Standard sampler: row_kernels.rs:799-919.  Mirostat 2: :672-797.  weighted_pick: :609-660.
+ * result = [status, token]: 1 sampled, 2 no finite logit (emit_sampler_guards, :518-545).
+ * *margin (optional) = the smallest relative gap of any comparison that decided the outcome; a caller comparing
+ * against another exp / log2 implementation can set cases with a tiny margin aside. */
+typedef struct {
+    uint32_t kind, top_k;
+    float temperature, repetition_penalty, top_p, min_p, tau, eta, random;
+} fo_sampler_params;
+
+static void fo_gap(float *margin, float a, float b) {
+    if (!margin) return;
+    float m = fmaxf(fmaxf(fabsf(a), fabsf(b)), 1e-30f);
+    float g = fabsf(a - b) / m;
+    if (g < *margin) *margin = g;
+}
+
+int fo_process_logits(const float *x, size_t n, float temperature, float penalty, const uint32_t *prev, uint32_t n_prev,
+                      float *out) {
+    for (size_t t = 0; t < n; t++) {
+        float v = x[t];
+        if (isfinite(v)) {
+            int repeated = 0;
+            for (uint32_t j = 0; j < n_prev; j++) repeated |= prev[j] == (uint32_t)t;
+            if (repeated && penalty > 1.0f) v = v <= 0.0f ? v * penalty : v / penalty;
+            if (temperature != 0.0f) v = v / temperature;
+        }
+        out[t] = v; /* what is not finite here is skipped by the top-k */
+    }
+    return 0;
+}
+
+int fo_sample_token(const float *logits, size_t n, const fo_sampler_params *p, const uint32_t *prev, uint32_t n_prev,
+                    float *mu_state, uint32_t *result, uint32_t *ids, float *vals, float *margin) {
+    const float eps = 1.0e-20f;
+    int k = (int)p->top_k;
+    if (k < 1 || k > 256) return -1;
+    float *proc = (float *)malloc(n * sizeof(float));
+    if (!proc) return -2;
+    fo_process_logits(logits, n, p->temperature, p->repetition_penalty, prev, n_prev, proc);
+    int found = fo_top_k(proc, n, k, ids, vals);
+    free(proc);
+    for (int i = found; i < k; i++) { ids[i] = 0xFFFFFFFFu; vals[i] = -FLT_MAX; }
+    if (margin) *margin = 1.0f;
+    if (ids[0] == 0xFFFFFFFFu) { result[0] = 2; result[1] = 0; return 0; }
+    float w[256] = {0};
+    for (int i = 0; i < k; i++) w[i] = expf(vals[i] - vals[0]);
+    int cutoff = k;
+    float cutoff_sum = 0.f, mu = 0.f;
+    if (p->kind == 1) {
+        float total = 0.f;
+        for (int i = 0; i < k; i++) total += w[i];
+        total = fmaxf(total, eps);
+        mu = *mu_state;
+        for (int i = 0; i < k; i++) {
+            float pr = fmaxf(w[i] / total, eps);
+            float surprise = log2f(pr) * -1.0f;
+            fo_gap(margin, surprise, mu);
+            if (surprise > mu) { cutoff = i > 1 ? i : 1; break; }
+        }
+        for (int i = 0; i < cutoff; i++) cutoff_sum += w[i];
+    } else {
+        float filtered = 0.f;
+        for (int i = 0; i < k; i++) {
+            fo_gap(margin, w[i], p->min_p);
+            if (w[i] >= p->min_p) filtered += w[i];
+        }
+        float target = fmaxf(filtered, eps) * p->top_p;
+        for (int i = 0; i < k; i++) {
+            if (w[i] >= p->min_p) {
+                cutoff_sum += w[i];
+                fo_gap(margin, cutoff_sum, target);
+                if (cutoff_sum >= target) { cutoff = i + 1; break; }
+            } else { cutoff = i; break; }
+        }
+        if (cutoff == 0) { cutoff = 1; cutoff_sum = w[0]; }
+    }
+    cutoff_sum = fmaxf(cutoff_sum, eps);
+    float threshold = p->random * cutoff_sum;
+    uint32_t token = ids[0];
+    float prob = w[0] / cutoff_sum, cum = 0.f;
+    for (int i = 0; i < cutoff; i++) {
+        cum += w[i];
+        fo_gap(margin, cum, threshold);
+        if (cum >= threshold) { token = ids[i]; prob = w[i] / cutoff_sum; break; }
+    }
+    if (p->kind == 1) {
+        float surprise = log2f(fmaxf(prob, eps)) * -1.0f;
+        float error = surprise - p->tau;
+        float correction = p->eta * error;
+        *mu_state = mu - correction;
+    }
+    result[0] = 1;
+    result[1] = token;
+    return 0;
 }
 
 /* fusor/src/layers/embedding.rs:43-89: out[t,:] = dequantize(W)[id[t],:] */

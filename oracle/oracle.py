@@ -292,6 +292,34 @@ def top_k(x, k: int):
     return list(zip(ids[:n].tolist(), vals[:n].tolist()))
 
 
+class SamplerParams(C.Structure):
+    _fields_ = [("kind", C.c_uint32), ("top_k", C.c_uint32), ("temperature", C.c_float), ("repetition_penalty", C.c_float),
+                ("top_p", C.c_float), ("min_p", C.c_float), ("tau", C.c_float), ("eta", C.c_float), ("random", C.c_float)]
+
+
+def sample_token(logits, kind: int, top_k: int, temperature=1.0, repetition_penalty=1.0, top_p=1.0, min_p=0.0, tau=5.0,
+                 eta=0.1, random=0.0, previous=(), mu=None):
+    """Device sampler of fusor-ml/core/src/sampling restated: returns a dict with `token` (None when no logit is
+    finite), `ids` / `values` (processed top-k, sorted), `mu` (after the update) and `margin` (smallest relative
+    gap of a deciding comparison)."""
+    x = _f32(logits).reshape(-1)
+    prev = np.ascontiguousarray(previous, np.uint32)
+    p = SamplerParams(kind, top_k, temperature, repetition_penalty, top_p, min_p, tau, eta, random)
+    ids, vals = np.empty(top_k, np.uint32), np.empty(top_k, np.float32)
+    res = np.zeros(2, np.uint32)
+    mu_c, margin = C.c_float(0.0 if mu is None else mu), C.c_float(1.0)
+    L = lib()
+    L.fo_sample_token.argtypes = [C.POINTER(C.c_float), C.c_size_t, C.POINTER(SamplerParams), C.POINTER(C.c_uint32),
+                                  C.c_uint32, C.POINTER(C.c_float), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32),
+                                  C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    rc = L.fo_sample_token(_p(x, C.c_float), x.size, C.byref(p), _p(prev, C.c_uint32), prev.size, C.byref(mu_c),
+                           _p(res, C.c_uint32), _p(ids, C.c_uint32), _p(vals, C.c_float), C.byref(margin))
+    if rc:
+        raise ValueError(f"fo_sample_token: {rc}")
+    return {"token": int(res[1]) if res[0] == 1 else None, "status": int(res[0]), "ids": ids, "values": vals,
+            "mu": mu_c.value, "margin": margin.value}
+
+
 def argmax(x) -> int:
     x = _f32(x).reshape(-1)
     return int(lib().fo_argmax(_p(x, C.c_float), x.size))

@@ -191,3 +191,57 @@ def test_decoder_errors(dev):
         m.load_tensor("blk.0.attn_q.weight", synth.Q4_K, 16, 256, synth.random_weight(synth.Q4_K, 16, 256, 1))
     with pytest.raises(FusorHipError, match="unknown tensor"):
         m.load_tensor("blk.0.nope.weight", synth.Q4_K, 16, 256, synth.random_weight(synth.Q4_K, 16, 256, 1))
+
+
+@pytest.mark.parametrize("use_graph", [True, False], ids=["graph", "eager"])
+@pytest.mark.parametrize("kind", ["standard", "mirostat2"])
+def test_sampled_decode_matches_checker(dev, oracle, use_graph, kind):
+    """Sampled decode with the token resident on the device (models/kalosm-llama/src/model/inference.rs:38-173)
+    against the checker fed the same tokens: at every step the checker's sampler, on the checker's logits, with the
+    same window of previous ids and the same random number, must pick the id the device picked, unless its own
+    deciding comparison is closer than the logit tolerance allows (relative gap below 2e-2) or the two ids' processed
+    logits are within 1e-2 of each other."""
+    from kalosm_amd.fusor import GpuMirostat2SamplerParams, GpuStandardSamplerParams
+    cfg = HD128
+    m, ref = build_pair(dev, oracle, cfg, sigma=2e-2, fuse_qkv=True, fuse_gate_up=True, use_graph=use_graph)
+    rng = np.random.default_rng(11)
+    prompt = rng.integers(0, cfg["vocab"], 12)
+    wl = ref.forward(prompt)
+    m.forward(prompt)
+    history = prompt.tolist()
+    first = int(np.argmax(wl))
+    rounds = [(10, 24, 1.3, 16), (10, 24, 1.3, 16), (7, 40, 1.6, 5)]        # steps, top_k, penalty, window
+    mu = 6.0
+    close = 0
+    for rnd_i, (steps, k, pen, window) in enumerate(rounds):
+        randoms = rng.random(steps).astype(np.float32)
+        if kind == "standard":
+            p = GpuStandardSamplerParams(k, 0.9, pen, 0.95, 0.01, 0.0)
+        else:
+            p = GpuMirostat2SamplerParams(k, 0.9, pen, 4.0, 0.2, 0.0)
+        got, ms, mu_after = m.decode_sampled(first, steps, p, randoms, previous_tokens=history, repetition_range=window, mu=mu)
+        t, mu_ref, exact = first, mu, True
+        for i in range(steps):
+            history.append(t)
+            wl = ref.forward([t])
+            prev = history[-window:]
+            if kind == "standard":
+                want = oracle.sample_token(wl, 0, k, 0.9, pen, 0.95, 0.01, random=float(randoms[i]), previous=prev)
+            else:
+                want = oracle.sample_token(wl, 1, k, 0.9, pen, tau=4.0, eta=0.2, random=float(randoms[i]), previous=prev, mu=mu_ref)
+                mu_ref = want["mu"]
+            g = int(got[i])
+            if g != want["token"]:
+                vals = dict(zip(want["ids"].tolist(), want["values"].tolist()))
+                near = g in vals and abs(vals[g] - vals[want["token"]]) < 1e-2
+                assert want["margin"] < 2e-2 or near, (rnd_i, i, g, want["token"], want["margin"])
+                close += 1
+                exact = False
+            t = g
+        if kind == "mirostat2" and exact:
+            assert mu_after == pytest.approx(mu_ref, rel=1e-3, abs=1e-3)
+        mu = mu_after
+        first = t
+    assert close <= 3
+    # the cache the sampled steps wrote gives the checker's logits through the eager path
+    assert_close(m.forward([first]), ref.forward([first]), what="logits after the sampled steps", abs_tol=1e-2, rel_tol=1e-3)

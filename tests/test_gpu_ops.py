@@ -387,3 +387,99 @@ def test_attention_batch_key_mask(dev, oracle, dtype):
     got2 = Tensor.from_slice(dev, q, dtype).flash_attention(Tensor.from_slice(dev, k2, dtype), Tensor.from_slice(dev, v, dtype),
                                                             0.125, (Tensor.from_slice(dev, mask), MaskKind.BatchKeyMask)).as_slice()
     assert np.array_equal(got[1], got2[1])
+
+
+def test_sample_token_reference_answers(dev):
+    """The answers the reference's sampler tests store (fusor-ml/core/src/sampling/tests.rs:192-318,
+    models/kalosm-llama/src/sampler.rs:384-441), through the library."""
+    from kalosm_amd.fusor import GpuMirostat2Sampler, GpuMirostat2SamplerParams, GpuStandardSamplerParams
+    flat = Tensor.from_slice(dev, np.ones(4, np.float32))
+    s = GpuMirostat2Sampler(dev, 10.0)
+    tok, ids, vals = flat.sample_mirostat2_token(s, [], GpuMirostat2SamplerParams(4, 1.0, 1.0, 5.0, 0.1, 0.8), want_candidates=True)
+    assert tok == 0 and ids.tolist() == [3, 2, 1, 0] and vals.tolist() == [1.0] * 4
+    assert s.mu == pytest.approx(10.0 - 0.1 * (2.0 - 5.0), rel=1e-6)      # four equal candidates: surprise 2 bits
+    assert flat.sample_standard_token([], GpuStandardSamplerParams(4, 1.0, 1.0, 0.5, 0.0, 0.8)) == 2
+    t = Tensor.from_slice(dev, np.array([9.0, 8.5, 7.0, 6.0, 2.5, 0.25, -1.0, -3.0], np.float32))
+    assert t.sample_mirostat2_token(GpuMirostat2Sampler(dev, 10.0), [], GpuMirostat2SamplerParams(4, 1.0, 1.0, 5.0, 0.1, 0.0)) == 0
+    t = Tensor.from_slice(dev, np.array([-5.0, -4.0, -3.0, 0.0], np.float32))
+    for rnd in (0.0, 0.5, 0.999):
+        assert t.sample_standard_token([], GpuStandardSamplerParams(4, 1.0, 1.0, 1.0, 0.1, rnd)) == 3
+    t = Tensor.from_slice(dev, np.array([9.0, 7.5, 7.0, 4.0, 3.5, 1.0], np.float32))
+    assert t.sample_mirostat2_token(GpuMirostat2Sampler(dev, 3.0), [], GpuMirostat2SamplerParams(5, 1.0, 1.0, 5.0, 0.1, 0.65)) == 0
+    # processors: temperature 0.5, penalty 2, previous {0, 3, 9} (tests.rs:61-136)
+    values = np.array([4.0, -2.0, 3.5, 8.0, np.nan, 1.0, 5.0, -1.5, 6.5, 7.0, -np.inf, 0.5], np.float32)
+    _, ids, vals = Tensor.from_slice(dev, values).sample_standard_token(
+        [0, 3, 9], GpuStandardSamplerParams(5, 0.5, 2.0, 1.0, 0.0, 0.0), want_candidates=True)
+    assert ids.tolist() == [8, 6, 3, 9, 2] and vals.tolist() == [13.0, 10.0, 8.0, 7.0, 7.0]
+    none = Tensor.from_slice(dev, np.array([np.nan, np.inf, -np.inf], np.float32))
+    assert none.sample_standard_token([], GpuStandardSamplerParams(2, 1.0, 1.0, 1.0, 0.0, 0.5)) is None
+    with pytest.raises(Exception):
+        flat.sample_standard_token([], GpuStandardSamplerParams(257, 1.0, 1.0, 1.0, 0.0, 0.5))
+    with pytest.raises(Exception):
+        flat.sample_standard_token([], GpuStandardSamplerParams(0, 1.0, 1.0, 1.0, 0.0, 0.5))
+
+
+@pytest.mark.parametrize("n", [12, 1000, 5000, 128256])
+def test_sample_token_matches_checker(dev, oracle, n):
+    """Both device samplers against the checker on random logits: the processed top-k candidates are bit-equal; the
+    sampled id is equal wherever the checker's deciding comparisons have a relative gap above 1e-4 (exp and log2
+    come from different libraries on the two sides); the Mirostat state follows to 1e-5.  Values are compared as
+    numbers: the candidates' values are rebuilt from the sort keys, which hold -0.0 as 0.0."""
+    from kalosm_amd.fusor import GpuMirostat2Sampler, GpuMirostat2SamplerParams, GpuStandardSamplerParams
+    rng = np.random.default_rng(n)
+    compared = 0
+    for case in range(40):
+        x = (rng.standard_normal(n) * rng.choice([0.5, 2.0, 6.0])).astype(np.float32)
+        if case % 5 == 0:
+            x[rng.integers(0, n, max(1, n // 20))] = [np.nan, np.inf, -np.inf][case % 3]
+        if case % 7 == 0:
+            x = np.round(x)                                            # ties
+        k = int(rng.choice([1, 2, 7, 40, 64, 256]))
+        temp = float(rng.choice([0.0, 0.7, 1.0, 1.3]))
+        pen = float(rng.choice([1.0, 1.1, 1.5, 0.5]))
+        n_prev = int(rng.choice([0, 1, 30, 64, 100]))
+        prev = rng.integers(0, n, n_prev)
+        if n_prev:
+            prev[: min(n_prev, 8)] = np.argsort(-np.nan_to_num(x, nan=-1e30, posinf=-1e30))[: min(n_prev, 8)]  # hit candidates
+            rng.shuffle(prev)
+        rnd = float(rng.random()) if case % 9 else 0.0
+        t = Tensor.from_slice(dev, x)
+        used = prev[-64:]
+        if case % 2 == 0:
+            top_p, min_p = float(rng.choice([1.0, 0.9, 0.5, 0.1])), float(rng.choice([0.0, 0.05, 0.3]))
+            got, ids, vals = t.sample_standard_token(prev, GpuStandardSamplerParams(k, temp, pen, top_p, min_p, rnd), want_candidates=True)
+            want = oracle.sample_token(x, 0, k, temp, pen, top_p, min_p, random=rnd, previous=used)
+        else:
+            mu0, tau, eta = float(rng.choice([1.0, 3.0, 10.0])), float(rng.choice([3.0, 5.0])), float(rng.choice([0.1, 0.3]))
+            s = GpuMirostat2Sampler(dev, mu0)
+            got, ids, vals = t.sample_mirostat2_token(s, prev, GpuMirostat2SamplerParams(k, temp, pen, tau, eta, rnd), want_candidates=True)
+            want = oracle.sample_token(x, 1, k, temp, pen, tau=tau, eta=eta, random=rnd, previous=used, mu=mu0)
+        what = (n, case, k, temp, pen, n_prev, rnd)
+        assert ids.tolist() == want["ids"].tolist(), what
+        live = want["ids"] != 0xFFFFFFFF
+        assert np.array_equal(vals[live], want["values"][live]), what        # a processed -0.0 comes back as 0.0
+        if want["margin"] > 1e-4:
+            compared += 1
+            assert got == want["token"], what
+            if case % 2 and want["token"] is not None:
+                assert s.mu == pytest.approx(want["mu"], rel=1e-5, abs=1e-5), what
+    assert compared >= 30
+
+
+def test_sample_token_previous_gpu_token(dev, oracle):
+    """The id another kernel left in device memory joins the previous tokens as their last entry
+    (fixed_previous_tokens_data_with_gpu_tail, fusor-ml/core/src/sampling/processors.rs:45-81): 63 host ids + 1."""
+    from kalosm_amd.fusor import GpuStandardSamplerParams
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal(500).astype(np.float32) * 3
+    order = np.argsort(-x)
+    tail = Tensor.from_slice(dev, np.array([order[0]], np.uint32), "u32")
+    host = np.concatenate([[order[1]], rng.integers(400, 500, 70), [order[2]]]).astype(np.uint32)   # order[1] falls out of the 63
+    p = GpuStandardSamplerParams(16, 1.0, 1.8, 1.0, 0.0, 0.4)
+    got, ids, vals = Tensor.from_slice(dev, x).sample_standard_token(host, p, previous_gpu_token=tail, want_candidates=True)
+    want = oracle.sample_token(x, 0, 16, 1.0, 1.8, random=0.4, previous=np.concatenate([host[-63:], [order[0]]]))
+    assert ids.tolist() == want["ids"].tolist() and np.array_equal(vals, want["values"])
+    assert got == want["token"]
+    seen = dict(zip(ids.tolist(), vals.tolist()))
+    assert seen[int(order[1])] == x[order[1]]                       # outside the window: not penalised
+    assert seen.get(int(order[0]), None) != x[order[0]]             # the device-side id is penalised
