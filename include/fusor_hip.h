@@ -375,6 +375,10 @@ fh_status fh_llama_destroy(fh_llama *m);
 fh_status fh_llama_load_tensor(fh_llama *m, const char *name, uint32_t ggml_type, int64_t n,
                                int64_t k, const void *bytes, size_t len);
 /* Fuse/concatenate what the config asks for and allocate the step buffers; call once after loading. */
+/* The `rope_scaling` argument of Model::from_gguf (models/kalosm-llama/src/raw/mod.rs:264-285, kept in the
+ * LlamaConfig, :120): long-context scaling of the RoPE inverse frequencies (raw/rope.rs:20-38), applied when
+ * fh_llama_finalize builds the tables, before the rope_freqs.weight factors.  NULL: none.  Call before finalize. */
+fh_status fh_llama_set_rope_scaling(fh_llama *m, const fh_rope_scaling *scaling);
 fh_status fh_llama_finalize(fh_llama *m);
 fh_status fh_llama_reset(fh_llama *m);
 /* Run `count` new tokens at the current position; logits_host (optional, [vocab]) and

@@ -202,6 +202,7 @@ extern "C" {
     pub fn fh_llama_create(dev: *mut FhDevice, cfg: *const FhLlamaConfig, out: *mut *mut FhLlama) -> FhStatus;
     pub fn fh_llama_destroy(m: *mut FhLlama) -> FhStatus;
     pub fn fh_llama_load_tensor(m: *mut FhLlama, name: *const c_char, ggml_type: u32, n: i64, k: i64, bytes: *const c_void, len: usize) -> FhStatus;
+    pub fn fh_llama_set_rope_scaling(m: *mut FhLlama, scaling: *const FhRopeScaling) -> FhStatus;
     pub fn fh_llama_finalize(m: *mut FhLlama) -> FhStatus;
     pub fn fh_llama_reset(m: *mut FhLlama) -> FhStatus;
     pub fn fh_llama_forward(m: *mut FhLlama, tokens_host: *const u32, count: i32, logits_host: *mut f32, hidden_host: *mut f32) -> FhStatus;

@@ -108,6 +108,7 @@ SIGNATURES = {
     "fh_llama_create": [_p, C.POINTER(LlamaConfig), _pp],
     "fh_llama_destroy": [_p],
     "fh_llama_load_tensor": [_p, C.c_char_p, _u32, _i64, _i64, _p, _sz],
+    "fh_llama_set_rope_scaling": [_p, C.POINTER(RopeScaling)],
     "fh_llama_finalize": [_p],
     "fh_llama_reset": [_p],
     "fh_llama_forward": [_p, _p, _i32, _p, _p],

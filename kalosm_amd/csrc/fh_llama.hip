@@ -26,6 +26,8 @@ struct fh_llama {
     float *out_norm = nullptr;
     float *cos_t = nullptr, *sin_t = nullptr;
     std::vector<float> rope_freq_weight; // rope_freqs.weight when the file has one
+    bool has_rope_scaling = false;
+    fh_rope_scaling rope_scaling = {};
     fh_kvcache *cache = nullptr;
     bool finalized = false;
     int pos = 0;
@@ -67,6 +69,18 @@ extern "C" fh_status fh_llama_create(fh_device *dev, const fh_llama_config *cfg,
     m->c = *cfg;
     m->layers.resize(cfg->n_layers);
     *out = m;
+    return FH_OK;
+}
+
+extern "C" fh_status fh_llama_set_rope_scaling(fh_llama *m, const fh_rope_scaling *scaling) {
+    FH_REQUIRE(m, "NULL decoder");
+    FH_REQUIRE(!m->finalized, "the RoPE tables are built by fh_llama_finalize: set the scaling before it");
+    if (scaling) {
+        FH_REQUIRE(scaling->factor != 0.0f && scaling->low_freq_factor != 0.0f && scaling->high_freq_factor != 0.0f,
+                   "rope scaling factors must not be zero");
+        m->rope_scaling = *scaling;
+    }
+    m->has_rope_scaling = scaling != nullptr;
     return FH_OK;
 }
 
@@ -214,8 +228,8 @@ extern "C" fh_status fh_llama_finalize(fh_llama *m) {
     size_t tbl = (size_t)c.ctx * (c.head_dim / 2) * 4;
     FH_TRY(fh_malloc(m->dev, tbl, (void **)&m->cos_t));
     FH_TRY(fh_malloc(m->dev, tbl, (void **)&m->sin_t));
-    FH_TRY(fh_rope_tables_weighted(m->dev, c.head_dim, c.ctx, c.theta,
-                                   m->rope_freq_weight.empty() ? nullptr : m->rope_freq_weight.data(), m->cos_t, m->sin_t));
+    FH_TRY(fh_rope_tables_scaled(m->dev, c.head_dim, c.ctx, c.theta, m->has_rope_scaling ? &m->rope_scaling : nullptr,
+                                 m->rope_freq_weight.empty() ? nullptr : m->rope_freq_weight.data(), m->cos_t, m->sin_t));
     FH_TRY(fh_kvcache_create(m->dev, c.n_layers, c.n_kv_heads, c.head_dim, c.ctx, c.kv_dtype, &m->cache));
     FH_TRY(fh_malloc(m->dev, (size_t)c.vocab * 4, (void **)&m->logits));
     FH_TRY(fh_malloc(m->dev, 256, (void **)&m->tok_dev));

@@ -51,10 +51,11 @@ class Model:
 
     @staticmethod
     def from_gguf(device: Device, source, ctx: Optional[int] = None, kv_dtype: str = "f32", fuse_qkv: bool = True,
-                  fuse_gate_up: bool = True, use_graph: bool = True) -> "Model":
+                  fuse_gate_up: bool = True, use_graph: bool = True, rope_scaling=None) -> "Model":
         """Model::from_gguf for the Llama architecture (raw/mod.rs:284-648): parameters from the metadata, every
         decoder tensor from the file.  `source` is a path or an open `GgufMetadata`; `ctx` caps the context
-        length (and with it the KV cache) below the file's `context_length`."""
+        length (and with it the KV cache) below the file's `context_length`; `rope_scaling` is the reference's
+        argument of that name: (factor, high_freq_factor, low_freq_factor, original_max_position_embeddings)."""
         from .gguf import GgufMetadata
         g = source if isinstance(source, GgufMetadata) else GgufMetadata.read(source)
         c = LlamaConfig()
@@ -65,8 +66,16 @@ class Model:
             cfg["ctx"] = min(cfg["ctx"], int(ctx))
         m = Model(device, cfg, kv_dtype=kv_dtype, fuse_qkv=fuse_qkv, fuse_gate_up=fuse_gate_up, use_graph=use_graph)
         check(device._lib.fh_llama_load_gguf(m._h, g._h))
+        if rope_scaling is not None:
+            m.set_rope_scaling(*rope_scaling)
         m.finalize()
         return m
+
+    def set_rope_scaling(self, factor: float, high_freq_factor: float, low_freq_factor: float,
+                         original_max_position_embeddings: int) -> None:
+        """RopeScalingConfig (raw/mod.rs:163-169); before `finalize`."""
+        sc = _lib.RopeScaling(factor, high_freq_factor, low_freq_factor, original_max_position_embeddings)
+        check(self.device._lib.fh_llama_set_rope_scaling(self._h, C.byref(sc)))
 
     def finalize(self) -> None:
         check(self.device._lib.fh_llama_finalize(self._h))

@@ -995,6 +995,10 @@ void fo_llama_set_layer_types(fo_llama *m, int l, const int *types) {
 void fo_llama_set_rope_freq_weight(fo_llama *m, const float *w) {
     fo_rope_tables_weighted(m->c.head_dim, m->c.ctx, m->c.theta, w, m->cosv, m->sinv);
 }
+/* scaling = {factor, high_freq_factor, low_freq_factor, original_max_position_embeddings} or NULL; w or NULL */
+void fo_llama_set_rope(fo_llama *m, const float *scaling, const float *w) {
+    fo_rope_tables_scaled(m->c.head_dim, m->c.ctx, m->c.theta, scaling, w, m->cosv, m->sinv);
+}
 void fo_llama_set_globals(fo_llama *m, const uint8_t *embd, const float *out_norm, const uint8_t *output) {
     m->embd = embd; m->out_norm = out_norm; m->output = output;
 }

@@ -375,6 +375,13 @@ class Llama:
                 lib().fo_llama_set_layer_types(self._h, l, arr)
         if "rope_freqs.weight" in weights:
             lib().fo_llama_set_rope_freq_weight(self._h, f32("rope_freqs.weight"))
+        if cfg.get("rope_scaling") is not None:     # (factor, high_freq_factor, low_freq_factor, original_max_position)
+            sc = np.asarray(cfg["rope_scaling"], np.float32)
+            self._keep.append(sc)
+            L = lib()
+            L.fo_llama_set_rope.argtypes = [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+            L.fo_llama_set_rope(self._h, _p(sc, C.c_float),
+                                f32("rope_freqs.weight") if "rope_freqs.weight" in weights else None)
 
     def reset(self):
         lib().fo_llama_reset(self._h)

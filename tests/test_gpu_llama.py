@@ -245,3 +245,48 @@ def test_sampled_decode_matches_checker(dev, oracle, use_graph, kind):
     assert close <= 3
     # the cache the sampled steps wrote gives the checker's logits through the eager path
     assert_close(m.forward([first]), ref.forward([first]), what="logits after the sampled steps", abs_tol=1e-2, rel_tol=1e-3)
+
+
+@pytest.mark.parametrize("rope_freqs", [True, False], ids=["with-rope_freqs", "plain"])
+def test_decoder_with_rope_scaling(dev, oracle, tmp_path, rope_freqs):
+    """The `rope_scaling` argument of Model::from_gguf (models/kalosm-llama/src/raw/mod.rs:264-285): the decoder's
+    RoPE tables use the scaled inverse frequencies (raw/rope.rs:20-38), then the rope_freqs.weight factors.  With
+    original_max_position_embeddings 32 and low_freq_factor 1 every frequency whose wavelength exceeds 32
+    positions is divided by 8, so the logits differ from the unscaled decoder's from position 1 on."""
+    from test_gguf_reader import TINY, llama_file
+    from oracle import gguf_ref
+    scaling = (8.0, 4.0, 1.0, 32)
+    data, weights, types = llama_file(TINY, seed=7, rope_freqs=rope_freqs)
+    m = Model.from_gguf(dev, _bytes_source(data, tmp_path), ctx=80, rope_scaling=scaling)
+    plain = Model.from_gguf(dev, _bytes_source(data, tmp_path), ctx=80)
+    r = gguf_ref.GgufRef(data)
+    rw = {}
+    for name, (ty, shape, off) in r.tensors.items():
+        raw = r.tensor_bytes(name)
+        if len(shape) == 1:
+            raw = raw.view(np.float32) if ty == 0 else raw.view(np.float16).astype(np.float32)
+        rw[name.decode()] = raw
+    ocfg = dict(m.cfg, type_attn=synth.Q4_K, type_ffn_gate_up=synth.Q4_K, type_ffn_down=synth.Q6_K,
+                type_embd=types["token_embd.weight"], type_output=types["output.weight"],
+                tensor_types={n.decode(): t for n, (t, _, _) in r.tensors.items()}, rope_scaling=scaling)
+    ref = oracle.Llama(ocfg, rw)
+    prompt = np.random.default_rng(4).integers(0, TINY["vocab"], 40)
+    lg = m.forward(prompt)
+    wl = ref.forward(prompt)
+    assert_close(lg, wl, what="prefill logits with scaled RoPE")
+    assert np.abs(plain.forward(prompt) - wl).max() > 50 * np.abs(lg - wl).max()    # the scaling is not a no-op
+    tok = oracle.argmax(wl)
+    got, _ = m.decode_greedy(tok, 12)
+    want, t = [], tok
+    for _ in range(12):
+        t = oracle.argmax(ref.forward([t]))
+        want.append(t)
+    assert got.tolist() == want
+    with pytest.raises(Exception):
+        m.set_rope_scaling(*scaling)            # the tables are built: too late
+
+
+def _bytes_source(data, tmp_path):
+    p = tmp_path / f"m{len(list(tmp_path.iterdir()))}.gguf"
+    p.write_bytes(data)
+    return str(p)
