@@ -396,8 +396,8 @@ extern "C" fh_status fh_argmax(fh_device *dev, const float *x_dev, int64_t count
 // ------------------------------------------------------------------------------ top-k
 // Tensor::top_k_pairs(k), fusor-ml/fusor/src/lib.rs:416-447: the k largest FINITE logits in descending order, ties
 // to the larger token id.  (value, id) becomes one 64-bit key whose unsigned order is that order (-0.0 ranks with
-// +0.0, as the reference's float compare does); every workgroup sorts 1024 keys in LDS (bitonic, descending) and
-// keeps its first k; passes repeat over the survivors until one workgroup is left.
+// +0.0, as the reference's float compare does); every workgroup sorts 1024 keys (bitonic, descending, two keys per
+// thread) and keeps its first k; passes repeat over the survivors until one workgroup is left.
 __device__ __forceinline__ uint64_t topk_key(float v, uint32_t id) {
     uint32_t b = __float_as_uint(v);
     if ((b & 0x7F800000u) == 0x7F800000u) return 0; // infinities and NaNs are skipped
@@ -508,7 +508,7 @@ __global__ __launch_bounds__(512) void k_topk_pass(const float *__restrict__ x, 
                                                    int64_t n_in, int k, int last, uint64_t *__restrict__ keys_out,
                                                    uint32_t *__restrict__ ids_out, float *__restrict__ vals_out,
                                                    uint32_t *__restrict__ found_out, TopkProc proc, TopkSample samp) {
-    __shared__ uint64_t s[1024];
+    __shared__ uint64_t s[2048];
     __shared__ uint32_t s_prev[64];
     __shared__ float s_w[256];
     const int tid = threadIdx.x;
@@ -520,8 +520,13 @@ __global__ __launch_bounds__(512) void k_topk_pass(const float *__restrict__ x, 
         if (tid < 64) s_prev[tid] = (uint32_t)tid < n_prev ? proc.prev[tid] : 0u;
         __syncthreads();
     }
-    for (int i = tid; i < 1024; i += 512) {
-        const int64_t idx = base + i;
+    // Thread t holds the keys at positions 2t and 2t + 1 of the bitonic network (which input lands where does not
+    // matter): partners at distance 1 are in its own registers, up to distance 64 in its wavefront (lane exchange),
+    // beyond that in another wavefront (through LDS, two buffers in turn so that one barrier per stage is enough).
+    uint64_t kk[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const int64_t idx = base + tid + 512 * h;
         uint64_t key = 0ull;
         if (idx < n_in) {
             if (FIRST) {
@@ -537,20 +542,45 @@ __global__ __launch_bounds__(512) void k_topk_pass(const float *__restrict__ x, 
                 key = keys_in[idx];
             }
         }
-        s[i] = key;
+        kk[h] = key;
+    }
+    int flip = 0;
+#pragma unroll
+    for (int size = 2; size <= 1024; size <<= 1) {
+        const bool down = ((2 * tid) & size) == 0; // this run is sorted descending
+#pragma unroll
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            if (stride == 1) {
+                if ((kk[0] < kk[1]) == down) {
+                    const uint64_t t = kk[0];
+                    kk[0] = kk[1];
+                    kk[1] = t;
+                }
+                continue;
+            }
+            const int m = stride >> 1; // distance in threads
+            uint64_t o[2];
+            if (stride <= 64) {
+                o[0] = __shfl_xor(kk[0], m);
+                o[1] = __shfl_xor(kk[1], m);
+            } else {
+                uint64_t *buf = s + 1024 * flip;
+                flip ^= 1;
+                buf[2 * tid] = kk[0];
+                buf[2 * tid + 1] = kk[1];
+                __syncthreads();
+                o[0] = buf[2 * (tid ^ m)];
+                o[1] = buf[2 * (tid ^ m) + 1];
+            }
+            const bool keep_max = ((tid & m) == 0) == down;
+#pragma unroll
+            for (int h = 0; h < 2; h++) kk[h] = keep_max ? (kk[h] > o[h] ? kk[h] : o[h]) : (kk[h] < o[h] ? kk[h] : o[h]);
+        }
     }
     __syncthreads();
-    for (int size = 2; size <= 1024; size <<= 1)
-        for (int stride = size >> 1; stride > 0; stride >>= 1) {
-            const int a = 2 * tid - (tid & (stride - 1)), b = a + stride;
-            const uint64_t va = s[a], vb = s[b];
-            const bool down = (a & size) == 0; // this run is sorted descending
-            if ((va < vb) == down) {
-                s[a] = vb;
-                s[b] = va;
-            }
-            __syncthreads();
-        }
+    s[2 * tid] = kk[0];
+    s[2 * tid + 1] = kk[1];
+    __syncthreads();
     if (!last) {
         for (int i = tid; i < k; i += 512) keys_out[(int64_t)blockIdx.x * k + i] = s[i];
         return;
