@@ -553,9 +553,11 @@ extern "C" fh_status fh_llama_decode_sampled(fh_llama *m, uint32_t first_token, 
     int done = 0;
     if (m->c.use_graph) {
         // the captured step holds the sampler's parameters and the window size as kernel arguments
+        fh_sampler_params want = *params;
+        want.random = 0.f; // every step takes its number from randoms_host
         const bool same = m->samp_exec && m->samp_capacity == m->cache->capacity && m->samp_range == range &&
-                          memcmp(&m->samp_params, params, sizeof(*params)) == 0;
-        m->samp_params = *params;
+                          memcmp(&m->samp_params, &want, sizeof(want)) == 0;
+        m->samp_params = want;
         m->samp_range = range;
         if (!same) {
             FH_TRY(fh_timer_start(dev));
