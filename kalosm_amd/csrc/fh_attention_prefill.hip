@@ -200,22 +200,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 }
             }
         }
-        // ---- mask, running max: register r of half kt is key t0 + 32 kt + 16 (r / 8) + 8 g + r % 8
+        // ---- mask, running max: register r of half kt is key t0 + 32 kt + 16 (r / 8) + 8 g + r % 8.  Only a tile
+        // that reaches past some query's last visible key needs the compare (one branch for the wavefront).
         const int lim = causal ? (qi + off < skv - 1 ? qi + off : skv - 1) : skv - 1; // last visible key
         float mx = -INFINITY;
+        if (__any(t0 + BN - 1 > lim)) {
 #pragma unroll
-        for (int kt = 0; kt < 2; kt++)
+            for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int key = t0 + 32 * kt + 16 * (r >> 3) + 8 * g + (r & 7);
-                const float s = key <= lim ? st[kt][r] * sc2 : -INFINITY;
-                st[kt][r] = s;
-                mx = fmaxf(mx, s);
-            }
-        mx = ap_swap32_max(mx);
+                for (int r = 0; r < 16; r++) {
+                    const int key = t0 + 32 * kt + 16 * (r >> 3) + 8 * g + (r & 7);
+                    const float sv = key <= lim ? st[kt][r] : -INFINITY;
+                    st[kt][r] = sv;
+                    mx = fmaxf(mx, sv);
+                }
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[kt][r]);
+        }
+        // the scale (> 0) is applied inside the exponent: p = 2^(s * sc2 - m), one multiply-add per score
+        mx = ap_swap32_max(mx) * sc2;
         const float m_new = fmaxf(m_run, mx);
         const bool dead = m_new == -INFINITY; // nothing visible yet (only queries past the end)
-        const float alpha = dead ? 1.f : exp2f(m_run - m_new);
+        const float alpha = dead ? 1.f : __builtin_amdgcn_exp2f(m_run - m_new);
+        const float m_sub = dead ? 0.f : -m_new; // dead rows: 2^(-inf - 0) = 0
         float ps = 0.f;
         half8 pb[2][2], pl[SPLIT ? 2 : 1][2];
 #pragma unroll
@@ -225,7 +235,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 fh_half t[8], tl[8];
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    const float p = dead ? 0.f : exp2f(st[kt][8 * s2 + e] - m_new);
+                    const float p = __builtin_amdgcn_exp2f(fmaf(st[kt][8 * s2 + e], sc2, m_sub)); // arguments <= 0
                     ps += p;
                     t[e] = (fh_half)p;
                     if constexpr (SPLIT) tl[e] = (fh_half)(p - (float)t[e]);
@@ -235,11 +245,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
         l_run = l_run * alpha + ap_swap32_sum(ps);
         m_run = m_new;
-        // ---- O^T = O^T * alpha + V^T . P^T
+        // ---- O^T = O^T * alpha + V^T . P^T (once the maxima have settled no lane of the wavefront rescales)
+        const bool rescale = __any(alpha != 1.f);
 #pragma unroll
         for (int dt = 0; dt < DT; dt++) {
+            if (rescale) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[dt][r] *= alpha;
+                for (int r = 0; r < 16; r++) acc[dt][r] *= alpha;
+            }
             const fh_half *vp = sV + (dt * 32 + li) * VS + 8 * g;
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
