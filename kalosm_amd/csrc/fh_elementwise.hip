@@ -341,9 +341,11 @@ __device__ __forceinline__ void amax_merge(float &v, uint32_t &id, float ov, uin
 }
 // Stage 1 (pv != NULL): workgroup b scans its slice of x and writes its best (value, id) to pv/pi[b].
 // Stage 2 (pv == NULL in the launch of one workgroup): x is the partial values, xi their ids.
+// The last stage can also finish a decode step (tail.ids != NULL): the id becomes the next step's input (0 when
+// no logit was finite), is appended to the step's output list, and the KV cache's device-side length goes up by one.
 __global__ __launch_bounds__(1024) void k_argmax(const float *__restrict__ x, const uint32_t *__restrict__ xi, int64_t n,
                                                   uint32_t *__restrict__ out, float *__restrict__ pv,
-                                                  uint32_t *__restrict__ pi) {
+                                                  uint32_t *__restrict__ pi, FhStepTail tail) {
     __shared__ float sv[16];
     __shared__ uint32_t si[16];
     float v = 0.f;
@@ -374,20 +376,29 @@ __global__ __launch_bounds__(1024) void k_argmax(const float *__restrict__ x, co
             pi[blockIdx.x] = id;
         } else {
             *out = id;
+            if (tail.ids) {
+                tail.ids[0] = id == 0xFFFFFFFFu ? 0u : id;
+                tail.out_tokens[*tail.step] = id;
+                *tail.step = *tail.step + 1;
+                *tail.kv_len = *tail.kv_len + 1;
+            }
         }
     }
 }
 extern "C" fh_status fh_argmax(fh_device *dev, const float *x_dev, int64_t count, uint32_t *id_dev) {
+    return fh_argmax_step(dev, x_dev, count, id_dev, FhStepTail{});
+}
+fh_status fh_argmax_step(fh_device *dev, const float *x_dev, int64_t count, uint32_t *id_dev, FhStepTail tail) {
     FH_REQUIRE(dev && x_dev && id_dev, "NULL argument");
     FH_REQUIRE(count > 0 && count < 0xFFFFFFFFll, "count %lld out of range", (long long)count);
     if (count <= 8192) {
-        k_argmax<<<dim3(1), dim3(1024), 0, dev->stream>>>(x_dev, nullptr, count, id_dev, nullptr, nullptr);
+        k_argmax<<<dim3(1), dim3(1024), 0, dev->stream>>>(x_dev, nullptr, count, id_dev, nullptr, nullptr, tail);
     } else {
         const int parts = 128;
         float *pv = (float *)dev->small_buf;
         uint32_t *pi = (uint32_t *)(pv + parts);
-        k_argmax<<<dim3(parts), dim3(256), 0, dev->stream>>>(x_dev, nullptr, count, nullptr, pv, pi);
-        k_argmax<<<dim3(1), dim3(128), 0, dev->stream>>>(pv, pi, parts, id_dev, nullptr, nullptr);
+        k_argmax<<<dim3(parts), dim3(256), 0, dev->stream>>>(x_dev, nullptr, count, nullptr, pv, pi, FhStepTail{});
+        k_argmax<<<dim3(1), dim3(128), 0, dev->stream>>>(pv, pi, parts, id_dev, nullptr, nullptr, tail);
     }
     FH_HIP(hipGetLastError());
     return FH_OK;
@@ -725,7 +736,6 @@ extern "C" fh_status fh_kvcache_destroy(fh_kvcache *c) {
 }
 
 __global__ void k_set_int(int *p, int v) { *p = v; }
-__global__ void k_inc_int(int *p) { *p = *p + 1; }
 
 extern "C" fh_status fh_kvcache_reset(fh_kvcache *c) {
     FH_REQUIRE(c, "NULL argument");
@@ -937,13 +947,6 @@ fh_status fh_rope_kv_decode(fh_kvcache *c, int layer, const float *q, const floa
         k_rope_kv_decode<fh_half><<<grid, 256, 0, s>>>(q, k, v, hq, hk, d, cos_t, sin_t, table_rows, c->len_dev, q_out,
                                                        (fh_half *)c->k + layer * plane, (fh_half *)c->v + layer * plane,
                                                        c->capacity);
-    FH_HIP(hipGetLastError());
-    return FH_OK;
-}
-
-// End of a graph-replayed decode step: advance the device-side length.
-fh_status fh_kvcache_advance_dev(fh_kvcache *c) {
-    k_inc_int<<<1, 1, 0, c->dev->stream>>>(c->len_dev);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }

@@ -194,7 +194,6 @@ size_t fh_dtype_size(int dtype);
 fh_status fh_kvcache_reserve(fh_kvcache *c, int required);
 // append reading the write position from c->len_dev (graph friendly), s == 1
 fh_status fh_kvcache_append_devpos(fh_kvcache *c, int layer, const float *k, const float *v, int64_t sh);
-fh_status fh_kvcache_advance_dev(fh_kvcache *c);
 fh_status fh_launch_q4k_m1_ropekv(const fh_qmatrix *q, const float *x, const float *nw, float eps, fh_kvcache *c,
                                   int layer, int hq, const float *cos_t, const float *sin_t, int table_rows,
                                   float *q_out);
@@ -214,6 +213,14 @@ fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *
 fh_status fh_rope_pair_devpos(fh_device *dev, const float *q, const float *k, int hq, int hk, int d,
                               const float *cos_t, const float *sin_t, int table_rows,
                               const int *pos_dev, float *q_out, float *k_out);
+// End of a device-side decode step, done by the last stage of the greedy pick (all pointers device memory).
+struct FhStepTail {
+    uint32_t *ids = nullptr;        // next step's input id
+    uint32_t *out_tokens = nullptr; // the step's output list
+    int *step = nullptr;            // its fill count
+    int *kv_len = nullptr;          // KV cache length
+};
+fh_status fh_argmax_step(fh_device *dev, const float *x_dev, int64_t count, uint32_t *id_dev, FhStepTail tail);
 // Sampler with every per-step input in device memory (fh_elementwise.hip); fh_sample_token is its host-input form.
 fh_status fh_sample_token_dev(fh_device *dev, const float *logits_dev, int64_t count, const fh_sampler_params *p,
                               const uint32_t *prev_dev, const uint32_t *prev_len_dev, uint32_t n_prev,

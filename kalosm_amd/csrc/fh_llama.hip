@@ -426,21 +426,13 @@ extern "C" fh_status fh_llama_forward(fh_llama *m, const uint32_t *tokens_host, 
     return FH_OK;
 }
 
-__global__ void k_store_token(const uint32_t *tok, uint32_t *ids, uint32_t *out, int *step) {
-    uint32_t t = *tok;
-    ids[0] = t == 0xFFFFFFFFu ? 0u : t; // next step's input (a non-finite logits row yields id 0)
-    out[*step] = t;
-    *step = *step + 1;
-}
 __global__ void k_set_u32(uint32_t *p, uint32_t v) { *p = v; }
 
 static fh_status decode_step_enqueue(fh_llama *m) {
     FH_TRY(run_layers(m, 1, true));
-    FH_TRY(fh_kvcache_advance_dev(m->cache));
-    FH_TRY(fh_argmax(m->dev, m->logits, m->c.vocab, m->tok_dev));
-    k_store_token<<<1, 1, 0, m->dev->stream>>>(m->tok_dev, m->ids, m->out_tok_dev, m->step_dev);
-    FH_HIP(hipGetLastError());
-    return FH_OK;
+    // the last stage of the pick also stores the token, feeds it to the next step and advances the cache length
+    return fh_argmax_step(m->dev, m->logits, m->c.vocab, m->tok_dev,
+                          FhStepTail{m->ids, m->out_tok_dev, m->step_dev, m->cache->len_dev});
 }
 
 extern "C" fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, int32_t steps, uint32_t *out_tokens_host,
@@ -495,7 +487,8 @@ extern "C" fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, i
 // device memory and feeds the next step; it also joins the window of previous ids that the repetition penalty
 // looks at (membership only, so the window is a ring).
 __global__ void k_store_sampled(const uint32_t *result, uint32_t *ids, uint32_t *out, int *step, uint32_t *prev,
-                                uint32_t range) {
+                                uint32_t range, int *kv_len) {
+    *kv_len = *kv_len + 1;
     const uint32_t t = result[0] == FH_SAMPLE_STATUS_SAMPLED ? result[1] : 0xFFFFFFFFu;
     const uint32_t next = t == 0xFFFFFFFFu ? 0u : t;
     ids[0] = next;
@@ -511,11 +504,11 @@ __global__ void k_store_sampled(const uint32_t *result, uint32_t *ids, uint32_t 
 
 static fh_status sampled_step_enqueue(fh_llama *m) {
     FH_TRY(run_layers(m, 1, true));
-    FH_TRY(fh_kvcache_advance_dev(m->cache));
     uint32_t *sd = m->samp_dev;
     FH_TRY(fh_sample_token_dev(m->dev, m->logits, m->c.vocab, &m->samp_params, sd, sd + 64, 0, (const float *)(sd + 128),
                                m->step_dev, (float *)(sd + 66), sd + 68, nullptr, nullptr));
-    k_store_sampled<<<1, 1, 0, m->dev->stream>>>(sd + 68, m->ids, m->out_tok_dev, m->step_dev, sd, m->samp_range);
+    k_store_sampled<<<1, 1, 0, m->dev->stream>>>(sd + 68, m->ids, m->out_tok_dev, m->step_dev, sd, m->samp_range,
+                                                m->cache->len_dev);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
