@@ -402,8 +402,9 @@ impl Drop for HipLlama {
     }
 }
 impl HipLlama {
-    /// `Model::from_gguf` (raw/mod.rs:284-648) for architecture `llama`; `max_context` caps the KV cache.
-    pub fn from_gguf(dev: &HipDevice, file: &HipGguf, max_context: Option<usize>) -> Result<Self> {
+    /// `Model::from_gguf` (raw/mod.rs:284-648) for architecture `llama`; `max_context` caps the KV cache,
+    /// `rope_scaling` is the reference's argument of that name (raw/mod.rs:271).
+    pub fn from_gguf(dev: &HipDevice, file: &HipGguf, max_context: Option<usize>, rope_scaling: Option<sys::FhRopeScaling>) -> Result<Self> {
         let mut config = sys::FhLlamaConfig::default();
         check(unsafe { sys::fh_llama_config_from_gguf(file.raw, &mut config) })?;
         if let Some(c) = max_context {
@@ -419,6 +420,9 @@ impl HipLlama {
         {
             let _g = dev.lock();
             check(unsafe { sys::fh_llama_load_gguf(model.raw, file.raw) })?;
+            if let Some(scaling) = rope_scaling.as_ref() {
+                check(unsafe { sys::fh_llama_set_rope_scaling(model.raw, scaling) })?;
+            }
             check(unsafe { sys::fh_llama_finalize(model.raw) })?;
         }
         Ok(model)
@@ -435,6 +439,31 @@ impl HipLlama {
         let mut out = vec![0u32; steps];
         let _g = self.dev.lock();
         check(unsafe { sys::fh_llama_decode_greedy(self.raw, first_token, steps as i32, out.as_mut_ptr(), ptr::null_mut()) })?;
+        Ok(out)
+    }
+    /// Sampled decoding with the token resident on the device (models/kalosm-llama/src/model/inference.rs:38-173):
+    /// `randoms` holds one uniform number per step (the host RNG of the reference's sampler draws them),
+    /// `previous` the token history before `first_token`, `repetition_range` the window of the penalty (at most 64);
+    /// `mu` is the Mirostat state, updated in place (unused by the standard sampler).  A step without a finite
+    /// logit yields `u32::MAX`.
+    pub fn decode_sampled(
+        &mut self,
+        first_token: u32,
+        params: &sys::FhSamplerParams,
+        randoms: &[f32],
+        previous: &[u32],
+        repetition_range: u32,
+        mu: &mut f32,
+    ) -> Result<Vec<u32>> {
+        let mut out = vec![0u32; randoms.len()];
+        let _g = self.dev.lock();
+        check(unsafe {
+            sys::fh_llama_decode_sampled(
+                self.raw, first_token, randoms.len() as i32, params, randoms.as_ptr(),
+                if previous.is_empty() { ptr::null() } else { previous.as_ptr() }, previous.len() as u32,
+                repetition_range, mu, out.as_mut_ptr(), ptr::null_mut(),
+            )
+        })?;
         Ok(out)
     }
     /// `KvCache::reset` for every layer.
