@@ -290,12 +290,16 @@ template <typename TQ, typename TKV, int D>
 static fh_status decode_dispatch_g(fh_device *dev, int G, const void *q, int64_t q_sb, int64_t q_sh, const void *k,
                                    const void *v, int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int b, int hq, int hkv,
                                    int skv, const int *len_dev, float scale, const float *mask, void *out) {
+    // any group size up to 8 (Llama-3.2-3B has 24 query heads on 8 KV heads: groups of 3)
+#define FH_DECODE_G(G_)                                                                                                  \
+    case G_:                                                                                                            \
+        return decode_launch<TQ, TKV, D, G_>(dev, q, q_sb, q_sh, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, skv, len_dev, scale, \
+                                             mask, out)
     switch (G) {
-    case 1: return decode_launch<TQ, TKV, D, 1>(dev, q, q_sb, q_sh, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, skv, len_dev, scale, mask, out);
-    case 2: return decode_launch<TQ, TKV, D, 2>(dev, q, q_sb, q_sh, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, skv, len_dev, scale, mask, out);
-    case 4: return decode_launch<TQ, TKV, D, 4>(dev, q, q_sb, q_sh, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, skv, len_dev, scale, mask, out);
-    case 8: return decode_launch<TQ, TKV, D, 8>(dev, q, q_sb, q_sh, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, skv, len_dev, scale, mask, out);
+        FH_DECODE_G(1); FH_DECODE_G(2); FH_DECODE_G(3); FH_DECODE_G(4);
+        FH_DECODE_G(5); FH_DECODE_G(6); FH_DECODE_G(7); FH_DECODE_G(8);
     }
+#undef FH_DECODE_G
     return FH_ERR_UNSUPPORTED;
 }
 
@@ -320,7 +324,7 @@ static fh_status attn_typed(fh_device *dev, const void *q, int64_t q_sb, int64_t
         }
         if (st != FH_ERR_UNSUPPORTED) return st;
     }
-    if (sq == 1 && aligned && (d == 128 || d == 64) && (G == 1 || G == 2 || G == 4 || G == 8) &&
+    if (sq == 1 && aligned && (d == 128 || d == 64) && G <= 8 &&
         mask_kind != FH_MASK_BATCH_KEY) {
         const float *mrow = mask_kind == FH_MASK_ADDITIVE ? mask : nullptr;
         fh_status st = d == 128 ? decode_dispatch_g<TQ, TKV, 128>(dev, G, q, q_sb, q_sh, k, v, kv_sb, kv_sh, kv_st, b, hq,

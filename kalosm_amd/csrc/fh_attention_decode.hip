@@ -598,7 +598,8 @@ static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void
                         int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req, int waves_req,
                         bool q_f16) {
     const int gtot = hq / hkv;
-    if (d != 128 || (gtot != 1 && gtot != 2 && gtot != 4 && gtot != 8) || kv_st % 8 || kv_sh % 8) return FH_ERR_UNSUPPORTED;
+    // any number of query heads per KV head: a workgroup takes 1, 2, 4 or 8 of them, whichever divides the group
+    if (d != 128 || gtot < 1 || kv_st % 8 || kv_sh % 8) return FH_ERR_UNSUPPORTED;
     // query heads per workgroup: the arithmetic of a workgroup grows with them, the K and V reads do not; one
     // (the workgroups of a KV head then share the rows through the L2) measured best on MI355X for 4 heads per KV
     // head at contexts of some hundred keys: 256 workgroups instead of 64

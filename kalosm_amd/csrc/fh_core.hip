@@ -171,6 +171,7 @@ fh_status fh_dev_scratch(fh_device *dev, void **buf, size_t *cap, size_t need) {
     size_t want = need < (1u << 20) ? (1u << 20) : need;
     FH_HIP(hipMalloc(buf, want));
     *cap = want;
+    dev->scratch_gen++;
     return FH_OK;
 }
 
@@ -201,6 +202,7 @@ struct fh_graph {
     fh_device *dev = nullptr;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    uint64_t scratch_gen = 0; // dev->scratch_gen when the capture ended
 };
 
 extern "C" fh_status fh_graph_begin(fh_device *dev) {
@@ -229,12 +231,16 @@ extern "C" fh_status fh_graph_end(fh_device *dev, fh_graph **out) {
     r->dev = dev;
     r->graph = g;
     r->exec = ex;
+    r->scratch_gen = dev->scratch_gen;
     *out = r;
     return FH_OK;
 }
 
 extern "C" fh_status fh_graph_launch(fh_graph *g) {
     FH_REQUIRE(g && g->exec, "NULL graph");
+    if (g->scratch_gen != g->dev->scratch_gen)
+        FH_FAIL(FH_ERR_INVALID, "the device's scratch buffers were reallocated by a larger call since this graph was "
+                                "captured; its kernels hold the old addresses: capture it again");
     FH_HIP(hipGraphLaunch(g->exec, g->dev->stream));
     return FH_OK;
 }

@@ -50,6 +50,10 @@ struct fh_device {
     size_t ksplit_cap = 0;
     // 64 KB that never moves: partial results of small reductions (argmax)
     void *small_buf = nullptr;
+    // Counts the reallocations of act_buf / part_buf / ksplit_buf.  A captured graph holds their addresses as
+    // kernel arguments, so whoever keeps a graph records the value at capture and must not replay it after
+    // the value has changed.
+    uint64_t scratch_gen = 0;
     // options (fh_set_option)
     int64_t opt_matvec_kernel = 0;   // 0 auto, 1 generic VALU, 2 MFMA, 3 first-generation Q4_K MFMA, 4 batch MFMA
     int64_t opt_matvec_splitk = 0;   // 0 auto, else forced split count

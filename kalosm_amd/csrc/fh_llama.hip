@@ -42,6 +42,7 @@ struct fh_llama {
     hipGraphExec_t graph_exec = nullptr;
     hipGraph_t graph = nullptr;
     int captured_capacity = -1;
+    uint64_t captured_gen = 0, samp_gen = 0; // dev->scratch_gen at the captures
     // sampled decode state: [0..63] previous ids, [64] their count, [65] next slot, [66] Mirostat mu (f32),
     // [68..69] status and token of the last step, [128..] one random number per step
     uint32_t *samp_dev = nullptr;
@@ -64,6 +65,9 @@ extern "C" fh_status fh_llama_create(fh_device *dev, const fh_llama_config *cfg,
                "bad decoder configuration");
     FH_REQUIRE(cfg->n_heads % cfg->n_kv_heads == 0, "n_heads %d not divisible by n_kv_heads %d", cfg->n_heads, cfg->n_kv_heads);
     FH_REQUIRE(cfg->head_dim == 64 || cfg->head_dim == 128, "head_dim %d unsupported (64 or 128)", cfg->head_dim);
+    if (cfg->n_heads / cfg->n_kv_heads > 8)
+        FH_FAIL(FH_ERR_UNSUPPORTED, "%d query heads per KV head: the decode-step attention handles groups of at most 8",
+                cfg->n_heads / cfg->n_kv_heads);
     fh_llama *m = new fh_llama();
     m->dev = dev;
     m->c = *cfg;
@@ -452,7 +456,7 @@ extern "C" fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, i
         // One eager step sizes every scratch buffer and sets kernel attributes; the capture then
         // records launches only.  The graph depends on the cache capacity (strides), so it is
         // rebuilt when the capacity changed since the last capture.
-        if (!m->graph_exec || m->captured_capacity != m->cache->capacity) {
+        if (!m->graph_exec || m->captured_capacity != m->cache->capacity || m->captured_gen != dev->scratch_gen) {
             FH_TRY(fh_timer_start(dev));
             FH_TRY(decode_step_enqueue(m));
             done = 1;
@@ -466,6 +470,7 @@ extern "C" fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, i
             FH_HIP(e);
             FH_HIP(hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
             m->captured_capacity = m->cache->capacity;
+            m->captured_gen = dev->scratch_gen;
         } else {
             FH_TRY(fh_timer_start(dev));
         }
@@ -549,6 +554,7 @@ extern "C" fh_status fh_llama_decode_sampled(fh_llama *m, uint32_t first_token, 
         fh_sampler_params want = *params;
         want.random = 0.f; // every step takes its number from randoms_host
         const bool same = m->samp_exec && m->samp_capacity == m->cache->capacity && m->samp_range == range &&
+                          m->samp_gen == dev->scratch_gen &&
                           memcmp(&m->samp_params, &want, sizeof(want)) == 0;
         m->samp_params = want;
         m->samp_range = range;
@@ -567,6 +573,7 @@ extern "C" fh_status fh_llama_decode_sampled(fh_llama *m, uint32_t first_token, 
             FH_HIP(e);
             FH_HIP(hipGraphInstantiate(&m->samp_exec, m->samp_graph, nullptr, nullptr, 0));
             m->samp_capacity = m->cache->capacity;
+            m->samp_gen = dev->scratch_gen;
         } else {
             FH_TRY(fh_timer_start(dev));
         }

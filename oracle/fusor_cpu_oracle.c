@@ -26,19 +26,33 @@
  *                           matmul (gemm crate): accumulation order UNPINNED, tolerance only
  *   q_mat_mul ............. one-hot / zero / linearity invariants, float64 dense product
  *   q8_0 quantize/vec_dot . closed form, exact integer sums, round trip < 0.02
- *   attention ............. torch CPU scaled_dot_product_attention, softmax invariants
- *   rms_norm / rope / silu  numpy formulas from the reference's conformance host
- *                           references; RoPE golden sextets; inverse-frequency closed form;
+ *   attention ............. float64 textbook form and torch CPU scaled_dot_product_attention (none, causal,
+ *                           additive and per-batch key masks, grouped heads), causal row 0 = v_0, equal keys ->
+ *                           mean of V, grouped heads == repeated KV heads (tests/test_oracle_ops.py)
+ *   attention, f16 form ... one key -> v bit for bit, equal scores -> n * f16(1/n) * v, agreement with the f32
+ *                           form on short rows, and the stall of the f16 running sum on long rows
+ *   rms_norm .............. float64 formula of the reference's host check, residual and bias forms, zero row
+ *   rope rotation ......... complex multiplication in float64 (both pairings, start positions), unit vectors
+ *                           (signs and partner element), bit equality with the f32 host forms of the
+ *                           reference's conformance suite
+ *   rope tables ........... RoPE golden sextets; inverse-frequency closed form; composition of positions;
  *                           long-context scaling and rope_freqs weights against numpy
+ *   silu / swiglu / add3 .. float64 closed form, fixed points, operand order
+ *   embed_rows ............ rows of the independently dequantised table, bit for bit
+ *   causal mask ........... numpy triu with the cache offset
  *   argmax ................ tie and non-finite cases from the reference's rule
  *   samplers .............. the reference's stored answers (flat logits: Mirostat 2 with random 0.8 -> id 0, top_p 0.5
  *                           with random 0.8 -> id 2, min_p 0.1 -> id 3, processed order -> id 0), the processor
  *                           case of its test (temperature 0.5, penalty 2, previous {0, 3, 9}) worked by hand,
  *                           sampled frequencies against the softmax probabilities, and the Mirostat update
  *                           against the closed form on two-candidate cases
- *   decoder ............... PARITY UNPINNED in the reference (no stored logits);
- *                           pinned here only by composition of the pinned ops and an
- *                           independent numpy float64 decoder on a tiny configuration.
+ *   decoder ............... PARITY UNPINNED in the reference (no stored logits); pinned here by an independent
+ *                           float64 numpy decoder (textbook ops on independently dequantised weights: prefill,
+ *                           decode steps and a second chunk against the cache, groups of 1, 2 and 3 query heads
+ *                           per KV head) on a two-layer configuration (tests/test_oracle_ops.py)
+ *   Committed vectors: tests/golden/fusor_golden.npz (written by tests/golden/make_golden.py) holds edge blocks,
+ *   [64, 512] matvecs, attention / rope / rms_norm / swiglu cases, a tiny decoder's logits and the values the
+ *   reference's tests store; tests/test_golden.py holds this file to them.
  *   q_mat_mul summation order, attention dot order, expf/sinf/cosf/powf are
  *   machine/library dependent in the reference itself (pulp lane width, gemm
  *   crate, platform libm) and are held to tolerance, never to bit equality.
@@ -640,6 +654,56 @@ int fo_flash_attention(const float *q, const float *k, const float *v, int b, in
     if (nj == 1) { att_worker(&jobs[0]); return 0; }
     for (int i = 0; i < nj; i++) pthread_create(&th[i], NULL, att_worker, &jobs[i]);
     for (int i = 0; i < nj; i++) pthread_join(th[i], NULL);
+    return 0;
+}
+
+/* The reference's f16 instantiation of the same composite: every tensor op yields f16, i.e. the value is
+ * computed in f32 and rounded to f16 after EVERY op.  matmul: f32 sum over k, one rounding per output
+ * (cpu/src/matmul.rs:159-179); mul_scalar / + mask / - max / exp / div: one rounding each
+ * (cpu/src/pairwise.rs:157-160, cpu/src/elementwise.rs:222); the row sum folds left to right with a rounding
+ * to f16 after every add (cpu/src/reduce.rs:228-237), so once the running sum's f16 spacing exceeds twice an
+ * addend the addend is lost; max is exact.  q, k, v and out are f16 bit patterns; mask_kind 0 or 1 (the causal
+ * mask holds 0 / -inf, exact in f16).  Single-threaded: it exists to show what the f16 CPU path yields on small cases. */
+static float fo_r16(float x) { return fo_f16_to_f32(fo_f32_to_f16(x)); }
+int fo_flash_attention_f16(const uint16_t *q, const uint16_t *k, const uint16_t *v, int b, int h, int hkv, int sq,
+                           int skv, int d, float scale, int mask_kind, uint16_t *out) {
+    if (hkv <= 0 || h % hkv) return -1;
+    if (mask_kind != 0 && mask_kind != 1) return -2;
+    int groups = h / hkv;
+    float sc16 = fo_r16(scale); /* D::from_f32(scale) */
+    float *s = (float *)malloc((size_t)skv * sizeof(float));
+    for (int bh = 0; bh < b * h; bh++) {
+        int bi = bh / h, hi = bh % h, kh = hi / groups;
+        const uint16_t *qh = q + ((size_t)bi * h + hi) * sq * d;
+        const uint16_t *kk = k + ((size_t)bi * hkv + kh) * skv * d;
+        const uint16_t *vv = v + ((size_t)bi * hkv + kh) * skv * d;
+        uint16_t *oh = out + ((size_t)bi * h + hi) * sq * d;
+        for (int i = 0; i < sq; i++) {
+            float mx = -INFINITY;
+            for (int t = 0; t < skv; t++) {
+                float acc = 0.0f;
+                for (int c = 0; c < d; c++)
+                    acc += fo_f16_to_f32(qh[(size_t)i * d + c]) * fo_f16_to_f32(kk[(size_t)t * d + c]);
+                acc = fo_r16(acc);
+                acc = fo_r16(acc * sc16);
+                if (mask_kind == 1) acc = fo_r16(acc + ((t > i + (skv - sq)) ? -INFINITY : 0.0f));
+                s[t] = acc;
+                mx = acc > mx ? acc : mx;
+            }
+            float sum = 0.0f;
+            for (int t = 0; t < skv; t++) {
+                s[t] = fo_r16(expf(fo_r16(s[t] - mx)));
+                sum = fo_r16(sum + s[t]);
+            }
+            for (int t = 0; t < skv; t++) s[t] = fo_r16(s[t] / sum);
+            for (int c = 0; c < d; c++) {
+                float acc = 0.0f;
+                for (int t = 0; t < skv; t++) acc += s[t] * fo_f16_to_f32(vv[(size_t)t * d + c]);
+                oh[(size_t)i * d + c] = fo_f32_to_f16(acc);
+            }
+        }
+    }
+    free(s);
     return 0;
 }
 

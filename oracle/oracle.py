@@ -21,7 +21,9 @@ BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, 0: 4, 1: 2, 6: 22, 13: 
 
 def build(force: bool = False) -> str:
     """Compile the checker with the Makefile beside it."""
-    if force or not os.path.exists(_SO):
+    src = os.path.join(_HERE, "fusor_cpu_oracle.c")
+    stale = not os.path.exists(_SO) or os.path.getmtime(src) > os.path.getmtime(_SO)
+    if force or stale:
         subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s"])
     return _SO
 
@@ -197,6 +199,22 @@ def flash_attention(q, k, v, scale: float, mask_kind: int = MASK_NONE, mask=None
                                   scale, mask_kind, mp, _p(out, C.c_float), threads or default_threads())
     if rc:
         raise ValueError(f"fo_flash_attention rc={rc}")
+    return out
+
+
+def flash_attention_f16(q, k, v, scale: float, causal: bool = False) -> np.ndarray:
+    """The reference's f16 instantiation of the attention composite: f16 in, f16 out, a rounding to f16 after every
+    tensor op (see fo_flash_attention_f16).  Small cases only (one thread)."""
+    q, k, v = (np.ascontiguousarray(t, np.float16) for t in (q, k, v))
+    b, h, sq, d = q.shape
+    _, hkv, skv, _ = k.shape
+    out = np.empty_like(q)
+    L = lib()
+    L.fo_flash_attention_f16.argtypes = [C.c_void_p] * 3 + [C.c_int] * 6 + [C.c_float, C.c_int, C.c_void_p]
+    rc = L.fo_flash_attention_f16(q.ctypes.data, k.ctypes.data, v.ctypes.data, b, h, hkv, sq, skv, d, scale,
+                                  1 if causal else 0, out.ctypes.data)
+    if rc:
+        raise ValueError(f"fo_flash_attention_f16 rc={rc}")
     return out
 
 

@@ -29,3 +29,13 @@ def oracle():
 
     o.build()
     return o
+
+
+@pytest.fixture(scope="session")
+def golden():
+    """The committed input / expected-output vectors (tests/golden/make_golden.py writes them)."""
+    import numpy as np
+
+    path = os.path.join(ROOT, "tests", "golden", "fusor_golden.npz")
+    with np.load(path, allow_pickle=False) as z:
+        return {k: z[k] for k in z.files}

@@ -46,9 +46,9 @@ def test_config1_other_formats_down_shape(dev, oracle, ty):
         assert_close(got, oracle.q_mat_mul(ty, x, raw, n, fast=True), what=f"{NAMES[ty]} m={m}")
 
 
-@pytest.mark.parametrize("s", [2048, 8192])
+@pytest.mark.parametrize("s", [512, 2048, 8192])
 def test_config3_causal_attention_long(dev, oracle, s):
-    """configs[3] at seq 2048 and 8192 (32 / 8 heads, d = 128, f16).  The checker would need minutes, so: 24 sampled
+    """configs[3] at seq 512, 2048 and 8192 (32 / 8 heads, d = 128, f16).  The checker would need minutes, so: 24 sampled
     query rows per length (first, last, tile and block boundaries, random) against the float64 textbook form computed
     for those rows only, plus the exact property that causal row 0 returns v_0."""
     h, hkv, d = 32, 8, 128
@@ -142,3 +142,38 @@ def test_decoder_from_gguf_file_full_width(dev, oracle, tmp_path):
         t = oracle.argmax(ref.forward([t]))
         want.append(t)
     assert got.tolist() == want
+
+
+def test_config4_decoder_all_32_layers(dev, oracle):
+    """configs[4] at its real depth and widths: the 32-layer Llama-3-8B-architecture decoder with random-init Q4_K_M
+    weights against the checker's decoder on the same weights: prefill logits of a 48-token prompt, 16 greedy steps
+    replayed on the device, and the logits after them.  The checker needs about a second per token."""
+    cfg = dict(synth.LLAMA3_8B, ctx=1024)
+    weights = {}
+    m = Model.random_init(dev, cfg, seed=0, sigma=1e-4, keep=lambda n, a: weights.__setitem__(n, a))
+    ocfg = dict(cfg, type_attn=synth.Q4_K, type_ffn_gate_up=synth.Q4_K, type_ffn_down=synth.Q6_K, type_embd=synth.Q4_K,
+                type_output=synth.Q6_K)
+    ref = oracle.Llama(ocfg, weights)
+    prompt = np.random.default_rng(1).integers(0, cfg["vocab"], 32)
+    lg = m.forward(prompt)
+    wl = ref.forward(prompt)
+    assert_close(lg, wl, what="prefill logits, 32 layers")
+    tok = oracle.argmax(wl)
+    steps = 12
+    got, _ = m.decode_greedy(tok, steps)
+    want, t = [], tok
+    margins = []
+    for _ in range(steps):
+        wl = ref.forward([t])
+        srt = np.sort(wl)
+        margins.append(float(srt[-1] - srt[-2]))
+        t = oracle.argmax(wl)
+        want.append(t)
+    # a greedy pick is only defined up to the logit tolerance: a step whose two best logits are closer than 2e-2
+    # may legitimately differ, and every later token with it
+    for i, (g, w_) in enumerate(zip(got.tolist(), want)):
+        if g != w_:
+            assert margins[i] < 2e-2, f"step {i}: {g} != {w_} with a margin of {margins[i]}"
+            break
+    else:
+        assert_close(m.forward([want[-1]]), ref.forward([want[-1]]), what="logits after 12 device-side steps, 32 layers")

@@ -78,7 +78,7 @@ def test_decoder_matches_checker(dev, oracle, variant, cfg):
     assert_close(m.forward([want3[-1]]), ref.forward([want3[-1]]), what="logits after 40 device-side steps", **tol)
 
 
-@pytest.mark.parametrize("heads,kv_heads", [(4, 1), (4, 2), (8, 1), (2, 2)], ids=["g4", "g2", "g8", "g1"])
+@pytest.mark.parametrize("heads,kv_heads", [(4, 1), (4, 2), (8, 1), (2, 2), (6, 2)], ids=["g4", "g2", "g8", "g1", "g3"])
 @pytest.mark.parametrize("opts", [{}, dict(attn_heads=2), dict(attn_heads=4, attn_waves=8), dict(attn_splits=4, wo_tiles=1),
                                   dict(wo_tiles=2, down_tiles=2, matvec_tiles=2), dict(matvec_per=2, down_tiles=4),
                                   dict(attn_kernel=4), dict(attn_kernel=4, attn_heads=4, attn_waves=8)],
@@ -290,3 +290,65 @@ def _bytes_source(data, tmp_path):
     p = tmp_path / f"m{len(list(tmp_path.iterdir()))}.gguf"
     p.write_bytes(data)
     return str(p)
+
+
+def test_graph_decode_survives_scratch_reallocation(oracle):
+    """A captured decode step holds the device's scratch buffers as kernel arguments.  A larger call between two
+    decodes (here a 100-token prompt and a 300-row matmul whose k-split planes, activation planes and partial sums
+    outgrow the buffers the capture saw) reallocates them; the next decode must capture again instead of replaying
+    kernels that point at freed memory.  Own device handle, so the buffers start at their minimum size."""
+    from kalosm_amd.fusor import Device, FusorHipError, GpuStandardSamplerParams, QMatrix, Tensor
+    d = Device.gpu(0)
+    cfg = dict(n_layers=2, d_model=1024, n_heads=8, n_kv_heads=2, head_dim=128, ffn=2048, vocab=2048, ctx=512, eps=1e-5,
+               theta=500000.0)
+    m, ref = build_pair(d, oracle, cfg, seed=9)
+    rng = np.random.default_rng(3)
+
+    def greedy_ref(t, steps):
+        out = []
+        for _ in range(steps):
+            t = oracle.argmax(ref.forward([t]))
+            out.append(t)
+        return out
+
+    # a user graph over a small matvec, captured while the scratch is small
+    w = QMatrix.from_raw_bytes(d, (64, 512), synth.random_weight(synth.Q8_0, 64, 512, 1), synth.Q8_0)
+    xs = Tensor.from_slice(d, synth.random_activation(8, 512, 2))
+    ys = Tensor.zeros(d, (8, 64))
+    xs.q_mat_mul(w, out=ys)          # eager first: sizes what the capture needs
+    d.graph_begin()
+    xs.q_mat_mul(w, out=ys)
+    g = d.graph_end()
+    g.launch()
+    d.sync()
+
+    prompt = rng.integers(0, cfg["vocab"], 6)
+    wl = ref.forward(prompt)
+    m.forward(prompt)
+    first = oracle.argmax(wl)
+    p = GpuStandardSamplerParams(1, 1.0, 1.0, 1.0, 0.0, 0.0)      # top_k 1: the sampled step picks the argmax
+    got, _, _ = m.decode_sampled(first, 5, p, np.full(5, 0.5, np.float32), repetition_range=0)
+    assert got.tolist() == greedy_ref(first, 5)
+    last = int(got[-1])
+    got, _ = m.decode_greedy(last, 5)
+    assert got.tolist() == greedy_ref(last, 5)
+    # larger calls on the same device: every scratch buffer is outgrown
+    m.reset(); ref.reset()
+    long_prompt = rng.integers(0, cfg["vocab"], 100)
+    wl = ref.forward(long_prompt)
+    assert_close(m.forward(long_prompt), wl, what="100-token prefill logits")
+    big = QMatrix.from_raw_bytes(d, (2048, 4096), synth.random_weight(synth.Q4_K, 2048, 4096, 4), synth.Q4_K)
+    Tensor.from_slice(d, synth.random_activation(300, 4096, 5)).q_mat_mul(big).as_slice()
+    Tensor.from_slice(d, synth.random_activation(16, 4096, 6)).q_mat_mul(big).as_slice()
+    # same parameters, same cache capacity: only the reallocation can trigger the new capture
+    first = oracle.argmax(wl)
+    got, _, _ = m.decode_sampled(first, 6, p, np.full(6, 0.5, np.float32), repetition_range=0)
+    want = greedy_ref(first, 6)
+    assert got.tolist() == want
+    got2, _ = m.decode_greedy(want[-1], 6)
+    assert got2.tolist() == greedy_ref(want[-1], 6)
+    # the user graph is refused with an error that says why
+    with pytest.raises(FusorHipError, match="captured"):
+        g.launch()
+    del g, m
+    d.sync()

@@ -130,12 +130,13 @@ def test_tile_matmul_bf16_activations(dev, oracle, ty, m):
         assert_close(got, want, what=f"bf16 {NAMES[ty]} m={m} kernel option {force}")
 
 
+@pytest.mark.parametrize("m", [512, 2048])
 @pytest.mark.parametrize("ty", [Q6_K, Q8_0], ids=lambda t: NAMES[t])
-def test_prefill_shape_spot_check(dev, oracle, ty):
-    """Full prefill shape (m = 512, k = 4096, n = 14336, bf16 activations): 64 output columns spread over the matrix
-    against the checker, and the sum over all outputs of a row against x . (sum of weight rows) -- a checksum that
-    every output element enters."""
-    m, k, n = 512, 4096, 14336
+def test_prefill_shape_spot_check(dev, oracle, ty, m):
+    """Full prefill shapes (m = 512 and 2048, k = 4096, n = 14336, bf16 activations): 64 output columns spread over the
+    matrix against the checker, and the sum over all outputs of a row against x . (sum of weight rows) -- a checksum
+    that every output element enters."""
+    k, n = 4096, 14336
     raw = synth.random_weight(ty, n, k, seed=100 + ty)
     xb, xf = bf16_round(synth.random_activation(m, k, seed=101))
     q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
@@ -252,10 +253,11 @@ def test_q8_activation_matmul_mfma(dev, oracle, m, n, k):
     assert np.array_equal(old.as_slice().view(np.uint32), want.view(np.uint32))
 
 
-def test_q8_activation_matmul_prefill_shape(dev, oracle):
-    """configs[2], integer variant, full shape (m = 512, k = 4096, n = 14336): 48 sampled weight rows against the
-    checker bit for bit, every output finite."""
-    m, k, n = 512, 4096, 14336
+@pytest.mark.parametrize("m", [512, 2048])
+def test_q8_activation_matmul_prefill_shape(dev, oracle, m):
+    """configs[2], integer variant, full shapes (m = 512 and 2048, k = 4096, n = 14336): 48 sampled weight rows against
+    the checker bit for bit, every output finite."""
+    k, n = 4096, 14336
     raw = synth.random_weight(Q8_0, n, k, seed=210)
     x = synth.random_activation(m, k, seed=211)
     q = QMatrix.from_raw_bytes(dev, (n, k), raw, Q8_0)
