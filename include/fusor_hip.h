@@ -243,6 +243,23 @@ fh_status fh_flash_attention_ex(fh_device *dev, int32_t q_dtype, int32_t kv_dtyp
                                 int32_t d, float scale, int32_t mask_kind, const float *mask_dev,
                                 void *out_dev);
 
+/* One query position per head against skv cached keys (b = 1, sq = 1, head_dim 128, no mask), for callers that
+ * cannot allocate: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No
+ * counterpart in the reference.  fh_flash_attention keeps the partial results of its key parts in a buffer the
+ * library grows with hipMalloc; this variant keeps them in a file-scope device array of 540 672 bytes (64 query
+ * heads x 16 key parts x 132 floats) that every GPU the library runs on holds until the process ends, and calls
+ * no hipMalloc, hipFree or other allocating routine.  q and out are [hq, 128] contiguous, of q_dtype; k and v are
+ * [hkv, skv, 128] views of kv_dtype with head stride kv_sh and position stride kv_st (elements, multiples of 8).
+ * Same kernels and the same cut of the key range as fh_flash_attention, so the same bits.  hq x parts beyond the
+ * array (more than 64 heads at 16 parts) is FH_ERR_INVALID with a message; shapes outside the list above are
+ * FH_ERR_UNSUPPORTED.  All calls on one GPU share the array: calls that overlap on one GPU (two streams, two
+ * device handles, two threads) race; calls on one handle's stream are ordered and safe.  Nothing needs clearing
+ * between calls: every slot the merge reads is written by the same call first. */
+fh_status fh_flash_attention_decode_static(fh_device *dev, int32_t q_dtype, int32_t kv_dtype,
+                                           const void *q_dev, const void *k_dev, const void *v_dev,
+                                           int64_t kv_sh, int64_t kv_st, int32_t hq, int32_t hkv, int32_t d,
+                                           float scale, int32_t skv, void *out_dev);
+
 /* -------------------------------------------------------------------- glue
  * silu(g) * u, fusor-ml/fusor/src/composite/activations.rs:47-65 + raw/attention_layer.rs:195 */
 fh_status fh_swiglu(fh_device *dev, const float *gate_dev, const float *up_dev, float *y_dev,

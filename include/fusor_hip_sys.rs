@@ -172,6 +172,7 @@ extern "C" {
     pub fn fh_kvcache_view(c: *const FhKvCache, layer: i32, len: *mut i32, capacity: *mut i32, k_dev: *mut *const c_void, v_dev: *mut *const c_void) -> FhStatus;
     pub fn fh_flash_attention(dev: *mut FhDevice, dtype: i32, q_dev: *const c_void, q_sb: i64, q_sh: i64, q_st: i64, k_dev: *const c_void, v_dev: *const c_void, kv_sb: i64, kv_sh: i64, kv_st: i64, b: i32, hq: i32, hkv: i32, sq: i32, skv: i32, d: i32, scale: f32, mask_kind: i32, mask_dev: *const f32, out_dev: *mut c_void) -> FhStatus;
     pub fn fh_flash_attention_ex(dev: *mut FhDevice, q_dtype: i32, kv_dtype: i32, q_dev: *const c_void, q_sb: i64, q_sh: i64, q_st: i64, k_dev: *const c_void, v_dev: *const c_void, kv_sb: i64, kv_sh: i64, kv_st: i64, b: i32, hq: i32, hkv: i32, sq: i32, skv: i32, d: i32, scale: f32, mask_kind: i32, mask_dev: *const f32, out_dev: *mut c_void) -> FhStatus;
+    pub fn fh_flash_attention_decode_static(dev: *mut FhDevice, q_dtype: i32, kv_dtype: i32, q_dev: *const c_void, k_dev: *const c_void, v_dev: *const c_void, kv_sh: i64, kv_st: i64, hq: i32, hkv: i32, d: i32, scale: f32, skv: i32, out_dev: *mut c_void) -> FhStatus;
     pub fn fh_swiglu(dev: *mut FhDevice, gate_dev: *const f32, up_dev: *const f32, y_dev: *mut f32, count: i64) -> FhStatus;
     pub fn fh_add3(dev: *mut FhDevice, a_dev: *const f32, b_dev: *const f32, c_dev: *const f32, y_dev: *mut f32, count: i64) -> FhStatus;
     pub fn fh_transpose_shd(dev: *mut FhDevice, x_dev: *const f32, s: i32, h: i32, d: i32, y_dev: *mut f32) -> FhStatus;

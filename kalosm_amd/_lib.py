@@ -93,6 +93,7 @@ SIGNATURES = {
                            _f32, _i32, _p, _p],
     "fh_flash_attention_ex": [_p, _i32, _i32, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _i32, _i32,
                               _i32, _i32, _f32, _i32, _p, _p],
+    "fh_flash_attention_decode_static": [_p, _i32, _i32, _p, _p, _p, _i64, _i64, _i32, _i32, _i32, _f32, _i32, _p],
     "fh_swiglu": [_p, _p, _p, _p, _i64],
     "fh_add3": [_p, _p, _p, _p, _p, _i64],
     "fh_transpose_shd": [_p, _p, _i32, _i32, _i32, _p],

@@ -509,7 +509,7 @@ template <typename TKV, int G, int NWV>
 static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const void *v, int64_t kv_sh, int64_t kv_st,
                            int hq, int hkv, float scale, const int *len_dev, int max_len, float *out, int *splits_out,
                            int gtot, int len_host = 0, int splits_req = 0, bool out_f16 = false, bool one_pass = false,
-                           bool q_f16 = false) {
+                           bool q_f16 = false, float *part_fixed = nullptr) {
     constexpr int D = 128;
     // splits: 8 measured best from a few hundred to a few thousand keys (MI355X); it is also the most the output
     // projection merges while staging its input.  The option allows 4 .. 16; a caller with a long cache and its
@@ -519,21 +519,26 @@ static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const 
     if (splits_req > 0) S = splits_req;
     FH_REQUIRE(!q_f16 || (one_pass && G <= 4), "an f16 query needs the one-pass kernel");
     if (one_pass && G <= 4) {
-        FH_TRY(fh_dev_scratch(dev, (void **)&dev->part_buf, &dev->part_cap, (size_t)hq * S * (D + 4) * 4));
+        // partial results: the device's growable buffer, or a buffer the caller fixed (no allocation then)
+        float *part = part_fixed;
+        if (!part) {
+            FH_TRY(fh_dev_scratch(dev, (void **)&dev->part_buf, &dev->part_cap, (size_t)hq * S * (D + 4) * 4));
+            part = dev->part_buf;
+        }
         k_attn_decode_1p<TKV, (G <= 4 ? G : 4), NWV><<<dim3((unsigned)S, (unsigned)hkv, (unsigned)(gtot / G)), dim3(64 * NWV), 0,
                                                        dev->stream>>>(q, q_f16 ? 1 : 0, (const TKV *)k, (const TKV *)v, kv_sh,
-                                                                      kv_st, len_dev, len_host, scale, max_len, gtot,
-                                                                      dev->part_buf);
+                                                                      kv_st, len_dev, len_host, scale, max_len, gtot, part);
         FH_HIP(hipGetLastError());
         if (splits_out) *splits_out = S;
         if (out) {
             if (out_f16)
-                k_attn_combine_dl<D, fh_half><<<dim3((unsigned)hq), dim3(D), 0, dev->stream>>>(dev->part_buf, S, (fh_half *)out);
-            else k_attn_combine_dl<D><<<dim3((unsigned)hq), dim3(D), 0, dev->stream>>>(dev->part_buf, S, out);
+                k_attn_combine_dl<D, fh_half><<<dim3((unsigned)hq), dim3(D), 0, dev->stream>>>(part, S, (fh_half *)out);
+            else k_attn_combine_dl<D><<<dim3((unsigned)hq), dim3(D), 0, dev->stream>>>(part, S, out);
             FH_HIP(hipGetLastError());
         }
         return FH_OK;
     }
+    FH_REQUIRE(!part_fixed, "a fixed partial buffer needs the one-pass kernel");
     const int chunk_max = (((max_len + 15) / 16 + S - 1) / S) * 16; // most local rows of a split
     const size_t lds = ((size_t)G * chunk_max + (size_t)NWV * G * D) * 4;
     FH_REQUIRE(lds <= 150 * 1024, "KV capacity %d too large for the decode attention kernel", max_len);
@@ -569,7 +574,7 @@ fh_status fh_attention_combine_dl(fh_device *dev, int hq, int splits, float *out
 static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v, int64_t kv_sh,
                         int64_t kv_st, int hq, int hkv, int d, float scale, const int *len_dev, int max_len, float *out,
                         int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req = 0, int waves_req = 0,
-                        bool q_f16 = false);
+                        bool q_f16 = false, float *part_fixed = nullptr);
 
 fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v,
                                      int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale,
@@ -593,10 +598,59 @@ fh_status fh_attention_decode_hostlen(fh_device *dev, int kv_dtype, const void *
                   skv - 1, splits, out_f16, heads, skv > 2048 ? 8 : 0, q_f16);
 }
 
+// ------------------------------------------------------------------------------ no allocation at call time
+// The partial results of the key parts normally live in a buffer the library grows with hipMalloc.  Callers that
+// must not allocate (a stream under graph capture, a serving loop that forbids it) use the entry point below: its
+// partials live in this array, which exists once per GPU from the moment the library's code is loaded there until
+// the process ends.  Room for 64 query heads x 16 key parts x (128 + 4) floats.
+#define FH_STATIC_SCRATCH_BYTES (64 * 16 * (128 + 4) * 4)
+static __device__ __align__(256) unsigned char fh_static_scratch[FH_STATIC_SCRATCH_BYTES];
+
+// Called by fh_device_create with the device current: in host code the array's name is only a stand-in, its
+// address on THIS device comes from the runtime and is kept in the device handle.
+fh_status fh_static_scratch_init(fh_device *dev) {
+    void *p = nullptr;
+    FH_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(fh_static_scratch)));
+    FH_REQUIRE(p, "hipGetSymbolAddress returned no address for the static scratch");
+    dev->static_scratch = p;
+    dev->static_scratch_bytes = FH_STATIC_SCRATCH_BYTES;
+    return FH_OK;
+}
+
+extern "C" fh_status fh_flash_attention_decode_static(fh_device *dev, int32_t q_dtype, int32_t kv_dtype,
+                                                      const void *q_dev, const void *k_dev, const void *v_dev,
+                                                      int64_t kv_sh, int64_t kv_st, int32_t hq, int32_t hkv, int32_t d,
+                                                      float scale, int32_t skv, void *out_dev) {
+    FH_REQUIRE(dev && q_dev && k_dev && v_dev && out_dev, "NULL argument");
+    FH_REQUIRE(dev->static_scratch, "the device handle has no static scratch");
+    FH_REQUIRE(hq > 0 && hkv > 0 && skv > 0, "empty attention operand");
+    FH_REQUIRE(hq % hkv == 0, "number of Q heads (%d) must be divisible by number of K/V heads (%d)", hq, hkv);
+    const bool qh = q_dtype == FH_F16, kh = kv_dtype == FH_F16;
+    FH_REQUIRE((qh || q_dtype == FH_F32) && (kh || kv_dtype == FH_F32), "dtype must be FH_F32 or FH_F16");
+    if (qh && !kh) FH_FAIL(FH_ERR_UNSUPPORTED, "f16 queries with an f32 KV are not supported");
+    if (d != 128 || kv_st % 8 || kv_sh % 8)
+        FH_FAIL(FH_ERR_UNSUPPORTED, "the allocation-free decode attention needs head_dim 128 and K / V strides that are "
+                                    "multiples of 8 elements (got d = %d, strides %lld, %lld)", d, (long long)kv_sh,
+                (long long)kv_st);
+    // the same cut of the key range as fh_flash_attention makes for one query position
+    int splits = skv <= 2048 ? 8 : 16;
+    if (dev->opt_attn_splits > 0) splits = dev->opt_attn_splits > 128 ? 128 : (int)dev->opt_attn_splits;
+    const size_t need = (size_t)hq * splits * (128 + 4) * 4;
+    if (need > dev->static_scratch_bytes)
+        FH_FAIL(FH_ERR_INVALID, "%d query heads x %d key parts need %zu bytes of partial results; the static scratch "
+                                "holds %zu (at most 64 heads x 16 parts): use fh_flash_attention", hq, splits, need,
+                dev->static_scratch_bytes);
+    const int heads = dev->opt_attn_heads > 0 ? (int)dev->opt_attn_heads : (skv <= 2048 ? 1 : 2);
+    // Every (head, part) slot the merge reads is written by this call's first kernel, parts without keys
+    // included, so nothing has to be cleared between calls.
+    return ad_any(dev, kv_dtype, (const float *)q_dev, k_dev, v_dev, kv_sh, kv_st, hq, hkv, d, scale, nullptr, skv,
+                  (float *)out_dev, nullptr, skv - 1, splits, qh, heads, skv > 2048 ? 8 : 0, qh, (float *)dev->static_scratch);
+}
+
 static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void *k, const void *v, int64_t kv_sh,
                         int64_t kv_st, int hq, int hkv, int d, float scale, const int *len_dev, int max_len, float *out,
                         int *splits_out, int len_host, int splits_req, bool out_f16, int heads_req, int waves_req,
-                        bool q_f16) {
+                        bool q_f16, float *part_fixed) {
     const int gtot = hq / hkv;
     // any number of query heads per KV head: a workgroup takes 1, 2, 4 or 8 of them, whichever divides the group
     if (d != 128 || gtot < 1 || kv_st % 8 || kv_sh % 8) return FH_ERR_UNSUPPORTED;
@@ -609,8 +663,9 @@ static fh_status ad_any(fh_device *dev, int kv_dtype, const float *q, const void
     // 8 wavefronts per workgroup instead of 16
     const bool w8 = (dev->opt_attn_waves == 8 || (dev->opt_attn_waves == 0 && waves_req == 8)) && G <= 8;
     // the one-pass kernel unless attn_kernel = 4 asks for the two-pass one (or 8 heads per workgroup are wanted)
-    const bool one_pass = dev->opt_attn_kernel != 4;
-#define AD_ARGS dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out, gtot, len_host, splits_req, out_f16, one_pass, q_f16
+    const bool one_pass = dev->opt_attn_kernel != 4 || part_fixed;
+    if (part_fixed && G > 4) G = 4; // the one-pass kernel takes at most four query heads per workgroup
+#define AD_ARGS dev, q, k, v, kv_sh, kv_st, hq, hkv, scale, len_dev, max_len, out, splits_out, gtot, len_host, splits_req, out_f16, one_pass, q_f16, part_fixed
 #define AD_GO(TKV_)                                                                       \
     switch (G) {                                                                          \
     case 1: return w8 ? ad_launch<TKV_, 1, 8>(AD_ARGS) : ad_launch<TKV_, 1, 16>(AD_ARGS); \

@@ -50,6 +50,11 @@ extern "C" fh_status fh_device_create(int32_t ordinal, fh_device **out) {
     FH_HIP(hipEventCreate(&d->ev_start));
     FH_HIP(hipEventCreate(&d->ev_stop));
     FH_HIP(hipMalloc(&d->small_buf, 64 * 1024));
+    fh_status st = fh_static_scratch_init(d);
+    if (st != FH_OK) {
+        (void)fh_device_destroy(d);
+        return st;
+    }
     *out = d;
     return FH_OK;
 }

@@ -54,6 +54,10 @@ struct fh_device {
     // kernel arguments, so whoever keeps a graph records the value at capture and must not replay it after
     // the value has changed.
     uint64_t scratch_gen = 0;
+    // this GPU's copy of the library's file-scope scratch array (fh_attention_decode.hip), for the entry point that
+    // must not allocate
+    void *static_scratch = nullptr;
+    size_t static_scratch_bytes = 0;
     // options (fh_set_option)
     int64_t opt_matvec_kernel = 0;   // 0 auto, 1 generic VALU, 2 MFMA, 3 first-generation Q4_K MFMA, 4 batch MFMA
     int64_t opt_matvec_splitk = 0;   // 0 auto, else forced split count
@@ -75,6 +79,7 @@ struct fh_device {
 };
 
 fh_status fh_dev_scratch(fh_device *dev, void **buf, size_t *cap, size_t need);
+fh_status fh_static_scratch_init(fh_device *dev); // with dev->ordinal current
 
 // ---------------------------------------------------------------- weights
 // Device layouts.  All of them hold exactly the bits of the GGUF block stream,

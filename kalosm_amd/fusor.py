@@ -314,6 +314,20 @@ class Tensor:
                                                      hq, hkv, sq, skv, d, scale, kind, mptr, C.c_void_p(out.ptr)))
         return out
 
+    def flash_attention_decode_static(self, k: "Tensor", v: "Tensor", scale: float, out: Optional["Tensor"] = None) -> "Tensor":
+        """fh_flash_attention_decode_static: one query position per head ([1, hq, 1, 128]) against the cached keys, with
+        the partial results in the library's static device array (no allocation at call time; `out` must be given
+        for the call to allocate nothing on the Python side either)."""
+        b, hq, sq, d = self.shape
+        _, hkv, skv, _ = k.shape
+        assert b == 1 and sq == 1 and v.shape == k.shape
+        if out is None:
+            out = Tensor(self.device, (1, hq, 1, d), self.dtype)
+        check(self.device._lib.fh_flash_attention_decode_static(
+            self.device._h, F16 if self.dtype == "f16" else F32, F16 if k.dtype == "f16" else F32, C.c_void_p(self.ptr),
+            C.c_void_p(k.ptr), C.c_void_p(v.ptr), skv * d, d, hq, hkv, d, scale, skv, C.c_void_p(out.ptr)))
+        return out
+
     def silu_mul(self, up: "Tensor") -> "Tensor":
         """silu(self) * up (activations.rs:47-65, raw/attention_layer.rs:195)"""
         out = Tensor(self.device, self.shape, "f32")
