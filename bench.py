@@ -5,18 +5,26 @@ A step is one pass of the Q4_K decode matvec (batch 1) over the four Llama-3-8B 
 (4096x4096 q/o, 1024x4096 k/v, 14336x4096 gate/up, 4096x14336 down), activations f32 N(0,1), weights
 random Q4_K super-blocks (f16 d/dmin ~ N(0, 0.02), 6-bit scales/mins, uniform nibbles), all resident in
 HBM before the timed region.  Each shape rotates over enough distinct weight buffers to exceed the
-256 MB last-level cache, so the bytes really come from HBM.
+256 MB last-level cache, so the bytes really come from HBM.  The K launches of a shape are one recorded train;
+the train is replayed `--trains` times and the median replay is the shape's time (K steps are timed, the
+repetitions only steady the number).
 
 Prints ONE JSON line: whole-path GB/s (algorithmic bytes / device time), the roofline of the dominant
-kernel and the CPU checker timed on the host cores beside it.  The same line carries, under "e2e", the second
-half of the metric: tokens/s of the random-init Q4_K_M Llama-3-8B-architecture decoder (512-token prompt, 256
-greedy steps, batch 1; about 10 s including the weight upload; --no-e2e skips it).
+kernel and the CPU checker timed on the host cores beside it.  The same line carries the other benchmark
+configurations, each with its own roofline entry: "batch" (configs[1] at 4 and 16 rows), "prefill"
+(configs[2]: bf16 x Q6_K / Q8_0 and the Q8_0 x Q8 integer variant at 512 and 2048 rows; configs[3]: causal
+attention at 512 / 2048 / 8192 and single-query attention against 1024 / 4096 / 16384 cached keys) and "e2e"
+(configs[4]: tokens/s of the random-init Q4_K_M Llama-3-8B-architecture decoder, 512-token prompt, 256 greedy
+steps, batch 1, with its greedy tokens checked against the CPU checker on a short prompt outside the timed
+region).  --no-legs / --no-e2e skip them.
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import re
+import statistics
 import sys
 import time
 
@@ -27,19 +35,116 @@ sys.path.insert(0, ROOT)
 
 SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]  # (n, k)
 HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+MFMA_I8_PEAK_TOPS = 5000.0
 ROTATE_BYTES = 640 << 20  # > 2x the 256 MB Infinity Cache
-# HBM bytes per launch (average of the four shapes) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this
-# workload at batch 1, scaled by what the same counters read for a 256 MiB device copy (FETCH_SIZE x2.000,
-# WRITE_SIZE x1.000); a measured constant, to be re-measured when the kernel changes.
-TRAFFIC_BYTES_PER_LAUNCH = 19766426
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "q4k_matvec_m1_llama_shapes.md")
 
 
-def prefill_legs(dev) -> dict:
+def measured_traffic():
+    """HBM bytes per launch of the headline kernel as the tracked counter profile states them (rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE scaled by a copy of known size), with the commit the profile was taken at."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None, None
+    m = re.search(r"traffic_bytes_per_launch\s*=\s*(\d+)", text)
+    c = re.search(r"measured_at_commit\s*=\s*([0-9a-f]{7,40})", text)
+    return (int(m.group(1)) if m else None), (c.group(1) if c else None)
+
+
+def timed_trains(dev, enqueue, trains: int, use_graph: bool = True):
+    """Median device milliseconds of `trains` runs of the launch sequence `enqueue()` (recorded once and replayed
+    unless use_graph is off)."""
+    ms = []
+    if use_graph:
+        dev.graph_begin()
+        enqueue()
+        g = dev.graph_end()
+        g.launch()          # one untimed replay
+        dev.sync()
+        for _ in range(trains):
+            dev.timer_start()
+            g.launch()
+            ms.append(dev.timer_stop())
+        del g
+    else:
+        for _ in range(trains):
+            dev.timer_start()
+            enqueue()
+            ms.append(dev.timer_stop())
+    return statistics.median(ms), ms
+
+
+def matvec_sets(dev, ty, m: int):
+    from kalosm_amd import synth
+    from kalosm_amd.fusor import QMatrix, Tensor
+
+    sets = []
+    for si, (n, k) in enumerate(SHAPES):
+        wbytes = n * (k // 256) * 144
+        copies = max(2, -(-ROTATE_BYTES // wbytes))
+        raw = synth.random_weight(ty, n, k, seed=1000 + si)
+        qs = [QMatrix.from_raw_bytes(dev, (n, k), raw, ty) for _ in range(copies)]
+        x = Tensor.from_slice(dev, synth.random_activation(m, k, seed=2000 + si))
+        y = Tensor(dev, (m, n), "f32")
+        sets.append(dict(n=n, k=k, qs=qs, x=x, y=y, raw=raw, bytes=synth.matvec_bytes(ty, n, k, m)))
+    return sets
+
+
+def run_shape(s, launches, offset=0):
+    qs, x, y = s["qs"], s["x"], s["y"]
+    for i in range(launches):
+        x.q_mat_mul(qs[(offset + i) % len(qs)], out=y)
+
+
+def batch_leg(dev, sets_m1, steps: int, warmup: int, trains: int) -> list:
+    """configs[1] at 4 and 16 activation rows: the same four shapes and weight rotation, HBM bound (the weights are
+    still read once per call)."""
+    from kalosm_amd import synth
+    from kalosm_amd.fusor import Tensor
+
+    out = []
+    for m in (4, 16):
+        tot_ms, tot_bytes, per = 0.0, 0, []
+        for si, s in enumerate(sets_m1):
+            n, k = s["n"], s["k"]
+            t = dict(s, x=Tensor.from_slice(dev, synth.random_activation(m, k, seed=2100 + si)), y=Tensor(dev, (m, n), "f32"),
+                     bytes=synth.matvec_bytes(synth.Q4_K, n, k, m))
+            run_shape(t, warmup)
+            dev.sync()
+            ms, _ = timed_trains(dev, lambda: run_shape(t, steps, offset=warmup), trains)
+            tot_ms += ms
+            tot_bytes += t["bytes"]
+            per.append({"n": n, "k": k, "us_per_launch": round(ms * 1e3 / steps, 3)})
+        gbs = tot_bytes * steps / (tot_ms * 1e-3) / 1e9
+        out.append({"rows": m, "GBps": round(gbs, 1), "shapes": per,
+                    "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                 "frac": round(gbs / HBM_PEAK_GBS, 4)}})
+    return out
+
+
+def prefill_legs(dev, trains: int) -> dict:
     """configs[2]: Y = X . W^T with bf16 X [m, 4096] and Q6_K / Q8_0 W [14336, 4096]; configs[3]: causal attention,
-    f16, 32 query heads on 8 KV heads, head_dim 128.  Device time per call from events around 5 calls; TFLOP/s counts
-    2 m n k (matmul) and 4 s^2 d h / 2 (causal attention) against the 2.5 PFLOP/s dense f16 MFMA peak."""
+    f16, 32 query heads on 8 KV heads, head_dim 128, and its decode variant.  Median device time of `trains` calls;
+    TFLOP/s counts 2 m n k (matmul) and 4 s^2 d h / 2 (causal attention) against the 2.5 PFLOP/s dense f16 MFMA peak
+    (5 POP/s for the int8 variant); the decode variant counts K and V bytes against the 8 TB/s HBM peak."""
     from kalosm_amd import synth
     from kalosm_amd.fusor import MaskKind, QMatrix, Tensor
+
+    def med(fn):
+        for _ in range(2):
+            fn()
+        dev.sync()
+        ts = []
+        for _ in range(trains):
+            dev.timer_start()
+            fn()
+            ts.append(dev.timer_stop())
+        return statistics.median(ts)
+
+    def mfma(tf, peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s"):
+        return {"bound": "mfma", "achieved": round(tf, 1), "peak": peak, "unit": unit, "frac": round(tf / peak, 4)}
 
     res = {"matmul": [], "attention": [], "attention_decode": []}
     n, k = 14336, 4096
@@ -48,62 +153,35 @@ def prefill_legs(dev) -> dict:
         for m in (512, 2048):
             x = Tensor.from_slice(dev, synth.to_bf16_bits(synth.random_activation(m, k, seed=8)), dtype="bf16")
             y = Tensor(dev, (m, n), "f32")
-            for _ in range(2):
-                x.q_mat_mul(q, out=y)
-            dev.sync()
-            dev.timer_start()
-            for _ in range(5):
-                x.q_mat_mul(q, out=y)
-            ms = dev.timer_stop() / 5
+            ms = med(lambda: x.q_mat_mul(q, out=y))
             tf = 2.0 * m * n * k / ms / 1e9
             res["matmul"].append({"weights": name, "activations": "bf16", "m": m, "n": n, "k": k,
-                                  "us": round(ms * 1e3, 1), "TFLOPs": round(tf, 1),
-                                  "frac_mfma_peak": round(tf / 2500.0, 4)})
+                                  "us": round(ms * 1e3, 1), "roofline": mfma(tf)})
             if ty == synth.Q8_0:  # the integer variant: f32 activations quantised per 32 inside the call, int8 MFMA
                 xf = Tensor.from_slice(dev, synth.random_activation(m, k, seed=8))
-                for _ in range(2):
-                    xf.q_mat_mul_q8(q, out=y)
-                dev.sync()
-                dev.timer_start()
-                for _ in range(5):
-                    xf.q_mat_mul_q8(q, out=y)
-                ms = dev.timer_stop() / 5
+                ms = med(lambda: xf.q_mat_mul_q8(q, out=y))
                 tf = 2.0 * m * n * k / ms / 1e9
                 res["matmul"].append({"weights": name, "activations": "Q8_0 per 32 (int8 MFMA)", "m": m, "n": n, "k": k,
-                                      "us": round(ms * 1e3, 1), "TOPs": round(tf, 1),
-                                      "frac_int8_mfma_peak": round(tf / 5000.0, 4)})
+                                      "us": round(ms * 1e3, 1), "roofline": mfma(tf, MFMA_I8_PEAK_TOPS, "TOP/s")})
     # the decoder's own prefill projections with few output tiles (k split over workgroups): f32 activations
     for ty, name, n2, k2 in ((synth.Q4_K, "Q4_K", 4096, 4096), (synth.Q6_K, "Q6_K", 4096, 14336)):
         q = QMatrix.from_raw_bytes(dev, (n2, k2), synth.random_weight(ty, n2, k2, seed=9), ty)
         m = 512
         xf = Tensor.from_slice(dev, synth.random_activation(m, k2, seed=10))
         y = Tensor(dev, (m, n2), "f32")
-        for _ in range(2):
-            xf.q_mat_mul(q, out=y)
-        dev.sync()
-        dev.timer_start()
-        for _ in range(5):
-            xf.q_mat_mul(q, out=y)
-        ms = dev.timer_stop() / 5
+        ms = med(lambda: xf.q_mat_mul(q, out=y))
         tf = 2.0 * m * n2 * k2 / ms / 1e9
         res["matmul"].append({"weights": name, "activations": "f32", "m": m, "n": n2, "k": k2, "us": round(ms * 1e3, 1),
-                              "TFLOPs": round(tf, 1), "frac_mfma_peak": round(tf / 2500.0, 4)})
+                              "roofline": mfma(tf)})
     h, hkv, d = 32, 8, 128
     for s in (512, 2048, 8192):
         rng = np.random.default_rng(s)
         qt, kt, vt = (Tensor.from_slice(dev, rng.standard_normal((1, hh, s, d)).astype(np.float16), "f16")
                       for hh in (h, hkv, hkv))
         ot = Tensor(dev, (1, h, s, d), "f16")
-        for _ in range(2):
-            qt.flash_attention(kt, vt, 1 / np.sqrt(d), MaskKind.Causal, out=ot)
-        dev.sync()
-        dev.timer_start()
-        for _ in range(5):
-            qt.flash_attention(kt, vt, 1 / np.sqrt(d), MaskKind.Causal, out=ot)
-        ms = dev.timer_stop() / 5
+        ms = med(lambda: qt.flash_attention(kt, vt, 1 / np.sqrt(d), MaskKind.Causal, out=ot))
         tf = 4.0 * s * s * d * h / 2 / ms / 1e9
-        res["attention"].append({"seq": s, "us": round(ms * 1e3, 1), "TFLOPs": round(tf, 1),
-                                 "frac_mfma_peak": round(tf / 2500.0, 4)})
+        res["attention"].append({"seq": s, "us": round(ms * 1e3, 1), "roofline": mfma(tf)})
     # configs[3], decode variant: one query per head against a cache of L keys (f16 K / V), HBM bound:
     # bytes = K and V once (2 * hkv * L * d * 2) + the query and the output (2 * h * d * 2); caches rotate over
     # more than the Infinity Cache
@@ -118,36 +196,104 @@ def prefill_legs(dev) -> dict:
             kvs.append((Tensor.from_slice(dev, base_k, "f16"), Tensor.from_slice(dev, base_v, "f16")))
         qt = Tensor.from_slice(dev, rng.standard_normal((1, h, 1, d)).astype(np.float16), "f16")
         ot = Tensor(dev, (1, h, 1, d), "f16")
-        reps = 200
-        for i in range(20):
-            qt.flash_attention(*kvs[i % len(kvs)], 1 / np.sqrt(d), None, out=ot)
+        reps = 100
+
+        def train(off=0):
+            for i in range(reps):
+                qt.flash_attention(*kvs[(off + i) % len(kvs)], 1 / np.sqrt(d), None, out=ot)
+
+        train()
         dev.sync()
-        dev.timer_start()
-        for i in range(reps):
-            qt.flash_attention(*kvs[i % len(kvs)], 1 / np.sqrt(d), None, out=ot)
-        ms = dev.timer_stop() / reps
+        ms, _ = timed_trains(dev, lambda: train(7), trains)
+        ms /= reps
         nbytes = kv_bytes + 2 * h * d * 2
+        gbs = nbytes / ms / 1e6
         res["attention_decode"].append({"kv_len": L, "us": round(ms * 1e3, 2), "bytes": nbytes,
-                                        "GBps": round(nbytes / ms / 1e6, 1), "frac_hbm_peak": round(nbytes / ms / 1e6 / 8000.0, 4),
-                                        "cache_copies_rotated": len(kvs)})
+                                        "cache_copies_rotated": len(kvs),
+                                        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                                                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4)}})
         del kvs
     return res
+
+
+def calibration(dev, trains: int, use_graph: bool) -> dict:
+    """What one dependent launch costs on this device whatever the kernel does: an empty kernel, and a plain
+    streaming read of the byte counts of the benchmark's matrices (rotating like the weights do)."""
+    from kalosm_amd.fusor import Tensor
+    import ctypes as C
+
+    L = 100
+    out = {"launches_per_train": L, "empty_us": {}, "read": []}
+    for wg, th in ((1, 64), (256, 1024)):
+        ms, _ = timed_trains(dev, lambda: [dev._lib.fh_probe_empty(dev._h, wg, th) for _ in range(L)], trains, use_graph)
+        out["empty_us"]["%dx%d" % (wg, th)] = round(ms * 1e3 / L, 3)
+    total = 768 << 20
+    buf = Tensor(dev, (total,), "u8")
+    dev._lib.fh_memset(dev._h, C.c_void_p(buf.ptr), 1, total)
+    for nbytes in (2359296, 9437184, 33030144, 66060288, 430940160):
+        used = nbytes // 16384 * 16384
+        copies = max(1, total // used)
+
+        def train():
+            for i in range(L):
+                dev._lib.fh_probe_read(dev._h, C.c_void_p(buf.ptr + (i % copies) * used), used)
+
+        train()
+        dev.sync()
+        ms, _ = timed_trains(dev, train, trains, use_graph)
+        us = ms * 1e3 / L
+        out["read"].append({"bytes": used, "us": round(us, 3), "GBps": round(used / us / 1e3, 1)})
+    return out
+
+
+def e2e_check(model, weights, cfg, prompt_len=16, steps=8):
+    """The decoder that was just timed against the CPU checker's decoder on the same weights, outside the timed
+    region: logits of a short prompt within tolerance and the greedy ids that follow (a step whose two best checker
+    logits are closer than 2e-2 may differ)."""
+    from kalosm_amd import synth
+    from oracle import oracle
+
+    ocfg = dict(cfg, type_attn=synth.Q4_K, type_ffn_gate_up=synth.Q4_K, type_ffn_down=synth.Q6_K, type_embd=synth.Q4_K,
+                type_output=synth.Q6_K)
+    ref = oracle.Llama(ocfg, weights)
+    prompt = np.random.default_rng(99).integers(0, cfg["vocab"], prompt_len)
+    model.reset()
+    lg = model.forward(prompt)
+    wl = ref.forward(prompt)
+    diff = np.abs(lg - wl)
+    ok = bool(((diff <= 1e-2) | (diff <= 1e-3 * np.maximum(np.abs(lg), np.abs(wl)))).all())
+    tok = oracle.argmax(wl)
+    got, _ = model.decode_greedy(tok, steps)
+    want, t, agree = [], tok, 0
+    for i in range(steps):
+        w2 = ref.forward([t])
+        srt = np.sort(w2)
+        t = oracle.argmax(w2)
+        want.append(t)
+        if int(got[i]) != t:
+            ok = ok and float(srt[-1] - srt[-2]) < 2e-2
+            break
+        agree += 1
+    return {"ok": ok, "prompt_len": prompt_len, "logits_max_abs_err": float(diff.max()), "greedy_steps_checked": steps,
+            "greedy_steps_equal": agree, "tokens": [int(x) for x in got[:steps]], "checker_tokens": want}
 
 
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--m", type=int, default=1, help="activation rows (decode batch)")
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--trains", type=int, default=7, help="replays of each shape's K-launch train; the median is reported")
+    ap.add_argument("--m", type=int, default=1, help="activation rows (decode batch) of the headline leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
-    ap.add_argument("--e2e", action="store_true", help="(default) also run the 8B-architecture decoder and report tok/s")
-    ap.add_argument("--no-e2e", action="store_true", help="skip the 8B-architecture decoder leg (about 10 s)")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the 8B-architecture decoder leg")
+    ap.add_argument("--no-e2e-check", action="store_true", help="skip the decoder's comparison with the CPU checker")
+    ap.add_argument("--no-legs", action="store_true", help="skip the batch, prefill and attention legs")
     ap.add_argument("--e2e-eager", action="store_true",
-                    help="also run 32 decode steps of the decoder with stream launches (for a kernel tracer)")
-    ap.add_argument("--prefill", action="store_true",
-                    help="also time the prefill matmul (configs[2]) and the causal prefill attention (configs[3])")
+                    help="run 32 decode steps of the decoder with stream launches instead (for a kernel tracer)")
+    ap.add_argument("--prefill", action="store_true", help="(default) kept for older command lines")
     ap.add_argument("--no-graph", action="store_true", help="launch on the stream instead of replaying a recorded graph")
+    ap.add_argument("--calib", action="store_true", help="also time an empty kernel and plain streaming reads")
     ap.add_argument("--calib-copy", action="store_true", help="append 4 device copies of 256 MiB (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -156,53 +302,25 @@ def main() -> int:
         return 2
 
     from kalosm_amd import synth
-    from kalosm_amd.fusor import Device, QMatrix, Tensor
+    from kalosm_amd.fusor import Device, Tensor
 
     dev = Device.gpu(0)
     info = dev.info()
     m = args.m
     ty = synth.Q4_K
+    sets = matvec_sets(dev, ty, m)
 
-    # ---- resident inputs
-    sets = []
-    for si, (n, k) in enumerate(SHAPES):
-        wbytes = n * (k // 256) * 144
-        copies = max(2, -(-ROTATE_BYTES // wbytes))
-        raw = synth.random_weight(ty, n, k, seed=1000 + si)
-        qs = [QMatrix.from_raw_bytes(dev, (n, k), raw, ty) for _ in range(copies)]
-        x = Tensor.from_slice(dev, synth.random_activation(m, k, seed=2000 + si))
-        y = Tensor(dev, (m, n), "f32")
-        sets.append(dict(n=n, k=k, qs=qs, x=x, y=y, raw=raw, bytes=synth.matvec_bytes(ty, n, k, m)))
-
-    def run_shape(s, launches, offset=0):
-        qs, x, y = s["qs"], s["x"], s["y"]
-        for i in range(launches):
-            x.q_mat_mul(qs[(offset + i) % len(qs)], out=y)
-
-    # ---- warmup, then the timed steps (per shape trains inside one bracketed region)
-    # The K launches of a shape are recorded once and replayed as one submission (the reference submits one
-    # command buffer per resolve); host launch overhead of the Python/ctypes loop stays out of the device time.
+    # ---- warmup, then the timed steps.  The K launches of a shape are recorded once and replayed as one submission
+    # (the reference submits one command buffer per resolve); the Python/ctypes loop stays out of the device time.
     for s in sets:
         run_shape(s, args.warmup)
     dev.sync()
-    per_shape_ms = []
-    if args.no_graph:  # plain stream launches (for runs under a kernel tracer, which does not follow graph replays)
-        t_wall0 = time.perf_counter()
-        for s in sets:
-            dev.timer_start()
-            run_shape(s, args.steps, offset=args.warmup)
-            per_shape_ms.append(dev.timer_stop())
-    else:
-        graphs = []
-        for s in sets:
-            dev.graph_begin()
-            run_shape(s, args.steps, offset=args.warmup)
-            graphs.append(dev.graph_end())
-        t_wall0 = time.perf_counter()
-        for g in graphs:
-            dev.timer_start()
-            g.launch()
-            per_shape_ms.append(dev.timer_stop())
+    per_shape_ms, all_ms = [], []
+    t_wall0 = time.perf_counter()
+    for s in sets:
+        ms, every = timed_trains(dev, lambda: run_shape(s, args.steps, offset=args.warmup), args.trains, not args.no_graph)
+        per_shape_ms.append(ms)
+        all_ms.append(every)
     if args.calib_copy:  # a device-to-device copy of known size, to scale the FETCH_SIZE / WRITE_SIZE counters
         nbytes = 256 << 20
         a, b = Tensor(dev, (nbytes,), "u8"), Tensor(dev, (nbytes,), "u8")
@@ -215,9 +333,11 @@ def main() -> int:
     step_bytes = sum(s["bytes"] for s in sets)
     value = step_bytes * args.steps / (total_ms * 1e-3) / 1e9
     shapes_out = []
-    for s, ms in zip(sets, per_shape_ms):
+    for s, ms, every in zip(sets, per_shape_ms, all_ms):
         us = ms * 1e3 / args.steps
         shapes_out.append({"n": s["n"], "k": s["k"], "us_per_launch": round(us, 3),
+                           "us_per_launch_min_max": [round(min(every) * 1e3 / args.steps, 3),
+                                                     round(max(every) * 1e3 / args.steps, 3)],
                            "GBps": round(s["bytes"] / (us * 1e-6) / 1e9, 1),
                            "frac_hbm_peak": round(s["bytes"] / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
     # dominant kernel: the Q4_K MFMA matvec k_qmv_q4k_m1, one launch per matvec (activation staging is inside it);
@@ -226,23 +346,29 @@ def main() -> int:
     launches = args.steps * len(sets)
     avg_us = total_ms * 1e3 / launches
     achieved = (step_bytes / len(sets)) / (avg_us * 1e-6) / 1e9
+    traffic, traffic_commit = measured_traffic()
     out = {
         "metric": "Q4_K matvec GB/s (% HBM peak); Q4_K_M 8B-arch decode tok/s, batch 1, 1 GPU",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "trains": args.trains,
         "ms_per_step": round(total_ms / args.steps, 6), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: Q4_K decode matvec at Llama-3-8B layer shapes "
                                "(4096x4096, 1024x4096, 14336x4096, 4096x14336), batch %d, one launch each per step" % m,
                    "batch": m, "weights_rotated_bytes_per_shape": ROTATE_BYTES, "device": info["name"],
-                   "compute_units": info["compute_units"]},
+                   "compute_units": info["compute_units"],
+                   "timing": "median of %d replays of each shape's %d-launch train" % (args.trains, args.steps)},
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "shapes": shapes_out,
         "wall_ms_timed_region": round(wall_ms, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH if m == 1 else None,
-                     "kernel": "k_qmv_q4k_m1 (instances <1,1>, <2,1>, <1,4>: tiles, blocks per wavefront)", "avg_launch_us": round(avg_us, 3),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic if m == 1 else None,
+                     "traffic_source": ("profiles/%s at commit %s" % (os.path.basename(TRAFFIC_PROFILE), traffic_commit))
+                     if traffic and m == 1 else None,
+                     "kernel": "k_qmv_q4k_m1", "avg_launch_us": round(avg_us, 3),
                      "algorithmic_bytes_per_launch": step_bytes // len(sets)},
     }
+    rc = 0
 
     # ---- CPU baseline: the checker's q_mat_mul (a C restatement of fusor-ml/cpu, not the Rust binary),
     # same shapes and inputs, all host cores, bounded repetitions
@@ -280,17 +406,35 @@ def main() -> int:
             worst = max(worst, float(diff.max()))
         out["parity_max_abs_err"] = worst
 
-    if not args.no_e2e and not args.e2e_eager:
-        from kalosm_amd import e2e
-        out["e2e"] = e2e.run(dev)
+    if args.calib:
+        out["calibration"] = calibration(dev, args.trains, not args.no_graph)
+    if not args.no_legs:
+        out["batch"] = batch_leg(dev, sets, args.steps, args.warmup, args.trains)
+    for s in sets:
+        s["qs"].clear()
+    del sets
+    if not args.no_legs:
+        out["prefill"] = prefill_legs(dev, max(3, min(args.trains, 5)))
+
     if args.e2e_eager:
         from kalosm_amd import e2e
         out["e2e_eager"] = e2e.run(dev, steps=32, repeats=1, use_graph=False)
-    if args.prefill:
-        out["prefill"] = prefill_legs(dev)
+    elif not args.no_e2e:
+        from kalosm_amd import e2e
+        check = not (args.no_e2e_check or args.no_cpu)
+        weights = {}
+        res, model, cfg = e2e.run(dev, keep=(lambda n_, a: weights.__setitem__(n_, a)) if check else None, return_model=True)
+        res["roofline"] = {"bound": "hbm", "achieved": res["weights_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": res["frac_hbm_peak"]}
+        if check:
+            res["checker"] = e2e_check(model, weights, cfg)
+            if not res["checker"]["ok"]:
+                print("bench.py: the decoder's logits / greedy tokens differ from the CPU checker's", file=sys.stderr)
+                rc = 1
+        out["e2e"] = res
 
     print(json.dumps(out))
-    return 0
+    return rc
 
 
 if __name__ == "__main__":

@@ -94,6 +94,12 @@ fh_status fh_copy(fh_device *dev, void *dst_dev, const void *src_dev, size_t byt
 fh_status fh_timer_start(fh_device *dev);
 fh_status fh_timer_stop(fh_device *dev, float *elapsed_ms); /* blocks until the stream reaches it */
 
+/* Measurement probes (same purpose as the timestamp queries above): an empty kernel of `workgroups` x `threads`,
+ * and a plain streaming read of `bytes` (a multiple of 16384) from src_dev.  A benchmark prices the matvec kernels
+ * against what these cost on the same device in the same launch pattern. */
+fh_status fh_probe_empty(fh_device *dev, int32_t workgroups, int32_t threads);
+fh_status fh_probe_read(fh_device *dev, const void *src_dev, size_t bytes);
+
 /* Record-and-replay of a sequence of operator calls (the reference records a lazy graph and submits one
  * command buffer per resolve, fusor-ml/core/src/compute_graph/resolve/run.rs).  Between begin and end the
  * operator calls on `dev` are captured into a hipGraph instead of running; fh_graph_launch replays them.

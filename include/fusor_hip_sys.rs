@@ -142,6 +142,8 @@ extern "C" {
     pub fn fh_copy(dev: *mut FhDevice, dst_dev: *mut c_void, src_dev: *const c_void, bytes: usize) -> FhStatus;
     pub fn fh_timer_start(dev: *mut FhDevice) -> FhStatus;
     pub fn fh_timer_stop(dev: *mut FhDevice, elapsed_ms: *mut f32) -> FhStatus;
+    pub fn fh_probe_empty(dev: *mut FhDevice, workgroups: i32, threads: i32) -> FhStatus;
+    pub fn fh_probe_read(dev: *mut FhDevice, src_dev: *const c_void, bytes: usize) -> FhStatus;
     pub fn fh_graph_begin(dev: *mut FhDevice) -> FhStatus;
     pub fn fh_graph_end(dev: *mut FhDevice, out: *mut *mut FhGraph) -> FhStatus;
     pub fn fh_graph_launch(g: *mut FhGraph) -> FhStatus;

@@ -63,6 +63,8 @@ SIGNATURES = {
     "fh_copy": [_p, _p, _p, _sz],
     "fh_timer_start": [_p],
     "fh_timer_stop": [_p, C.POINTER(_f32)],
+    "fh_probe_empty": [_p, _i32, _i32],
+    "fh_probe_read": [_p, _p, C.c_size_t],
     "fh_graph_begin": [_p],
     "fh_graph_end": [_p, _pp],
     "fh_graph_launch": [_p],

@@ -162,6 +162,41 @@ extern "C" fh_status fh_timer_stop(fh_device *dev, float *elapsed_ms) {
     return FH_OK;
 }
 
+// ---------------------------------------------------------------- measurement probes
+// What a launch costs on this device before any arithmetic: an empty kernel, and a plain streaming read (16 bytes
+// per lane and request, 4 KB per wavefront, four requests in flight per lane).  The matvec kernels are priced
+// against these, not only against the nominal HBM peak.
+__global__ void k_probe_empty(uint32_t *p) {
+    if (p && threadIdx.x == 9999) *p = 1;
+}
+__global__ __launch_bounds__(256) void k_probe_read(const uint4 *__restrict__ src, uint32_t *out) {
+    const size_t wave = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint4 *p = src + wave * 256 + (threadIdx.x & 63);
+    uint4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) v[u] = p[u * 64];
+    uint32_t a = 0;
+#pragma unroll
+    for (int u = 0; u < 4; u++) a ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    if (a == 0x12345678u) out[0] = a; // keeps the loads alive; practically never true
+}
+
+extern "C" fh_status fh_probe_empty(fh_device *dev, int32_t workgroups, int32_t threads) {
+    FH_REQUIRE(dev && workgroups > 0 && threads > 0 && threads <= 1024, "bad probe launch");
+    k_probe_empty<<<dim3((unsigned)workgroups), dim3((unsigned)threads), 0, dev->stream>>>((uint32_t *)dev->small_buf);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+extern "C" fh_status fh_probe_read(fh_device *dev, const void *src_dev, size_t bytes) {
+    FH_REQUIRE(dev && src_dev, "NULL argument");
+    FH_REQUIRE(bytes >= 16384 && bytes % 16384 == 0 && bytes / 16384 <= 0x7FFFFFFFu, "bytes must be a multiple of 16384");
+    k_probe_read<<<dim3((unsigned)(bytes / 16384)), dim3(256), 0, dev->stream>>>((const uint4 *)src_dev,
+                                                                              (uint32_t *)dev->small_buf);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
 fh_status fh_dev_scratch(fh_device *dev, void **buf, size_t *cap, size_t need) {
     if (*cap >= need) return FH_OK;
     if (dev->capturing)

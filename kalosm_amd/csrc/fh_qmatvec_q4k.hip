@@ -69,6 +69,10 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     // SwiGLU with one tile per wavefront: the "tile" is rows 8h .. 8h+7 of a gate tile (columns 0-7 of the MFMA) and
     // the same rows of the matching up tile (columns 8-15), h = workgroup parity: workgroups half as heavy as with a
     // whole gate and a whole up tile, which divides the Llama FFN evenly over the compute units
+    // Q4_K: the sums of the activations per sub-block (they multiply the block minimums) come from one more MFMA per
+    // block, whose B operand is the constant code 1 and whose A operand is the whole image (every row at once),
+    // instead of from adds and lane exchanges in the staging
+    constexpr bool ONES = FMT == FH_Q4_K;
     constexpr bool HP = EPI == FH_EPI_SWIGLU && TPW == 1;
     constexpr int NT = (EPI == FH_EPI_SWIGLU && !HP) ? 2 : 1;
     constexpr int TOUT = TPW / NT; // output tiles of the workgroup
@@ -206,7 +210,9 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
             ss += s2;
             v = make_float4(v.x * wv[i].x, v.y * wv[i].y, v.z * wv[i].z, v.w * wv[i].w);
         }
-        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        float amax;
+        asm("v_max3_f32 %0, |%1|, |%2|, |%3|" : "=v"(amax) : "v"(v.x), "v"(v.y), "v"(v.z));
+        asm("v_max_f32_e64 %0, %1, |%2|" : "=v"(amax) : "v"(amax), "v"(v.w));
         // non-negative floats order like their bit patterns: the cross-lane maximum is an integer one
         uint32_t am = __float_as_uint(amax);
         am = max(am, dpp_u32<DPP_XOR1>(am));
@@ -221,28 +227,33 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         e = e > 100 ? 100 : (e < -100 ? -100 : e);
         const int eo = e - (FMT == FH_Q8_0 ? 0 : 4 * (FMT == FH_Q4_0 ? half : s & 1)); // high nibbles: codes x 16
         const float sc = __uint_as_float((uint32_t)(eo + 127) << 23);
-        const float xq[4] = {v.x, v.y, v.z, v.w};
-        _Float16 hi[4], lo[4];
-#pragma unroll
-        for (int c = 0; c < 4; c++) { // x * sc is exact (a power of two), so the fused form rounds like the split one
-            hi[c] = (_Float16)(xq[c] * sc);
-            lo[c] = (_Float16)__builtin_fmaf(xq[c], sc, -(float)hi[c]);
-        }
-        const _Float16 oh[4] = {hi[0], hi[2], hi[1], hi[3]}, ol[4] = {lo[0], lo[2], lo[1], lo[3]};
+        // hi = f16(x * sc), lo = f16(x * sc - hi) (x * sc is exact, a power of two, so the fused form rounds once),
+        // written straight into the halves of the packed words in operand order (elements 0, 2 | 1, 3)
         uint2 ph, pl;
-        __builtin_memcpy(&ph, oh, 8);
-        __builtin_memcpy(&pl, ol, 8);
+        asm("v_fma_mixlo_f16 %0, %1, %2, 0" : "=v"(ph.x) : "v"(v.x), "v"(sc));
+        asm("v_fma_mixlo_f16 %0, %1, %2, 0" : "=v"(ph.y) : "v"(v.y), "v"(sc));
+        asm("v_fma_mixhi_f16 %0, %1, %2, 0" : "+v"(ph.x) : "v"(v.z), "v"(sc));
+        asm("v_fma_mixhi_f16 %0, %1, %2, 0" : "+v"(ph.y) : "v"(v.w), "v"(sc));
+        asm("v_fma_mixlo_f16 %0, %1, %2, -%3 op_sel_hi:[0,0,1]" : "=v"(pl.x) : "v"(v.x), "v"(sc), "v"(ph.x));
+        asm("v_fma_mixlo_f16 %0, %1, %2, -%3 op_sel_hi:[0,0,1]" : "=v"(pl.y) : "v"(v.y), "v"(sc), "v"(ph.y));
+        asm("v_fma_mixhi_f16 %0, %1, %2, -%3 op_sel:[0,0,1] op_sel_hi:[0,0,1]" : "+v"(pl.x) : "v"(v.z), "v"(sc), "v"(ph.x));
+        asm("v_fma_mixhi_f16 %0, %1, %2, -%3 op_sel:[0,0,1] op_sel_hi:[0,0,1]" : "+v"(pl.y) : "v"(v.w), "v"(sc), "v"(ph.y));
         uint2 *dst = (uint2 *)(img + b * Q4K_IMG + (s * 4 + gg) * 2);
         dst[half] = ph;     // hi
         dst[2 + half] = pl; // lo
         if (lane == 0) img[b * Q4K_IMG + 64] = make_uint4(0, 0, 0, 0);
-        float s4 = (v.x + v.y) + (v.z + v.w);
-        s4 += dpp_f32<DPP_XOR1>(s4);
-        s4 += dpp_f32<DPP_XOR2>(s4);
-        s4 += dpp_f32<DPP_HALF_MIRROR>(s4);
-        if ((lane & 7) == 0) {
-            sf[b * 16 + s] = s4;
-            sf[b * 16 + 8 + s] = __uint_as_float((uint32_t)((FMT == FH_Q8_0 ? 0 : 24) - e + 127) << 23);
+        const float fct = __uint_as_float((uint32_t)((FMT == FH_Q8_0 ? 0 : 24) - e + 127) << 23);
+        if constexpr (ONES) {
+            if ((lane & 7) == 0) sf[b * 16 + 8 + s] = fct;
+        } else {
+            float s4 = (v.x + v.y) + (v.z + v.w);
+            s4 += dpp_f32<DPP_XOR1>(s4);
+            s4 += dpp_f32<DPP_XOR2>(s4);
+            s4 += dpp_f32<DPP_HALF_MIRROR>(s4);
+            if ((lane & 7) == 0) {
+                sf[b * 16 + s] = s4;
+                sf[b * 16 + 8 + s] = fct;
+            }
         }
     }
     if (IN == 1) {
@@ -258,8 +269,8 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     // per-lane operand address of each step: its own sub-block's (hi|lo) in step mysb, the zero slot otherwise.
     // Lanes with (lane >> 1) % 8 == st are bits 2 st, 2 st + 1 of every 16.
     uint32_t pa[8];
+    const uint32_t own = lds_addr(img + b0 * MR * Q4K_IMG + (mysb * 4 + g) * 2 + part);
     {
-        const uint32_t own = lds_addr(img + b0 * MR * Q4K_IMG + (mysb * 4 + g) * 2 + part);
         const uint32_t zero = lds_addr(img + b0 * MR * Q4K_IMG + 64);
 #pragma unroll
         for (int st = 0; st < 8; st++) pa[st] = sel_lanes(0x0003000300030003ull << (2 * st), own, zero);
@@ -291,6 +302,21 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         for (int tp = 0; tp < TPW; tp++)
 #pragma unroll
             for (int mr = 0; mr < MR; mr++) dd[tp][mr] = floatx4{0.f, 0.f, 0.f, 0.f};
+        // rows 2s, 2s + 1 of dsum: the sum of the staged hi / lo values of sub-block s (the same in every
+        // column, so one product serves all tiles)
+        floatx4 dsum[ONES ? MR : 1];
+        if constexpr (ONES) {
+            const uint4 one = make_uint4(0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u); // f16 1.0
+            half8 ov;
+            __builtin_memcpy(&ov, &one, 16);
+#pragma unroll
+            for (int mr = 0; mr < MR; mr++) {
+                const uint4 ao = lds_read16(own + (r * MR + mr) * Q4K_IMG * 16);
+                half8 av;
+                __builtin_memcpy(&av, &ao, 16);
+                dsum[mr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, ov, floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+            }
+        }
 #pragma unroll
         for (int st = 0; st < 8; st++) {
             const int t = (r * 8 + st) * MR;
@@ -330,8 +356,14 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         }
 #pragma unroll
         for (int mr = 0; mr < MR; mr++) {
-            const float2 sx = *(const float2 *)(psf + (r * MR + mr) * 16);
             const float2 fc = *(const float2 *)(psf + (r * MR + mr) * 16 + 8);
+            float2 sx;
+            if constexpr (ONES) { // odd sub-blocks are staged 16 times lower (their codes are 16 times higher)
+                sx.x = (dsum[mr][0] + dsum[mr][1]) * (fc.x * 0x1p-24f);
+                sx.y = (dsum[mr][2] + dsum[mr][3]) * (fc.y * 0x1p-20f);
+            } else {
+                sx = *(const float2 *)(psf + (r * MR + mr) * 16);
+            }
 #pragma unroll
             for (int tp = 0; tp < TPW; tp++) {
                 const uint4 h = w[tp][r].h;

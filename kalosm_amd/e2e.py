@@ -12,10 +12,12 @@ from .llama import Model
 
 def run(dev, cfg: dict | None = None, prompt_len: int = 512, steps: int = 256, seed: int = 0, sigma: float = 1e-4,
         kv_dtype: str = "f32", repeats: int = 2, prefill_chunk: int = 512, use_graph: bool = True,
-        sampled: bool = True) -> dict:
+        sampled: bool = True, keep=None, return_model: bool = False):
+    """`keep(name, array)` receives every weight tensor as it is generated (for a caller that checks the decoder
+    against something else afterwards); with return_model the result is (report, model, cfg)."""
     cfg = dict(cfg or synth.LLAMA3_8B)
     t0 = time.perf_counter()
-    m = Model.random_init(dev, cfg, seed=seed, sigma=sigma, kv_dtype=kv_dtype, use_graph=use_graph)
+    m = Model.random_init(dev, cfg, seed=seed, sigma=sigma, kv_dtype=kv_dtype, use_graph=use_graph, keep=keep)
     load_s = time.perf_counter() - t0
     rng = np.random.default_rng(seed + 1)
     prompt = rng.integers(0, cfg["vocab"], prompt_len)
@@ -54,9 +56,10 @@ def run(dev, cfg: dict | None = None, prompt_len: int = 512, steps: int = 256, s
                 sbest, stoks = ms, out
         samp = {"sampler": "mirostat2 top_k 64 temperature 0.8 penalty 1.3 window 64", "tok_per_s": round(steps / (sbest * 1e-3), 1),
                 "ms_per_token": round(sbest / steps, 4), "distinct_tokens": int(len(set(stoks.tolist())))}
-    return {"tok_per_s": round(tok_s, 1), "ms_per_token": round(best / steps, 4), "steps": steps,
+    report = {"tok_per_s": round(tok_s, 1), "ms_per_token": round(best / steps, 4), "steps": steps,
             "prompt_len": prompt_len, "graph_replay": use_graph, "prefill_ms_host_clock": round(prefill_ms, 1), "kv_dtype": kv_dtype,
             "weight_bytes_per_token": wbytes, "weights_GBps": round(wbytes * tok_s / 1e9, 1),
             "frac_hbm_peak": round(wbytes * tok_s / 8e12, 4), "load_seconds": round(load_s, 1),
             "first_tokens": [int(t) for t in toks[:8]], "config": {k: cfg[k] for k in ("n_layers", "d_model", "ffn", "vocab")},
             "sampled": samp}
+    return (report, m, cfg) if return_model else report
