@@ -227,6 +227,20 @@ fh_status fh_kvcache_append(fh_kvcache *c, int32_t layer, const float *k_dev, co
 fh_status fh_kvcache_view(const fh_kvcache *c, int32_t layer, int32_t *len, int32_t *capacity,
                           const void **k_dev, const void **v_dev);
 
+/* ------------------------------------------------------------------ dense matmul
+ * Tensor::matmul, fusor-ml/fusor/src/lib.rs:1094-1103 (CPU form fusor-ml/cpu/src/matmul.rs:226-352; f16:
+ * :159-179): C[b] = A[b] . B[b] with A [batch, m, k], B [batch, k, n], C contiguous [batch, m, n]; dtype FH_F32 or
+ * FH_F16 for all three.  A and B are views: element (b, i, j) of A is a_dev[b * a_sb + i * a_sr + j * a_sc] (element
+ * strides), likewise B, so transposed or sliced operands need no copy by the caller (the reference copies
+ * non-contiguous operands to scratch first, matmul.rs:299-328).  f32 operands are multiplied as exact two-term f16
+ * splits of values normalised per row of A and per column of B on the matrix cores with f32 accumulation (the
+ * reference's gemm kernel order is not pinned: results agree to f32 rounding); f16 results are rounded once from the
+ * f32 sum like the reference's f16 instantiation.  Dense F16 / F32 weight matrices of fh_qmatmul run through the
+ * same tiles from 17 activation rows on. */
+fh_status fh_matmul(fh_device *dev, int32_t dtype, const void *a_dev, int64_t a_sb, int64_t a_sr, int64_t a_sc,
+                    const void *b_dev, int64_t b_sb, int64_t b_sr, int64_t b_sc, int32_t batch, int32_t m,
+                    int32_t k, int32_t n, void *c_dev);
+
 /* --------------------------------------------------------------- attention
  * Tensor<4>::flash_attention(&k, &v, scale, Option<(&mask, MaskKind)>),
  * fusor-ml/fusor/src/composite/flash_attention.rs:58-109 (GQA: kv head = h / (hq / hkv)).

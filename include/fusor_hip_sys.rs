@@ -172,6 +172,7 @@ extern "C" {
     pub fn fh_kvcache_reset(c: *mut FhKvCache) -> FhStatus;
     pub fn fh_kvcache_append(c: *mut FhKvCache, layer: i32, k_dev: *const f32, v_dev: *const f32, sh: i64, st: i64, s: i32) -> FhStatus;
     pub fn fh_kvcache_view(c: *const FhKvCache, layer: i32, len: *mut i32, capacity: *mut i32, k_dev: *mut *const c_void, v_dev: *mut *const c_void) -> FhStatus;
+    pub fn fh_matmul(dev: *mut FhDevice, dtype: i32, a_dev: *const c_void, a_sb: i64, a_sr: i64, a_sc: i64, b_dev: *const c_void, b_sb: i64, b_sr: i64, b_sc: i64, batch: i32, m: i32, k: i32, n: i32, c_dev: *mut c_void) -> FhStatus;
     pub fn fh_flash_attention(dev: *mut FhDevice, dtype: i32, q_dev: *const c_void, q_sb: i64, q_sh: i64, q_st: i64, k_dev: *const c_void, v_dev: *const c_void, kv_sb: i64, kv_sh: i64, kv_st: i64, b: i32, hq: i32, hkv: i32, sq: i32, skv: i32, d: i32, scale: f32, mask_kind: i32, mask_dev: *const f32, out_dev: *mut c_void) -> FhStatus;
     pub fn fh_flash_attention_ex(dev: *mut FhDevice, q_dtype: i32, kv_dtype: i32, q_dev: *const c_void, q_sb: i64, q_sh: i64, q_st: i64, k_dev: *const c_void, v_dev: *const c_void, kv_sb: i64, kv_sh: i64, kv_st: i64, b: i32, hq: i32, hkv: i32, sq: i32, skv: i32, d: i32, scale: f32, mask_kind: i32, mask_dev: *const f32, out_dev: *mut c_void) -> FhStatus;
     pub fn fh_flash_attention_decode_static(dev: *mut FhDevice, q_dtype: i32, kv_dtype: i32, q_dev: *const c_void, k_dev: *const c_void, v_dev: *const c_void, kv_sh: i64, kv_st: i64, hq: i32, hkv: i32, d: i32, scale: f32, skv: i32, out_dev: *mut c_void) -> FhStatus;

@@ -91,6 +91,7 @@ SIGNATURES = {
     "fh_kvcache_reset": [_p],
     "fh_kvcache_append": [_p, _i32, _p, _p, _i64, _i64, _i32],
     "fh_kvcache_view": [_p, _i32, C.POINTER(_i32), C.POINTER(_i32), _pp, _pp],
+    "fh_matmul": [_p, _i32, _p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _p],
     "fh_flash_attention": [_p, _i32, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32,
                            _f32, _i32, _p, _p],
     "fh_flash_attention_ex": [_p, _i32, _i32, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _i32, _i32,

@@ -118,6 +118,9 @@ struct fh_qmatrix {
     int rec_bytes = 0;
     uint8_t *data = nullptr; // device
     size_t bytes = 0;
+    // dense f32 rows on the matrix cores: a power of two that brings the largest |w| into [2^14, 2^15), so that the
+    // f16 pair hi + lo of w * wscale keeps 22 bits for every value that matters next to the largest one
+    float wscale = 1.f;
 };
 
 // Weight types kept in the file's own row-major block order (no tiled re-layout): dense f32 / f16 rows and the
@@ -159,9 +162,10 @@ struct QView {
     const uint8_t *data;
     int64_t n, k, kb, recs;
     int rec_bytes;
+    float wscale = 1.f, winv = 1.f; // dense f32 rows: decode multiplies by wscale, the store by winv
 };
 static inline QView fh_view(const fh_qmatrix *q) {
-    QView v{q->data, q->n, q->k, q->kb, q->recs, q->rec_bytes};
+    QView v{q->data, q->n, q->k, q->kb, q->recs, q->rec_bytes, q->wscale, 1.f / q->wscale};
     return v;
 }
 
@@ -173,6 +177,8 @@ fh_status fh_launch_qmatvec_batch(const fh_qmatrix *q, const float *x, int m, fl
                                   const float *b);
 fh_status fh_launch_qmm_q8_mfma(const fh_qmatrix *q, const float *x, int m, float *y);
 fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y);
+// power of two for fh_qmatrix::wscale from the largest |w| of `count` f32 values on the device (blocking)
+fh_status fh_dense_wscale(fh_device *dev, const float *w_dev, int64_t count, float *wscale);
 enum { FH_EPI_NONE = 0, FH_EPI_ADD2 = 1, FH_EPI_SWIGLU = 2, FH_EPI_ROPEKV = 3, FH_EPI_ACC = 4 };
 fh_status fh_launch_q4k_rows(const fh_qmatrix *q, const float *x, int m, float *y, int epi, const float *a, const float *b);
 fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b);

@@ -129,6 +129,13 @@ extern "C" fh_status fh_qmatrix_from_gguf_bytes(fh_device *dev, uint32_t ggml_ty
             FH_FAIL(FH_ERR_HIP, "upload of a [%lld, %lld] type-%u weight failed: %s", (long long)n, (long long)k, ggml_type,
                     hipGetErrorString(e));
         }
+        if (ggml_type == FH_W_F32) { // for the matrix-core path of dense f32 rows
+            fh_status ws = fh_dense_wscale(dev, (const float *)q->data, n * k, &q->wscale);
+            if (ws != FH_OK) {
+                fh_qmatrix_free(q);
+                return ws;
+            }
+        }
         *out = q;
         return FH_OK;
     }
@@ -208,6 +215,7 @@ extern "C" fh_status fh_qmatrix_concat_rows(fh_device *dev, const fh_qmatrix *co
             FH_FAIL(FH_ERR_HIP, "hipMemcpyAsync failed: %s", hipGetErrorString(e));
         }
         off += parts[i]->bytes;
+        if (i == 0 || parts[i]->wscale < q->wscale) q->wscale = parts[i]->wscale; // the largest |w| decides
     }
     *out = q;
     return FH_OK;

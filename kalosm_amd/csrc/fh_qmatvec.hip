@@ -395,7 +395,10 @@ static fh_status qmm_check(const fh_qmatrix *q, const void *x, int m, const void
 extern "C" fh_status fh_qmatmul(const fh_qmatrix *q, const float *x_dev, int32_t m, float *y_dev) {
     FH_TRY(qmm_check(q, x_dev, m, y_dev));
     const int64_t mk = q->dev->opt_matmul_kernel;
-    if (((m > 16 && mk != 1) || mk >= 2) && !fh_is_plain(q->type)) return fh_launch_qmatmul_tile(q, x_dev, 0, m, y_dev);
+    // dense f16 / f32 weight rows (core/src/quantized/matmul/kernel.rs:132-193 routes them to the dense matmul) take
+    // the matrix-core tiles as well once there are rows to fill them
+    const bool dense = (q->type == FH_W_F16 || q->type == FH_W_F32) && q->k % 32 == 0;
+    if (((m > 16 && mk != 1) || mk >= 2) && (!fh_is_plain(q->type) || dense)) return fh_launch_qmatmul_tile(q, x_dev, 0, m, y_dev);
     return fh_launch_qmatvec(q, x_dev, m, y_dev, FH_EPI_NONE, nullptr, nullptr);
 }
 

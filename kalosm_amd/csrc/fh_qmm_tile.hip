@@ -16,15 +16,18 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 #define QMM_LDK 40 // halfs per LDS row: 32 + 8 padding (80 B stride: 16-byte reads of 16 rows hit 16 distinct chunks)
 
 // ------------------------------------------------------------------------------ activation planes
-// One workgroup per row.  xh / xl are [m, k] f16, rs[m] = 2^-e undoes the normalisation at the store.
-template <bool BF16>
-__global__ __launch_bounds__(256) void k_act_split(const void *__restrict__ xin, int k, _Float16 *__restrict__ xh,
-                                                    _Float16 *__restrict__ xl, float *__restrict__ rs) {
+// One workgroup per row.  xh / xl are [m, kp] f16 (zero from k to kp), rs[m] = 2^-e undoes the normalisation at the
+// store.  IN: 0 f32, 1 bf16, 2 f16 input; element c of row r is at r * srow + c * scol.
+template <int IN>
+__global__ __launch_bounds__(256) void k_act_split(const void *__restrict__ xin, int64_t srow, int64_t scol, int k, int kp,
+                                                    _Float16 *__restrict__ xh, _Float16 *__restrict__ xl,
+                                                    float *__restrict__ rs) {
     __shared__ float sh[4];
-    const int64_t off = (int64_t)blockIdx.x * k;
+    const int64_t off = (int64_t)blockIdx.x * srow, oo = (int64_t)blockIdx.x * kp;
     auto ld = [&](int c) -> float {
-        if (BF16) return __uint_as_float((uint32_t)((const uint16_t *)xin)[off + c] << 16);
-        return ((const float *)xin)[off + c];
+        if (IN == 1) return __uint_as_float((uint32_t)((const uint16_t *)xin)[off + c * scol] << 16);
+        if (IN == 2) return (float)((const _Float16 *)xin)[off + c * scol];
+        return ((const float *)xin)[off + c * scol];
     };
     float amax = 0.f;
     for (int c = threadIdx.x; c < k; c += 256) amax = fmaxf(amax, fabsf(ld(c)));
@@ -36,13 +39,38 @@ __global__ __launch_bounds__(256) void k_act_split(const void *__restrict__ xin,
     int e = 141 - (int)((__float_as_uint(amax) >> 23) & 0xFFu); // 14 - floor(log2 amax); zero / inf / nan clamp
     e = e > 100 ? 100 : (e < -100 ? -100 : e);
     const float sc = __uint_as_float((uint32_t)(e + 127) << 23);
-    for (int c = threadIdx.x; c < k; c += 256) {
-        const float v = ld(c) * sc;
+    for (int c = threadIdx.x; c < kp; c += 256) {
+        const float v = c < k ? ld(c) * sc : 0.f;
         const _Float16 h = (_Float16)v;
-        xh[off + c] = h;
-        if (!BF16) xl[off + c] = (_Float16)(v - (float)h);
+        xh[oo + c] = h;
+        if (IN != 1) xl[oo + c] = (_Float16)(v - (float)h);
     }
     if (threadIdx.x == 0) rs[blockIdx.x] = __uint_as_float((uint32_t)(127 - e) << 23);
+}
+
+// Rows of a dense right-hand side as the tile kernel's "weights": row r (one output column of the product) scaled by
+// its own power of two into the f16 range, written as f32 [rows, kp] (zero from k to kp); cs[r] = 2^-e for the store.
+template <bool F16>
+__global__ __launch_bounds__(256) void k_dense_rows(const void *__restrict__ bin, int64_t srow, int64_t scol, int k, int kp,
+                                                     float *__restrict__ out, float *__restrict__ cs) {
+    __shared__ float sh[4];
+    const int64_t off = (int64_t)blockIdx.x * srow, oo = (int64_t)blockIdx.x * kp;
+    auto ld = [&](int c) -> float {
+        if (F16) return (float)((const _Float16 *)bin)[off + c * scol];
+        return ((const float *)bin)[off + c * scol];
+    };
+    float amax = 0.f;
+    for (int c = threadIdx.x; c < k; c += 256) amax = fmaxf(amax, fabsf(ld(c)));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+    int e = 141 - (int)((__float_as_uint(amax) >> 23) & 0xFFu);
+    e = e > 100 ? 100 : (e < -100 ? -100 : e);
+    const float sc = __uint_as_float((uint32_t)(e + 127) << 23);
+    for (int c = threadIdx.x; c < kp; c += 256) out[oo + c] = c < k ? ld(c) * sc : 0.f;
+    if (threadIdx.x == 0) cs[blockIdx.x] = __uint_as_float((uint32_t)(127 - e) << 23);
 }
 
 // ------------------------------------------------------------------------------ weight slab decode
@@ -52,7 +80,22 @@ template <int T>
 __device__ __forceinline__ void decode8(const QView &q, int64_t tile16, int j, int g, int ks, float *w, int &p0, int &p1) {
     p0 = 8 * g;     // position of w[0..3]
     p1 = 8 * g + 4; // position of w[4..7]
-    if (T == FH_Q8_0) {
+    if (T == FH_W_F32 || T == FH_W_F16) { // dense rows [n][k]: row-major, no blocks
+        int64_t row = tile16 * 16 + j;
+        if (row >= q.n) row = q.n - 1; // rows past the end repeat the last one and are never stored
+        const int64_t at = row * q.k + (int64_t)ks * 32 + 8 * g;
+        if (T == FH_W_F32) {
+            const float4 a = *(const float4 *)((const float *)q.data + at), b = *(const float4 *)((const float *)q.data + at + 4);
+            w[0] = a.x * q.wscale; w[1] = a.y * q.wscale; w[2] = a.z * q.wscale; w[3] = a.w * q.wscale;
+            w[4] = b.x * q.wscale; w[5] = b.y * q.wscale; w[6] = b.z * q.wscale; w[7] = b.w * q.wscale;
+        } else {
+            const uint4 u = *(const uint4 *)((const _Float16 *)q.data + at);
+            _Float16 h[8];
+            __builtin_memcpy(h, &u, 16);
+#pragma unroll
+            for (int i = 0; i < 8; i++) w[i] = (float)h[i];
+        }
+    } else if (T == FH_Q8_0) {
         const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 1)) * 1088;
         const int u = ks & 1;
         const uint2 c = *(const uint2 *)(rec + (g * 16 + j) * 16 + 8 * u);
@@ -116,7 +159,8 @@ template <int T, int NTERM, int WGN, int WGM, int FN, int FM>
 __global__ __launch_bounds__(64 * WGN * WGM) void k_qmm_tile(QView q, const _Float16 *__restrict__ xh,
                                                               const _Float16 *__restrict__ xl,
                                                               const float *__restrict__ rs, int m,
-                                                              float *__restrict__ y) {
+                                                              float *__restrict__ y,
+                                                              const float *__restrict__ cs = nullptr) {
     constexpr int TN = WGN * FN * 32, TM = WGM * FM * 32, NTH = 64 * WGN * WGM;
     __shared__ __attribute__((aligned(16))) _Float16 s_ah[TN * QMM_LDK], s_al[TN * QMM_LDK], s_bh[TM * QMM_LDK];
     __shared__ __attribute__((aligned(16))) _Float16 s_bl[NTERM == 2 ? TM * QMM_LDK : 8];
@@ -215,7 +259,7 @@ __global__ __launch_bounds__(64 * WGN * WGM) void k_qmm_tile(QView q, const _Flo
     for (int b = 0; b < FM; b++) {
         const int mm = m0 + (wm * FM + b) * 32 + (lane & 31);
         if (mm >= m) continue;
-        const float s = rs[mm];
+        const float s = rs[mm] * q.winv;
 #pragma unroll
         for (int a = 0; a < FN; a++) {
             const int64_t nb = n0 + (wn * FN + a) * 32 + 4 * (lane >> 5);
@@ -224,6 +268,12 @@ __global__ __launch_bounds__(64 * WGN * WGM) void k_qmm_tile(QView q, const _Flo
                 const int64_t nn = nb + 8 * r4;
                 float4 v = make_float4(acc[a][b][4 * r4] * s, acc[a][b][4 * r4 + 1] * s, acc[a][b][4 * r4 + 2] * s,
                                        acc[a][b][4 * r4 + 3] * s);
+                if (cs) { // a dense right-hand side: every output column has its own factor
+                    v.x *= cs[nn < q.n ? nn : q.n - 1];
+                    v.y *= cs[nn + 1 < q.n ? nn + 1 : q.n - 1];
+                    v.z *= cs[nn + 2 < q.n ? nn + 2 : q.n - 1];
+                    v.w *= cs[nn + 3 < q.n ? nn + 3 : q.n - 1];
+                }
                 float *dst = y + (int64_t)mm * q.n + nn;
                 if (vec && nn + 3 < q.n) {
                     *(float4 *)dst = v;
@@ -571,11 +621,28 @@ static fh_status qmm_launch_t(const fh_qmatrix *q, const _Float16 *xh, const _Fl
     return FH_OK;
 }
 
+// dense f16 / f32 weight rows: the plain tile kernel (its weight "decode" is a load), tile shape by row count
+template <int T, int NTERM>
+static fh_status qmm_launch_dense(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const float *rs, int m,
+                                  float *y, const float *cs = nullptr) {
+    hipStream_t s = q->dev->stream;
+    QView v = fh_view(q);
+    const unsigned gn = (unsigned)((q->n + 127) / 128);
+    FH_REQUIRE((m + 63) / 64 <= 65535, "m = %d too large for one launch", m);
+    if (m <= 32) k_qmm_tile<T, NTERM, 4, 1, 1, 1><<<dim3(gn, 1), 256, 0, s>>>(v, xh, xl, rs, m, y, cs);
+    else if (m <= 64 || (int64_t)gn * ((m + 127) / 128) < (int64_t)q->dev->compute_units)
+        k_qmm_tile<T, NTERM, 2, 2, 2, 1><<<dim3(gn, (unsigned)((m + 63) / 64)), 256, 0, s>>>(v, xh, xl, rs, m, y, cs);
+    else k_qmm_tile<T, NTERM, 2, 2, 2, 2><<<dim3(gn, (unsigned)((m + 127) / 128)), 256, 0, s>>>(v, xh, xl, rs, m, y, cs);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
 fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y) {
     fh_device *dev = q->dev;
     const int64_t K = q->k;
-    if (fh_is_plain(q->type))
-        FH_FAIL(FH_ERR_UNSUPPORTED, "type %u has no matrix-core matmul (f32 activations run through fh_qmatmul)", q->type);
+    if (fh_is_plain(q->type) && ((q->type != FH_W_F16 && q->type != FH_W_F32) || K % 32 != 0))
+        FH_FAIL(FH_ERR_UNSUPPORTED, "type %u with k = %lld has no matrix-core matmul (it runs through fh_qmatmul)", q->type,
+                (long long)K);
     FH_REQUIRE((m + 127) / 128 <= 65535, "m = %d too large for one launch", m);
     // planes: xh | xl | rs
     const size_t plane = ((size_t)m * K * 2 + 255) & ~(size_t)255;
@@ -584,8 +651,8 @@ fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf
     _Float16 *xh = (_Float16 *)dev->act_buf;
     _Float16 *xl = x_is_bf16 ? nullptr : (_Float16 *)((uint8_t *)dev->act_buf + plane);
     float *rs = (float *)((uint8_t *)dev->act_buf + plane * (x_is_bf16 ? 1 : 2));
-    if (x_is_bf16) k_act_split<true><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, (int)K, xh, xl, rs);
-    else k_act_split<false><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, (int)K, xh, xl, rs);
+    if (x_is_bf16) k_act_split<1><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, K, 1, (int)K, (int)K, xh, xl, rs);
+    else k_act_split<0><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, K, 1, (int)K, (int)K, xh, xl, rs);
     FH_HIP(hipGetLastError());
 #define QMM_GO(T_)                                                              \
     return x_is_bf16 ? qmm_launch_t<T_, 1>(q, xh, xl, rs, m, y) : qmm_launch_t<T_, 2>(q, xh, xl, rs, m, y)
@@ -594,7 +661,82 @@ fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf
     case FH_Q8_0: QMM_GO(FH_Q8_0);
     case FH_Q4_K: QMM_GO(FH_Q4_K);
     case FH_Q6_K: QMM_GO(FH_Q6_K);
+    case FH_W_F16: return x_is_bf16 ? qmm_launch_dense<FH_W_F16, 1>(q, xh, xl, rs, m, y) : qmm_launch_dense<FH_W_F16, 2>(q, xh, xl, rs, m, y);
+    case FH_W_F32: return x_is_bf16 ? qmm_launch_dense<FH_W_F32, 1>(q, xh, xl, rs, m, y) : qmm_launch_dense<FH_W_F32, 2>(q, xh, xl, rs, m, y);
     }
 #undef QMM_GO
     FH_FAIL(FH_ERR_UNSUPPORTED, "unsupported type %u", q->type);
+}
+
+// ------------------------------------------------------------------------------ dense matmul
+// largest |w| of a dense f32 weight -> the power of two that brings it into [2^14, 2^15)
+__global__ __launch_bounds__(256) void k_amax_bits(const float *__restrict__ w, int64_t count, uint32_t *__restrict__ out) {
+    uint32_t a = 0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256)
+        a = max(a, __float_as_uint(w[i]) & 0x7FFFFFFFu);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) a = max(a, (uint32_t)__shfl_xor((int)a, o, 64));
+    if ((threadIdx.x & 63) == 0) atomicMax(out, a); // integer maximum: the order does not matter
+}
+
+fh_status fh_dense_wscale(fh_device *dev, const float *w_dev, int64_t count, float *wscale) {
+    uint32_t *slot = (uint32_t *)dev->small_buf;
+    FH_TRY(fh_memset(dev, slot, 0, 4));
+    const int64_t blocks = (count + 255) / 256;
+    k_amax_bits<<<dim3((unsigned)(blocks > 1024 ? 1024 : blocks)), dim3(256), 0, dev->stream>>>(w_dev, count, slot);
+    FH_HIP(hipGetLastError());
+    uint32_t bits = 0;
+    FH_TRY(fh_download(dev, &bits, slot, 4));
+    int e = 141 - (int)((bits >> 23) & 0xFFu);
+    e = e > 100 ? 100 : (e < -100 ? -100 : e);
+    const uint32_t sb = (uint32_t)(e + 127) << 23;
+    __builtin_memcpy(wscale, &sb, 4);
+    return FH_OK;
+}
+
+// Tensor::matmul (fusor-ml/fusor/src/lib.rs:1094-1103; CPU form fusor-ml/cpu/src/matmul.rs:226-352, f16 form :159-179):
+// C[b] = A[b] . B[b] for strided views A [batch, m, k] and B [batch, k, n].  Both operands become exact two-term
+// f16 splits of values normalised per row of A and per column of B (as the reference copies non-contiguous operands to
+// scratch first, :299-328), the product runs on the matrix cores with f32 accumulation, f16 results are rounded once.
+extern "C" fh_status fh_matmul(fh_device *dev, int32_t dtype, const void *a_dev, int64_t a_sb, int64_t a_sr, int64_t a_sc,
+                               const void *b_dev, int64_t b_sb, int64_t b_sr, int64_t b_sc, int32_t batch, int32_t m,
+                               int32_t k, int32_t n, void *c_dev) {
+    FH_REQUIRE(dev && a_dev && b_dev && c_dev, "NULL argument");
+    FH_REQUIRE(dtype == FH_F32 || dtype == FH_F16, "dtype must be FH_F32 or FH_F16");
+    FH_REQUIRE(batch > 0 && m > 0 && k > 0 && n > 0, "empty matmul operand [%d, %d, %d] @ [.., %d, %d]", batch, m, k, k, n);
+    const bool h16 = dtype == FH_F16;
+    const int kp = (k + 31) / 32 * 32;
+    const size_t plane = ((size_t)m * kp * 2 + 255) & ~(size_t)255;
+    FH_TRY(fh_dev_scratch(dev, &dev->act_buf, &dev->act_cap, 2 * plane + (size_t)m * 4 + 256));
+    const size_t bt = ((size_t)n * kp * 4 + 255) & ~(size_t)255, csb = ((size_t)n * 4 + 255) & ~(size_t)255;
+    FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, bt + csb + (h16 ? (size_t)m * n * 4 : 0)));
+    _Float16 *xh = (_Float16 *)dev->act_buf, *xl = (_Float16 *)((uint8_t *)dev->act_buf + plane);
+    float *rs = (float *)((uint8_t *)dev->act_buf + 2 * plane);
+    float *btp = dev->ksplit_buf, *cs = (float *)((uint8_t *)dev->ksplit_buf + bt);
+    float *c32 = (float *)((uint8_t *)dev->ksplit_buf + bt + csb);
+    const size_t esz = h16 ? 2 : 4;
+    fh_qmatrix qt; // the packed right-hand side viewed as dense f32 weight rows [n, kp]
+    qt.dev = dev;
+    qt.type = FH_W_F32;
+    qt.n = n;
+    qt.k = kp;
+    qt.n_pad = n;
+    qt.kb = kp;
+    qt.rec_bytes = 4;
+    qt.data = (uint8_t *)btp;
+    for (int bi = 0; bi < batch; bi++) {
+        const uint8_t *ab = (const uint8_t *)a_dev + (size_t)bi * a_sb * esz, *bb = (const uint8_t *)b_dev + (size_t)bi * b_sb * esz;
+        if (h16) {
+            k_act_split<2><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(ab, a_sr, a_sc, k, kp, xh, xl, rs);
+            k_dense_rows<true><<<dim3((unsigned)n), dim3(256), 0, dev->stream>>>(bb, b_sc, b_sr, k, kp, btp, cs);
+        } else {
+            k_act_split<0><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(ab, a_sr, a_sc, k, kp, xh, xl, rs);
+            k_dense_rows<false><<<dim3((unsigned)n), dim3(256), 0, dev->stream>>>(bb, b_sc, b_sr, k, kp, btp, cs);
+        }
+        FH_HIP(hipGetLastError());
+        float *dst = h16 ? c32 : (float *)c_dev + (size_t)bi * m * n;
+        FH_TRY((qmm_launch_dense<FH_W_F32, 2>(&qt, xh, xl, rs, m, dst, cs)));
+        if (h16) FH_TRY(fh_cast_f32_f16(dev, c32, (_Float16 *)c_dev + (size_t)bi * m * n, (int64_t)m * n));
+    }
+    return FH_OK;
 }

@@ -228,6 +228,30 @@ class Tensor:
             check(L.fh_qmatmul(w._h, C.c_void_p(self.ptr), m, C.c_void_p(out.ptr)))
         return out
 
+    def matmul(self, rhs: "Tensor", rhs_transposed: bool = False, out: Optional["Tensor"] = None) -> "Tensor":
+        """Tensor::matmul (fusor-ml/fusor/src/lib.rs:1094-1103): [.., M, K] @ [.., K, N] -> [.., M, N], f32 or f16, batched
+        over the leading dimensions (which must match).  With rhs_transposed the right operand is the lazy transpose
+        of a contiguous [.., N, K] tensor (the strided view the reference's `transpose` hands to matmul)."""
+        if len(self.shape) < 2 or len(rhs.shape) != len(self.shape):
+            raise FusorHipError(_lib.FH_ERR_INVALID, "Matrix multiplication requires at least 2 dimensions and equal ranks")
+        if self.dtype != rhs.dtype or self.dtype not in ("f32", "f16"):
+            raise FusorHipError(_lib.FH_ERR_INVALID, "matmul operands must both be f32 or both f16")
+        m, k = self.shape[-2:]
+        if rhs_transposed:
+            n, k2 = rhs.shape[-2:]
+            b_sr, b_sc = 1, k2
+        else:
+            k2, n = rhs.shape[-2:]
+            b_sr, b_sc = n, 1
+        if k != k2 or tuple(self.shape[:-2]) != tuple(rhs.shape[:-2]):
+            raise FusorHipError(_lib.FH_ERR_INVALID, f"matmul shapes {self.shape} and {rhs.shape} do not agree")
+        batch = int(np.prod(self.shape[:-2])) if len(self.shape) > 2 else 1
+        if out is None:
+            out = Tensor(self.device, (*self.shape[:-2], m, n), self.dtype)
+        check(self.device._lib.fh_matmul(self.device._h, F16 if self.dtype == "f16" else F32, C.c_void_p(self.ptr), m * k, k, 1,
+                                         C.c_void_p(rhs.ptr), k * n, b_sr, b_sc, batch, m, k, n, C.c_void_p(out.ptr)))
+        return out
+
     def q_mat_mul_add2(self, w: "QMatrix", first: "Tensor", second: "Tensor",
                        out: Optional["Tensor"] = None) -> "Tensor":
         """(x.W^T + first) + second, the decode epilogue of raw/attention_layer.rs:147-174."""

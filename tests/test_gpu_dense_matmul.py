@@ -1,0 +1,118 @@
+"""Dense matmul on the matrix cores (Tensor::matmul, fusor/src/lib.rs:1094-1103) against float64 numpy at the shapes of
+the reference's own `matmul_*_match_host_reference` cases (conformance/src/suite/native/matmul_conv_pool.rs:11-653), and
+dense F16 / F32 weight matrices through q_mat_mul."""
+import numpy as np
+import pytest
+
+from refgen import assert_close
+from kalosm_amd import synth
+from kalosm_amd.fusor import FusorHipError, QMatrix, Tensor
+
+pytestmark = pytest.mark.gpu
+
+
+def test_small_fixed_regression(dev):
+    """matmul_small_fixed_regression: [[1,2,3],[4,5,6]] @ [[1,2],[3,4],[5,6]] = [[22,28],[49,64]], tolerance 1e-6."""
+    a = Tensor.from_slice(dev, np.float32([[1, 2, 3], [4, 5, 6]]))
+    b = Tensor.from_slice(dev, np.float32([[1, 2], [3, 4], [5, 6]]))
+    got = a.matmul(b).as_slice()
+    assert np.abs(got - np.float32([[22, 28], [49, 64]])).max() <= 1e-6
+
+
+@pytest.mark.parametrize("m,k,n", [(256, 128, 64), (256, 256, 256), (256, 128, 256), (1, 64, 1), (1, 300, 77), (5, 1, 9),
+                                   (130, 33, 257), (512, 4096, 128)])
+def test_matmul_matches_float64(dev, m, k, n):
+    """matmul_match_host_reference (uniform(-3, 3) operands, [256, 128 | 256] @ [.., 64 | 256], tolerance 1e-2 there) and
+    the single-output / multi-output matrix-vector variants; shapes that are not multiples of any tile."""
+    rng = np.random.default_rng(m + k + n)
+    a = rng.uniform(-3, 3, (m, k)).astype(np.float32)
+    b = rng.uniform(-3, 3, (k, n)).astype(np.float32)
+    got = Tensor.from_slice(dev, a).matmul(Tensor.from_slice(dev, b)).as_slice()
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    # f32 accuracy: a few ulps of the row-column scale, far inside the reference's 1e-2
+    assert np.abs(got - want).max() <= 4e-6 * np.sqrt(k) * 9 + 1e-6
+
+
+def test_matmul_keeps_f32_accuracy_over_magnitudes(dev):
+    """Rows of A and columns of B of very different magnitude (1e-6 .. 1e6) and tiny values beside large ones: the
+    per-row / per-column normalisation keeps every output at f32 accuracy relative to its own row-column scale."""
+    rng = np.random.default_rng(7)
+    m, k, n = 96, 160, 80
+    a = rng.standard_normal((m, k)) * (10.0 ** rng.uniform(-6, 6, (m, 1)))
+    b = rng.standard_normal((k, n)) * (10.0 ** rng.uniform(-6, 6, (1, n)))
+    a[3, ::2] *= 1e-7
+    a, b = a.astype(np.float32), b.astype(np.float32)
+    got = Tensor.from_slice(dev, a).matmul(Tensor.from_slice(dev, b)).as_slice().astype(np.float64)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    scale = np.sqrt((a.astype(np.float64) ** 2).sum(1))[:, None] * np.sqrt((b.astype(np.float64) ** 2).sum(0))[None, :]
+    assert (np.abs(got - want) <= 2e-6 * scale).all()
+
+
+def test_batched_and_attention_shaped(dev):
+    """matmul_batched_3d / matmul_attention_4d ([1, 2, 16, 16], data ((i + seed) % 31 - 15) * 0.05, tolerance 1e-3)."""
+    def data(seed, shape):
+        i = np.arange(int(np.prod(shape)))
+        return ((((i + seed) % 31) - 15) * 0.05).astype(np.float32).reshape(shape)
+    a, b = data(0, (1, 2, 16, 16)), data(7, (1, 2, 16, 16))
+    got = Tensor.from_slice(dev, a).matmul(Tensor.from_slice(dev, b)).as_slice()
+    assert np.abs(got - a.astype(np.float64) @ b.astype(np.float64)).max() < 1e-5
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal((3, 4, 20, 48)).astype(np.float32)
+    b = rng.standard_normal((3, 4, 48, 36)).astype(np.float32)
+    got = Tensor.from_slice(dev, a).matmul(Tensor.from_slice(dev, b)).as_slice()
+    assert got.shape == (3, 4, 20, 36)
+    assert np.abs(got - a.astype(np.float64) @ b.astype(np.float64)).max() < 3e-5
+
+
+def test_transposed_operand_and_identity(dev):
+    """matmul_transposed_operand (the right operand is the lazy transpose of a contiguous tensor) and
+    matmul_identity_matrix."""
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal((40, 72)).astype(np.float32)
+    bt = rng.standard_normal((24, 72)).astype(np.float32)            # contiguous [N, K]
+    got = Tensor.from_slice(dev, a).matmul(Tensor.from_slice(dev, bt), rhs_transposed=True).as_slice()
+    assert np.abs(got - a.astype(np.float64) @ bt.astype(np.float64).T).max() < 3e-5
+    eye = np.eye(72, dtype=np.float32)
+    got = Tensor.from_slice(dev, a).matmul(Tensor.from_slice(dev, eye)).as_slice()
+    assert np.abs(got - a).max() <= 2.0 ** -22 * np.abs(a).max()    # one product per output: the two-term split keeps 22 bits
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 64, 64), (64, 96, 64), (33, 70, 100)])
+def test_f16_matmul(dev, oracle, m, n, k):
+    """f16_matmul_{64x64x64, 64x96x64}_matches_host_reference (tolerance 5e-2 there).  The reference's f16 form sums in
+    f32 and rounds once (cpu/src/matmul.rs:159-179); products of f16 values are exact, so the result is the correctly
+    rounded f16 of the f32-accumulated sum: at most one f16 ulp from the float64 sum rounded to f16."""
+    def data(seed, total):
+        i = np.arange(total)
+        return ((((i + seed) % 31) - 15) * 0.05).astype(np.float32).astype(np.float16)
+    a, b = data(0, m * k).reshape(m, k), data(7, k * n).reshape(k, n)
+    got = Tensor.from_slice(dev, a, "f16").matmul(Tensor.from_slice(dev, b, "f16")).as_slice()
+    want = (a.astype(np.float64) @ b.astype(np.float64))
+    assert got.dtype == np.float16
+    ulp = np.maximum(np.abs(want), 2.0 ** -14) * 2.0 ** -10
+    assert (np.abs(got.astype(np.float64) - want) <= ulp).all()
+
+
+@pytest.mark.parametrize("ty", [synth.W_F32, synth.W_F16], ids=["F32", "F16"])
+@pytest.mark.parametrize("m", [1, 9, 17, 200])
+def test_dense_weight_rows_through_q_mat_mul(dev, oracle, ty, m):
+    """F16 / F32 "quantized" weights (the reference dequantises them and calls the dense matmul, fusor/src/lib.rs:
+    1184-1215): few rows through the per-row kernel, 17 rows and more through the matrix-core tiles; both against the
+    checker and float64."""
+    n, k = 150, 512
+    raw = synth.random_weight(ty, n, k, seed=31 + ty)
+    w = (raw.view(np.float32) if ty == synth.W_F32 else raw.view(np.float16).astype(np.float32)).reshape(n, k)
+    x = synth.random_activation(m, k, seed=m)
+    got = Tensor.from_slice(dev, x).q_mat_mul(QMatrix.from_raw_bytes(dev, (n, k), raw, ty)).as_slice()
+    want = x.astype(np.float64) @ w.astype(np.float64).T
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 3e-6 * scale
+    assert_close(got, oracle.q_mat_mul(ty, x, raw, n), what=f"dense rows m={m}")
+
+
+def test_matmul_errors(dev):
+    a = Tensor.zeros(dev, (4, 8))
+    with pytest.raises(FusorHipError, match="do not agree"):
+        a.matmul(Tensor.zeros(dev, (7, 3)))
+    with pytest.raises(FusorHipError, match="both"):
+        a.matmul(Tensor.zeros(dev, (8, 3), "f16"))
