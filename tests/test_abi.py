@@ -82,3 +82,52 @@ def test_rust_declarations_cover_the_header():
     c_fields = re.findall(r"\b([a-z_0-9]+)\s*[,;]", cfg)
     rs_cfg = re.search(r"pub struct FhLlamaConfig \{([^{}]*)\}", rs).group(1)
     assert c_fields == re.findall(r"pub ([a-z_0-9]+):", rs_cfg)
+
+
+C_TO_RUST = {"int32_t": "i32", "int64_t": "i64", "uint8_t": "u8", "uint16_t": "u16", "uint32_t": "u32", "uint64_t": "u64",
+             "size_t": "usize", "float": "f32", "double": "f64", "void": "c_void", "char": "c_char", "int": "i32",
+             "fh_status": "FhStatus", "fh_device": "FhDevice", "fh_qmatrix": "FhQMatrix", "fh_kvcache": "FhKvCache",
+             "fh_llama": "FhLlama", "fh_graph": "FhGraph", "fh_gguf": "FhGguf", "fh_llama_config": "FhLlamaConfig",
+             "fh_rope_scaling": "FhRopeScaling", "fh_sampler_params": "FhSamplerParams",
+             "fh_gguf_tensor": "FhGgufTensor"}
+
+
+def c_param_to_rust(param: str) -> str:
+    """`const float *x_dev` -> `*const f32`; `fh_qmatrix **out` -> `*mut *mut FhQMatrix`; `int32_t m` -> `i32`."""
+    t = " ".join(param.replace("*", " * ").split())
+    toks = t.split(" ")
+    const = toks[0] == "const"
+    if const:
+        toks = toks[1:]
+    base, rest = toks[0], toks[1:]
+    stars = rest.count("*")
+    if rest and "const" in rest:          # `const fh_qmatrix *const *parts`: a const pointer level
+        const_levels = True
+    else:
+        const_levels = False
+    out = C_TO_RUST[base]
+    for level in range(stars):
+        innermost = level == 0
+        is_const = const if innermost else const_levels
+        out = ("*const " if is_const else "*mut ") + out
+    return out
+
+
+def test_rust_declarations_have_the_header_types():
+    """Every parameter of every function in include/fusor_hip_sys.rs has the Rust type its C declaration dictates
+    (pointer depth, constness, integer width), not only the same count."""
+    text = open(os.path.join(ROOT, "include", "fusor_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    rs = open(os.path.join(ROOT, "include", "fusor_hip_sys.rs")).read()
+    rust = {name: args for name, args in re.findall(r"pub fn (fh_[a-z0-9_]+)\(([^)]*)\)", rs)}
+    checked = 0
+    for name, args in re.findall(r"\b(fh_[a-z0-9_]+)\s*\(([^;{}]*?)\)\s*;", text, flags=re.S):
+        args = " ".join(args.split())
+        c_params = [] if args == "void" else [a.strip() for a in args.split(",")]
+        r_params = [a.strip().split(":", 1)[1].strip() for a in rust[name].split(",")] if rust[name].strip() else []
+        assert len(c_params) == len(r_params), name
+        for cp, rp in zip(c_params, r_params):
+            want = c_param_to_rust(cp)
+            assert want == rp, f"{name}: `{cp}` should be `{want}` in Rust, found `{rp}`"
+            checked += 1
+    assert checked > 400
