@@ -163,7 +163,11 @@ fh_status fh_q8_0_quantize(fh_device *dev, const float *x_dev, int64_t count, vo
 
 /* Kernel selection override for measurement (the reference's FUSOR_* tile overrides,
  * fusor-ml/tile-ir-kernels/src/dispatch.rs:15-20).  key/value pairs documented in the README of
- * the csrc directory; unknown keys give FH_ERR_INVALID. */
+ * the csrc directory; unknown keys give FH_ERR_INVALID.
+ * "deterministic" = 1: the decoder's device-side decode steps never add k-split partial sums with float atomics
+ * (the output projection and the Q6_K down projection otherwise do, which makes the last bits of a step vary
+ * from run to run): every run then gives the same bits, as the reference's CPU path does on one machine, at
+ * about a tenth of the decode rate.  Every other entry point is deterministic as it is. */
 fh_status fh_set_option(fh_device *dev, const char *key, int64_t value);
 
 /* -------------------------------------------------------------------- norm

@@ -234,7 +234,9 @@ extern "C" fh_status fh_set_option(fh_device *dev, const char *key, int64_t valu
     else if (!strcmp(key, "attn_waves")) dev->opt_attn_waves = value;
     else if (!strcmp(key, "attn_heads")) dev->opt_attn_heads = value;
     else if (!strcmp(key, "down_tiles")) dev->opt_down_tiles = value;
+    else if (!strcmp(key, "deterministic")) dev->opt_deterministic = value;
     else FH_FAIL(FH_ERR_INVALID, "unknown option '%s'", key);
+    dev->opt_gen++;
     return FH_OK;
 }
 

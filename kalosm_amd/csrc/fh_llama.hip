@@ -43,6 +43,7 @@ struct fh_llama {
     hipGraph_t graph = nullptr;
     int captured_capacity = -1;
     uint64_t captured_gen = 0, samp_gen = 0; // dev->scratch_gen at the captures
+    uint64_t captured_opt = 0, samp_opt = 0; // dev->opt_gen at the captures (options pick the kernels of a step)
     // sampled decode state: [0..63] previous ids, [64] their count, [65] next slot, [66] Mirostat mu (f32),
     // [68..69] status and token of the last step, [128..] one random number per step
     uint32_t *samp_dev = nullptr;
@@ -328,7 +329,7 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
             else if (ast == FH_OK && merge_in_wo) {
                 // first choice: x += Wo . att with k split over small workgroups; the residual stream then already
                 // holds x + attn for the FFN norm and the final sum ((ffn + attn) + residual, raw/mod.rs:1036)
-                fh_status st = dev->opt_wo_acc == 1 ? FH_ERR_UNSUPPORTED
+                fh_status st = (dev->opt_wo_acc == 1 || dev->opt_deterministic) ? FH_ERR_UNSUPPORTED
                                                     : fh_launch_q4k_m1_attn_acc(l.wo, dev->part_buf, nsplit, m->x);
                 xacc = st == FH_OK;
                 if (st == FH_ERR_UNSUPPORTED) st = fh_launch_q4k_m1_attn(l.wo, dev->part_buf, nsplit, m->attn_out);
@@ -362,7 +363,8 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
             // On request (down_splitk = 3; measured slower on MI355X) SwiGLU moves into the staging of a split-k Q6_K down
             // projection: the gate | up
             // projection then runs in its plain (fastest) form and writes both halves.
-            late_swiglu = l.down->type == FH_Q6_K && dev->opt_down_splitk == 3 && l.down->kb % 4 == 0 && l.down->kb >= 8;
+            late_swiglu = l.down->type == FH_Q6_K && dev->opt_down_splitk == 3 && !dev->opt_deterministic &&
+                          l.down->kb % 4 == 0 && l.down->kb >= 8;
             fh_status st = late_swiglu ? fh_launch_q4k_m1_norm(l.gate_up, hin, hres, l.ffn_norm, c.eps, m->gu, FH_EPI_NONE,
                                                                nullptr, nullptr)
                                        : fh_launch_q4k_m1_norm(l.gate_up, hin, hres, l.ffn_norm, c.eps, m->act,
@@ -389,7 +391,7 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
             if (late_swiglu) { // x += down(silu(gate) * up) + attn
                 st = fh_launch_q6k_m1_acc(l.down, m->gu, m->gu + F, m->x, hadd);
                 if (st == FH_ERR_UNSUPPORTED) FH_TRY(fh_swiglu(dev, m->gu, m->gu + F, m->act, F));
-            } else if (fuse && l.down->type == FH_Q6_K && dev->opt_down_splitk != 1) {
+            } else if (fuse && l.down->type == FH_Q6_K && dev->opt_down_splitk != 1 && !dev->opt_deterministic) {
                 st = fh_launch_q6k_m1_acc(l.down, m->act, nullptr, m->x, hadd); // x += down(act) [+ attn]
             }
             if (st == FH_ERR_UNSUPPORTED && xacc) { // x already holds x + attn
@@ -456,7 +458,8 @@ extern "C" fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, i
         // One eager step sizes every scratch buffer and sets kernel attributes; the capture then
         // records launches only.  The graph depends on the cache capacity (strides), so it is
         // rebuilt when the capacity changed since the last capture.
-        if (!m->graph_exec || m->captured_capacity != m->cache->capacity || m->captured_gen != dev->scratch_gen) {
+        if (!m->graph_exec || m->captured_capacity != m->cache->capacity || m->captured_gen != dev->scratch_gen ||
+            m->captured_opt != dev->opt_gen) {
             FH_TRY(fh_timer_start(dev));
             FH_TRY(decode_step_enqueue(m));
             done = 1;
@@ -471,6 +474,7 @@ extern "C" fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, i
             FH_HIP(hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
             m->captured_capacity = m->cache->capacity;
             m->captured_gen = dev->scratch_gen;
+            m->captured_opt = dev->opt_gen;
         } else {
             FH_TRY(fh_timer_start(dev));
         }
@@ -554,7 +558,7 @@ extern "C" fh_status fh_llama_decode_sampled(fh_llama *m, uint32_t first_token, 
         fh_sampler_params want = *params;
         want.random = 0.f; // every step takes its number from randoms_host
         const bool same = m->samp_exec && m->samp_capacity == m->cache->capacity && m->samp_range == range &&
-                          m->samp_gen == dev->scratch_gen &&
+                          m->samp_gen == dev->scratch_gen && m->samp_opt == dev->opt_gen &&
                           memcmp(&m->samp_params, &want, sizeof(want)) == 0;
         m->samp_params = want;
         m->samp_range = range;
@@ -574,6 +578,7 @@ extern "C" fh_status fh_llama_decode_sampled(fh_llama *m, uint32_t first_token, 
             FH_HIP(hipGraphInstantiate(&m->samp_exec, m->samp_graph, nullptr, nullptr, 0));
             m->samp_capacity = m->cache->capacity;
             m->samp_gen = dev->scratch_gen;
+            m->samp_opt = dev->opt_gen;
         } else {
             FH_TRY(fh_timer_start(dev));
         }

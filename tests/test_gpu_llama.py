@@ -352,3 +352,37 @@ def test_graph_decode_survives_scratch_reallocation(oracle):
         g.launch()
     del g, m
     d.sync()
+
+
+def test_deterministic_option_gives_identical_bits(dev, oracle):
+    """The default decode step adds the k-split partial sums of the output projection and of the Q6_K down projection
+    with float atomics, so the last bits of its hidden state depend on the arrival order.  With the `deterministic`
+    option the step uses the ordered kernels: three runs of 24 replayed steps must give bit-identical logits and the
+    checker's tokens; afterwards the default step is captured again (options are part of the capture key)."""
+    cfg = dict(HD128, n_heads=8, n_kv_heads=2, d_model=1024, ffn=2048)
+    m, ref = build_pair(dev, oracle, cfg, seed=12)
+    prompt = np.random.default_rng(8).integers(0, cfg["vocab"], 10)
+    wl = ref.forward(prompt)
+    first = oracle.argmax(wl)
+    want, t = [], first
+    for _ in range(24):
+        t = oracle.argmax(ref.forward([t]))
+        want.append(t)
+
+    def run():
+        m.reset()
+        m.forward(prompt)
+        got, _ = m.decode_greedy(first, 24)
+        return got.tolist(), m.forward([int(got[-1])])
+
+    dev.set_option("deterministic", 1)
+    try:
+        runs = [run() for _ in range(3)]
+    finally:
+        dev.set_option("deterministic", 0)
+    for toks, lg in runs:
+        assert toks == want
+        assert np.array_equal(lg.view(np.uint32), runs[0][1].view(np.uint32))
+    toks, lg = run()                       # default kernels again: same tokens, logits within tolerance
+    assert toks == want
+    assert_close(lg, runs[0][1], what="default step against the deterministic one")
