@@ -3,8 +3,17 @@
 // Reference: fusor-ml/fusor/src/composite/flash_attention.rs:58-236 (semantics; causal mask as MaskKind::Causal
 // with the queries aligned to the END of the keys), fusor-ml/core/src/row_program.rs:1210-1382 (the fused kernel).
 //
-// grid (query blocks of 128, q heads, batch); 4 wavefronts, each owning 32 query rows.  KV tiles of 64 keys go
-// through LDS as f16: K as [key][d], V transposed to [d][key].  Both products are computed TRANSPOSED with
+// grid (q heads / HW, query blocks of 128, batch); 4 x HW wavefronts, each owning 32 query rows of one head: the HW
+// (1 or 2) heads of a workgroup share a KV head, so a KV tile is fetched and staged once for 128 x HW query rows.
+// KV tiles of 64 keys go through LDS as f16, both as [key][d] rows written with 16-byte stores; the V^T operand
+// of the second product is read with the transposing LDS load of gfx950 (ds_read_b64_tr_b16: the 16 lanes of a
+// group supply 4 keys x 16 dims and receive, per lane, one dim of the 4 keys).  Two LDS buffers and one barrier per
+// tile: tile t+1 is written to the other buffer right after the first product of tile t (its LDS writes and the
+// request for tile t+2 then run under the softmax arithmetic).
+// What bounds the loop (measured per stage): the first product is matrix-core bound, the softmax vector-ALU bound
+// (both wavefronts of a SIMD are in it together) and the second product bound by the transposing LDS loads, which
+// run at half the rate of plain 16-byte loads.
+// Both products are computed TRANSPOSED with
 // v_mfma_f32_32x32x16_f16 so that a lane always stands for ONE query (the accumulator column):
 //   S^T (keys x queries) = K . Q^T      A = K rows, B = Q^T kept in registers for the whole kernel
 //   O^T (d x queries)    = V^T . P^T    A = V^T rows, B = P^T = the S^T accumulator, exponentiated, as f16
@@ -60,21 +69,33 @@ __device__ __forceinline__ void ap_split8(const float *x, fh_half *hi, fh_half *
     }
 }
 
-template <typename TQ, typename TKV, int D, bool SPLIT = false>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_attn_prefill(const TQ *__restrict__ q, int64_t q_sb, int64_t q_sh, int64_t q_st,
+typedef short short4v __attribute__((ext_vector_type(4)));
+// Eight halfs of the V^T operand: keys k .. k+7 of the dim this lane stands for (two transposing loads of 4 keys).
+__device__ __forceinline__ half8 ap_vt8(const fh_half *p, int row_stride) {
+    const short4v a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(uintptr_t)(uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p);
+    const short4v b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(uintptr_t)(uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)(p + 4 * row_stride));
+    half8 r;
+    __builtin_memcpy(&r, &a, 8);
+    __builtin_memcpy((char *)&r + 8, &b, 8);
+    return r;
+}
+
+template <typename TQ, typename TKV, int D, bool SPLIT = false, int HW = 1>
+__global__ __launch_bounds__(256 * HW) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_attn_prefill(const TQ *__restrict__ q, int64_t q_sb, int64_t q_sh, int64_t q_st,
                                                        const TKV *__restrict__ k, const TKV *__restrict__ v,
                                                        int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int hq, int hkv,
                                                        int sq, int skv, float scale, int causal, TQ *__restrict__ out) {
-    constexpr int BN = 64, KS = D + 8, VS = BN + 8, DT = D / 32, KSTEPS = D / 16, CH = D / 8; // CH: 8-element chunks per row
+    constexpr int BN = 64, KS = D + 8, VS = D + 16, DT = D / 32, KSTEPS = D / 16, CH = D / 8; // CH: 8-element chunks per row
     constexpr int NP = SPLIT ? 2 : 1; // operand planes: hi (, lo)
-    __shared__ __attribute__((aligned(16))) fh_half sK[NP * BN * KS];
-    __shared__ __attribute__((aligned(16))) fh_half sV[NP * D * VS];
+    constexpr int NTH = 256 * HW, KBUF = NP * BN * KS, VBUF = NP * BN * VS; // halfs per buffer
+    extern __shared__ __attribute__((aligned(16))) fh_half ap_lds[]; // [2 buffers][K planes | V planes]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
-    const int h = blockIdx.y, bi = blockIdx.z, kh = h / (hq / hkv);
-    // causal: the last query blocks see the most keys; they are dispatched first so that the short ones fill the tail
-    const int qb0 = (causal ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x) * 128;
-    const int qi = qb0 + wave * 32 + li; // this lane's query row
-    const int off = skv - sq;            // causal: query i sees keys 0 .. i + off
+    const int h = (int)blockIdx.x * HW + (wave >> 2), bi = blockIdx.z, kh = h / (hq / hkv);
+    // causal: the last query blocks see the most keys; with the block index on the slow grid axis ALL heads of the
+    // longest block are dispatched first and the short blocks fill the tail
+    const int qb0 = (causal ? (int)(gridDim.y - 1 - blockIdx.y) : (int)blockIdx.y) * 128;
+    const int qi = qb0 + (wave & 3) * 32 + li; // this lane's query row
+    const int off = skv - sq;                  // causal: query i sees keys 0 .. i + off
     const TKV *kb = k + bi * kv_sb + kh * kv_sh, *vb = v + bi * kv_sb + kh * kv_sh;
 
     // Q^T operand, once: lane (query li, k-slots 8g .. 8g+7 of every 16-wide step of d)
@@ -110,45 +131,37 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int last = (qb0 + 127 < sq ? qb0 + 127 : sq - 1) + off + 1;
         kend = last < skv ? last : skv;
     }
-    // The next KV tile is requested (into registers, as f16) before the current one is multiplied.
-    constexpr int NCH = BN * CH / 256; // 8-element pieces of K (and of V) per thread and tile
-    uint4 kreg[NCH], vreg[NCH];
-    float4 kraw[SPLIT ? 2 * NCH : 1], vraw[SPLIT ? 2 * NCH : 1]; // SPLIT: the f32 values wait in registers
+    // A KV tile waits in registers (as f16; SPLIT: as the f32 values) from one tile before it is written to LDS.
+    // Piece c = tid + NTH i of a tile: key c / CH, d chunk c % CH - consecutive threads along d, K and V alike.
+    constexpr int NCH = BN * CH / NTH;
+    uint4 kreg[SPLIT ? 1 : NCH], vreg[SPLIT ? 1 : NCH];
+    float4 kraw[SPLIT ? 2 * NCH : 1], vraw[SPLIT ? 2 * NCH : 1];
     auto fetch = [&](int t0) {
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
-            const int c = tid + 256 * i;
-            fh_half t[8];
-            const int kkey = c / CH, kdc = c % CH; // K: consecutive threads along d (coalesced rows)
-            if constexpr (SPLIT) { // rows past the end repeat the last one: their scores are masked, their P is 0
-                const float *kp = (const float *)kb + (int64_t)(t0 + kkey < skv ? t0 + kkey : skv - 1) * kv_st + 8 * kdc;
+            const int c = tid + NTH * i, key = c / CH, dc = c % CH;
+            // rows past the end repeat the last one (no branch): their scores are masked and their P is 0
+            const int64_t row = (int64_t)(t0 + key < skv ? t0 + key : skv - 1) * kv_st + 8 * dc;
+            if constexpr (SPLIT) {
+                const float *kp = (const float *)kb + row, *vp = (const float *)vb + row;
                 kraw[2 * i] = *(const float4 *)kp;
                 kraw[2 * i + 1] = *(const float4 *)(kp + 4);
-                const int vk = c % BN, vd = c / BN;
-                const float *vp = (const float *)vb + (int64_t)(t0 + vk < skv ? t0 + vk : skv - 1) * kv_st + 8 * vd;
                 vraw[2 * i] = *(const float4 *)vp;
                 vraw[2 * i + 1] = *(const float4 *)(vp + 4);
-                continue;
+            } else {
+                fh_half t[8];
+                ap_load8(kb + row, t);
+                __builtin_memcpy(&kreg[i], t, 16);
+                ap_load8(vb + row, t);
+                __builtin_memcpy(&vreg[i], t, 16);
             }
-            if (t0 + kkey < skv) ap_load8(kb + (int64_t)(t0 + kkey) * kv_st + 8 * kdc, t);
-            else {
-#pragma unroll
-                for (int e = 0; e < 8; e++) t[e] = (fh_half)0.f;
-            }
-            __builtin_memcpy(&kreg[i], t, 16);
-            const int vkey = c % BN, vdc = c / BN; // V: a lane keeps one key, so its 2-byte LDS stores are contiguous
-            if (t0 + vkey < skv) ap_load8(vb + (int64_t)(t0 + vkey) * kv_st + 8 * vdc, t);
-            else {
-#pragma unroll
-                for (int e = 0; e < 8; e++) t[e] = (fh_half)0.f;
-            }
-            __builtin_memcpy(&vreg[i], t, 16);
         }
     };
-    auto stash = [&]() { // K tile -> sK[key][d], V tile -> sV[d][key]
+    auto stash = [&](int buf) { // K tile -> sK[key][d], V tile -> sV[key][d]
+        fh_half *sK = ap_lds + buf * (KBUF + VBUF), *sV = sK + KBUF;
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
-            const int c = tid + 256 * i;
+            const int c = tid + NTH * i, key = c / CH, dc = c % CH;
             if constexpr (SPLIT) {
                 const float kx[8] = {kraw[2 * i].x, kraw[2 * i].y, kraw[2 * i].z, kraw[2 * i].w,
                                      kraw[2 * i + 1].x, kraw[2 * i + 1].y, kraw[2 * i + 1].z, kraw[2 * i + 1].w};
@@ -157,69 +170,107 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 uint4 uh, ul;
                 __builtin_memcpy(&uh, hi, 16);
                 __builtin_memcpy(&ul, lo, 16);
-                *(uint4 *)(sK + (c / CH) * KS + 8 * (c % CH)) = uh;
-                *(uint4 *)(sK + BN * KS + (c / CH) * KS + 8 * (c % CH)) = ul;
+                *(uint4 *)(sK + key * KS + 8 * dc) = uh;
+                *(uint4 *)(sK + BN * KS + key * KS + 8 * dc) = ul;
                 const float vx[8] = {vraw[2 * i].x, vraw[2 * i].y, vraw[2 * i].z, vraw[2 * i].w,
                                      vraw[2 * i + 1].x, vraw[2 * i + 1].y, vraw[2 * i + 1].z, vraw[2 * i + 1].w};
                 ap_split8(vx, hi, lo);
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    sV[(8 * (c / BN) + e) * VS + (c % BN)] = hi[e];
-                    sV[D * VS + (8 * (c / BN) + e) * VS + (c % BN)] = lo[e];
-                }
-                continue;
+                __builtin_memcpy(&uh, hi, 16);
+                __builtin_memcpy(&ul, lo, 16);
+                *(uint4 *)(sV + key * VS + 8 * dc) = uh;
+                *(uint4 *)(sV + BN * VS + key * VS + 8 * dc) = ul;
+            } else {
+                *(uint4 *)(sK + key * KS + 8 * dc) = kreg[i];
+                *(uint4 *)(sV + key * VS + 8 * dc) = vreg[i];
             }
-            *(uint4 *)(sK + (c / CH) * KS + 8 * (c % CH)) = kreg[i];
-            fh_half t[8];
-            __builtin_memcpy(t, &vreg[i], 16);
-#pragma unroll
-            for (int e = 0; e < 8; e++) sV[(8 * (c / BN) + e) * VS + (c % BN)] = t[e];
         }
     };
-    if (kend > 0) fetch(0);
-    for (int t0 = 0; t0 < kend; t0 += BN) {
-        __syncthreads(); // the previous tile is consumed
-        stash();
-        __syncthreads();
-        if (t0 + BN < kend) fetch(t0 + BN);
+    // V^T operand addressing: the 16 lanes of a group supply keys (8 g + s / 4) and dims (16 * (group & 1) + 4 * (s % 4))
+    // .. +3 and receive dim 16 * (group & 1) + s of keys 8 g .. 8 g + 3
+    const int vt_off = (8 * g + ((lane & 15) >> 2)) * VS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    // The Q loads must have landed before the loop: a wait for them inside the loop would also wait, every tile, for
+    // the KV loads issued after them (the memory counter is in order).
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+        asm volatile("" ::"v"(qf[ks]));
+        if constexpr (SPLIT) asm volatile("" ::"v"(ql[ks]));
+    }
+    const int lim = causal ? (qi + off < skv - 1 ? qi + off : skv - 1) : skv - 1; // this query's last visible key
+    if (kend > 0) {
+        fetch(0);
+        stash(0);
+        if (BN < kend) fetch(BN);
+    }
+    __syncthreads();
+
+    const float ninf = -INFINITY;
+    for (int t0 = 0, it = 0; t0 < kend; t0 += BN, it++) {
+        const fh_half *sK = ap_lds + (it & 1) * (KBUF + VBUF), *sV = sK + KBUF;
         // ---- S^T = K . Q^T for the two 32-key halves of the tile
         floatx16 st[2];
 #pragma unroll
-        for (int kt = 0; kt < 2; kt++) {
+        for (int r = 0; r < 16; r++) st[0][r] = st[1][r] = 0.f;
+        if constexpr (!SPLIT) {
+            // product i: key half i % 2, d step i / 2; the K operands are requested eight products ahead
+            const fh_half *ap = sK + prow * KS + 8 * g;
+            constexpr int NI = 2 * KSTEPS, AHEAD = 8;
+            half8 ka[AHEAD];
 #pragma unroll
-            for (int r = 0; r < 16; r++) st[kt][r] = 0.f;
-            const fh_half *ap = sK + (kt * 32 + prow) * KS + 8 * g;
+            for (int i = 0; i < AHEAD; i++) ka[i] = *(const half8 *)(ap + (i & 1) * 32 * KS + 16 * (i >> 1));
 #pragma unroll
-            for (int ks = 0; ks < KSTEPS; ks++) {
-                const half8 a = *(const half8 *)(ap + 16 * ks);
-                st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], st[kt], 0, 0, 0);
-                if constexpr (SPLIT) {
+            for (int i = 0; i < NI; i++) {
+                st[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[i % AHEAD], qf[i >> 1], st[i & 1], 0, 0, 0);
+                if (i + AHEAD < NI) ka[i % AHEAD] = *(const half8 *)(ap + (i & 1) * 32 * KS + 16 * ((i + AHEAD) >> 1));
+            }
+            __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+#pragma unroll
+            for (int i = 0; i < NI - AHEAD; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++) {
+                const fh_half *ap = sK + (kt * 32 + prow) * KS + 8 * g;
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ks++) {
+                    const half8 a = *(const half8 *)(ap + 16 * ks);
+                    st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], st[kt], 0, 0, 0);
                     const half8 al = *(const half8 *)(ap + BN * KS + 16 * ks);
                     st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, qf[ks], st[kt], 0, 0, 0);
                     st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, ql[ks], st[kt], 0, 0, 0);
                 }
             }
         }
-        // ---- mask, running max: register r of half kt is key t0 + 32 kt + 16 (r / 8) + 8 g + r % 8.  Only a tile
-        // that reaches past some query's last visible key needs the compare (one branch for the wavefront).
-        const int lim = causal ? (qi + off < skv - 1 ? qi + off : skv - 1) : skv - 1; // last visible key
-        float mx = -INFINITY;
+        // ---- tile t+1 goes into the other buffer (last read before the barrier that ended the previous tile) and
+        // tile t+2 is requested: the LDS writes and the loads run under the softmax arithmetic
+        // (the scheduler may not mix the stages: the operands prefetched for one product and the tile in flight would
+        // otherwise be live together with the scores)
+        __builtin_amdgcn_sched_barrier(0);
+        if (t0 + BN < kend) stash((it + 1) & 1);
+        if (t0 + 2 * BN < kend) fetch(t0 + 2 * BN);
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- mask, running max: register r of half kt is key t0 + 32 kt + 16 (r / 8) + 8 g + r % 8
+        // Only a tile that reaches past some query's last visible key pays for the compares (one branch for the
+        // wavefront); the select works in place, so the common path has no register copies at the join.
         if (__any(t0 + BN - 1 > lim)) {
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int key = t0 + 32 * kt + 16 * (r >> 3) + 8 * g + (r & 7);
-                    const float sv = key <= lim ? st[kt][r] : -INFINITY;
-                    st[kt][r] = sv;
-                    mx = fmaxf(mx, sv);
+                    asm volatile("v_cmp_le_i32 vcc, %1, %2\n\tv_cndmask_b32 %0, %3, %0, vcc"
+                                 : "+v"(st[kt][r])
+                                 : "v"(key), "v"(lim), "v"(ninf)
+                                 : "vcc");
                 }
-        } else {
-#pragma unroll
-            for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[kt][r]);
         }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[kt][r]);
         // the scale (> 0) is applied inside the exponent: p = 2^(s * sc2 - m), one multiply-add per score
         mx = ap_swap32_max(mx) * sc2;
         const float m_new = fmaxf(m_run, mx);
@@ -246,27 +297,51 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         l_run = l_run * alpha + ap_swap32_sum(ps);
         m_run = m_new;
         // ---- O^T = O^T * alpha + V^T . P^T (once the maxima have settled no lane of the wavefront rescales)
-        const bool rescale = __any(alpha != 1.f);
+        __builtin_amdgcn_sched_barrier(0);
+        if (__any(alpha != 1.f)) {
 #pragma unroll
-        for (int dt = 0; dt < DT; dt++) {
-            if (rescale) {
+            for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[dt][r] *= alpha;
+        }
+        if constexpr (!SPLIT) {
+            // product j: d tile j % DT, key step j / DT (= 2 kt + s2): consecutive products go to different
+            // accumulators; the V^T operand is requested eight products ahead
+            const fh_half *vp = sV + vt_off;
+            constexpr int NJ = 4 * DT, AHEAD = 8;
+            half8 va[AHEAD];
+#pragma unroll
+            for (int j = 0; j < AHEAD; j++) va[j] = ap_vt8(vp + 32 * (j % DT) + 16 * (j / DT) * VS, VS);
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                const int c = j / DT;
+                acc[j % DT] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[j % AHEAD], pb[c >> 1][c & 1], acc[j % DT], 0, 0, 0);
+                if (j + AHEAD < NJ) va[j % AHEAD] = ap_vt8(vp + 32 * ((j + AHEAD) % DT) + 16 * ((j + AHEAD) / DT) * VS, VS);
             }
-            const fh_half *vp = sV + (dt * 32 + li) * VS + 8 * g;
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * AHEAD, 0);
 #pragma unroll
-            for (int kt = 0; kt < 2; kt++)
+            for (int j = 0; j < NJ - AHEAD; j++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
+        } else {
 #pragma unroll
-                for (int s2 = 0; s2 < 2; s2++) {
-                    const half8 a = *(const half8 *)(vp + 32 * kt + 16 * s2);
-                    acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[kt][s2], acc[dt], 0, 0, 0);
-                    if constexpr (SPLIT) {
-                        const half8 al = *(const half8 *)(vp + D * VS + 32 * kt + 16 * s2);
+            for (int dt = 0; dt < DT; dt++) {
+                const fh_half *vp = sV + vt_off + 32 * dt;
+#pragma unroll
+                for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                    for (int s2 = 0; s2 < 2; s2++) {
+                        const half8 a = ap_vt8(vp + (32 * kt + 16 * s2) * VS, VS);
+                        acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[kt][s2], acc[dt], 0, 0, 0);
+                        const half8 al = ap_vt8(vp + BN * VS + (32 * kt + 16 * s2) * VS, VS);
                         acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, pb[kt][s2], acc[dt], 0, 0, 0);
                         acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pl[kt][s2], acc[dt], 0, 0, 0);
                     }
-                }
+            }
         }
+        __syncthreads(); // tile t+1 is staged, and nobody reads this tile's buffer any more
     }
     // ---- store: lane = query, register r of d-tile dt is d = 32 dt + 8 (r / 4) + 4 g + r % 4
     if (qi < sq) {
@@ -281,21 +356,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+template <typename TQ, typename TKV, int D, bool SPLIT, int HW>
+static fh_status ap_launch_k(fh_device *dev, const void *q, int64_t q_sb, int64_t q_sh, int64_t q_st, const void *k,
+                             const void *v, int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int b, int hq, int hkv, int sq,
+                             int skv, float scale, int causal, void *out) {
+    constexpr int LDS = 2 * (SPLIT ? 2 : 1) * 64 * (D + 8 + D + 16) * 2; // two buffers of K and V planes, bytes
+    static_assert(LDS <= 160 * 1024, "KV tiles exceed the LDS of a compute unit");
+    auto kern = k_attn_prefill<TQ, TKV, D, SPLIT, HW>;
+    static bool raised[64] = {}; // per kernel instance and device: allow more than 64 KB of dynamic LDS
+    const bool known = dev->ordinal >= 0 && dev->ordinal < 64;
+    if (!known || !raised[dev->ordinal]) {
+        FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        if (known) raised[dev->ordinal] = true;
+    }
+    dim3 grid((unsigned)(hq / HW), (unsigned)((sq + 127) / 128), (unsigned)b);
+    kern<<<grid, 256 * HW, LDS, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k, (const TKV *)v, kv_sb,
+                                               kv_sh, kv_st, hq, hkv, sq, skv, scale, causal, (TQ *)out);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
 template <typename TQ, typename TKV, bool SPLIT = false>
 static fh_status ap_launch(fh_device *dev, const void *q, int64_t q_sb, int64_t q_sh, int64_t q_st, const void *k,
                            const void *v, int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int b, int hq, int hkv, int sq,
                            int skv, int d, float scale, int causal, void *out) {
-    dim3 grid((unsigned)((sq + 127) / 128), (unsigned)hq, (unsigned)b);
-    if (d == 128)
-        k_attn_prefill<TQ, TKV, 128, SPLIT><<<grid, 256, 0, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k,
-                                                                    (const TKV *)v, kv_sb, kv_sh, kv_st, hq, hkv, sq, skv,
-                                                                    scale, causal, (TQ *)out);
-    else
-        k_attn_prefill<TQ, TKV, 64, SPLIT><<<grid, 256, 0, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k,
-                                                                   (const TKV *)v, kv_sb, kv_sh, kv_st, hq, hkv, sq, skv,
-                                                                   scale, causal, (TQ *)out);
-    FH_HIP(hipGetLastError());
-    return FH_OK;
+    // Two heads of one KV group share the staged tiles when the launch still has enough workgroups without the
+    // split: short prompts are bound by the longest workgroup and by how many compute units have one at all.
+    const long wgs = (long)hq * ((sq + 127) / 128) * b;
+    const bool pair = (hq / hkv) % 2 == 0 && wgs >= 4096;
+#define FH_AP(D, HW) ap_launch_k<TQ, TKV, D, SPLIT, HW>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, scale, causal, out)
+    if (d == 128) return pair ? FH_AP(128, 2) : FH_AP(128, 1);
+    return pair ? FH_AP(64, 2) : FH_AP(64, 1);
+#undef FH_AP
 }
 
 // FH_ERR_UNSUPPORTED when the shape is not one this kernel is written for (the caller keeps the generic kernel).
@@ -304,7 +396,7 @@ fh_status fh_attention_prefill_mfma(fh_device *dev, int q_dtype, int kv_dtype, c
                                     int64_t kv_sh, int64_t kv_st, int b, int hq, int hkv, int sq, int skv, int d,
                                     float scale, int mask_kind, void *out) {
     if ((d != 128 && d != 64) || hq % hkv || (mask_kind != FH_MASK_NONE && mask_kind != FH_MASK_CAUSAL)) return FH_ERR_UNSUPPORTED;
-    if (q_st % 8 || q_sh % 8 || q_sb % 8 || kv_st % 8 || kv_sh % 8 || kv_sb % 8 || hq > 65535 || b > 65535) return FH_ERR_UNSUPPORTED;
+    if (q_st % 8 || q_sh % 8 || q_sb % 8 || kv_st % 8 || kv_sh % 8 || kv_sb % 8 || (sq + 127) / 128 > 65535 || b > 65535) return FH_ERR_UNSUPPORTED;
     if (mask_kind == FH_MASK_CAUSAL && skv < sq) return FH_ERR_UNSUPPORTED;
     const int causal = mask_kind == FH_MASK_CAUSAL;
     if (q_dtype == FH_F16 && kv_dtype == FH_F16)
