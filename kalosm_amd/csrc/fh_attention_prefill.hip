@@ -383,7 +383,7 @@ static fh_status ap_launch(fh_device *dev, const void *q, int64_t q_sb, int64_t 
     // Two heads of one KV group share the staged tiles when the launch still has enough workgroups without the
     // split: short prompts are bound by the longest workgroup and by how many compute units have one at all.
     const long wgs = (long)hq * ((sq + 127) / 128) * b;
-    const bool pair = (hq / hkv) % 2 == 0 && wgs >= 4096;
+    const bool pair = (hq / hkv) % 2 == 0 && wgs >= 1024;
 #define FH_AP(D, HW) ap_launch_k<TQ, TKV, D, SPLIT, HW>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, scale, causal, out)
     if (d == 128) return pair ? FH_AP(128, 2) : FH_AP(128, 1);
     return pair ? FH_AP(64, 2) : FH_AP(64, 1);
