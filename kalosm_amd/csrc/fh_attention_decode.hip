@@ -582,11 +582,92 @@ fh_status fh_attention_decode_devlen(fh_device *dev, int kv_dtype, const float *
     return ad_any(dev, kv_dtype, q, k, v, kv_sh, kv_st, hq, hkv, d, scale, len_dev, max_len, out, splits_out, 0, 0, false);
 }
 
+// Merge of many parts: four thread groups of 128 take every fourth part each (a quarter of the dependent load
+// rounds of k_attn_combine_dl), then add up through LDS.
+template <typename TO>
+__global__ __launch_bounds__(512) void k_attn_combine_wide(const float *__restrict__ part, int splits, TO *__restrict__ out) {
+    constexpr int D = 128, PG = 4;
+    __shared__ float s_m[128], s_w[128], s_num[PG][D], s_den[PG];
+    const int64_t h = blockIdx.x;
+    const int t = threadIdx.x & 127, pg = threadIdx.x >> 7;
+    const float *pp = part + h * splits * (D + 4);
+    float m = -INFINITY, l = 0.f;
+    if (pg == 0) {
+        if (t < splits) {
+            m = pp[t * (D + 4) + D];
+            l = pp[t * (D + 4) + D + 1];
+        }
+        s_m[t] = m;
+    }
+    __syncthreads();
+    float mx = -INFINITY;
+    for (int s = 0; s < splits; s++) mx = fmaxf(mx, s_m[s]);
+    __syncthreads();
+    if (pg == 0) {
+        const float w = (m == -INFINITY) ? 0.f : __expf(m - mx);
+        s_w[t] = w;
+        s_m[t] = l * w; // reuse: weighted denominators
+    }
+    __syncthreads();
+    float num = 0.f, den = 0.f;
+    int s = pg;
+    for (; s + 7 * PG < splits; s += 8 * PG) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = pp[(s + u * PG) * (D + 4) + t];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            num = fmaf(v[u], s_w[s + u * PG], num);
+            den += s_m[s + u * PG];
+        }
+    }
+    for (; s < splits; s += PG) {
+        num = fmaf(pp[s * (D + 4) + t], s_w[s], num);
+        den += s_m[s];
+    }
+    s_num[pg][t] = num;
+    if (t == 0) s_den[pg] = den;
+    __syncthreads();
+    if (pg == 0) {
+        num = (s_num[0][t] + s_num[1][t]) + (s_num[2][t] + s_num[3][t]);
+        den = (s_den[0] + s_den[1]) + (s_den[2] + s_den[3]);
+        out[h * D + t] = (TO)(num / den);
+    }
+}
+
+// Merge `splits` partials per head ([hq][splits][132] floats) into out [hq, 128], f32 or f16.
+fh_status fh_attention_combine_parts(fh_device *dev, const float *part, int hq, int splits, void *out, bool out_f16) {
+    FH_REQUIRE(splits >= 1 && splits <= 128, "the merge takes 1 .. 128 parts");
+    if (splits > 16) {
+        if (out_f16) k_attn_combine_wide<fh_half><<<dim3((unsigned)hq), dim3(512), 0, dev->stream>>>(part, splits, (fh_half *)out);
+        else k_attn_combine_wide<float><<<dim3((unsigned)hq), dim3(512), 0, dev->stream>>>(part, splits, (float *)out);
+    } else if (out_f16) k_attn_combine_dl<128, fh_half><<<dim3((unsigned)hq), dim3(128), 0, dev->stream>>>(part, splits, (fh_half *)out);
+    else k_attn_combine_dl<128><<<dim3((unsigned)hq), dim3(128), 0, dev->stream>>>(part, splits, (float *)out);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
 // One f32 query per head against `skv` cached keys known on the host; `out` is f32 or f16 [hq, d].  The key
 // range is cut into more parts the longer it is (every part is a workgroup per KV head and query-head group).
 fh_status fh_attention_decode_hostlen(fh_device *dev, int kv_dtype, const void *q, bool q_f16, const void *k,
                                       const void *v, int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale,
                                       int skv, void *out, bool out_f16) {
+    // long f16 caches: the matrix-core kernel (attn_kernel = 5 forces it from 32 keys up, any other non-zero value keeps the vector-ALU kernels)
+    const int mfma_min = dev->opt_attn_kernel == 5 ? 32 : 4096;
+    if (kv_dtype == FH_F16 && d == 128 && hq % hkv == 0 && hq / hkv <= 16 && skv >= mfma_min &&
+        (dev->opt_attn_kernel == 0 || dev->opt_attn_kernel == 5) && dev->opt_attn_heads == 0 && kv_st % 8 == 0 && kv_sh % 8 == 0) {
+        // parts: four wavefronts each, two chunks of 32 keys per wavefront, at most 128 parts for the merge (measured on
+        // MI355X, 32 / 8 heads: 19.2 us against 22.0 us of the vector-ALU kernel at 16384 keys, level at 4096)
+        const int nct = (skv + 31) / 32;
+        int splits = dev->opt_attn_splits > 0 ? (int)dev->opt_attn_splits : nct / 8;
+        splits = splits < 1 ? 1 : (splits > 128 ? 128 : splits);
+        FH_TRY(fh_dev_scratch(dev, (void **)&dev->part_buf, &dev->part_cap, (size_t)hq * splits * (128 + 4) * 4));
+        fh_status st = fh_attention_decode_mfma(dev, q, q_f16, k, v, kv_sh, kv_st, hq, hkv, d, scale, skv, splits, dev->part_buf);
+        if (st != FH_ERR_UNSUPPORTED) {
+            if (st != FH_OK) return st;
+            return fh_attention_combine_parts(dev, dev->part_buf, hq, splits, out, out_f16);
+        }
+    }
     if (q_f16 && (dev->opt_attn_kernel == 4 || (dev->opt_attn_heads > 4))) return FH_ERR_UNSUPPORTED; // caller widens q
     int splits = skv <= 2048 ? 8 : 16;
     if (dev->opt_attn_splits > 0) splits = dev->opt_attn_splits > 128 ? 128 : (int)dev->opt_attn_splits;

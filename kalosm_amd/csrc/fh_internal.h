@@ -189,6 +189,10 @@ fh_status fh_launch_q4k_m1_norm(const fh_qmatrix *q, const float *x, const float
 fh_status fh_launch_q4k_m1_attn(const fh_qmatrix *q, const float *part, int nsplit, float *y);
 fh_status fh_launch_q4k_m1_attn_acc(const fh_qmatrix *q, const float *part, int nsplit, float *y_inout);
 fh_status fh_attention_combine_dl(fh_device *dev, int hq, int splits, float *out);
+fh_status fh_attention_combine_parts(fh_device *dev, const float *part, int hq, int splits, void *out, bool out_f16);
+fh_status fh_attention_decode_mfma(fh_device *dev, const void *q, bool q_f16, const void *k, const void *v,
+                                   int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale, int skv,
+                                   int splits, float *part);
 fh_status fh_attention_decode_hostlen(fh_device *dev, int kv_dtype, const void *q, bool q_f16, const void *k,
                                       const void *v, int64_t kv_sh, int64_t kv_st, int hq, int hkv, int d, float scale,
                                       int skv, void *out, bool out_f16);

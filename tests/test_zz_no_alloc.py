@@ -1,7 +1,9 @@
 """The entry point that allocates nothing (fh_flash_attention_decode_static): its partial results live in the library's
 file-scope device array instead of a buffer grown with hipMalloc.  Checked through the C ABI against
-fh_flash_attention on the same inputs, bit for bit (same kernels, same cut of the key range), on two calls in a row,
-the second with a smaller input, so stale contents of the shared array would show."""
+fh_flash_attention on the same inputs on two calls in a row, the second with a smaller input, so stale contents of
+the shared array would show: bit for bit where both run the same kernels with the same cut of the key range (f32
+caches, short f16 caches), within the attention tolerance where fh_flash_attention takes its matrix-core kernel
+(f16 caches from 4096 keys)."""
 import numpy as np
 import pytest
 
@@ -22,8 +24,12 @@ def _case(dev, oracle, hq, hkv, L, dtype, seed):
     want = qt.flash_attention(kt, vt, scale).as_slice()
     out = Tensor.filled_bytes(dev, (1, hq, 1, 128), 0xFF, dtype)
     got = qt.flash_attention_decode_static(kt, vt, scale, out=out).as_slice()
-    assert np.array_equal(got.view(np.uint16 if dtype == "f16" else np.uint32),
-                          want.view(np.uint16 if dtype == "f16" else np.uint32)), f"hq={hq} L={L} {dtype}"
+    if dtype == "f16" and L >= 4096:
+        assert_close(got.astype(np.float32), want.astype(np.float32), abs_tol=1e-2, rel_tol=1e-3,
+                     what=f"static vs allocating decode attention hq={hq} L={L} {dtype}")
+    else:
+        assert np.array_equal(got.view(np.uint16 if dtype == "f16" else np.uint32),
+                              want.view(np.uint16 if dtype == "f16" else np.uint32)), f"hq={hq} L={L} {dtype}"
     ref = oracle.flash_attention(*(a.astype(np.float32) for a in (q, k, v)), scale)
     assert_close(got.astype(np.float32), ref, abs_tol=1e-2, rel_tol=1e-3, what=f"static decode attention hq={hq} L={L} {dtype}")
 
