@@ -10,6 +10,9 @@
 // group supply 4 keys x 16 dims and receive, per lane, one dim of the 4 keys).  Two LDS buffers and one barrier per
 // tile: tile t+1 is written to the other buffer right after the first product of tile t (its LDS writes and the
 // request for tile t+2 then run under the softmax arithmetic).
+// KS = 2 (short prompts: fewer workgroups than the device holds, and the launch lasts as long as the workgroup of the
+// last query block): eight wavefronts per query block, the second four take every other key tile with running
+// statistics of their own, and the two halves are merged through LDS at the end - half the tile steps per workgroup.
 // What bounds the loop (measured per stage): the first product is matrix-core bound, the softmax vector-ALU bound
 // (both wavefronts of a SIMD are in it together) and the second product bound by the transposing LDS loads, which
 // run at half the rate of plain 16-byte loads.
@@ -80,21 +83,23 @@ __device__ __forceinline__ half8 ap_vt8(const fh_half *p, int row_stride) {
     return r;
 }
 
-template <typename TQ, typename TKV, int D, bool SPLIT = false, int HW = 1>
-__global__ __launch_bounds__(256 * HW) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_attn_prefill(const TQ *__restrict__ q, int64_t q_sb, int64_t q_sh, int64_t q_st,
+template <typename TQ, typename TKV, int D, bool SPLIT = false, int HW = 1, int KS = 1>
+__global__ __launch_bounds__(256 * HW * KS) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_attn_prefill(const TQ *__restrict__ q, int64_t q_sb, int64_t q_sh, int64_t q_st,
                                                        const TKV *__restrict__ k, const TKV *__restrict__ v,
                                                        int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int hq, int hkv,
                                                        int sq, int skv, float scale, int causal, TQ *__restrict__ out) {
-    constexpr int BN = 64, KS = D + 8, VS = D + 16, DT = D / 32, KSTEPS = D / 16, CH = D / 8; // CH: 8-element chunks per row
+    constexpr int BN = 64, KS_ = D + 8, VS = D + 16, DT = D / 32, KSTEPS = D / 16, CH = D / 8; // CH: 8-element chunks per row
     constexpr int NP = SPLIT ? 2 : 1; // operand planes: hi (, lo)
-    constexpr int NTH = 256 * HW, KBUF = NP * BN * KS, VBUF = NP * BN * VS; // halfs per buffer
+    static_assert(HW * KS <= 2 && !(SPLIT && KS == 2), "eight wavefronts at most; split operands leave no room for two tiles");
+    constexpr int NTH = 256 * HW * KS, KBUF = NP * BN * KS_, VBUF = NP * BN * VS, TILE = KBUF + VBUF; // halfs per staged tile
     extern __shared__ __attribute__((aligned(16))) fh_half ap_lds[]; // [2 buffers][K planes | V planes]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
-    const int h = (int)blockIdx.x * HW + (wave >> 2), bi = blockIdx.z, kh = h / (hq / hkv);
+    const int kset = KS == 2 ? wave >> 2 : 0; // which key tiles of a step this wavefront multiplies
+    const int h = (int)blockIdx.x * HW + (HW == 2 ? wave >> 2 : 0), bi = blockIdx.z, kh = h / (hq / hkv);
     // causal: the last query blocks see the most keys; with the block index on the slow grid axis ALL heads of the
     // longest block are dispatched first and the short blocks fill the tail
     const int qb0 = (causal ? (int)(gridDim.y - 1 - blockIdx.y) : (int)blockIdx.y) * 128;
-    const int qi = qb0 + (wave & 3) * 32 + li; // this lane's query row
+    const int qi = qb0 + (wave & 3) * 32 + li; // this lane's query row (KS = 2: both groups have the same rows)
     const int off = skv - sq;                  // causal: query i sees keys 0 .. i + off
     const TKV *kb = k + bi * kv_sb + kh * kv_sh, *vb = v + bi * kv_sb + kh * kv_sh;
 
@@ -133,13 +138,13 @@ __global__ __launch_bounds__(256 * HW) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     // A KV tile waits in registers (as f16; SPLIT: as the f32 values) from one tile before it is written to LDS.
     // Piece c = tid + NTH i of a tile: key c / CH, d chunk c % CH - consecutive threads along d, K and V alike.
-    constexpr int NCH = BN * CH / NTH;
+    constexpr int NCH = KS * BN * CH / NTH;
     uint4 kreg[SPLIT ? 1 : NCH], vreg[SPLIT ? 1 : NCH];
     float4 kraw[SPLIT ? 2 * NCH : 1], vraw[SPLIT ? 2 * NCH : 1];
     auto fetch = [&](int t0) {
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
-            const int c = tid + NTH * i, key = c / CH, dc = c % CH;
+            const int c = tid + NTH * i, key = c / CH, dc = c % CH; // key 0 .. KS * BN - 1: the KS tiles of a step
             // rows past the end repeat the last one (no branch): their scores are masked and their P is 0
             const int64_t row = (int64_t)(t0 + key < skv ? t0 + key : skv - 1) * kv_st + 8 * dc;
             if constexpr (SPLIT) {
@@ -158,10 +163,10 @@ __global__ __launch_bounds__(256 * HW) __attribute__((amdgpu_waves_per_eu(2, 2))
         }
     };
     auto stash = [&](int buf) { // K tile -> sK[key][d], V tile -> sV[key][d]
-        fh_half *sK = ap_lds + buf * (KBUF + VBUF), *sV = sK + KBUF;
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
-            const int c = tid + NTH * i, key = c / CH, dc = c % CH;
+            const int c = tid + NTH * i, kk = c / CH, key = kk % BN, dc = c % CH;
+            fh_half *sK = ap_lds + (buf * KS + kk / BN) * TILE, *sV = sK + KBUF;
             if constexpr (SPLIT) {
                 const float kx[8] = {kraw[2 * i].x, kraw[2 * i].y, kraw[2 * i].z, kraw[2 * i].w,
                                      kraw[2 * i + 1].x, kraw[2 * i + 1].y, kraw[2 * i + 1].z, kraw[2 * i + 1].w};
@@ -170,8 +175,8 @@ __global__ __launch_bounds__(256 * HW) __attribute__((amdgpu_waves_per_eu(2, 2))
                 uint4 uh, ul;
                 __builtin_memcpy(&uh, hi, 16);
                 __builtin_memcpy(&ul, lo, 16);
-                *(uint4 *)(sK + key * KS + 8 * dc) = uh;
-                *(uint4 *)(sK + BN * KS + key * KS + 8 * dc) = ul;
+                *(uint4 *)(sK + key * KS_ + 8 * dc) = uh;
+                *(uint4 *)(sK + BN * KS_ + key * KS_ + 8 * dc) = ul;
                 const float vx[8] = {vraw[2 * i].x, vraw[2 * i].y, vraw[2 * i].z, vraw[2 * i].w,
                                      vraw[2 * i + 1].x, vraw[2 * i + 1].y, vraw[2 * i + 1].z, vraw[2 * i + 1].w};
                 ap_split8(vx, hi, lo);
@@ -180,7 +185,7 @@ __global__ __launch_bounds__(256 * HW) __attribute__((amdgpu_waves_per_eu(2, 2))
                 *(uint4 *)(sV + key * VS + 8 * dc) = uh;
                 *(uint4 *)(sV + BN * VS + key * VS + 8 * dc) = ul;
             } else {
-                *(uint4 *)(sK + key * KS + 8 * dc) = kreg[i];
+                *(uint4 *)(sK + key * KS_ + 8 * dc) = kreg[i];
                 *(uint4 *)(sV + key * VS + 8 * dc) = vreg[i];
             }
         }
@@ -199,28 +204,31 @@ __global__ __launch_bounds__(256 * HW) __attribute__((amdgpu_waves_per_eu(2, 2))
     if (kend > 0) {
         fetch(0);
         stash(0);
-        if (BN < kend) fetch(BN);
+        if (KS * BN < kend) fetch(KS * BN);
     }
     __syncthreads();
 
     const float ninf = -INFINITY;
-    for (int t0 = 0, it = 0; t0 < kend; t0 += BN, it++) {
-        const fh_half *sK = ap_lds + (it & 1) * (KBUF + VBUF), *sV = sK + KBUF;
+    for (int ts = 0, it = 0; ts < kend; ts += KS * BN, it++) { // a step: KS tiles, one per group of four wavefronts
+        const int t0 = ts + kset * BN;
+        // a group without a tile in the last step multiplies the staged rows (clamped, finite) with every key masked
+        const int lim_t = (KS == 1 || t0 < kend) ? lim : -1;
+        const fh_half *sK = ap_lds + ((it & 1) * KS + kset) * TILE, *sV = sK + KBUF;
         // ---- S^T = K . Q^T for the two 32-key halves of the tile
         floatx16 st[2];
 #pragma unroll
         for (int r = 0; r < 16; r++) st[0][r] = st[1][r] = 0.f;
         if constexpr (!SPLIT) {
             // product i: key half i % 2, d step i / 2; the K operands are requested eight products ahead
-            const fh_half *ap = sK + prow * KS + 8 * g;
+            const fh_half *ap = sK + prow * KS_ + 8 * g;
             constexpr int NI = 2 * KSTEPS, AHEAD = 8;
             half8 ka[AHEAD];
 #pragma unroll
-            for (int i = 0; i < AHEAD; i++) ka[i] = *(const half8 *)(ap + (i & 1) * 32 * KS + 16 * (i >> 1));
+            for (int i = 0; i < AHEAD; i++) ka[i] = *(const half8 *)(ap + (i & 1) * 32 * KS_ + 16 * (i >> 1));
 #pragma unroll
             for (int i = 0; i < NI; i++) {
                 st[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[i % AHEAD], qf[i >> 1], st[i & 1], 0, 0, 0);
-                if (i + AHEAD < NI) ka[i % AHEAD] = *(const half8 *)(ap + (i & 1) * 32 * KS + 16 * ((i + AHEAD) >> 1));
+                if (i + AHEAD < NI) ka[i % AHEAD] = *(const half8 *)(ap + (i & 1) * 32 * KS_ + 16 * ((i + AHEAD) >> 1));
             }
             __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
 #pragma unroll
@@ -232,12 +240,12 @@ __global__ __launch_bounds__(256 * HW) __attribute__((amdgpu_waves_per_eu(2, 2))
         } else {
 #pragma unroll
             for (int kt = 0; kt < 2; kt++) {
-                const fh_half *ap = sK + (kt * 32 + prow) * KS + 8 * g;
+                const fh_half *ap = sK + (kt * 32 + prow) * KS_ + 8 * g;
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ks++) {
                     const half8 a = *(const half8 *)(ap + 16 * ks);
                     st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], st[kt], 0, 0, 0);
-                    const half8 al = *(const half8 *)(ap + BN * KS + 16 * ks);
+                    const half8 al = *(const half8 *)(ap + BN * KS_ + 16 * ks);
                     st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, qf[ks], st[kt], 0, 0, 0);
                     st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, ql[ks], st[kt], 0, 0, 0);
                 }
@@ -248,13 +256,13 @@ __global__ __launch_bounds__(256 * HW) __attribute__((amdgpu_waves_per_eu(2, 2))
         // (the scheduler may not mix the stages: the operands prefetched for one product and the tile in flight would
         // otherwise be live together with the scores)
         __builtin_amdgcn_sched_barrier(0);
-        if (t0 + BN < kend) stash((it + 1) & 1);
-        if (t0 + 2 * BN < kend) fetch(t0 + 2 * BN);
+        if (ts + KS * BN < kend) stash((it + 1) & 1);
+        if (ts + 2 * KS * BN < kend) fetch(ts + 2 * KS * BN);
         __builtin_amdgcn_sched_barrier(0);
         // ---- mask, running max: register r of half kt is key t0 + 32 kt + 16 (r / 8) + 8 g + r % 8
         // Only a tile that reaches past some query's last visible key pays for the compares (one branch for the
         // wavefront); the select works in place, so the common path has no register copies at the join.
-        if (__any(t0 + BN - 1 > lim)) {
+        if (__any(t0 + BN - 1 > lim_t)) {
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
@@ -262,7 +270,7 @@ __global__ __launch_bounds__(256 * HW) __attribute__((amdgpu_waves_per_eu(2, 2))
                     const int key = t0 + 32 * kt + 16 * (r >> 3) + 8 * g + (r & 7);
                     asm volatile("v_cmp_le_i32 vcc, %1, %2\n\tv_cndmask_b32 %0, %3, %0, vcc"
                                  : "+v"(st[kt][r])
-                                 : "v"(key), "v"(lim), "v"(ninf)
+                                 : "v"(key), "v"(lim_t), "v"(ninf)
                                  : "vcc");
                 }
         }
@@ -343,6 +351,30 @@ __global__ __launch_bounds__(256 * HW) __attribute__((amdgpu_waves_per_eu(2, 2))
         }
         __syncthreads(); // tile t+1 is staged, and nobody reads this tile's buffer any more
     }
+    if constexpr (KS == 2) {
+        // ---- the second group hands its statistics and output over: [value][query wavefront][lane] floats in the
+        // tile buffers (the barrier that ended the last step has passed: nobody reads them any more)
+        float *sm = (float *)ap_lds;
+        const int slot = (wave & 3) * 64 + lane;
+        if (kset == 1) {
+            sm[slot] = m_run;
+            sm[256 + slot] = l_run;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) sm[(2 + dt * 16 + r) * 256 + slot] = acc[dt][r];
+        }
+        __syncthreads();
+        if (kset == 1) return;
+        const float m1 = sm[slot], l1 = sm[256 + slot];
+        const float mm = fmaxf(m_run, m1), ref = mm == -INFINITY ? 0.f : mm;
+        const float f0 = __builtin_amdgcn_exp2f(m_run - ref), f1 = __builtin_amdgcn_exp2f(m1 - ref);
+        l_run = l_run * f0 + l1 * f1;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[dt][r] = acc[dt][r] * f0 + sm[(2 + dt * 16 + r) * 256 + slot] * f1;
+    }
     // ---- store: lane = query, register r of d-tile dt is d = 32 dt + 8 (r / 4) + 4 g + r % 4
     if (qi < sq) {
         const float inv = 1.0f / l_run;
@@ -356,13 +388,14 @@ __global__ __launch_bounds__(256 * HW) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
 }
 
-template <typename TQ, typename TKV, int D, bool SPLIT, int HW>
+template <typename TQ, typename TKV, int D, bool SPLIT, int HW, int KS = 1>
 static fh_status ap_launch_k(fh_device *dev, const void *q, int64_t q_sb, int64_t q_sh, int64_t q_st, const void *k,
                              const void *v, int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int b, int hq, int hkv, int sq,
                              int skv, float scale, int causal, void *out) {
-    constexpr int LDS = 2 * (SPLIT ? 2 : 1) * 64 * (D + 8 + D + 16) * 2; // two buffers of K and V planes, bytes
+    constexpr int LDS = 2 * KS * (SPLIT ? 2 : 1) * 64 * (D + 8 + D + 16) * 2; // two buffers of KS tiles (K and V planes), bytes
+    static_assert(KS == 1 || LDS >= (2 + (D / 32) * 16) * 256 * 4, "the merge of the key groups reuses the tile buffers");
     static_assert(LDS <= 160 * 1024, "KV tiles exceed the LDS of a compute unit");
-    auto kern = k_attn_prefill<TQ, TKV, D, SPLIT, HW>;
+    auto kern = k_attn_prefill<TQ, TKV, D, SPLIT, HW, KS>;
     static bool raised[64] = {}; // per kernel instance and device: allow more than 64 KB of dynamic LDS
     const bool known = dev->ordinal >= 0 && dev->ordinal < 64;
     if (!known || !raised[dev->ordinal]) {
@@ -370,7 +403,7 @@ static fh_status ap_launch_k(fh_device *dev, const void *q, int64_t q_sb, int64_
         if (known) raised[dev->ordinal] = true;
     }
     dim3 grid((unsigned)(hq / HW), (unsigned)((sq + 127) / 128), (unsigned)b);
-    kern<<<grid, 256 * HW, LDS, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k, (const TKV *)v, kv_sb,
+    kern<<<grid, 256 * HW * KS, LDS, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k, (const TKV *)v, kv_sb,
                                                kv_sh, kv_st, hq, hkv, sq, skv, scale, causal, (TQ *)out);
     FH_HIP(hipGetLastError());
     return FH_OK;
@@ -384,9 +417,15 @@ static fh_status ap_launch(fh_device *dev, const void *q, int64_t q_sb, int64_t 
     // split: short prompts are bound by the longest workgroup and by how many compute units have one at all.
     const long wgs = (long)hq * ((sq + 127) / 128) * b;
     const bool pair = (hq / hkv) % 2 == 0 && wgs >= 1024;
-#define FH_AP(D, HW) ap_launch_k<TQ, TKV, D, SPLIT, HW>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, scale, causal, out)
-    if (d == 128) return pair ? FH_AP(128, 2) : FH_AP(128, 1);
-    return pair ? FH_AP(64, 2) : FH_AP(64, 1);
+#define FH_AP(D, HW, KS) ap_launch_k<TQ, TKV, D, SPLIT, HW, KS>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, scale, causal, out)
+    if constexpr (!SPLIT) {
+        // short prompts: every workgroup is resident at once (two of four wavefronts per compute unit) and the launch
+        // lasts as long as the last query block's - its key tiles are shared out over two groups of wavefronts
+        const bool halves = wgs <= 2L * dev->compute_units && skv > 128;
+        if (halves) return d == 128 ? FH_AP(128, 1, 2) : FH_AP(64, 1, 2);
+    }
+    if (d == 128) return pair ? FH_AP(128, 2, 1) : FH_AP(128, 1, 1);
+    return pair ? FH_AP(64, 2, 1) : FH_AP(64, 1, 1);
 #undef FH_AP
 }
 
