@@ -124,6 +124,30 @@ def batch_leg(dev, sets_m1, steps: int, warmup: int, trains: int) -> list:
     return out
 
 
+def decoder_shapes_leg(dev, steps: int, warmup: int, trains: int) -> list:
+    """The two fused matrices a decode step of the 8B architecture launches besides the four layer shapes of
+    configs[1]: q|k|v (6144 x 4096) and gate|up (28672 x 4096), plain matvec, batch 1, weights rotated over 640 MB."""
+    from kalosm_amd import synth
+    from kalosm_amd.fusor import QMatrix, Tensor
+
+    out = []
+    for si, (n, k) in enumerate(((6144, 4096), (28672, 4096))):
+        wbytes = n * (k // 256) * 144
+        copies = max(2, -(-ROTATE_BYTES // wbytes))
+        raw = synth.random_weight(synth.Q4_K, n, k, seed=1100 + si)
+        s = dict(qs=[QMatrix.from_raw_bytes(dev, (n, k), raw, synth.Q4_K) for _ in range(copies)],
+                 x=Tensor.from_slice(dev, synth.random_activation(1, k, seed=2200 + si)), y=Tensor(dev, (1, n), "f32"))
+        nbytes = synth.matvec_bytes(synth.Q4_K, n, k, 1)
+        run_shape(s, warmup)
+        dev.sync()
+        ms, _ = timed_trains(dev, lambda: run_shape(s, steps, offset=warmup), trains)
+        us = ms * 1e3 / steps
+        out.append({"n": n, "k": k, "us_per_launch": round(us, 3), "GBps": round(nbytes / us / 1e3, 1),
+                    "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+        del s
+    return out
+
+
 def prefill_legs(dev, trains: int) -> dict:
     """configs[2]: Y = X . W^T with bf16 X [m, 4096] and Q6_K / Q8_0 W [14336, 4096]; configs[3]: causal attention,
     f16, 32 query heads on 8 KV heads, head_dim 128, and its decode variant.  Median device time of `trains` calls;
@@ -414,6 +438,7 @@ def main() -> int:
         s["qs"].clear()
     del sets
     if not args.no_legs:
+        out["decoder_shapes"] = decoder_shapes_leg(dev, args.steps, args.warmup, args.trains)
         out["prefill"] = prefill_legs(dev, max(3, min(args.trains, 5)))
 
     if args.e2e_eager:
