@@ -416,12 +416,14 @@ static fh_status ap_launch(fh_device *dev, const void *q, int64_t q_sb, int64_t 
     // Two heads of one KV group share the staged tiles when the launch still has enough workgroups without the
     // split: short prompts are bound by the longest workgroup and by how many compute units have one at all.
     const long wgs = (long)hq * ((sq + 127) / 128) * b;
-    const bool pair = (hq / hkv) % 2 == 0 && wgs >= 1024;
+    // attn_kernel = 6 / 7 / 8 force the workgroup shape (two heads / two key groups / plain) whatever the size: tests
+    const int64_t force = dev->opt_attn_kernel;
+    const bool pair = (hq / hkv) % 2 == 0 && (force == 6 || (force != 7 && force != 8 && wgs >= 1024));
 #define FH_AP(D, HW, KS) ap_launch_k<TQ, TKV, D, SPLIT, HW, KS>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, scale, causal, out)
     if constexpr (!SPLIT) {
         // short prompts: every workgroup is resident at once (two of four wavefronts per compute unit) and the launch
         // lasts as long as the last query block's - its key tiles are shared out over two groups of wavefronts
-        const bool halves = wgs <= 2L * dev->compute_units && skv > 128;
+        const bool halves = force == 7 || (force != 6 && force != 8 && wgs <= 2L * dev->compute_units && skv > 128);
         if (halves) return d == 128 ? FH_AP(128, 1, 2) : FH_AP(64, 1, 2);
     }
     if (d == 128) return pair ? FH_AP(128, 2, 1) : FH_AP(128, 1, 1);

@@ -319,6 +319,31 @@ def test_attention_prefill_f32_split(dev, oracle, sq, skv, causal, d):
     assert_close(got, rows, abs_tol=1e-3, rel_tol=1e-4, what="vs the exact row kernel")
 
 
+@pytest.mark.parametrize("force", [6, 7, 8])
+@pytest.mark.parametrize("sq,skv,causal,d", [(300, 300, True, 128), (129, 700, True, 128), (257, 190, False, 128),
+                                             (64, 65, True, 64), (384, 384, True, 64), (33, 200, True, 128)])
+def test_attention_prefill_workgroup_shapes(dev, oracle, force, sq, skv, causal, d):
+    """The three workgroup shapes of the matrix-core kernel on the same ragged inputs, whatever the dispatch would
+    pick for the size (attn_kernel = 6: two heads of a KV group share the staged tiles; 7: the key tiles of a query
+    block shared out over two groups of wavefronts and merged; 8: four wavefronts, one head): f16 and f32 queries on an
+    f16 cache, causal with the queries at the end of a longer cache, odd tile counts (a group without a tile in the last
+    step), a single query block."""
+    h, hkv = 8, 2
+    rng = np.random.default_rng(sq * 31 + skv * 7 + d + force)
+    scale = 1 / np.sqrt(d)
+    q = rng.standard_normal((1, h, sq, d)).astype(np.float16)
+    k = rng.standard_normal((1, hkv, skv, d)).astype(np.float16)
+    v = rng.standard_normal((1, hkv, skv, d)).astype(np.float16)
+    qf, kf, vf = (a.astype(np.float32) for a in (q, k, v))
+    want = oracle.flash_attention(qf, kf, vf, scale, oracle.MASK_CAUSAL if causal else oracle.MASK_NONE, None)
+    dev.set_option("attn_kernel", force)
+    try:
+        got = run_attn(dev, q, k, v, scale, MaskKind.Causal if causal else None, dtype="f16")
+    finally:
+        dev.set_option("attn_kernel", 0)
+    assert_close(got, want, abs_tol=1e-2, rel_tol=1e-3, what=f"f16 prefill shape {force}: {sq}x{skv}x{d}")
+
+
 def test_attention_prefill_f32_on_request(dev, oracle):
     """f32 operands through the same kernel (rounded to f16 inside, f32 out), and the invariants that do not depend
     on the rounding: V constant -> output constant, causal row 0 -> v_0."""
