@@ -157,11 +157,15 @@ def prefill_legs(dev, trains: int) -> dict:
     from kalosm_amd.fusor import MaskKind, QMatrix, Tensor
 
     def med(fn):
-        for _ in range(2):
+        # warm-up: at least three calls and 50 ms of them (the device drops its clocks while the host prepares the next
+        # case's inputs; the first calls after that run slower than the steady state the figure is about)
+        t0, calls = time.perf_counter(), 0
+        while calls < 3 or time.perf_counter() - t0 < 0.05:
             fn()
-        dev.sync()
+            dev.sync()
+            calls += 1
         ts = []
-        for _ in range(trains):
+        for _ in range(max(trains, 7)):
             dev.timer_start()
             fn()
             ts.append(dev.timer_stop())
