@@ -531,6 +531,213 @@ __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__re
     }
 }
 
+// ------------------------------------------------------------------------------ integer codes, scale after the MFMA
+// Q8_0 and Q4_0 (one f16 scale per 32 weights = one k step): the weight operand is the integer code itself
+// (-128 .. 127, -8 .. 7: exact in f16, ONE term instead of the hi + lo pair of a dequantised weight), the products of
+// a step are collected in a zeroed accumulator and the block scale is applied to it in f32:
+//   acc += d[n, step] * sum_k x[m, k] * code[n, k]
+// which is the reference's sum with d factored out of each block.  The roles of the MFMA operands are swapped against
+// k_qmm_tile2 (A = activations, B = weights), so a lane holds ONE weight row of the output tile and d is a per-lane
+// scalar: 16 multiply-adds per lane, block and 32 x 32 tile against two MFMAs saved.  Same tile (128 weight rows x 256
+// activation rows, 8 wavefronts of 64 x 64), same pipeline (raw bytes and activation slab of step s+2 in registers,
+// step s+1 decoded into the second LDS buffer, one barrier per step).
+typedef _Float16 qmm_half2 __attribute__((ext_vector_type(2)));
+
+template <int T, int NTERM, int WM>
+__global__ __launch_bounds__(128 * WM) void k_qmm_tile2i(QView q, const _Float16 *__restrict__ xh,
+                                                    const _Float16 *__restrict__ xl, const float *__restrict__ rs,
+                                                    int m, float *__restrict__ y) {
+    static_assert(T == FH_Q8_0 || T == FH_Q4_0, "formats with one scale per 32 weights");
+    // WM = 4: eight wavefronts, 256 activation rows; WM = 2: four wavefronts, 128 activation rows - two such workgroups
+    // share a compute unit and are at different points of their steps (one's MFMAs under the other's scaling and staging)
+    constexpr int WN = 2, FN = 2, FM = 2, TN = WN * FN * 32, TM = WM * FM * 32, NT = 128 * WM, NA = 512 / NT;
+    constexpr int A_H = TN * QMM_LDK, B_H = TM * QMM_LDK;       // halfs per plane
+    constexpr int BUF = A_H + NTERM * B_H + 2 * TN;            // halfs per buffer: codes, x hi (, x lo), TN f32 scales
+    extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31;
+    const int wn = wave / WM, wm = wave % WM;
+    const int64_t n0 = (int64_t)blockIdx.x * TN;
+    const int m0 = blockIdx.y * TM;
+    const int K = (int)q.k, ksteps = K / 32;
+    const int64_t tiles16 = (q.n + 15) / 16;
+    // weight duty: NA items (row, lane group) of 8 codes per step; activation duty: two 16-byte pieces per plane and step
+    const int a_g = tid & 3, a_j = (tid >> 2) & 15;
+    int a_row[NA];
+    int64_t a_tile[NA];
+#pragma unroll
+    for (int u = 0; u < NA; u++) {
+        a_row[u] = (tid >> 2) + u * (NT / 4);
+        a_tile[u] = (n0 >> 4) + (a_row[u] >> 4);
+        if (a_tile[u] >= tiles16) a_tile[u] = tiles16 - 1; // rows past the end decode a valid tile and are never stored
+    }
+    const int b_c = tid & 3, b_row0 = tid >> 2, b_row1 = b_row0 + TM / 2;
+    const int64_t b_off0 = (int64_t)(m0 + b_row0 < m ? m0 + b_row0 : m - 1) * K + b_c * 8;
+    const int64_t b_off1 = (int64_t)(m0 + b_row1 < m ? m0 + b_row1 : m - 1) * K + b_c * 8;
+    struct Slab {
+        QmmRaw raw[NA];
+        uint4 h0, h1, l0, l1;
+    } s0, s1;
+    auto fetch = [&](Slab &sl, int ks) {
+#pragma unroll
+        for (int u = 0; u < NA; u++) qmm_load_raw<T>(q, a_tile[u], a_j, a_g, ks, sl.raw[u]);
+        sl.h0 = *(const uint4 *)(xh + b_off0 + ks * 32);
+        sl.h1 = *(const uint4 *)(xh + b_off1 + ks * 32);
+        if (NTERM == 2) {
+            sl.l0 = *(const uint4 *)(xl + b_off0 + ks * 32);
+            sl.l1 = *(const uint4 *)(xl + b_off1 + ks * 32);
+        }
+    };
+    // two code bytes (already 0 .. 255 resp. 0 .. 15) under the high byte 0x64 are the halfs 1024 + u; minus the bias
+    auto codes2 = [&](uint32_t bytes, uint32_t sel, float bias) -> uint32_t {
+        const uint32_t w = __builtin_amdgcn_perm(0x64646464u, bytes, sel);
+        qmm_half2 h;
+        __builtin_memcpy(&h, &w, 4);
+        h = h - qmm_half2{(_Float16)bias, (_Float16)bias};
+        uint32_t o;
+        __builtin_memcpy(&o, &h, 4);
+        return o;
+    };
+    auto stage = [&](const Slab &sl, int ks) {
+        _Float16 *buf = smem + (ks & 1) * BUF;
+#pragma unroll
+        for (int u = 0; u < NA; u++) {
+        if (T == FH_Q8_0) { // bytes 0 .. 3 of a, then of b: positions 8 g .. 8 g + 7 of the step
+            const uint32_t ua = sl.raw[u].a ^ 0x80808080u, ub = sl.raw[u].b ^ 0x80808080u;
+            uint4 c;
+            c.x = codes2(ua, 0x04010400u, 1152.f);
+            c.y = codes2(ua, 0x04030402u, 1152.f);
+            c.z = codes2(ub, 0x04010400u, 1152.f);
+            c.w = codes2(ub, 0x04030402u, 1152.f);
+            *(uint4 *)(buf + a_row[u] * QMM_LDK + 8 * a_g) = c;
+        } else { // low nibbles: positions 4 g .. 4 g + 3, high nibbles: 16 + 4 g .. 16 + 4 g + 3
+            const uint32_t lo = sl.raw[u].a & 0x0F0F0F0Fu, hi = (sl.raw[u].a >> 4) & 0x0F0F0F0Fu;
+            uint2 c0, c1;
+            c0.x = codes2(lo, 0x04010400u, 1032.f);
+            c0.y = codes2(lo, 0x04030402u, 1032.f);
+            c1.x = codes2(hi, 0x04010400u, 1032.f);
+            c1.y = codes2(hi, 0x04030402u, 1032.f);
+            *(uint2 *)(buf + a_row[u] * QMM_LDK + 4 * a_g) = c0;
+            *(uint2 *)(buf + a_row[u] * QMM_LDK + 16 + 4 * a_g) = c1;
+        }
+        ((float *)(buf + A_H + NTERM * B_H))[a_row[u]] = fh_h2f((uint16_t)sl.raw[u].h.x); // the four threads of a row: same value
+        }
+        *(uint4 *)(buf + A_H + b_row0 * QMM_LDK + b_c * 8) = sl.h0;
+        *(uint4 *)(buf + A_H + b_row1 * QMM_LDK + b_c * 8) = sl.h1;
+        if (NTERM == 2) {
+            *(uint4 *)(buf + A_H + B_H + b_row0 * QMM_LDK + b_c * 8) = sl.l0;
+            *(uint4 *)(buf + A_H + B_H + b_row1 * QMM_LDK + b_c * 8) = sl.l1;
+        }
+    };
+    floatx16 acc[FN][FM];
+#pragma unroll
+    for (int a = 0; a < FN; a++)
+#pragma unroll
+        for (int b = 0; b < FM; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
+
+    fetch(s0, 0);
+    if (ksteps > 1) fetch(s1, 1);
+    stage(s0, 0);
+    auto kstep = [&](int ks, Slab &mine, const Slab &other) {
+        if (ks < ksteps) {
+            __syncthreads(); // buffer ks & 1 is complete; the other one is no longer read
+            fetch(mine, ks + 2 < ksteps ? ks + 2 : ksteps - 1); // (no branch in the step: past the end, a repeat)
+            const _Float16 *buf = smem + (ks & 1) * BUF;
+            floatx16 part[FN][FM];
+#pragma unroll
+            for (int a = 0; a < FN; a++)
+#pragma unroll
+                for (int b = 0; b < FM; b++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) part[a][b][r] = 0.f;
+            // all operands of the step first (12 or 16 reads of 16 bytes), then the products weight tile by weight tile:
+            // the scaling of tile a runs under the MFMAs of tile a + 1 (a wavefront hides vector instructions under its
+            // own MFMAs), the scaling of the last tile under the decode of the next slab
+            half8 wc[2][FN], xhv[2][FM], xlv[2][FM];
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++) {
+                const int ko = kk * 16 + 8 * (lane >> 5);
+#pragma unroll
+                for (int a = 0; a < FN; a++) wc[kk][a] = *(const half8 *)(buf + ((wn * FN + a) * 32 + li) * QMM_LDK + ko);
+#pragma unroll
+                for (int b = 0; b < FM; b++) {
+                    const int row = (wm * FM + b) * 32 + li;
+                    xhv[kk][b] = *(const half8 *)(buf + A_H + row * QMM_LDK + ko);
+                    if (NTERM == 2) xlv[kk][b] = *(const half8 *)(buf + A_H + B_H + row * QMM_LDK + ko);
+                }
+            }
+            const float *sd = (const float *)(buf + A_H + NTERM * B_H);
+            float dl[FN];
+#pragma unroll
+            for (int a = 0; a < FN; a++) dl[a] = sd[(wn * FN + a) * 32 + li]; // the lane's weight rows
+#pragma unroll
+            for (int a = 0; a < FN; a++) {
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                    for (int b = 0; b < FM; b++) {
+                        part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xhv[kk][b], wc[kk][a], part[a][b], 0, 0, 0);
+                        if (NTERM == 2)
+                            part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xlv[kk][b], wc[kk][a], part[a][b], 0, 0, 0);
+                    }
+            }
+#pragma unroll
+            for (int a = 0; a < FN; a++)
+#pragma unroll
+                for (int b = 0; b < FM; b++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[a][b][r] = fmaf(part[a][b][r], dl[a], acc[a][b][r]);
+            stage(other, ks + 1 < ksteps ? ks + 1 : ks); // (no branch: the last step stages a repeat nobody reads)
+            {
+                constexpr int MPT = 2 * FM * NTERM; // MFMAs per weight tile
+                __builtin_amdgcn_sched_group_barrier(0x100, 2 * (FN + NTERM * FM) + FN, 0); // the operand and scale reads
+                __builtin_amdgcn_sched_group_barrier(0x008, MPT, 0);                          // tile 0
+#pragma unroll
+                for (int a = 1; a < FN; a++)
+#pragma unroll
+                    for (int i = 0; i < MPT; i++) { // tile a, with the 16 FM multiply-adds of tile a - 1 spread under it
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, 16 * FM / MPT, 0);
+                    }
+            }
+        }
+    };
+    for (int ks0 = 0; ks0 < ksteps; ks0 += 2) { // the register sets alternate: no indexing survives into the code
+        kstep(ks0, s0, s1);
+        kstep(ks0 + 1, s1, s0);
+    }
+    // lane = weight row n (column of the MFMA result), register r = activation row 8 (r / 4) + 4 (lane / 32) + r % 4
+#pragma unroll
+    for (int a = 0; a < FN; a++) {
+        const int64_t nn = n0 + (wn * FN + a) * 32 + li;
+        if (nn >= q.n) continue;
+#pragma unroll
+        for (int b = 0; b < FM; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int mm = m0 + (wm * FM + b) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (mm < m) y[(int64_t)mm * q.n + nn] = acc[a][b][r] * rs[mm];
+            }
+    }
+}
+
+template <int T, int NTERM, int WM>
+static fh_status qmm_launch_tile2i(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const float *rs, int m,
+                                   float *y) {
+    constexpr int TM = WM * 64;
+    constexpr size_t lds = 2 * (size_t)(128 * QMM_LDK + NTERM * TM * QMM_LDK + 2 * 128) * 2;
+    static bool attr_done = false;
+    if (!attr_done) {
+        FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2i<T, NTERM, WM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_done = true;
+    }
+    dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + TM - 1) / TM));
+    k_qmm_tile2i<T, NTERM, WM><<<grid, 128 * WM, lds, q->dev->stream>>>(fh_view(q), xh, xl, rs, m, y);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
 // y = sum of the partial planes of a k-split product, in plane order (deterministic)
 __global__ void k_qmm_sum_planes(const float4 *__restrict__ part, int planes, int64_t n4, float4 *__restrict__ y) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -581,8 +788,16 @@ static fh_status qmm_launch_t(const fh_qmatrix *q, const _Float16 *xh, const _Fl
     // (opt_matmul_kernel = 3: never, 4: always 256)
     const int64_t tn = (q->n + 127) / 128, cus = q->dev->compute_units;
     const int64_t mk = q->dev->opt_matmul_kernel;
-    if (mk == 4 || (m > 128 && tn * ((m + 255) / 256) * 5 >= cus * 4 && mk != 3))
+    if (mk == 4 || mk == 8 || (m > 128 && tn * ((m + 255) / 256) * 5 >= cus * 4 && mk != 3)) { // 8: as 4, integer codes
+        // one scale per 32 weights: integer codes and the scale after the MFMA (matmul_kernel = 6 keeps the split form)
+        if constexpr (T == FH_Q8_0 || T == FH_Q4_0) {
+            // (matmul_kernel = 7: four wavefronts and 128 activation rows per workgroup, two workgroups per compute unit:
+            // measured slower, 596 against 496 µs for 2048 x 14336 x 4096)
+            if (mk == 7) return qmm_launch_tile2i<T, NTERM, 2>(q, xh, xl, rs, m, y);
+            if (mk != 6 && mk != 4) return qmm_launch_tile2i<T, NTERM, 4>(q, xh, xl, rs, m, y);
+        }
         return qmm_launch_tile2<T, NTERM, 2, 2, 2>(q, xh, xl, rs, m, y);
+    }
     if (m > 64 && mk != 3 && mk != 5) {
         // too few tiles for the device: split k over workgroups rather than shrink the tile (every tile row of
         // workgroups decodes the weights again), as long as a split keeps 16 steps; the partial planes are summed

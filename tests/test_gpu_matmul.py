@@ -130,6 +130,38 @@ def test_tile_matmul_bf16_activations(dev, oracle, ty, m):
         assert_close(got, want, what=f"bf16 {NAMES[ty]} m={m} kernel option {force}")
 
 
+@pytest.mark.parametrize("act", ["f32", "bf16"])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_0], ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("m,n,k", [(256, 128, 256), (300, 200, 96), (129, 1000, 1024), (513, 130, 4096)])
+def test_integer_code_tile_kernel(dev, oracle, ty, act, m, n, k):
+    """Q8_0 / Q4_0 through the tile kernel that multiplies the integer codes and applies the block scale to the
+    accumulated block (matmul_kernel = 8 selects it whatever the size; the dispatch takes it for large products): ragged
+    tiles in both directions, an odd number of k steps, both activation forms; against the checker, and one-hot
+    activations pick single dequantised weights exactly."""
+    raw = synth.random_weight(ty, n, k, seed=m + n + k)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    xa = synth.random_activation(m, k, seed=7)
+    if act == "bf16":
+        bits = synth.to_bf16_bits(xa)
+        xa = (bits.astype(np.uint32) << 16).view(np.float32)
+        x = Tensor.from_slice(dev, bits, dtype="bf16")
+    else:
+        x = Tensor.from_slice(dev, xa)
+    want = oracle.q_mat_mul(ty, xa, raw, n)
+    dev.set_option("matmul_kernel", 8)
+    try:
+        got = x.q_mat_mul(q).as_slice()
+        onehot = np.zeros((m, k), dtype=np.float32)
+        cols = (np.arange(m) * 37 + 5) % k
+        onehot[np.arange(m), cols] = 0.5
+        picked = Tensor.from_slice(dev, onehot).q_mat_mul(q).as_slice()
+    finally:
+        dev.set_option("matmul_kernel", 0)
+    assert_close(got, want, abs_tol=1e-2, rel_tol=1e-3, what=f"integer-code tile {NAMES[ty]} {act} {m}x{n}x{k}")
+    deq = oracle.dequantize(ty, raw).reshape(n, k)
+    assert np.array_equal(picked, 0.5 * deq[:, cols].T), "one-hot activations pick dequantised weights exactly"
+
+
 @pytest.mark.parametrize("m", [512, 2048])
 @pytest.mark.parametrize("ty", [Q6_K, Q8_0], ids=lambda t: NAMES[t])
 def test_prefill_shape_spot_check(dev, oracle, ty, m):
