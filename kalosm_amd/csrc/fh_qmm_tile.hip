@@ -722,6 +722,222 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2i(QView q, const _Float16
     }
 }
 
+// The integer-code kernel with two blocks of 32 weights per step (64 of k): half as many workgroup barriers and
+// operand-read latencies per weight, one 16-byte load per weight item and step (the repack keeps the two blocks'
+// codes of a lane side by side). One activation plane only (f16 / bf16 activations); k must be a multiple of 64.
+template <int T, int WM>
+__global__ __launch_bounds__(128 * WM) void k_qmm_tile2j(QView q, const _Float16 *__restrict__ xh,
+                                                    const float *__restrict__ rs, int m, float *__restrict__ y) {
+    static_assert(T == FH_Q8_0 || T == FH_Q4_0, "formats with one scale per 32 weights");
+    // An LDS row is 64 halfs = eight 16-byte pieces; piece c of row r sits at position c ^ sw(r), sw(r) = bit 1 of r
+    // (as bit 2) and bits 2 .. 3 of r: the 16-byte reads of 16 consecutive rows at one c, the 64-byte code writes of four
+    // consecutive rows and the 128-byte activation writes of two rows all cover the 64 banks once
+    constexpr int LDK = 64;
+    auto sw = [](int row) { return ((row >> 1) & 1) << 2 | ((row >> 2) & 3); };
+    constexpr int WN = 2, FN = 2, FM = 2, TN = WN * FN * 32, TM = WM * FM * 32, NT = 128 * WM, NA = 512 / NT;
+    constexpr int A_H = TN * LDK, B_H = TM * LDK; // halfs per plane
+    constexpr int BUF = A_H + B_H + 4 * TN;       // halfs per buffer: codes, activations, 2 TN f32 scales
+    extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31;
+    const int wn = wave / WM, wm = wave % WM;
+    const int64_t n0 = (int64_t)blockIdx.x * TN;
+    const int m0 = blockIdx.y * TM;
+    const int K = (int)q.k, ksteps = K / 64;
+    const int64_t tiles16 = (q.n + 15) / 16;
+    const int a_g = tid & 3, a_j = (tid >> 2) & 15;
+    int a_row[NA];
+    const uint8_t *a_rec[NA];
+#pragma unroll
+    for (int u = 0; u < NA; u++) {
+        a_row[u] = (tid >> 2) + u * (NT / 4);
+        int64_t t = (n0 >> 4) + (a_row[u] >> 4);
+        if (t >= tiles16) t = tiles16 - 1; // rows past the end decode a valid tile and are never stored
+        a_rec[u] = q.data + t * q.recs * (T == FH_Q8_0 ? 1088 : 1152);
+    }
+    // activation duty: four 16-byte pieces per step, the eight threads of a row cover its 128 bytes
+    const int b_c = tid & 7;
+    int64_t b_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int row = m0 + (tid >> 3) + i * (NT / 8);
+        b_off[i] = (int64_t)(row < m ? row : m - 1) * K + b_c * 8;
+    }
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    struct Slab {
+        uint32_t c0[NA], c1[NA], c2[NA], c3[NA], d[NA];
+        u32x4 h[4];
+    } sl;
+    auto fetch = [&](int ks) {
+#pragma unroll
+        for (int u = 0; u < NA; u++) {
+            if (T == FH_Q8_0) { // a record holds 64 of k: this step
+                const uint8_t *rec = a_rec[u] + (int64_t)ks * 1088;
+                const u32x4 c = *(const u32x4 *)(rec + (a_g * 16 + a_j) * 16);
+                sl.c0[u] = c.x, sl.c1[u] = c.y, sl.c2[u] = c.z, sl.c3[u] = c.w;
+                sl.d[u] = *(const uint32_t *)(rec + 1024 + 4 * a_j);
+            } else { // a record holds 128 of k: two steps
+                const uint8_t *rec = a_rec[u] + (int64_t)(ks >> 1) * 1152;
+                const uint2 c = *(const uint2 *)(rec + (a_g * 16 + a_j) * 16 + 8 * (ks & 1));
+                sl.c0[u] = c.x, sl.c1[u] = c.y;
+                sl.d[u] = *(const uint32_t *)(rec + 1024 + 8 * a_j + 4 * (ks & 1));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) sl.h[i] = *(const u32x4 *)(xh + b_off[i] + ks * 64);
+    };
+    // two code bytes (already 0 .. 255 resp. 0 .. 15) under the high byte 0x64 are the halfs 1024 + u; minus the bias
+    auto codes2 = [&](uint32_t bytes, uint32_t sel, float bias) -> uint32_t {
+        const uint32_t w = __builtin_amdgcn_perm(0x64646464u, bytes, sel);
+        qmm_half2 h;
+        __builtin_memcpy(&h, &w, 4);
+        h = h - qmm_half2{(_Float16)bias, (_Float16)bias};
+        uint32_t o;
+        __builtin_memcpy(&o, &h, 4);
+        return o;
+    };
+    auto stage = [&](int ks) {
+        _Float16 *buf = smem + (ks & 1) * BUF;
+        float *sd = (float *)(buf + A_H + B_H);
+#pragma unroll
+        for (int u = 0; u < NA; u++) {
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                _Float16 *dst = buf + a_row[u] * LDK;
+                const int sr = sw(a_row[u]);
+                if (T == FH_Q8_0) { // bytes 0 .. 3 of the first word, then of the second: positions 8 g .. 8 g + 7
+                    const uint32_t ua = (blk ? sl.c2[u] : sl.c0[u]) ^ 0x80808080u;
+                    const uint32_t ub = (blk ? sl.c3[u] : sl.c1[u]) ^ 0x80808080u;
+                    uint4 c;
+                    c.x = codes2(ua, 0x04010400u, 1152.f);
+                    c.y = codes2(ua, 0x04030402u, 1152.f);
+                    c.z = codes2(ub, 0x04010400u, 1152.f);
+                    c.w = codes2(ub, 0x04030402u, 1152.f);
+                    *(uint4 *)(dst + 8 * ((4 * blk + a_g) ^ sr)) = c;
+                } else { // low nibbles: positions 4 g .. 4 g + 3, high nibbles: 16 + 4 g .. 16 + 4 g + 3
+                    const uint32_t w = blk ? sl.c1[u] : sl.c0[u];
+                    const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+                    uint2 c0, c1;
+                    c0.x = codes2(lo, 0x04010400u, 1032.f);
+                    c0.y = codes2(lo, 0x04030402u, 1032.f);
+                    c1.x = codes2(hi, 0x04010400u, 1032.f);
+                    c1.y = codes2(hi, 0x04030402u, 1032.f);
+                    *(uint2 *)(dst + 8 * ((4 * blk + (a_g >> 1)) ^ sr) + 4 * (a_g & 1)) = c0;
+                    *(uint2 *)(dst + 8 * ((4 * blk + 2 + (a_g >> 1)) ^ sr) + 4 * (a_g & 1)) = c1;
+                }
+                sd[blk * TN + a_row[u]] = fh_h2f((uint16_t)(sl.d[u] >> (16 * blk))); // the four threads of a row: same value
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int row = (tid >> 3) + i * (NT / 8);
+            *(u32x4 *)(buf + A_H + row * LDK + 8 * (b_c ^ sw(row))) = sl.h[i];
+        }
+    };
+    floatx16 acc[FN][FM];
+#pragma unroll
+    for (int a = 0; a < FN; a++)
+#pragma unroll
+        for (int b = 0; b < FM; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
+
+    auto compute = [&](int ks) {
+        const _Float16 *buf = smem + (ks & 1) * BUF;
+        const float *sd = (const float *)(buf + A_H + B_H);
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++) {
+            floatx16 part[FN][FM];
+#pragma unroll
+            for (int a = 0; a < FN; a++)
+#pragma unroll
+                for (int b = 0; b < FM; b++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) part[a][b][r] = 0.f;
+            half8 wc[2][FN], xhv[2][FM];
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++) {
+                const int ko = 8 * ((4 * blk + 2 * kk + (lane >> 5)) ^ sw(li)); // (tile bases are multiples of 32 rows)
+#pragma unroll
+                for (int a = 0; a < FN; a++) wc[kk][a] = *(const half8 *)(buf + ((wn * FN + a) * 32 + li) * LDK + ko);
+#pragma unroll
+                for (int b = 0; b < FM; b++) xhv[kk][b] = *(const half8 *)(buf + A_H + ((wm * FM + b) * 32 + li) * LDK + ko);
+            }
+            float dl[FN];
+#pragma unroll
+            for (int a = 0; a < FN; a++) dl[a] = sd[blk * TN + (wn * FN + a) * 32 + li]; // the lane's weight rows
+#pragma unroll
+            for (int a = 0; a < FN; a++)
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                    for (int b = 0; b < FM; b++)
+                        part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xhv[kk][b], wc[kk][a], part[a][b], 0, 0, 0);
+#pragma unroll
+            for (int a = 0; a < FN; a++)
+#pragma unroll
+                for (int b = 0; b < FM; b++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[a][b][r] = fmaf(part[a][b][r], dl[a], acc[a][b][r]);
+        }
+        {
+            // block 0: reads, weight tile 0, weight tile 1 over the multiply-adds of tile 0; block 1: reads, tile 0 over
+            // the multiply-adds of block 0's tile 1, tile 1 over those of its tile 0; the last 32 run under the decode
+            constexpr int MPT = 2 * FM;
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * (FN + FM) + FN, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, MPT, 0);
+#pragma unroll
+            for (int i = 0; i < MPT; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 16 * FM / MPT, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * (FN + FM) + FN, 0);
+#pragma unroll
+            for (int i = 0; i < 2 * MPT; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 16 * FM / MPT, 0);
+            }
+        }
+    };
+    fetch(0);
+    stage(0);
+    // (A schedule in which the second wavefront of every SIMD runs half a step behind the first - one multiplies while
+    // the other decodes and stages, two barriers per step - was measured slower: 422 against 378 us at 2048 x 14336 x 4096.)
+    for (int ks = 0; ks < ksteps; ks++) {
+        __syncthreads(); // buffer ks & 1 is complete; the other one is no longer read
+        fetch(ks + 1 < ksteps ? ks + 1 : ks); // (no branch in the step: past the end, a repeat)
+        compute(ks);
+        stage(ks + 1); // (no branch: the last step stages a repeat nobody reads)
+    }
+    // lane = weight row n (column of the MFMA result), register r = activation row 8 (r / 4) + 4 (lane / 32) + r % 4
+#pragma unroll
+    for (int a = 0; a < FN; a++) {
+        const int64_t nn = n0 + (wn * FN + a) * 32 + li;
+        if (nn >= q.n) continue;
+#pragma unroll
+        for (int b = 0; b < FM; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int mm = m0 + (wm * FM + b) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (mm < m) y[(int64_t)mm * q.n + nn] = acc[a][b][r] * rs[mm];
+            }
+    }
+}
+
+template <int T, int WM>
+static fh_status qmm_launch_tile2j(const fh_qmatrix *q, const _Float16 *xh, const float *rs, int m, float *y) {
+    constexpr int TM = WM * 64;
+    constexpr size_t lds = 2 * (size_t)(128 * 64 + TM * 64 + 4 * 128) * 2;
+    static bool attr_done = false;
+    if (!attr_done) {
+        FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2j<T, WM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_done = true;
+    }
+    dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + TM - 1) / TM));
+    k_qmm_tile2j<T, WM><<<grid, 128 * WM, lds, q->dev->stream>>>(fh_view(q), xh, rs, m, y);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
 template <int T, int NTERM, int WM>
 static fh_status qmm_launch_tile2i(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const float *rs, int m,
                                    float *y) {
@@ -788,12 +1004,15 @@ static fh_status qmm_launch_t(const fh_qmatrix *q, const _Float16 *xh, const _Fl
     // (opt_matmul_kernel = 3: never, 4: always 256)
     const int64_t tn = (q->n + 127) / 128, cus = q->dev->compute_units;
     const int64_t mk = q->dev->opt_matmul_kernel;
-    if (mk == 4 || mk == 8 || (m > 128 && tn * ((m + 255) / 256) * 5 >= cus * 4 && mk != 3)) { // 8: as 4, integer codes
+    if (mk == 4 || mk == 8 || mk == 9 || (m > 128 && tn * ((m + 255) / 256) * 5 >= cus * 4 && mk != 3)) { // 8, 9: as 4, integer codes
         // one scale per 32 weights: integer codes and the scale after the MFMA (matmul_kernel = 6 keeps the split form)
         if constexpr (T == FH_Q8_0 || T == FH_Q4_0) {
             // (matmul_kernel = 7: four wavefronts and 128 activation rows per workgroup, two workgroups per compute unit:
             // measured slower, 596 against 496 µs for 2048 x 14336 x 4096)
             if (mk == 7) return qmm_launch_tile2i<T, NTERM, 2>(q, xh, xl, rs, m, y);
+            if constexpr (NTERM == 1) // (matmul_kernel = 9: one block of 32 per step also for one activation plane)
+                if (mk != 6 && mk != 4 && mk != 9 && q->k % 64 == 0)
+                    return qmm_launch_tile2j<T, 4>(q, xh, rs, m, y);
             if (mk != 6 && mk != 4) return qmm_launch_tile2i<T, NTERM, 4>(q, xh, xl, rs, m, y);
         }
         return qmm_launch_tile2<T, NTERM, 2, 2, 2>(q, xh, xl, rs, m, y);

@@ -132,11 +132,13 @@ def test_tile_matmul_bf16_activations(dev, oracle, ty, m):
 
 @pytest.mark.parametrize("act", ["f32", "bf16"])
 @pytest.mark.parametrize("ty", [Q8_0, Q4_0], ids=lambda t: NAMES[t])
-@pytest.mark.parametrize("m,n,k", [(256, 128, 256), (300, 200, 96), (129, 1000, 1024), (513, 130, 4096)])
-def test_integer_code_tile_kernel(dev, oracle, ty, act, m, n, k):
-    """Q8_0 / Q4_0 through the tile kernel that multiplies the integer codes and applies the block scale to the
-    accumulated block (matmul_kernel = 8 selects it whatever the size; the dispatch takes it for large products): ragged
-    tiles in both directions, an odd number of k steps, both activation forms; against the checker, and one-hot
+@pytest.mark.parametrize("m,n,k", [(256, 128, 256), (300, 200, 96), (300, 200, 192), (129, 1000, 1024), (513, 130, 4096)])
+@pytest.mark.parametrize("force", [8, 9])
+def test_integer_code_tile_kernel(dev, oracle, ty, act, m, n, k, force):
+    """Q8_0 / Q4_0 through the tile kernels that multiply the integer codes and apply the block scale to the
+    accumulated block (matmul_kernel = 8 selects them whatever the size; the dispatch takes them for large products):
+    64 of k per step for one activation plane (bf16) and k a multiple of 64, 32 of k per step otherwise (f32, k = 96,
+    or matmul_kernel = 9); ragged tiles in both directions, odd numbers of steps; against the checker, and one-hot
     activations pick single dequantised weights exactly."""
     raw = synth.random_weight(ty, n, k, seed=m + n + k)
     q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
@@ -148,13 +150,16 @@ def test_integer_code_tile_kernel(dev, oracle, ty, act, m, n, k):
     else:
         x = Tensor.from_slice(dev, xa)
     want = oracle.q_mat_mul(ty, xa, raw, n)
-    dev.set_option("matmul_kernel", 8)
+    dev.set_option("matmul_kernel", force)
     try:
         got = x.q_mat_mul(q).as_slice()
         onehot = np.zeros((m, k), dtype=np.float32)
         cols = (np.arange(m) * 37 + 5) % k
         onehot[np.arange(m), cols] = 0.5
-        picked = Tensor.from_slice(dev, onehot).q_mat_mul(q).as_slice()
+        if act == "bf16":  # 0.5 is a bf16 value: the same kernel as above picks the weights
+            picked = Tensor.from_slice(dev, synth.to_bf16_bits(onehot), dtype="bf16").q_mat_mul(q).as_slice()
+        else:
+            picked = Tensor.from_slice(dev, onehot).q_mat_mul(q).as_slice()
     finally:
         dev.set_option("matmul_kernel", 0)
     assert_close(got, want, abs_tol=1e-2, rel_tol=1e-3, what=f"integer-code tile {NAMES[ty]} {act} {m}x{n}x{k}")
