@@ -9,6 +9,7 @@
 // v_mfma_f32_32x32x16_f16 as  w_hi*x_hi + w_lo*x_hi (+ w_hi*x_lo)  with f32 accumulation, so the only
 // deviation from the f32 reference is the summation order and the 2^-22 residues.
 #include "fh_blocks.h"
+#include <type_traits>
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -21,7 +22,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 template <int IN>
 __global__ __launch_bounds__(256) void k_act_split(const void *__restrict__ xin, int64_t srow, int64_t scol, int k, int kp,
                                                     _Float16 *__restrict__ xh, _Float16 *__restrict__ xl,
-                                                    float *__restrict__ rs) {
+                                                    float *__restrict__ rs, _Float16 *__restrict__ xs = nullptr) {
     __shared__ float sh[4];
     const int64_t off = (int64_t)blockIdx.x * srow, oo = (int64_t)blockIdx.x * kp;
     auto ld = [&](int c) -> float {
@@ -44,6 +45,18 @@ __global__ __launch_bounds__(256) void k_act_split(const void *__restrict__ xin,
         const _Float16 h = (_Float16)v;
         xh[oo + c] = h;
         if (IN != 1) xl[oo + c] = (_Float16)(v - (float)h);
+        if (xs) { // (kp is a multiple of 256 then) sums of the 32-groups of the normalised row, / 64, as hi + lo planes
+            float t = v;
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
+            if ((threadIdx.x & 31) == 0) {
+                t *= 0.015625f;
+                const _Float16 th = (_Float16)t;
+                const int64_t at = (int64_t)blockIdx.x * (kp >> 5) + (c >> 5);
+                xs[at] = th;
+                xs[at + (int64_t)gridDim.x * (kp >> 5)] = (_Float16)(t - (float)th);
+            }
+        }
     }
     if (threadIdx.x == 0) rs[blockIdx.x] = __uint_as_float((uint32_t)(127 - e) << 23);
 }
@@ -954,6 +967,208 @@ static fh_status qmm_launch_tile2i(const fh_qmatrix *q, const _Float16 *xh, cons
     return FH_OK;
 }
 
+// ------------------------------------------------------------------------------ Q4_K on integer codes
+// Q4_K: w = d * sc_s * q - dmin * m_s (sub-block s of 32, 8 per 256-block; q 0 .. 15, sc and m 0 .. 63).  The weight
+// operand is the integer sc_s * q (at most 945: exact in f16; a nibble under the byte 0x64 is the f16 1024 + q, and
+// one packed f16 fma (1024 + q) * sc - 1024 sc gives two codes), the products of a whole 256-block collect in one zeroed
+// accumulator, and the block's d is applied to it once (acc += d * part: 16 multiply-adds per lane, 32 x 32 tile and 256
+// of k, where the formats with a scale per 32 pay them per 32).  The offsets are one more MFMA per 256-block: the
+// integers m_s against the sums of the activations of each sub-block (prepared with the activation planes, / 64 to stay
+// in the f16 range, as hi + lo), scaled by -64 dmin.  One MFMA per counted product (two with f32 activations) instead
+// of two (three) in the split form.  Tile and pipeline as k_qmm_tile2i.
+// gridDim.z > 1: k split in runs of whole 256-blocks, partial planes at y + z * m * n.
+template <int NTERM>
+__global__ __launch_bounds__(512) void k_qmm_tile2k(QView q, const _Float16 *__restrict__ xh, const _Float16 *__restrict__ xl,
+                                                      const _Float16 *__restrict__ xs, const float *__restrict__ rs, int m,
+                                                      float *__restrict__ y) {
+    constexpr int WM = 4, WN = 2, FN = 2, FM = 2, TN = WN * FN * 32, TM = WM * FM * 32;
+    constexpr int A_H = TN * QMM_LDK, B_H = TM * QMM_LDK; // halfs per plane
+    constexpr int BUF = A_H + NTERM * B_H;                // halfs per buffer: codes, x hi (, x lo)
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers, then the per-256-block operands
+    _Float16 *s_mn = smem + 2 * BUF;            // [TN][8] offsets m_s as f16 integers
+    _Float16 *s_xs = s_mn + TN * 8;             // [2][TM][8] activation sums, hi and lo plane
+    float *s_d = (float *)(s_xs + 2 * TM * 8);  // [TN][2]: d, -64 dmin
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31;
+    const int wn = wave / WM, wm = wave % WM;
+    const int64_t n0 = (int64_t)blockIdx.x * TN;
+    const int m0 = blockIdx.y * TM;
+    const int K = (int)q.k, nsb = (K >> 8) / (int)gridDim.z, sb0 = (int)blockIdx.z * nsb; // 256-blocks of this workgroup
+    const int ksteps = nsb * 8, kbase = sb0 * 8;
+    y += (int64_t)blockIdx.z * m * q.n;
+    const int64_t tiles16 = (q.n + 15) / 16;
+    // weight duty: one item (row, lane group) of 8 codes per step; activation duty: two 16-byte pieces per plane and step;
+    // sums: threads 0 .. 255 the hi plane's 16 bytes of one row per 256-block, threads 256 .. 511 the lo plane's
+    const int a_g = tid & 3, a_j = (tid >> 2) & 15, a_row = tid >> 2;
+    int64_t a_tile = (n0 >> 4) + (a_row >> 4);
+    if (a_tile >= tiles16) a_tile = tiles16 - 1; // rows past the end decode a valid tile and are never stored
+    const uint8_t *a_rec = q.data + a_tile * q.recs * 2304;
+    const int b_c = tid & 3, b_row0 = tid >> 2, b_row1 = b_row0 + TM / 2;
+    const int64_t b_off0 = (int64_t)(m0 + b_row0 < m ? m0 + b_row0 : m - 1) * K + b_c * 8;
+    const int64_t b_off1 = (int64_t)(m0 + b_row1 < m ? m0 + b_row1 : m - 1) * K + b_c * 8;
+    const int x_row = tid & 255, x_pl = tid >> 8;
+    const _Float16 *x_src = xs + (int64_t)x_pl * m * (K >> 5) + (int64_t)(m0 + x_row < m ? m0 + x_row : m - 1) * (K >> 5);
+    struct Slab {
+        uint32_t a, b;
+        u32x4 h, h0, h1, l0, l1;
+    } s0, s1;
+    auto fetch = [&](Slab &sl, int ks) { // ks: step of this workgroup's range
+        const int g = kbase + ks, S = g >> 3, sb = g & 7;
+        const uint8_t *rec = a_rec + (int64_t)S * 2304;
+        const uint2 c = *(const uint2 *)(rec + 256 + (sb >> 2) * 1024 + (a_g * 16 + a_j) * 16 + 8 * ((sb >> 1) & 1));
+        sl.a = c.x, sl.b = c.y;
+        sl.h = *(const u32x4 *)(rec + 16 * a_j);
+        sl.h0 = *(const u32x4 *)(xh + b_off0 + g * 32);
+        sl.h1 = *(const u32x4 *)(xh + b_off1 + g * 32);
+        if (NTERM == 2) {
+            sl.l0 = *(const u32x4 *)(xl + b_off0 + g * 32);
+            sl.l1 = *(const u32x4 *)(xl + b_off1 + g * 32);
+        }
+    };
+    // two bytes (0 .. 63 each) under the high byte 0x64: the halfs 1024 + u
+    auto up2 = [&](uint32_t bytes, uint32_t sel) -> qmm_half2 {
+        const uint32_t w = __builtin_amdgcn_perm(0x64646464u, bytes, sel);
+        qmm_half2 h;
+        __builtin_memcpy(&h, &w, 4);
+        return h;
+    };
+    auto bits = [&](qmm_half2 h) -> uint32_t {
+        uint32_t o;
+        __builtin_memcpy(&o, &h, 4);
+        return o;
+    };
+    const qmm_half2 k1024 = {(_Float16)1024.f, (_Float16)1024.f};
+    // the slab of step ks (sub-block sb of its 256-block) into buffer ks & 1; with sb == 1 - at the end of the block's
+    // first step, when nobody reads the block before any more - the block's offsets, scales and sums (xsv) go along
+    auto stage = [&](const Slab &sl, int ks, u32x4 xsv) {
+        const int sb = (kbase + ks) & 7;
+        _Float16 *buf = smem + (ks & 1) * BUF;
+        const uint32_t scw = sb < 4 ? (sl.h.y & 0x3F3F3F3Fu) : ((sl.h.w & 0x0F0F0F0Fu) | ((sl.h.y >> 2) & 0x30303030u));
+        const uint32_t scb = (scw >> (8 * (sb & 3))) & 0xFFu;
+        const qmm_half2 sc2 = up2(scb | (scb << 16), 0x04020400u) - k1024;
+        const qmm_half2 nb = sc2 * qmm_half2{(_Float16)-1024.f, (_Float16)-1024.f}; // exact: at most 63 * 2^10
+        const int sh = 4 * (sb & 1);
+        const uint32_t wa = (sl.a >> sh) & 0x0F0F0F0Fu, wb = (sl.b >> sh) & 0x0F0F0F0Fu;
+        u32x4 c;
+        c.x = bits(__builtin_elementwise_fma(up2(wa, 0x04010400u), sc2, nb));
+        c.y = bits(__builtin_elementwise_fma(up2(wa, 0x04030402u), sc2, nb));
+        c.z = bits(__builtin_elementwise_fma(up2(wb, 0x04010400u), sc2, nb));
+        c.w = bits(__builtin_elementwise_fma(up2(wb, 0x04030402u), sc2, nb));
+        *(u32x4 *)(buf + a_row * QMM_LDK + 8 * a_g) = c;
+        *(u32x4 *)(buf + A_H + b_row0 * QMM_LDK + b_c * 8) = sl.h0;
+        *(u32x4 *)(buf + A_H + b_row1 * QMM_LDK + b_c * 8) = sl.h1;
+        if (NTERM == 2) {
+            *(u32x4 *)(buf + A_H + B_H + b_row0 * QMM_LDK + b_c * 8) = sl.l0;
+            *(u32x4 *)(buf + A_H + B_H + b_row1 * QMM_LDK + b_c * 8) = sl.l1;
+        }
+        if (sb == 1) {
+            const uint32_t m03 = sl.h.z & 0x3F3F3F3Fu, m47 = ((sl.h.w >> 4) & 0x0F0F0F0Fu) | ((sl.h.z >> 2) & 0x30303030u);
+            u32x4 mn;
+            mn.x = bits(up2(m03, 0x04010400u) - k1024);
+            mn.y = bits(up2(m03, 0x04030402u) - k1024);
+            mn.z = bits(up2(m47, 0x04010400u) - k1024);
+            mn.w = bits(up2(m47, 0x04030402u) - k1024);
+            *(u32x4 *)(s_mn + a_row * 8) = mn; // (the four threads of a row: the same values)
+            s_d[2 * a_row] = fh_h2f((uint16_t)(sl.h.x & 0xFFFF));
+            s_d[2 * a_row + 1] = -64.f * fh_h2f((uint16_t)(sl.h.x >> 16));
+            *(u32x4 *)(s_xs + (x_pl * TM + x_row) * 8) = xsv;
+        }
+    };
+    floatx16 acc[FN][FM], part[FN][FM];
+#pragma unroll
+    for (int a = 0; a < FN; a++)
+#pragma unroll
+        for (int b = 0; b < FM; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f, part[a][b][r] = 0.f;
+
+    auto kstep = [&](int ks, Slab &mine, const Slab &other) {
+        __syncthreads(); // buffer ks & 1 is complete; the other one is no longer read
+        // the sums of this step's 256-block (staged after the block's first step): requested before the slab, so that
+        // waiting for them does not wait for the slab
+        const u32x4 xsv = *(const u32x4 *)(x_src + ((kbase + ks) >> 3) * 8);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(mine, ks + 2 < ksteps ? ks + 2 : ksteps - 1); // (no branch around the requests: past the end, a repeat)
+        const _Float16 *buf = smem + (ks & 1) * BUF;
+        half8 wc[2][FN], xhv[2][FM], xlv[2][FM];
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+            const int ko = kk * 16 + 8 * (lane >> 5);
+#pragma unroll
+            for (int a = 0; a < FN; a++) wc[kk][a] = *(const half8 *)(buf + ((wn * FN + a) * 32 + li) * QMM_LDK + ko);
+#pragma unroll
+            for (int b = 0; b < FM; b++) {
+                const int row = (wm * FM + b) * 32 + li;
+                xhv[kk][b] = *(const half8 *)(buf + A_H + row * QMM_LDK + ko);
+                if (NTERM == 2) xlv[kk][b] = *(const half8 *)(buf + A_H + B_H + row * QMM_LDK + ko);
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < FN; a++)
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for (int b = 0; b < FM; b++) {
+                    part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xhv[kk][b], wc[kk][a], part[a][b], 0, 0, 0);
+                    if (NTERM == 2)
+                        part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xlv[kk][b], wc[kk][a], part[a][b], 0, 0, 0);
+                }
+        if (((kbase + ks) & 7) == 7) { // the 256-block is complete: its scale, then its offsets
+            half8 mnv[FN], xsh[FM], xsl[FM];
+            const half8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int a = 0; a < FN; a++) mnv[a] = lane < 32 ? *(const half8 *)(s_mn + ((wn * FN + a) * 32 + li) * 8) : zero8;
+#pragma unroll
+            for (int b = 0; b < FM; b++) {
+                const int row = (wm * FM + b) * 32 + li;
+                xsh[b] = lane < 32 ? *(const half8 *)(s_xs + row * 8) : zero8;
+                xsl[b] = lane < 32 ? *(const half8 *)(s_xs + (TM + row) * 8) : zero8;
+            }
+#pragma unroll
+            for (int a = 0; a < FN; a++) {
+                const float d = s_d[2 * ((wn * FN + a) * 32 + li)], nd = s_d[2 * ((wn * FN + a) * 32 + li) + 1];
+#pragma unroll
+                for (int b = 0; b < FM; b++) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[a][b][r] = fmaf(part[a][b][r], d, acc[a][b][r]);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) part[a][b][r] = 0.f;
+                    part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xsh[b], mnv[a], part[a][b], 0, 0, 0);
+                    part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xsl[b], mnv[a], part[a][b], 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[a][b][r] = fmaf(part[a][b][r], nd, acc[a][b][r]);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) part[a][b][r] = 0.f;
+                }
+            }
+        }
+        if (ks + 1 < ksteps) stage(other, ks + 1, xsv); // (the last step has nothing to stage)
+        // the sums are waited for in every step (they are the oldest request: the slab stays in flight), or the request
+        // would still be pending at the next barrier and the wait there would take the slab with it
+        asm volatile("" ::"v"(xsv));
+    };
+    fetch(s0, 0);
+    fetch(s1, 1);
+    stage(s0, 0, u32x4{0, 0, 0, 0});
+    for (int ks0 = 0; ks0 < ksteps; ks0 += 2) { // the register sets alternate: no indexing survives into the code
+        kstep(ks0, s0, s1);
+        kstep(ks0 + 1, s1, s0);
+    }
+    // lane = weight row n (column of the MFMA result), register r = activation row 8 (r / 4) + 4 (lane / 32) + r % 4
+#pragma unroll
+    for (int a = 0; a < FN; a++) {
+        const int64_t nn = n0 + (wn * FN + a) * 32 + li;
+        if (nn >= q.n) continue;
+#pragma unroll
+        for (int b = 0; b < FM; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int mm = m0 + (wm * FM + b) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (mm < m) y[(int64_t)mm * q.n + nn] = acc[a][b][r] * rs[mm];
+            }
+    }
+}
+
 // y = sum of the partial planes of a k-split product, in plane order (deterministic)
 __global__ void k_qmm_sum_planes(const float4 *__restrict__ part, int planes, int64_t n4, float4 *__restrict__ y) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -964,6 +1179,33 @@ __global__ void k_qmm_sum_planes(const float4 *__restrict__ part, int planes, in
         a = make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
     }
     y[i] = a;
+}
+
+template <int NTERM>
+static fh_status qmm_launch_tile2k(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const _Float16 *xs,
+                                   const float *rs, int m, float *y, int ksplit) {
+    constexpr size_t lds = 2 * (size_t)(128 * QMM_LDK + NTERM * 256 * QMM_LDK) * 2 + 128 * 8 * 2 + 2 * 256 * 8 * 2 + 128 * 2 * 4;
+    static bool attr_done = false;
+    if (!attr_done) {
+        FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2k<NTERM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_done = true;
+    }
+    dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + 255) / 256), (unsigned)ksplit);
+    float *dst = y;
+    if (ksplit > 1) {
+        fh_device *dev = q->dev;
+        FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, (size_t)ksplit * m * q->n * 4));
+        dst = dev->ksplit_buf;
+    }
+    k_qmm_tile2k<NTERM><<<grid, 512, lds, q->dev->stream>>>(fh_view(q), xh, xl, xs, rs, m, dst);
+    FH_HIP(hipGetLastError());
+    if (ksplit > 1) {
+        const int64_t n4 = (int64_t)m * q->n / 4;
+        k_qmm_sum_planes<<<dim3((unsigned)((n4 + 255) / 256)), 256, 0, q->dev->stream>>>((const float4 *)dst, ksplit, n4,
+                                                                                       (float4 *)y);
+        FH_HIP(hipGetLastError());
+    }
+    return FH_OK;
 }
 
 template <int T, int NTERM, int WN, int FN, int FM>
@@ -997,14 +1239,14 @@ static fh_status qmm_launch_tile2(const fh_qmatrix *q, const _Float16 *xh, const
 
 template <int T, int NTERM>
 static fh_status qmm_launch_t(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const float *rs, int m,
-                              float *y) {
+                              float *y, const _Float16 *xs) {
     hipStream_t s = q->dev->stream;
     QView v = fh_view(q);
     // the pipelined kernel with the tallest activation tile (256, 128, 64 rows) that still fills most of the device
     // (opt_matmul_kernel = 3: never, 4: always 256)
     const int64_t tn = (q->n + 127) / 128, cus = q->dev->compute_units;
     const int64_t mk = q->dev->opt_matmul_kernel;
-    if (mk == 4 || mk == 8 || mk == 9 || (m > 128 && tn * ((m + 255) / 256) * 5 >= cus * 4 && mk != 3)) { // 8, 9: as 4, integer codes
+    if (mk == 4 || mk == 8 || mk == 9 || mk == 10 || (m > 128 && tn * ((m + 255) / 256) * 5 >= cus * 4 && mk != 3)) { // 8, 9, 10: as 4, integer codes
         // one scale per 32 weights: integer codes and the scale after the MFMA (matmul_kernel = 6 keeps the split form)
         if constexpr (T == FH_Q8_0 || T == FH_Q4_0) {
             // (matmul_kernel = 7: four wavefronts and 128 activation rows per workgroup, two workgroups per compute unit:
@@ -1015,6 +1257,10 @@ static fh_status qmm_launch_t(const fh_qmatrix *q, const _Float16 *xh, const _Fl
                     return qmm_launch_tile2j<T, 4>(q, xh, rs, m, y);
             if (mk != 6 && mk != 4) return qmm_launch_tile2i<T, NTERM, 4>(q, xh, xl, rs, m, y);
         }
+        // Q4_K: integer codes sc * q, the 256-block's d after the MFMAs, the offsets as one more MFMA per block
+        if constexpr (T == FH_Q4_K)
+            if (mk != 6 && mk != 4 && xs) // (matmul_kernel = 10: k split in two where k allows it)
+                return qmm_launch_tile2k<NTERM>(q, xh, xl, xs, rs, m, y, mk == 10 && (q->k / 256) % 2 == 0 && (q->n & 3) == 0 ? 2 : 1);
         return qmm_launch_tile2<T, NTERM, 2, 2, 2>(q, xh, xl, rs, m, y);
     }
     if (m > 64 && mk != 3 && mk != 5) {
@@ -1031,7 +1277,11 @@ static fh_status qmm_launch_t(const fh_qmatrix *q, const _Float16 *xh, const _Fl
         };
         if (m > 128) {
             const int ks = split_for(tn * ((m + 255) / 256));
-            if (tn * ((m + 255) / 256) * ks * 5 >= cus * 4) return qmm_launch_tile2<T, NTERM, 2, 2, 2>(q, xh, xl, rs, m, y, ks);
+            if (tn * ((m + 255) / 256) * ks * 5 >= cus * 4) {
+                if constexpr (T == FH_Q4_K)
+                    if (mk != 6 && xs && (q->k / 256) % ks == 0) return qmm_launch_tile2k<NTERM>(q, xh, xl, xs, rs, m, y, ks);
+                return qmm_launch_tile2<T, NTERM, 2, 2, 2>(q, xh, xl, rs, m, y, ks);
+            }
         }
         const int ks = split_for(tn * ((m + 127) / 128));
         if (tn * ((m + 127) / 128) * ks * 5 >= cus * 4) return qmm_launch_tile2<T, NTERM, 2, 2, 1>(q, xh, xl, rs, m, y, ks);
@@ -1078,18 +1328,21 @@ fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf
         FH_FAIL(FH_ERR_UNSUPPORTED, "type %u with k = %lld has no matrix-core matmul (it runs through fh_qmatmul)", q->type,
                 (long long)K);
     FH_REQUIRE((m + 127) / 128 <= 65535, "m = %d too large for one launch", m);
-    // planes: xh | xl | rs
+    // planes: xh | xl | rs | (Q4_K: sums of the 32-groups, hi and lo)
     const size_t plane = ((size_t)m * K * 2 + 255) & ~(size_t)255;
-    const size_t need = plane * (x_is_bf16 ? 1 : 2) + (size_t)m * 4 + 256;
+    const size_t rs_bytes = ((size_t)m * 4 + 255) & ~(size_t)255;
+    const bool sums = q->type == FH_Q4_K && K % 256 == 0;
+    const size_t need = plane * (x_is_bf16 ? 1 : 2) + rs_bytes + (sums ? 2 * (size_t)m * (K / 32) * 2 : 0) + 256;
     FH_TRY(fh_dev_scratch(dev, &dev->act_buf, &dev->act_cap, need));
     _Float16 *xh = (_Float16 *)dev->act_buf;
     _Float16 *xl = x_is_bf16 ? nullptr : (_Float16 *)((uint8_t *)dev->act_buf + plane);
     float *rs = (float *)((uint8_t *)dev->act_buf + plane * (x_is_bf16 ? 1 : 2));
-    if (x_is_bf16) k_act_split<1><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, K, 1, (int)K, (int)K, xh, xl, rs);
-    else k_act_split<0><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, K, 1, (int)K, (int)K, xh, xl, rs);
+    _Float16 *xs = sums ? (_Float16 *)((uint8_t *)rs + rs_bytes) : nullptr;
+    if (x_is_bf16) k_act_split<1><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, K, 1, (int)K, (int)K, xh, xl, rs, xs);
+    else k_act_split<0><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, K, 1, (int)K, (int)K, xh, xl, rs, xs);
     FH_HIP(hipGetLastError());
 #define QMM_GO(T_)                                                              \
-    return x_is_bf16 ? qmm_launch_t<T_, 1>(q, xh, xl, rs, m, y) : qmm_launch_t<T_, 2>(q, xh, xl, rs, m, y)
+    return x_is_bf16 ? qmm_launch_t<T_, 1>(q, xh, xl, rs, m, y, xs) : qmm_launch_t<T_, 2>(q, xh, xl, rs, m, y, xs)
     switch (q->type) {
     case FH_Q4_0: QMM_GO(FH_Q4_0);
     case FH_Q8_0: QMM_GO(FH_Q8_0);

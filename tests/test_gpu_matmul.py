@@ -167,8 +167,44 @@ def test_integer_code_tile_kernel(dev, oracle, ty, act, m, n, k, force):
     assert np.array_equal(picked, 0.5 * deq[:, cols].T), "one-hot activations pick dequantised weights exactly"
 
 
+@pytest.mark.parametrize("act", ["f32", "bf16"])
+@pytest.mark.parametrize("m,n,k,force", [(256, 128, 256, 8), (300, 200, 512, 8), (129, 1000, 1024, 8), (513, 130, 4096, 8),
+                                          (300, 200, 512, 10), (257, 132, 3584, 10), (40, 128, 768, 10)])
+def test_q4k_integer_code_tile_kernel(dev, oracle, act, m, n, k, force):
+    """Q4_K through the tile kernel that multiplies the integer codes sc * q, applies the 256-block's d to the
+    accumulated block and takes the offsets from one more matrix-core product of the block minimums with the sums of
+    the activations per sub-block (matmul_kernel = 8 selects it whatever the size, 10 with k split over two workgroups and
+    the planes summed; the dispatch takes it for large products): ragged tiles in both directions, one and several
+    256-blocks, odd block counts per k part; against the checker, and one-hot activations pick single dequantised
+    weights to the last bits (the scale is applied to sc * q in one rounding instead of two)."""
+    raw = synth.random_weight(Q4_K, n, k, seed=m + n + k)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, Q4_K)
+    xa = synth.random_activation(m, k, seed=7)
+    onehot = np.zeros((m, k), dtype=np.float32)
+    cols = (np.arange(m) * 37 + 5) % k
+    onehot[np.arange(m), cols] = 0.5
+    if act == "bf16":
+        bits = synth.to_bf16_bits(xa)
+        xa = (bits.astype(np.uint32) << 16).view(np.float32)
+        x = Tensor.from_slice(dev, bits, dtype="bf16")
+        oh = Tensor.from_slice(dev, synth.to_bf16_bits(onehot), dtype="bf16")
+    else:
+        x = Tensor.from_slice(dev, xa)
+        oh = Tensor.from_slice(dev, onehot)
+    want = oracle.q_mat_mul(Q4_K, xa, raw, n)
+    dev.set_option("matmul_kernel", force)
+    try:
+        got = x.q_mat_mul(q).as_slice()
+        picked = oh.q_mat_mul(q).as_slice()
+    finally:
+        dev.set_option("matmul_kernel", 0)
+    assert_close(got, want, abs_tol=1e-2, rel_tol=1e-3, what=f"Q4_K integer-code tile {act} {m}x{n}x{k}")
+    deq = oracle.dequantize(Q4_K, raw).reshape(n, k)
+    assert np.abs(picked - 0.5 * deq[:, cols].T).max() <= 2e-6 * np.abs(deq).max()
+
+
 @pytest.mark.parametrize("m", [512, 2048])
-@pytest.mark.parametrize("ty", [Q6_K, Q8_0], ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("ty", [Q6_K, Q8_0, Q4_K], ids=lambda t: NAMES[t])
 def test_prefill_shape_spot_check(dev, oracle, ty, m):
     """Full prefill shapes (m = 512 and 2048, k = 4096, n = 14336, bf16 activations): 64 output columns spread over the
     matrix against the checker, and the sum over all outputs of a row against x . (sum of weight rows) -- a checksum
