@@ -14,6 +14,17 @@
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+// adds the two k halves of the tiles of a split last round (see k_qmm_tile2j) into y
+__global__ void k_qmm_tail_sum(const float *__restrict__ planes, int tail, int full, int tiles_n, int m, int64_t n,
+                               float *__restrict__ y);
+// Tiles of the last round of workgroups that are worth splitting along k: more tiles than compute units and a
+// remainder of at most half of them (matmul_kernel = 11: never)
+static int qmm_tail_tiles(const fh_device *dev, int tiles) {
+    const int cus = dev->compute_units;
+    const int tail = tiles > cus ? tiles % cus : 0;
+    return (tail * 2 > cus || dev->opt_matmul_kernel == 11) ? 0 : tail;
+}
+
 #define QMM_LDK 40 // halfs per LDS row: 32 + 8 padding (80 B stride: 16-byte reads of 16 rows hit 16 distinct chunks)
 
 // ------------------------------------------------------------------------------ activation planes
@@ -398,7 +409,8 @@ __device__ __forceinline__ void qmm_decode_raw(const QmmRaw &r, int g, int ks, f
 template <int T, int NTERM, int WN, int FN, int FM>
 __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__restrict__ xh,
                                                    const _Float16 *__restrict__ xl, const float *__restrict__ rs,
-                                                   int m, float *__restrict__ y) {
+                                                   int m, float *__restrict__ y, int tiles_n = 0, int full = 0, int tail = 0,
+                                                   float *__restrict__ planes = nullptr) {
     constexpr int WM = 8 / WN, TN = WN * FN * 32, TM = WM * FM * 32;
     static_assert(TN == 128, "512 threads decode 128 weight rows x 4 pieces per step");
     constexpr int NB = (TM * 4 + 511) / 512; // 16-byte activation pieces per thread, plane and step
@@ -407,11 +419,14 @@ __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__re
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int wn = wave / WM, wm = wave % WM;
-    const int64_t n0 = (int64_t)blockIdx.x * TN;
-    const int m0 = blockIdx.y * TM;
+    // tiles_n > 0: one-dimensional grid with the tiles of the last round split along k, as in k_qmm_tile2j
+    const int lin = (int)blockIdx.x, split = tiles_n > 0 && lin >= full, tile = split ? full + ((lin - full) >> 1) : lin;
+    const int64_t n0 = (int64_t)(tiles_n > 0 ? tile % tiles_n : (int)blockIdx.x) * TN;
+    const int m0 = (tiles_n > 0 ? tile / tiles_n : (int)blockIdx.y) * TM;
     // gridDim.z > 1: the k steps are split over workgroups, each writing its partial product to its own [m, n] plane
     // of y (the host sums the planes); a split holds an even number of steps, so LDS buffer parity is that of ks
-    const int K = (int)q.k, kper = K / 32 / (int)gridDim.z, kbeg = (int)blockIdx.z * kper, ksteps = kbeg + kper;
+    const int K = (int)q.k, kparts = split ? 2 : (int)gridDim.z, kpart = split ? (lin - full) & 1 : (int)blockIdx.z;
+    const int kper = K / 32 / kparts, kbeg = kpart * kper, ksteps = kbeg + kper;
     y += (size_t)blockIdx.z * (size_t)m * (size_t)q.n;
     const int64_t tiles16 = (q.n + 15) / 16;
     // this thread's weight duty: row a_row of the tile, lane group a_g (8 weights per step)
@@ -531,7 +546,9 @@ __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__re
                 const float4 v = make_float4(acc[a][b][4 * r4] * s, acc[a][b][4 * r4 + 1] * s, acc[a][b][4 * r4 + 2] * s,
                                              acc[a][b][4 * r4 + 3] * s);
                 float *dst = y + (int64_t)mm * q.n + nn;
-                if (vec && nn + 3 < q.n) {
+                if (split) {
+                    if (nn < q.n) *(float4 *)(planes + (((int64_t)kpart * tail + (tile - full)) * TM + (mm - m0)) * TN + (nn - n0)) = v;
+                } else if (vec && nn + 3 < q.n) {
                     *(float4 *)dst = v;
                 } else {
                     if (nn < q.n) dst[0] = v.x;
@@ -559,7 +576,8 @@ typedef _Float16 qmm_half2 __attribute__((ext_vector_type(2)));
 template <int T, int NTERM, int WM>
 __global__ __launch_bounds__(128 * WM) void k_qmm_tile2i(QView q, const _Float16 *__restrict__ xh,
                                                     const _Float16 *__restrict__ xl, const float *__restrict__ rs,
-                                                    int m, float *__restrict__ y) {
+                                                    int m, float *__restrict__ y, int tiles_n, int full, int tail,
+                                                    float *__restrict__ planes) {
     static_assert(T == FH_Q8_0 || T == FH_Q4_0, "formats with one scale per 32 weights");
     // WM = 4: eight wavefronts, 256 activation rows; WM = 2: four wavefronts, 128 activation rows - two such workgroups
     // share a compute unit and are at different points of their steps (one's MFMAs under the other's scaling and staging)
@@ -569,9 +587,12 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2i(QView q, const _Float16
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31;
     const int wn = wave / WM, wm = wave % WM;
-    const int64_t n0 = (int64_t)blockIdx.x * TN;
-    const int m0 = blockIdx.y * TM;
-    const int K = (int)q.k, ksteps = K / 32;
+    // tiles_n > 0: one-dimensional grid with the tiles of the last round split along k, as in k_qmm_tile2j
+    const int lin = (int)blockIdx.x, split = tiles_n > 0 && lin >= full, tile = split ? full + ((lin - full) >> 1) : lin;
+    const int64_t n0 = (int64_t)(tiles_n > 0 ? tile % tiles_n : (int)blockIdx.x) * TN;
+    const int m0 = (tiles_n > 0 ? tile / tiles_n : (int)blockIdx.y) * TM;
+    const int K = (int)q.k, kpart = split ? (lin - full) & 1 : 0;
+    const int kfirst = split && kpart ? K / 64 : 0, ksteps = split && !kpart ? K / 64 : K / 32; // steps [kfirst, ksteps)
     const int64_t tiles16 = (q.n + 15) / 16;
     // weight duty: NA items (row, lane group) of 8 codes per step; activation duty: two 16-byte pieces per plane and step
     const int a_g = tid & 3, a_j = (tid >> 2) & 15;
@@ -649,9 +670,9 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2i(QView q, const _Float16
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
 
-    fetch(s0, 0);
-    if (ksteps > 1) fetch(s1, 1);
-    stage(s0, 0);
+    fetch(s0, kfirst);
+    if (ksteps > kfirst + 1) fetch(s1, kfirst + 1);
+    stage(s0, kfirst);
     auto kstep = [&](int ks, Slab &mine, const Slab &other) {
         if (ks < ksteps) {
             __syncthreads(); // buffer ks & 1 is complete; the other one is no longer read
@@ -716,7 +737,7 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2i(QView q, const _Float16
             }
         }
     };
-    for (int ks0 = 0; ks0 < ksteps; ks0 += 2) { // the register sets alternate: no indexing survives into the code
+    for (int ks0 = kfirst; ks0 < ksteps; ks0 += 2) { // the register sets alternate: no indexing survives into the code
         kstep(ks0, s0, s1);
         kstep(ks0 + 1, s1, s0);
     }
@@ -729,8 +750,11 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2i(QView q, const _Float16
         for (int b = 0; b < FM; b++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int mm = m0 + (wm * FM + b) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (mm < m) y[(int64_t)mm * q.n + nn] = acc[a][b][r] * rs[mm];
+                const int ml = (wm * FM + b) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3), mm = m0 + ml;
+                if (mm >= m) continue;
+                const float v = acc[a][b][r] * rs[mm];
+                if (split) planes[(((int64_t)kpart * tail + (tile - full)) * TM + ml) * TN + (nn - n0)] = v;
+                else y[(int64_t)mm * q.n + nn] = v;
             }
     }
 }
@@ -738,9 +762,15 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2i(QView q, const _Float16
 // The integer-code kernel with two blocks of 32 weights per step (64 of k): half as many workgroup barriers and
 // operand-read latencies per weight, one 16-byte load per weight item and step (the repack keeps the two blocks'
 // codes of a lane side by side). One activation plane only (f16 / bf16 activations); k must be a multiple of 64.
+// One-dimensional grid: workgroup t < full owns output tile t (n tile t % tiles_n, m tile t / tiles_n) over all of k.
+// When the tiles do not fill the last round of workgroups on the device (tiles mod compute units at most half the
+// compute units), the host makes those last tiles two workgroups each, one per half of k, which together fill the round
+// for half its time: workgroup full + 2 u + h takes half h of tile full + u and writes the whole tile to
+// planes[h][u][TM][TN]; k_qmm_tail_sum adds the two halves into y.
 template <int T, int WM>
 __global__ __launch_bounds__(128 * WM) void k_qmm_tile2j(QView q, const _Float16 *__restrict__ xh,
-                                                    const float *__restrict__ rs, int m, float *__restrict__ y) {
+                                                    const float *__restrict__ rs, int m, float *__restrict__ y,
+                                                    int tiles_n, int full, int tail, float *__restrict__ planes) {
     static_assert(T == FH_Q8_0 || T == FH_Q4_0, "formats with one scale per 32 weights");
     // An LDS row is 64 halfs = eight 16-byte pieces; piece c of row r sits at position c ^ sw(r), sw(r) = bit 1 of r
     // (as bit 2) and bits 2 .. 3 of r: the 16-byte reads of 16 consecutive rows at one c, the 64-byte code writes of four
@@ -753,9 +783,11 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2j(QView q, const _Float16
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31;
     const int wn = wave / WM, wm = wave % WM;
-    const int64_t n0 = (int64_t)blockIdx.x * TN;
-    const int m0 = blockIdx.y * TM;
-    const int K = (int)q.k, ksteps = K / 64;
+    const int lin = (int)blockIdx.x, split = lin >= full, tile = split ? full + ((lin - full) >> 1) : lin;
+    const int64_t n0 = (int64_t)(tile % tiles_n) * TN;
+    const int m0 = (tile / tiles_n) * TM;
+    const int K = (int)q.k;
+    const int kfirst = split && ((lin - full) & 1) ? K / 128 : 0, ksteps = split && !((lin - full) & 1) ? K / 128 : K / 64;
     const int64_t tiles16 = (q.n + 15) / 16;
     const int a_g = tid & 3, a_j = (tid >> 2) & 15;
     int a_row[NA];
@@ -911,11 +943,11 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2j(QView q, const _Float16
             }
         }
     };
-    fetch(0);
-    stage(0);
+    fetch(kfirst);
+    stage(kfirst);
     // (A schedule in which the second wavefront of every SIMD runs half a step behind the first - one multiplies while
     // the other decodes and stages, two barriers per step - was measured slower: 422 against 378 us at 2048 x 14336 x 4096.)
-    for (int ks = 0; ks < ksteps; ks++) {
+    for (int ks = kfirst; ks < ksteps; ks++) { // steps [kfirst, ksteps)
         __syncthreads(); // buffer ks & 1 is complete; the other one is no longer read
         fetch(ks + 1 < ksteps ? ks + 1 : ks); // (no branch in the step: past the end, a repeat)
         compute(ks);
@@ -930,10 +962,27 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2j(QView q, const _Float16
         for (int b = 0; b < FM; b++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int mm = m0 + (wm * FM + b) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (mm < m) y[(int64_t)mm * q.n + nn] = acc[a][b][r] * rs[mm];
+                const int ml = (wm * FM + b) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3), mm = m0 + ml;
+                if (mm >= m) continue;
+                const float v = acc[a][b][r] * rs[mm]; // (a power of two: the halves may be scaled before they are added)
+                if (split) planes[(((int64_t)((lin - full) & 1) * tail + (tile - full)) * TM + ml) * TN + (nn - n0)] = v;
+                else y[(int64_t)mm * q.n + nn] = v;
             }
     }
+}
+
+// y tile = planes[0][u] + planes[1][u] for the tail tiles u of k_qmm_tile2j (256 x 128 tiles); one workgroup per 16 rows
+__global__ void k_qmm_tail_sum(const float *__restrict__ planes, int tail, int full, int tiles_n, int m, int64_t n,
+                               float *__restrict__ y) {
+    const int u = blockIdx.x >> 4, tile = full + u, row = ((blockIdx.x & 15) << 4) + (threadIdx.x >> 5), c4 = (threadIdx.x & 31) * 4;
+    const int mm = (tile / tiles_n) * 256 + row;
+    const int64_t nn = (int64_t)(tile % tiles_n) * 128 + c4;
+    if (mm >= m || nn >= n) return;
+    const float4 a = *(const float4 *)(planes + (((int64_t)u) * 256 + row) * 128 + c4);
+    const float4 b = *(const float4 *)(planes + (((int64_t)tail + u) * 256 + row) * 128 + c4);
+    float *dst = y + (int64_t)mm * n + nn;
+    const float s[4] = {a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w};
+    for (int i = 0; i < 4 && nn + i < n; i++) dst[i] = s[i];
 }
 
 template <int T, int WM>
@@ -945,9 +994,22 @@ static fh_status qmm_launch_tile2j(const fh_qmatrix *q, const _Float16 *xh, cons
         FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2j<T, WM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_done = true;
     }
-    dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + TM - 1) / TM));
-    k_qmm_tile2j<T, WM><<<grid, 128 * WM, lds, q->dev->stream>>>(fh_view(q), xh, rs, m, y);
+    fh_device *dev = q->dev;
+    const int tiles_n = (int)((q->n + 127) / 128), tiles = tiles_n * ((m + TM - 1) / TM);
+    // the last round of workgroups: split its tiles along k when they fill at most half the device
+    const int tail = (q->k % 128 != 0 || WM != 4) ? 0 : qmm_tail_tiles(dev, tiles);
+    float *planes = nullptr;
+    if (tail) {
+        FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, (size_t)2 * tail * TM * 128 * 4));
+        planes = dev->ksplit_buf;
+    }
+    k_qmm_tile2j<T, WM><<<dim3((unsigned)(tiles + tail)), 128 * WM, lds, dev->stream>>>(fh_view(q), xh, rs, m, y, tiles_n,
+                                                                                     tiles - tail, tail, planes);
     FH_HIP(hipGetLastError());
+    if (tail) {
+        k_qmm_tail_sum<<<dim3((unsigned)(tail * 16)), 512, 0, dev->stream>>>(planes, tail, tiles - tail, tiles_n, m, q->n, y);
+        FH_HIP(hipGetLastError());
+    }
     return FH_OK;
 }
 
@@ -962,7 +1024,21 @@ static fh_status qmm_launch_tile2i(const fh_qmatrix *q, const _Float16 *xh, cons
         attr_done = true;
     }
     dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + TM - 1) / TM));
-    k_qmm_tile2i<T, NTERM, WM><<<grid, 128 * WM, lds, q->dev->stream>>>(fh_view(q), xh, xl, rs, m, y);
+    if (WM == 4 && q->k % 128 == 0) { // split the tiles of a short last round along k
+        fh_device *dev = q->dev;
+        const int tiles = (int)(grid.x * grid.y), tail = qmm_tail_tiles(dev, tiles);
+        if (tail) {
+            FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, (size_t)2 * tail * 256 * 128 * 4));
+            k_qmm_tile2i<T, NTERM, WM><<<dim3((unsigned)(tiles + tail)), 128 * WM, lds, dev->stream>>>(
+                fh_view(q), xh, xl, rs, m, y, (int)grid.x, tiles - tail, tail, dev->ksplit_buf);
+            FH_HIP(hipGetLastError());
+            k_qmm_tail_sum<<<dim3((unsigned)(tail * 16)), 512, 0, dev->stream>>>(dev->ksplit_buf, tail, tiles - tail, (int)grid.x, m,
+                                                                                q->n, y);
+            FH_HIP(hipGetLastError());
+            return FH_OK;
+        }
+    }
+    k_qmm_tile2i<T, NTERM, WM><<<grid, 128 * WM, lds, q->dev->stream>>>(fh_view(q), xh, xl, rs, m, y, 0, 0, 0, nullptr);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
@@ -980,7 +1056,8 @@ static fh_status qmm_launch_tile2i(const fh_qmatrix *q, const _Float16 *xh, cons
 template <int NTERM>
 __global__ __launch_bounds__(512) void k_qmm_tile2k(QView q, const _Float16 *__restrict__ xh, const _Float16 *__restrict__ xl,
                                                       const _Float16 *__restrict__ xs, const float *__restrict__ rs, int m,
-                                                      float *__restrict__ y) {
+                                                      float *__restrict__ y, int tiles_n, int full, int tail,
+                                                      float *__restrict__ planes) {
     constexpr int WM = 4, WN = 2, FN = 2, FM = 2, TN = WN * FN * 32, TM = WM * FM * 32;
     constexpr int A_H = TN * QMM_LDK, B_H = TM * QMM_LDK; // halfs per plane
     constexpr int BUF = A_H + NTERM * B_H;                // halfs per buffer: codes, x hi (, x lo)
@@ -991,9 +1068,12 @@ __global__ __launch_bounds__(512) void k_qmm_tile2k(QView q, const _Float16 *__r
     float *s_d = (float *)(s_xs + 2 * TM * 8);  // [TN][2]: d, -64 dmin
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31;
     const int wn = wave / WM, wm = wave % WM;
-    const int64_t n0 = (int64_t)blockIdx.x * TN;
-    const int m0 = blockIdx.y * TM;
-    const int K = (int)q.k, nsb = (K >> 8) / (int)gridDim.z, sb0 = (int)blockIdx.z * nsb; // 256-blocks of this workgroup
+    // tiles_n > 0: one-dimensional grid with the tiles of the last round split along k, as in k_qmm_tile2j
+    const int lin = (int)blockIdx.x, split = tiles_n > 0 && lin >= full, tile = split ? full + ((lin - full) >> 1) : lin;
+    const int64_t n0 = (int64_t)(tiles_n > 0 ? tile % tiles_n : (int)blockIdx.x) * TN;
+    const int m0 = (tiles_n > 0 ? tile / tiles_n : (int)blockIdx.y) * TM;
+    const int kparts = split ? 2 : (int)gridDim.z, kpart = split ? (lin - full) & 1 : (int)blockIdx.z;
+    const int K = (int)q.k, nsb = (K >> 8) / kparts, sb0 = kpart * nsb; // 256-blocks of this workgroup
     const int ksteps = nsb * 8, kbase = sb0 * 8;
     y += (int64_t)blockIdx.z * m * q.n;
     const int64_t tiles16 = (q.n + 15) / 16;
@@ -1163,8 +1243,11 @@ __global__ __launch_bounds__(512) void k_qmm_tile2k(QView q, const _Float16 *__r
         for (int b = 0; b < FM; b++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int mm = m0 + (wm * FM + b) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (mm < m) y[(int64_t)mm * q.n + nn] = acc[a][b][r] * rs[mm];
+                const int ml = (wm * FM + b) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3), mm = m0 + ml;
+                if (mm >= m) continue;
+                const float v = acc[a][b][r] * rs[mm];
+                if (split) planes[(((int64_t)kpart * tail + (tile - full)) * TM + ml) * TN + (nn - n0)] = v;
+                else y[(int64_t)mm * q.n + nn] = v;
             }
     }
 }
@@ -1191,13 +1274,27 @@ static fh_status qmm_launch_tile2k(const fh_qmatrix *q, const _Float16 *xh, cons
         attr_done = true;
     }
     dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + 255) / 256), (unsigned)ksplit);
+    if (ksplit == 1 && q->k % 512 == 0) { // split the tiles of a short last round along k
+        fh_device *dev = q->dev;
+        const int tiles = (int)(grid.x * grid.y), tail = qmm_tail_tiles(dev, tiles);
+        if (tail) {
+            FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, (size_t)2 * tail * 256 * 128 * 4));
+            k_qmm_tile2k<NTERM><<<dim3((unsigned)(tiles + tail)), 512, lds, dev->stream>>>(
+                fh_view(q), xh, xl, xs, rs, m, y, (int)grid.x, tiles - tail, tail, dev->ksplit_buf);
+            FH_HIP(hipGetLastError());
+            k_qmm_tail_sum<<<dim3((unsigned)(tail * 16)), 512, 0, dev->stream>>>(dev->ksplit_buf, tail, tiles - tail, (int)grid.x, m,
+                                                                                q->n, y);
+            FH_HIP(hipGetLastError());
+            return FH_OK;
+        }
+    }
     float *dst = y;
     if (ksplit > 1) {
         fh_device *dev = q->dev;
         FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, (size_t)ksplit * m * q->n * 4));
         dst = dev->ksplit_buf;
     }
-    k_qmm_tile2k<NTERM><<<grid, 512, lds, q->dev->stream>>>(fh_view(q), xh, xl, xs, rs, m, dst);
+    k_qmm_tile2k<NTERM><<<grid, 512, lds, q->dev->stream>>>(fh_view(q), xh, xl, xs, rs, m, dst, 0, 0, 0, nullptr);
     FH_HIP(hipGetLastError());
     if (ksplit > 1) {
         const int64_t n4 = (int64_t)m * q->n / 4;
@@ -1220,6 +1317,20 @@ static fh_status qmm_launch_tile2(const fh_qmatrix *q, const _Float16 *xh, const
         attr_done = true;
     }
     dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + TM - 1) / TM), (unsigned)ksplit);
+    if (TM == 256 && ksplit == 1 && q->k % 128 == 0) { // split the tiles of a short last round along k
+        fh_device *dev = q->dev;
+        const int tiles = (int)(grid.x * grid.y), tail = qmm_tail_tiles(dev, tiles);
+        if (tail) {
+            FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, (size_t)2 * tail * 256 * 128 * 4));
+            k_qmm_tile2<T, NTERM, WN, FN, FM><<<dim3((unsigned)(tiles + tail)), 512, lds, dev->stream>>>(
+                fh_view(q), xh, xl, rs, m, y, (int)grid.x, tiles - tail, tail, dev->ksplit_buf);
+            FH_HIP(hipGetLastError());
+            k_qmm_tail_sum<<<dim3((unsigned)(tail * 16)), 512, 0, dev->stream>>>(dev->ksplit_buf, tail, tiles - tail, (int)grid.x, m,
+                                                                                q->n, y);
+            FH_HIP(hipGetLastError());
+            return FH_OK;
+        }
+    }
     float *dst = y;
     if (ksplit > 1) {
         fh_device *dev = q->dev;

@@ -167,6 +167,36 @@ def test_integer_code_tile_kernel(dev, oracle, ty, act, m, n, k, force):
     assert np.array_equal(picked, 0.5 * deq[:, cols].T), "one-hot activations pick dequantised weights exactly"
 
 
+@pytest.mark.parametrize("ty,act", [(Q8_0, "bf16"), (Q4_0, "bf16"), (Q8_0, "f32"), (Q6_K, "bf16"), (Q4_K, "bf16"), (Q4_K, "f32")],
+                         ids=lambda t: NAMES.get(t, t) if not isinstance(t, str) else t)
+def test_tile_kernels_split_last_round(dev, oracle, ty, act):
+    """More output tiles than compute units, the remainder at most half of them: the tiles of the last round are two
+    workgroups each, one per half of k, summed by a second launch (280 tiles of 256 x 128 on 256 compute units: 24 tiles
+    are split; ragged in both directions) - in every kernel with 256 x 128 tiles: integer codes with 64 and 32 of k per
+    step, the split form (Q6_K), Q4_K on integer codes with one and two activation planes.  Against the checker on sampled columns, and against the same product with
+    the split switched off (matmul_kernel = 11), which must agree to the rounding of one addition."""
+    m, n, k = 3333, 2556, 512
+    raw = synth.random_weight(ty, n, k, seed=77)
+    xb, xf = bf16_round(synth.random_activation(m, k, seed=78))
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    x = Tensor.from_slice(dev, xb, dtype="bf16") if act == "bf16" else Tensor.from_slice(dev, xf)
+    got = x.q_mat_mul(q).as_slice()
+    dev.set_option("matmul_kernel", 11)
+    try:
+        whole = x.q_mat_mul(q).as_slice()
+    finally:
+        dev.set_option("matmul_kernel", 0)
+    assert np.abs(got - whole).max() <= 1e-5 * np.abs(whole).max()
+    rows = (np.arange(96) * 53 + 7) % n
+    bpr = len(raw) // n
+    sub = np.concatenate([raw[r * bpr:(r + 1) * bpr] for r in rows])
+    want = oracle.q_mat_mul(ty, xf, sub, 96, fast=True)
+    assert_close(got[:, rows], want, what="sampled columns")
+    last = np.arange(n - 40, n)  # the split tiles are the last ones: the last columns of the last rows
+    sub = np.concatenate([raw[r * bpr:(r + 1) * bpr] for r in last])
+    assert_close(got[-300:, last], oracle.q_mat_mul(ty, xf[-300:], sub, 40, fast=True), what="last tiles")
+
+
 @pytest.mark.parametrize("act", ["f32", "bf16"])
 @pytest.mark.parametrize("m,n,k,force", [(256, 128, 256, 8), (300, 200, 512, 8), (129, 1000, 1024, 8), (513, 130, 4096, 8),
                                           (300, 200, 512, 10), (257, 132, 3584, 10), (40, 128, 768, 10)])
