@@ -1252,6 +1252,159 @@ __global__ __launch_bounds__(512) void k_qmm_tile2k(QView q, const _Float16 *__r
     }
 }
 
+// ------------------------------------------------------------------------------ Q6_K on integer codes
+// Q6_K: w = d * sc_g * (q - 32) (16-element groups g, sc int8, q 0 .. 63).  sc * (q - 32) needs 12 bits, one more than an
+// f16 holds, so the weight operand is two exact terms: (sc & ~15) * (q - 32) (a multiple of 16 up to 4096 in size) and
+// (sc & 15) * (q - 32) (at most 480), both accumulated into one zeroed accumulator over a whole 256-block, to which the
+// block's d is applied once.  As many MFMAs as the split form (two per product), but the decode is integer and packed
+// f16 work (the 6-bit codes of two weights come out of the tiled words as one 32-bit pattern under 0x6400 = the f16
+// pair 1024 + q) instead of f32 arithmetic and two-term rounding, and there is no rounding at all before the f32
+// accumulation.  One activation plane (f16 / bf16 activations); tile, pipeline, k split and the split last round as
+// k_qmm_tile2k.
+__global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__restrict__ xh, const float *__restrict__ rs,
+                                                      int m, float *__restrict__ y, int tiles_n, int full, int tail,
+                                                      float *__restrict__ planes) {
+    constexpr int WM = 4, WN = 2, FN = 2, FM = 2, TN = WN * FN * 32, TM = WM * FM * 32;
+    constexpr int A_H = TN * QMM_LDK, B_H = TM * QMM_LDK; // halfs per plane
+    constexpr int BUF = 2 * A_H + B_H;                    // halfs per buffer: codes (high part, low part), x
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers, then d per weight row
+    float *s_d = (float *)(smem + 2 * BUF);
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31;
+    const int wn = wave / WM, wm = wave % WM;
+    const int lin = (int)blockIdx.x, split = tiles_n > 0 && lin >= full, tile = split ? full + ((lin - full) >> 1) : lin;
+    const int64_t n0 = (int64_t)(tiles_n > 0 ? tile % tiles_n : (int)blockIdx.x) * TN;
+    const int m0 = (tiles_n > 0 ? tile / tiles_n : (int)blockIdx.y) * TM;
+    const int kparts = split ? 2 : (int)gridDim.z, kpart = split ? (lin - full) & 1 : (int)blockIdx.z;
+    const int K = (int)q.k, nsb = (K >> 8) / kparts, sb0 = kpart * nsb; // 256-blocks of this workgroup
+    const int ksteps = nsb * 8, kbase = sb0 * 8;
+    y += (int64_t)blockIdx.z * m * q.n;
+    const int64_t tiles16 = (q.n + 15) / 16;
+    const int a_g = tid & 3, a_j = (tid >> 2) & 15, a_row = tid >> 2;
+    int64_t a_tile = (n0 >> 4) + (a_row >> 4);
+    if (a_tile >= tiles16) a_tile = tiles16 - 1; // rows past the end decode a valid tile and are never stored
+    const uint8_t *a_rec = q.data + a_tile * q.recs * 3360;
+    const int b_c = tid & 3, b_row0 = tid >> 2, b_row1 = b_row0 + TM / 2;
+    const int64_t b_off0 = (int64_t)(m0 + b_row0 < m ? m0 + b_row0 : m - 1) * K + b_c * 8;
+    const int64_t b_off1 = (int64_t)(m0 + b_row1 < m ? m0 + b_row1 : m - 1) * K + b_c * 8;
+    struct Slab {
+        uint32_t a, b, sc, d;
+        u32x4 h0, h1;
+    } s0, s1;
+    auto fetch = [&](Slab &sl, int ks) { // ks: step of this workgroup's range
+        const int g = kbase + ks, t = g & 7;
+        const uint8_t *rec = a_rec + (int64_t)(g >> 3) * 3360;
+        sl.a = *(const uint32_t *)(rec + q6k_lword_off(a_j, t, a_g));
+        sl.b = *(const uint32_t *)(rec + q6k_hword_off(a_j, t, a_g));
+        sl.sc = rec[q6k_sc_off(a_j, 2 * t + (a_g >> 1))];
+        sl.d = fh_ld16(rec + q6k_d_off(a_j));
+        sl.h0 = *(const u32x4 *)(xh + b_off0 + g * 32);
+        sl.h1 = *(const u32x4 *)(xh + b_off1 + g * 32);
+    };
+    // the slab of step ks into buffer ks & 1; ODD: the parity of the step inside its 256-block (the two-bit parts of the
+    // codes sit at other places of their word in odd steps); with sub-block 1 the block's d goes along
+    auto stage = [&](const Slab &sl, int ks, auto oddc) {
+        constexpr bool ODD = decltype(oddc)::value;
+        _Float16 *buf = smem + (ks & 1) * BUF;
+        const int sc = (int)(int8_t)sl.sc;
+        const _Float16 fl = (_Float16)(float)(sc & 15), fh = (_Float16)(float)(sc & ~15); // exact: small integers
+        const qmm_half2 sl2 = {fl, fl}, sh2 = {fh, fh}, k1056 = {(_Float16)1056.f, (_Float16)1056.f};
+        u32x4 chi, clo;
+#pragma unroll
+        for (int p = 0; p < 4; p++) { // weights 2 p and 2 p + 1 of the item: positions 8 g + 2 p, + 1 of the step
+            const uint32_t lo4 = (sl.a >> (4 * p)) & 0x000F000Fu;
+            uint32_t hi2;
+            if (!ODD) hi2 = sl.b >> (2 * p);
+            else hi2 = p == 0 ? sl.b << 4 : (p == 1 ? sl.b << 2 : (p == 2 ? sl.b >> 8 : sl.b >> 10));
+            const uint32_t v = lo4 | (hi2 & 0x00300030u) | 0x64006400u; // the f16 pair 1024 + q
+            qmm_half2 h;
+            __builtin_memcpy(&h, &v, 4);
+            h = h - k1056; // q - 32
+            const qmm_half2 a = h * sh2, b = h * sl2;
+            uint32_t ua, ub;
+            __builtin_memcpy(&ua, &a, 4);
+            __builtin_memcpy(&ub, &b, 4);
+            chi[p] = ua, clo[p] = ub;
+        }
+        *(u32x4 *)(buf + a_row * QMM_LDK + 8 * a_g) = chi;
+        *(u32x4 *)(buf + A_H + a_row * QMM_LDK + 8 * a_g) = clo;
+        *(u32x4 *)(buf + 2 * A_H + b_row0 * QMM_LDK + b_c * 8) = sl.h0;
+        *(u32x4 *)(buf + 2 * A_H + b_row1 * QMM_LDK + b_c * 8) = sl.h1;
+        if (((kbase + ks) & 7) == 1) s_d[a_row] = fh_h2f((uint16_t)sl.d); // (the four threads of a row: the same value)
+    };
+    floatx16 acc[FN][FM], part[FN][FM];
+#pragma unroll
+    for (int a = 0; a < FN; a++)
+#pragma unroll
+        for (int b = 0; b < FM; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f, part[a][b][r] = 0.f;
+
+    auto kstep = [&](int ks, Slab &mine, const Slab &other, auto nextodd) {
+        __syncthreads(); // buffer ks & 1 is complete; the other one is no longer read
+        fetch(mine, ks + 2 < ksteps ? ks + 2 : ksteps - 1); // (no branch around the requests: past the end, a repeat)
+        const _Float16 *buf = smem + (ks & 1) * BUF;
+        half8 wh[2][FN], wl[2][FN], xv[2][FM];
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+            const int ko = kk * 16 + 8 * (lane >> 5);
+#pragma unroll
+            for (int a = 0; a < FN; a++) {
+                wh[kk][a] = *(const half8 *)(buf + ((wn * FN + a) * 32 + li) * QMM_LDK + ko);
+                wl[kk][a] = *(const half8 *)(buf + A_H + ((wn * FN + a) * 32 + li) * QMM_LDK + ko);
+            }
+#pragma unroll
+            for (int b = 0; b < FM; b++) xv[kk][b] = *(const half8 *)(buf + 2 * A_H + ((wm * FM + b) * 32 + li) * QMM_LDK + ko);
+        }
+#pragma unroll
+        for (int a = 0; a < FN; a++)
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for (int b = 0; b < FM; b++) {
+                    part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xv[kk][b], wh[kk][a], part[a][b], 0, 0, 0);
+                    part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xv[kk][b], wl[kk][a], part[a][b], 0, 0, 0);
+                }
+        if (((kbase + ks) & 7) == 7) { // the 256-block is complete: its scale
+#pragma unroll
+            for (int a = 0; a < FN; a++) {
+                const float d = s_d[(wn * FN + a) * 32 + li];
+#pragma unroll
+                for (int b = 0; b < FM; b++) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[a][b][r] = fmaf(part[a][b][r], d, acc[a][b][r]);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) part[a][b][r] = 0.f;
+                }
+            }
+        }
+        if (ks + 1 < ksteps) stage(other, ks + 1, nextodd); // (the last step has nothing to stage)
+    };
+    fetch(s0, 0);
+    fetch(s1, 1);
+    stage(s0, 0, std::false_type{});
+    for (int ks0 = 0; ks0 < ksteps; ks0 += 2) { // the register sets alternate: no indexing survives into the code
+        kstep(ks0, s0, s1, std::true_type{});
+        kstep(ks0 + 1, s1, s0, std::false_type{});
+    }
+    // lane = weight row n (column of the MFMA result), register r = activation row 8 (r / 4) + 4 (lane / 32) + r % 4
+#pragma unroll
+    for (int a = 0; a < FN; a++) {
+        const int64_t nn = n0 + (wn * FN + a) * 32 + li;
+        if (nn >= q.n) continue;
+#pragma unroll
+        for (int b = 0; b < FM; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int ml = (wm * FM + b) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3), mm = m0 + ml;
+                if (mm >= m) continue;
+                const float v = acc[a][b][r] * rs[mm];
+                if (split) planes[(((int64_t)kpart * tail + (tile - full)) * TM + ml) * TN + (nn - n0)] = v;
+                else y[(int64_t)mm * q.n + nn] = v;
+            }
+    }
+}
+
 // y = sum of the partial planes of a k-split product, in plane order (deterministic)
 __global__ void k_qmm_sum_planes(const float4 *__restrict__ part, int planes, int64_t n4, float4 *__restrict__ y) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1262,6 +1415,43 @@ __global__ void k_qmm_sum_planes(const float4 *__restrict__ part, int planes, in
         a = make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
     }
     y[i] = a;
+}
+
+static fh_status qmm_launch_tile2q(const fh_qmatrix *q, const _Float16 *xh, const float *rs, int m, float *y, int ksplit) {
+    constexpr size_t lds = 2 * (size_t)(2 * 128 * QMM_LDK + 256 * QMM_LDK) * 2 + 128 * 4;
+    static bool attr_done = false;
+    if (!attr_done) {
+        FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2q, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_done = true;
+    }
+    fh_device *dev = q->dev;
+    dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + 255) / 256), (unsigned)ksplit);
+    if (ksplit == 1 && q->k % 512 == 0) { // split the tiles of a short last round along k
+        const int tiles = (int)(grid.x * grid.y), tail = qmm_tail_tiles(dev, tiles);
+        if (tail) {
+            FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, (size_t)2 * tail * 256 * 128 * 4));
+            k_qmm_tile2q<<<dim3((unsigned)(tiles + tail)), 512, lds, dev->stream>>>(fh_view(q), xh, rs, m, y, (int)grid.x, tiles - tail,
+                                                                                 tail, dev->ksplit_buf);
+            FH_HIP(hipGetLastError());
+            k_qmm_tail_sum<<<dim3((unsigned)(tail * 16)), 512, 0, dev->stream>>>(dev->ksplit_buf, tail, tiles - tail, (int)grid.x, m,
+                                                                                q->n, y);
+            FH_HIP(hipGetLastError());
+            return FH_OK;
+        }
+    }
+    float *dst = y;
+    if (ksplit > 1) {
+        FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, (size_t)ksplit * m * q->n * 4));
+        dst = dev->ksplit_buf;
+    }
+    k_qmm_tile2q<<<grid, 512, lds, dev->stream>>>(fh_view(q), xh, rs, m, dst, 0, 0, 0, nullptr);
+    FH_HIP(hipGetLastError());
+    if (ksplit > 1) {
+        const int64_t n4 = (int64_t)m * q->n / 4;
+        k_qmm_sum_planes<<<dim3((unsigned)((n4 + 255) / 256)), 256, 0, dev->stream>>>((const float4 *)dst, ksplit, n4, (float4 *)y);
+        FH_HIP(hipGetLastError());
+    }
+    return FH_OK;
 }
 
 template <int NTERM>
@@ -1368,6 +1558,9 @@ static fh_status qmm_launch_t(const fh_qmatrix *q, const _Float16 *xh, const _Fl
                     return qmm_launch_tile2j<T, 4>(q, xh, rs, m, y);
             if (mk != 6 && mk != 4) return qmm_launch_tile2i<T, NTERM, 4>(q, xh, xl, rs, m, y);
         }
+        // Q6_K with one activation plane: two exact integer-code terms, the 256-block's d after the MFMAs
+        if constexpr (T == FH_Q6_K && NTERM == 1)
+            if (mk != 6 && mk != 4) return qmm_launch_tile2q(q, xh, rs, m, y, mk == 10 && (q->k / 256) % 2 == 0 && (q->n & 3) == 0 ? 2 : 1);
         // Q4_K: integer codes sc * q, the 256-block's d after the MFMAs, the offsets as one more MFMA per block
         if constexpr (T == FH_Q4_K)
             if (mk != 6 && mk != 4 && xs) // (matmul_kernel = 10: k split in two where k allows it)
@@ -1391,6 +1584,8 @@ static fh_status qmm_launch_t(const fh_qmatrix *q, const _Float16 *xh, const _Fl
             if (tn * ((m + 255) / 256) * ks * 5 >= cus * 4) {
                 if constexpr (T == FH_Q4_K)
                     if (mk != 6 && xs && (q->k / 256) % ks == 0) return qmm_launch_tile2k<NTERM>(q, xh, xl, xs, rs, m, y, ks);
+                if constexpr (T == FH_Q6_K && NTERM == 1)
+                    if (mk != 6 && (q->k / 256) % ks == 0) return qmm_launch_tile2q(q, xh, rs, m, y, ks);
                 return qmm_launch_tile2<T, NTERM, 2, 2, 2>(q, xh, xl, rs, m, y, ks);
             }
         }

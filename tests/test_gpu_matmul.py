@@ -167,6 +167,32 @@ def test_integer_code_tile_kernel(dev, oracle, ty, act, m, n, k, force):
     assert np.array_equal(picked, 0.5 * deq[:, cols].T), "one-hot activations pick dequantised weights exactly"
 
 
+@pytest.mark.parametrize("m,n,k,force", [(256, 128, 256, 8), (300, 200, 512, 8), (129, 1000, 1024, 8), (513, 130, 4096, 8),
+                                          (300, 200, 512, 10), (257, 132, 3584, 10), (40, 128, 768, 10)])
+def test_q6k_integer_code_tile_kernel(dev, oracle, m, n, k, force):
+    """Q6_K with bf16 activations through the tile kernel whose weight operand is two exact integer terms,
+    (sc & ~15) (q - 32) and (sc & 15) (q - 32), with the 256-block's d applied to the accumulated block (matmul_kernel =
+    8 selects it whatever the size, 10 with k split over two workgroups): ragged tiles, one and several 256-blocks,
+    even and odd steps; against the checker, and one-hot activations pick single dequantised weights (d * sc * (q - 32)
+    in one rounding where the reference rounds d * sc first)."""
+    raw = synth.random_weight(Q6_K, n, k, seed=m + n + k)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, Q6_K)
+    bits, xa = bf16_round(synth.random_activation(m, k, seed=7))
+    onehot = np.zeros((m, k), dtype=np.float32)
+    cols = (np.arange(m) * 37 + 5) % k
+    onehot[np.arange(m), cols] = 0.5
+    want = oracle.q_mat_mul(Q6_K, xa, raw, n)
+    dev.set_option("matmul_kernel", force)
+    try:
+        got = Tensor.from_slice(dev, bits, dtype="bf16").q_mat_mul(q).as_slice()
+        picked = Tensor.from_slice(dev, synth.to_bf16_bits(onehot), dtype="bf16").q_mat_mul(q).as_slice()
+    finally:
+        dev.set_option("matmul_kernel", 0)
+    assert_close(got, want, abs_tol=1e-2, rel_tol=1e-3, what=f"Q6_K integer-code tile {m}x{n}x{k}")
+    deq = oracle.dequantize(Q6_K, raw).reshape(n, k)
+    assert np.abs(picked - 0.5 * deq[:, cols].T).max() <= 2e-7 * np.abs(deq).max()
+
+
 @pytest.mark.parametrize("ty,act", [(Q8_0, "bf16"), (Q4_0, "bf16"), (Q8_0, "f32"), (Q6_K, "bf16"), (Q4_K, "bf16"), (Q4_K, "f32")],
                          ids=lambda t: NAMES.get(t, t) if not isinstance(t, str) else t)
 def test_tile_kernels_split_last_round(dev, oracle, ty, act):
