@@ -1264,9 +1264,13 @@ __global__ __launch_bounds__(512) void k_qmm_tile2k(QView q, const _Float16 *__r
 __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__restrict__ xh, const float *__restrict__ rs,
                                                       int m, float *__restrict__ y, int tiles_n, int full, int tail,
                                                       float *__restrict__ planes) {
+    // 64 of k (an even and an odd sub-block step of the tiled record) per step and workgroup barrier; LDS rows of 64 halfs
+    // with the 16-byte pieces XOR-swizzled as in k_qmm_tile2j
+    constexpr int LDK = 64;
+    auto sw = [](int row) { return ((row >> 1) & 1) << 2 | ((row >> 2) & 3); };
     constexpr int WM = 4, WN = 2, FN = 2, FM = 2, TN = WN * FN * 32, TM = WM * FM * 32;
-    constexpr int A_H = TN * QMM_LDK, B_H = TM * QMM_LDK; // halfs per plane
-    constexpr int BUF = 2 * A_H + B_H;                    // halfs per buffer: codes (high part, low part), x
+    constexpr int A_H = TN * LDK, B_H = TM * LDK; // halfs per plane
+    constexpr int BUF = 2 * A_H + B_H;            // halfs per buffer: codes (high part, low part), x
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers, then d per weight row
     float *s_d = (float *)(smem + 2 * BUF);
@@ -1277,60 +1281,73 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
     const int m0 = (tiles_n > 0 ? tile / tiles_n : (int)blockIdx.y) * TM;
     const int kparts = split ? 2 : (int)gridDim.z, kpart = split ? (lin - full) & 1 : (int)blockIdx.z;
     const int K = (int)q.k, nsb = (K >> 8) / kparts, sb0 = kpart * nsb; // 256-blocks of this workgroup
-    const int ksteps = nsb * 8, kbase = sb0 * 8;
+    const int ksteps = nsb * 4, kbase = sb0 * 4;                        // steps of 64
     y += (int64_t)blockIdx.z * m * q.n;
     const int64_t tiles16 = (q.n + 15) / 16;
-    const int a_g = tid & 3, a_j = (tid >> 2) & 15, a_row = tid >> 2;
+    const int a_g = tid & 3, a_j = (tid >> 2) & 15, a_row = tid >> 2, a_sw = sw(a_row);
     int64_t a_tile = (n0 >> 4) + (a_row >> 4);
     if (a_tile >= tiles16) a_tile = tiles16 - 1; // rows past the end decode a valid tile and are never stored
     const uint8_t *a_rec = q.data + a_tile * q.recs * 3360;
-    const int b_c = tid & 3, b_row0 = tid >> 2, b_row1 = b_row0 + TM / 2;
-    const int64_t b_off0 = (int64_t)(m0 + b_row0 < m ? m0 + b_row0 : m - 1) * K + b_c * 8;
-    const int64_t b_off1 = (int64_t)(m0 + b_row1 < m ? m0 + b_row1 : m - 1) * K + b_c * 8;
-    struct Slab {
-        uint32_t a, b, sc, d;
-        u32x4 h0, h1;
-    } s0, s1;
-    auto fetch = [&](Slab &sl, int ks) { // ks: step of this workgroup's range
-        const int g = kbase + ks, t = g & 7;
-        const uint8_t *rec = a_rec + (int64_t)(g >> 3) * 3360;
-        sl.a = *(const uint32_t *)(rec + q6k_lword_off(a_j, t, a_g));
-        sl.b = *(const uint32_t *)(rec + q6k_hword_off(a_j, t, a_g));
-        sl.sc = rec[q6k_sc_off(a_j, 2 * t + (a_g >> 1))];
-        sl.d = fh_ld16(rec + q6k_d_off(a_j));
-        sl.h0 = *(const u32x4 *)(xh + b_off0 + g * 32);
-        sl.h1 = *(const u32x4 *)(xh + b_off1 + g * 32);
-    };
-    // the slab of step ks into buffer ks & 1; ODD: the parity of the step inside its 256-block (the two-bit parts of the
-    // codes sit at other places of their word in odd steps); with sub-block 1 the block's d goes along
-    auto stage = [&](const Slab &sl, int ks, auto oddc) {
-        constexpr bool ODD = decltype(oddc)::value;
-        _Float16 *buf = smem + (ks & 1) * BUF;
-        const int sc = (int)(int8_t)sl.sc;
-        const _Float16 fl = (_Float16)(float)(sc & 15), fh = (_Float16)(float)(sc & ~15); // exact: small integers
-        const qmm_half2 sl2 = {fl, fl}, sh2 = {fh, fh}, k1056 = {(_Float16)1056.f, (_Float16)1056.f};
-        u32x4 chi, clo;
+    // activation duty: four 16-byte pieces per step, the eight threads of a row cover its 128 bytes
+    const int b_c = tid & 7;
+    int64_t b_off[4];
 #pragma unroll
-        for (int p = 0; p < 4; p++) { // weights 2 p and 2 p + 1 of the item: positions 8 g + 2 p, + 1 of the step
-            const uint32_t lo4 = (sl.a >> (4 * p)) & 0x000F000Fu;
-            uint32_t hi2;
-            if (!ODD) hi2 = sl.b >> (2 * p);
-            else hi2 = p == 0 ? sl.b << 4 : (p == 1 ? sl.b << 2 : (p == 2 ? sl.b >> 8 : sl.b >> 10));
-            const uint32_t v = lo4 | (hi2 & 0x00300030u) | 0x64006400u; // the f16 pair 1024 + q
-            qmm_half2 h;
-            __builtin_memcpy(&h, &v, 4);
-            h = h - k1056; // q - 32
-            const qmm_half2 a = h * sh2, b = h * sl2;
-            uint32_t ua, ub;
-            __builtin_memcpy(&ua, &a, 4);
-            __builtin_memcpy(&ub, &b, 4);
-            chi[p] = ua, clo[p] = ub;
+    for (int i = 0; i < 4; i++) {
+        const int row = m0 + (tid >> 3) + i * 64;
+        b_off[i] = (int64_t)(row < m ? row : m - 1) * K + b_c * 8;
+    }
+    struct Slab {
+        uint32_t a0, a1, b, sc0, sc1, d;
+        u32x4 h[4];
+    } sl;
+    auto fetch = [&](int ks) { // ks: step of this workgroup's range
+        const int g = kbase + ks, t = 2 * (g & 3); // the even sub-block step; t + 1 shares its word of two-bit parts
+        const uint8_t *rec = a_rec + (int64_t)(g >> 2) * 3360;
+        const uint2 a = *(const uint2 *)(rec + q6k_lword_off(a_j, t, a_g));
+        sl.a0 = a.x, sl.a1 = a.y;
+        sl.b = *(const uint32_t *)(rec + q6k_hword_off(a_j, t, a_g));
+        sl.sc0 = rec[q6k_sc_off(a_j, 2 * t + (a_g >> 1))];
+        sl.sc1 = rec[q6k_sc_off(a_j, 2 * t + 2 + (a_g >> 1))];
+        sl.d = fh_ld16(rec + q6k_d_off(a_j));
+#pragma unroll
+        for (int i = 0; i < 4; i++) sl.h[i] = *(const u32x4 *)(xh + b_off[i] + g * 64);
+    };
+    auto stage = [&](int ks) {
+        _Float16 *buf = smem + (ks & 1) * BUF;
+        const qmm_half2 k1056 = {(_Float16)1056.f, (_Float16)1056.f};
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++) { // blk = parity of the sub-block step: the two-bit parts sit elsewhere in odd steps
+            const int sc = (int)(int8_t)(blk ? sl.sc1 : sl.sc0);
+            const uint32_t aw = blk ? sl.a1 : sl.a0;
+            const _Float16 fl = (_Float16)(float)(sc & 15), fh = (_Float16)(float)(sc & ~15); // exact: small integers
+            const qmm_half2 sl2 = {fl, fl}, sh2 = {fh, fh};
+            u32x4 chi, clo;
+#pragma unroll
+            for (int p = 0; p < 4; p++) { // weights 2 p and 2 p + 1 of the item: positions 8 g + 2 p, + 1 of the sub-block
+                const uint32_t lo4 = (aw >> (4 * p)) & 0x000F000Fu;
+                uint32_t hi2;
+                if (!blk) hi2 = sl.b >> (2 * p);
+                else hi2 = p == 0 ? sl.b << 4 : (p == 1 ? sl.b << 2 : (p == 2 ? sl.b >> 8 : sl.b >> 10));
+                const uint32_t v = lo4 | (hi2 & 0x00300030u) | 0x64006400u; // the f16 pair 1024 + q
+                qmm_half2 h;
+                __builtin_memcpy(&h, &v, 4);
+                h = h - k1056; // q - 32
+                const qmm_half2 a = h * sh2, b = h * sl2;
+                uint32_t ua, ub;
+                __builtin_memcpy(&ua, &a, 4);
+                __builtin_memcpy(&ub, &b, 4);
+                chi[p] = ua, clo[p] = ub;
+            }
+            *(u32x4 *)(buf + a_row * LDK + 8 * ((4 * blk + a_g) ^ a_sw)) = chi;
+            *(u32x4 *)(buf + A_H + a_row * LDK + 8 * ((4 * blk + a_g) ^ a_sw)) = clo;
         }
-        *(u32x4 *)(buf + a_row * QMM_LDK + 8 * a_g) = chi;
-        *(u32x4 *)(buf + A_H + a_row * QMM_LDK + 8 * a_g) = clo;
-        *(u32x4 *)(buf + 2 * A_H + b_row0 * QMM_LDK + b_c * 8) = sl.h0;
-        *(u32x4 *)(buf + 2 * A_H + b_row1 * QMM_LDK + b_c * 8) = sl.h1;
-        if (((kbase + ks) & 7) == 1) s_d[a_row] = fh_h2f((uint16_t)sl.d); // (the four threads of a row: the same value)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int row = (tid >> 3) + i * 64;
+            *(u32x4 *)(buf + 2 * A_H + row * LDK + 8 * (b_c ^ sw(row))) = sl.h[i];
+        }
+        // the block's d, staged with its second step: nobody reads the previous block's any more
+        if (((kbase + ks) & 3) == 1) s_d[a_row] = fh_h2f((uint16_t)sl.d); // (the four threads of a row: the same value)
     };
     floatx16 acc[FN][FM], part[FN][FM];
 #pragma unroll
@@ -1340,32 +1357,37 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f, part[a][b][r] = 0.f;
 
-    auto kstep = [&](int ks, Slab &mine, const Slab &other, auto nextodd) {
+    fetch(0);
+    stage(0);
+    for (int ks = 0; ks < ksteps; ks++) {
         __syncthreads(); // buffer ks & 1 is complete; the other one is no longer read
-        fetch(mine, ks + 2 < ksteps ? ks + 2 : ksteps - 1); // (no branch around the requests: past the end, a repeat)
+        fetch(ks + 1 < ksteps ? ks + 1 : ks); // (no branch around the requests: past the end, a repeat)
         const _Float16 *buf = smem + (ks & 1) * BUF;
-        half8 wh[2][FN], wl[2][FN], xv[2][FM];
 #pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
-            const int ko = kk * 16 + 8 * (lane >> 5);
+        for (int blk = 0; blk < 2; blk++) {
+            half8 wh[2][FN], wl[2][FN], xv[2][FM];
 #pragma unroll
-            for (int a = 0; a < FN; a++) {
-                wh[kk][a] = *(const half8 *)(buf + ((wn * FN + a) * 32 + li) * QMM_LDK + ko);
-                wl[kk][a] = *(const half8 *)(buf + A_H + ((wn * FN + a) * 32 + li) * QMM_LDK + ko);
+            for (int kk = 0; kk < 2; kk++) {
+                const int ko = 8 * ((4 * blk + 2 * kk + (lane >> 5)) ^ sw(li)); // (tile bases are multiples of 32 rows)
+#pragma unroll
+                for (int a = 0; a < FN; a++) {
+                    wh[kk][a] = *(const half8 *)(buf + ((wn * FN + a) * 32 + li) * LDK + ko);
+                    wl[kk][a] = *(const half8 *)(buf + A_H + ((wn * FN + a) * 32 + li) * LDK + ko);
+                }
+#pragma unroll
+                for (int b = 0; b < FM; b++) xv[kk][b] = *(const half8 *)(buf + 2 * A_H + ((wm * FM + b) * 32 + li) * LDK + ko);
             }
 #pragma unroll
-            for (int b = 0; b < FM; b++) xv[kk][b] = *(const half8 *)(buf + 2 * A_H + ((wm * FM + b) * 32 + li) * QMM_LDK + ko);
+            for (int a = 0; a < FN; a++)
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                    for (int b = 0; b < FM; b++) {
+                        part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xv[kk][b], wh[kk][a], part[a][b], 0, 0, 0);
+                        part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xv[kk][b], wl[kk][a], part[a][b], 0, 0, 0);
+                    }
         }
-#pragma unroll
-        for (int a = 0; a < FN; a++)
-#pragma unroll
-            for (int kk = 0; kk < 2; kk++)
-#pragma unroll
-                for (int b = 0; b < FM; b++) {
-                    part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xv[kk][b], wh[kk][a], part[a][b], 0, 0, 0);
-                    part[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xv[kk][b], wl[kk][a], part[a][b], 0, 0, 0);
-                }
-        if (((kbase + ks) & 7) == 7) { // the 256-block is complete: its scale
+        if (((kbase + ks) & 3) == 3) { // the 256-block is complete: its scale
 #pragma unroll
             for (int a = 0; a < FN; a++) {
                 const float d = s_d[(wn * FN + a) * 32 + li];
@@ -1378,14 +1400,7 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
                 }
             }
         }
-        if (ks + 1 < ksteps) stage(other, ks + 1, nextodd); // (the last step has nothing to stage)
-    };
-    fetch(s0, 0);
-    fetch(s1, 1);
-    stage(s0, 0, std::false_type{});
-    for (int ks0 = 0; ks0 < ksteps; ks0 += 2) { // the register sets alternate: no indexing survives into the code
-        kstep(ks0, s0, s1, std::true_type{});
-        kstep(ks0 + 1, s1, s0, std::false_type{});
+        if (ks + 1 < ksteps) stage(ks + 1); // (the last step has nothing to stage)
     }
     // lane = weight row n (column of the MFMA result), register r = activation row 8 (r / 4) + 4 (lane / 32) + r % 4
 #pragma unroll
@@ -1418,7 +1433,7 @@ __global__ void k_qmm_sum_planes(const float4 *__restrict__ part, int planes, in
 }
 
 static fh_status qmm_launch_tile2q(const fh_qmatrix *q, const _Float16 *xh, const float *rs, int m, float *y, int ksplit) {
-    constexpr size_t lds = 2 * (size_t)(2 * 128 * QMM_LDK + 256 * QMM_LDK) * 2 + 128 * 4;
+    constexpr size_t lds = 2 * (size_t)(2 * 128 * 64 + 256 * 64) * 2 + 128 * 4;
     static bool attr_done = false;
     if (!attr_done) {
         FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2q, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
