@@ -72,6 +72,88 @@ __global__ __launch_bounds__(256) void k_act_split(const void *__restrict__ xin,
     if (threadIdx.x == 0) rs[blockIdx.x] = __uint_as_float((uint32_t)(127 - e) << 23);
 }
 
+// The same for contiguous rows with k a multiple of 8 and at most 16384: a thread holds its (up to 64) elements of
+// the row in registers between the maximum and the conversion, so the row is read once, in 16- or 32-byte loads, and
+// written in 16-byte stores.  Values, sums and scale are those of k_act_split.
+template <int IN>
+__global__ __launch_bounds__(256) void k_act_split_rows(const void *__restrict__ xin, int k, _Float16 *__restrict__ xh,
+                                                         _Float16 *__restrict__ xl, float *__restrict__ rs,
+                                                         _Float16 *__restrict__ xs) {
+    constexpr int NCH = 8; // chunks of 8 elements per thread
+    __shared__ float sh[4];
+    const int64_t oo = (int64_t)blockIdx.x * k;
+    const int nch = (k + 2047) / 2048;
+    float v[NCH][8];
+    float amax = 0.f;
+#pragma unroll
+    for (int it = 0; it < NCH; it++) {
+        const int c = (it * 256 + (int)threadIdx.x) * 8;
+        if (it < nch && c < k) {
+            if (IN == 1) {
+                const uint4 u = *(const uint4 *)((const uint16_t *)xin + oo + c);
+                const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    v[it][2 * e] = __uint_as_float(w[e] << 16);
+                    v[it][2 * e + 1] = __uint_as_float(w[e] & 0xFFFF0000u);
+                }
+            } else {
+                const float4 a = *(const float4 *)((const float *)xin + oo + c), b = *(const float4 *)((const float *)xin + oo + c + 4);
+                v[it][0] = a.x, v[it][1] = a.y, v[it][2] = a.z, v[it][3] = a.w;
+                v[it][4] = b.x, v[it][5] = b.y, v[it][6] = b.z, v[it][7] = b.w;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[it][e] = 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[it][e]));
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+    int e2 = 141 - (int)((__float_as_uint(amax) >> 23) & 0xFFu); // 14 - floor(log2 amax); zero / inf / nan clamp
+    e2 = e2 > 100 ? 100 : (e2 < -100 ? -100 : e2);
+    const float sc = __uint_as_float((uint32_t)(e2 + 127) << 23);
+#pragma unroll
+    for (int it = 0; it < NCH; it++) {
+        const int c = (it * 256 + (int)threadIdx.x) * 8;
+        const bool live = it < nch && c < k; // (uniform over the four threads of a 32-group: k is a multiple of 8 ... and of 32 with xs)
+        _Float16 h[8], l[8];
+        float t = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float w = v[it][e] * sc;
+            h[e] = (_Float16)w;
+            l[e] = (_Float16)(w - (float)h[e]);
+            t += w;
+        }
+        if (live) {
+            uint4 u;
+            __builtin_memcpy(&u, h, 16);
+            *(uint4 *)(xh + oo + c) = u;
+            if (IN != 1) {
+                __builtin_memcpy(&u, l, 16);
+                *(uint4 *)(xl + oo + c) = u;
+            }
+        }
+        if (xs) { // sums of the 32-groups (four neighbouring threads), / 64, as hi + lo planes
+            t += __shfl_xor(t, 1, 64);
+            t += __shfl_xor(t, 2, 64);
+            if (live && (threadIdx.x & 3) == 0) {
+                t *= 0.015625f;
+                const _Float16 th = (_Float16)t;
+                const int64_t at = (int64_t)blockIdx.x * (k >> 5) + (c >> 5);
+                xs[at] = th;
+                xs[at + (int64_t)gridDim.x * (k >> 5)] = (_Float16)(t - (float)th);
+            }
+        }
+    }
+    if (threadIdx.x == 0) rs[blockIdx.x] = __uint_as_float((uint32_t)(127 - e2) << 23);
+}
+
 // Rows of a dense right-hand side as the tile kernel's "weights": row r (one output column of the product) scaled by
 // its own power of two into the f16 range, written as f32 [rows, kp] (zero from k to kp); cs[r] = 2^-e for the store.
 template <bool F16>
@@ -1659,7 +1741,10 @@ fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf
     _Float16 *xl = x_is_bf16 ? nullptr : (_Float16 *)((uint8_t *)dev->act_buf + plane);
     float *rs = (float *)((uint8_t *)dev->act_buf + plane * (x_is_bf16 ? 1 : 2));
     _Float16 *xs = sums ? (_Float16 *)((uint8_t *)rs + rs_bytes) : nullptr;
-    if (x_is_bf16) k_act_split<1><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, K, 1, (int)K, (int)K, xh, xl, rs, xs);
+    const bool rows = K % 32 == 0 && K <= 16384 && ((uintptr_t)x & 15) == 0 && dev->opt_matmul_kernel != 12; // (12: the general kernel)
+    if (rows && x_is_bf16) k_act_split_rows<1><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, (int)K, xh, xl, rs, xs);
+    else if (rows) k_act_split_rows<0><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, (int)K, xh, xl, rs, xs);
+    else if (x_is_bf16) k_act_split<1><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, K, 1, (int)K, (int)K, xh, xl, rs, xs);
     else k_act_split<0><<<dim3((unsigned)m), dim3(256), 0, dev->stream>>>(x, K, 1, (int)K, (int)K, xh, xl, rs, xs);
     FH_HIP(hipGetLastError());
 #define QMM_GO(T_)                                                              \

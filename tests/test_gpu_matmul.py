@@ -167,6 +167,32 @@ def test_integer_code_tile_kernel(dev, oracle, ty, act, m, n, k, force):
     assert np.array_equal(picked, 0.5 * deq[:, cols].T), "one-hot activations pick dequantised weights exactly"
 
 
+@pytest.mark.parametrize("act", ["f32", "bf16"])
+@pytest.mark.parametrize("ty,k", [(Q8_0, 4096), (Q8_0, 96), (Q6_K, 14336), (Q4_K, 2304)], ids=lambda t: NAMES.get(t, t))
+def test_activation_planes_one_pass_kernel(dev, oracle, ty, k, act):
+    """The activation planes of the tile kernels come from a kernel that reads a contiguous row once (k a multiple of 32,
+    at most 16384) or from the general two-pass one (matmul_kernel = 12 forces it): the same
+    planes, so the same product bit for bit - except Q4_K, whose sub-block sums are added in another order."""
+    m, n = 150, 136
+    raw = synth.random_weight(ty, n, k, seed=k)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    xa = synth.random_activation(m, k, seed=3)
+    xa[7] = 0.0  # a row of zeros: the scale clamps
+    xa[9] *= 1e-30
+    x = Tensor.from_slice(dev, synth.to_bf16_bits(xa), dtype="bf16") if act == "bf16" else Tensor.from_slice(dev, xa)
+    dev.set_option("matmul_kernel", 2)
+    try:
+        one = x.q_mat_mul(q).as_slice()
+        dev.set_option("matmul_kernel", 12)
+        two = x.q_mat_mul(q).as_slice()
+    finally:
+        dev.set_option("matmul_kernel", 0)
+    if ty == Q4_K:
+        assert np.abs(one - two).max() <= 1e-5 * np.abs(two).max()
+    else:
+        assert np.array_equal(one, two)
+
+
 @pytest.mark.parametrize("m,n,k,force", [(256, 128, 256, 8), (300, 200, 512, 8), (129, 1000, 1024, 8), (513, 130, 4096, 8),
                                           (300, 200, 512, 10), (257, 132, 3584, 10), (40, 128, 768, 10)])
 def test_q6k_integer_code_tile_kernel(dev, oracle, m, n, k, force):
