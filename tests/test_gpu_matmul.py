@@ -219,15 +219,17 @@ def test_q6k_integer_code_tile_kernel(dev, oracle, m, n, k, force):
     assert np.abs(picked - 0.5 * deq[:, cols].T).max() <= 2e-7 * np.abs(deq).max()
 
 
-@pytest.mark.parametrize("ty,act", [(Q8_0, "bf16"), (Q4_0, "bf16"), (Q8_0, "f32"), (Q6_K, "bf16"), (Q4_K, "bf16"), (Q4_K, "f32")],
-                         ids=lambda t: NAMES.get(t, t) if not isinstance(t, str) else t)
-def test_tile_kernels_split_last_round(dev, oracle, ty, act):
+@pytest.mark.parametrize("n", [2556, 2555])
+@pytest.mark.parametrize("ty,act", [(Q8_0, "bf16"), (Q4_0, "bf16"), (Q8_0, "f32"), (Q6_K, "bf16"), (Q6_K, "f32"), (Q4_K, "bf16"),
+                                    (Q4_K, "f32")], ids=lambda t: NAMES.get(t, t) if not isinstance(t, str) else t)
+def test_tile_kernels_split_last_round(dev, oracle, ty, act, n):
     """More output tiles than compute units, the remainder at most half of them: the tiles of the last round are two
     workgroups each, one per half of k, summed by a second launch (280 tiles of 256 x 128 on 256 compute units: 24 tiles
-    are split; ragged in both directions) - in every kernel with 256 x 128 tiles: integer codes with 64 and 32 of k per
-    step, the split form (Q6_K), Q4_K on integer codes with one and two activation planes.  Against the checker on sampled columns, and against the same product with
-    the split switched off (matmul_kernel = 11), which must agree to the rounding of one addition."""
-    m, n, k = 3333, 2556, 512
+    are split; ragged in both directions, n a multiple of four or odd) - in every kernel with 256 x 128 tiles: integer
+    codes with 64 and 32 of k per step (Q8_0 / Q4_0), Q6_K on two integer terms (bf16) and on the split form (f32), Q4_K
+    on integer codes with one and two activation planes.  Against the checker on sampled columns, and against the same
+    product with the split switched off (matmul_kernel = 11), which must agree to the rounding of one addition."""
+    m, k = 3333, 512
     raw = synth.random_weight(ty, n, k, seed=77)
     xb, xf = bf16_round(synth.random_activation(m, k, seed=78))
     q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
