@@ -148,13 +148,17 @@ def decoder_shapes_leg(dev, steps: int, warmup: int, trains: int) -> list:
     return out
 
 
-def prefill_legs(dev, trains: int) -> dict:
+def prefill_legs(dev, trains: int, use_graph: bool = True) -> dict:
     """configs[2]: Y = X . W^T with bf16 X [m, 4096] and Q6_K / Q8_0 W [14336, 4096]; configs[3]: causal attention,
-    f16, 32 query heads on 8 KV heads, head_dim 128, and its decode variant.  Median device time of `trains` calls;
+    f16, 32 query heads on 8 KV heads, head_dim 128, and its decode variant.  Device time per call: the median over
+    `trains` replays of a recorded train of CALLS back-to-back calls (as the headline and the decode variant are timed:
+    a call in a pipeline of launches, not a lone launch between two events), all launches of a call included;
     TFLOP/s counts 2 m n k (matmul) and 4 s^2 d h / 2 (causal attention) against the 2.5 PFLOP/s dense f16 MFMA peak
     (5 POP/s for the int8 variant); the decode variant counts K and V bytes against the 8 TB/s HBM peak."""
     from kalosm_amd import synth
     from kalosm_amd.fusor import MaskKind, QMatrix, Tensor
+
+    CALLS = 8
 
     def med(fn):
         # warm-up: at least three calls and 50 ms of them (the device drops its clocks while the host prepares the next
@@ -164,17 +168,13 @@ def prefill_legs(dev, trains: int) -> dict:
             fn()
             dev.sync()
             calls += 1
-        ts = []
-        for _ in range(max(trains, 7)):
-            dev.timer_start()
-            fn()
-            ts.append(dev.timer_stop())
-        return statistics.median(ts)
+        ms, _ = timed_trains(dev, lambda: [fn() for _ in range(CALLS)], max(trains, 7), use_graph)
+        return ms / CALLS
 
     def mfma(tf, peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s"):
         return {"bound": "mfma", "achieved": round(tf, 1), "peak": peak, "unit": unit, "frac": round(tf / peak, 4)}
 
-    res = {"matmul": [], "attention": [], "attention_decode": []}
+    res = {"calls_per_train": CALLS, "matmul": [], "attention": [], "attention_decode": []}
     n, k = 14336, 4096
     for ty, name in ((synth.Q6_K, "Q6_K"), (synth.Q8_0, "Q8_0")):
         q = QMatrix.from_raw_bytes(dev, (n, k), synth.random_weight(ty, n, k, seed=7), ty)
@@ -443,7 +443,7 @@ def main() -> int:
     del sets
     if not args.no_legs:
         out["decoder_shapes"] = decoder_shapes_leg(dev, args.steps, args.warmup, args.trains)
-        out["prefill"] = prefill_legs(dev, max(3, min(args.trains, 5)))
+        out["prefill"] = prefill_legs(dev, max(3, min(args.trains, 5)), not args.no_graph)
 
     if args.e2e_eager:
         from kalosm_amd import e2e
