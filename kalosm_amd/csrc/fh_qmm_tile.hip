@@ -1141,7 +1141,11 @@ __global__ __launch_bounds__(512) void k_qmm_tile2k(QView q, const _Float16 *__r
                                                       float *__restrict__ y, int tiles_n, int full, int tail,
                                                       float *__restrict__ planes) {
     constexpr int WM = 4, WN = 2, FN = 2, FM = 2, TN = WN * FN * 32, TM = WM * FM * 32;
-    constexpr int A_H = TN * QMM_LDK, B_H = TM * QMM_LDK; // halfs per plane
+    // LDS rows of 32 halfs = four 16-byte pieces, piece c of row r at position c ^ ((r >> 2) & 3): the 16-byte reads of 16
+    // consecutive rows at one c and the 64-byte writes of four consecutive rows cover the 64 banks once (no padding)
+    constexpr int LDK = 32;
+    auto sw = [](int row) { return (row >> 2) & 3; };
+    constexpr int A_H = TN * LDK, B_H = TM * LDK; // halfs per plane
     constexpr int BUF = A_H + NTERM * B_H;                // halfs per buffer: codes, x hi (, x lo)
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers, then the per-256-block operands
@@ -1216,12 +1220,12 @@ __global__ __launch_bounds__(512) void k_qmm_tile2k(QView q, const _Float16 *__r
         c.y = bits(__builtin_elementwise_fma(up2(wa, 0x04030402u), sc2, nb));
         c.z = bits(__builtin_elementwise_fma(up2(wb, 0x04010400u), sc2, nb));
         c.w = bits(__builtin_elementwise_fma(up2(wb, 0x04030402u), sc2, nb));
-        *(u32x4 *)(buf + a_row * QMM_LDK + 8 * a_g) = c;
-        *(u32x4 *)(buf + A_H + b_row0 * QMM_LDK + b_c * 8) = sl.h0;
-        *(u32x4 *)(buf + A_H + b_row1 * QMM_LDK + b_c * 8) = sl.h1;
+        *(u32x4 *)(buf + a_row * LDK + 8 * (a_g ^ sw(a_row))) = c;
+        *(u32x4 *)(buf + A_H + b_row0 * LDK + 8 * (b_c ^ sw(b_row0))) = sl.h0;
+        *(u32x4 *)(buf + A_H + b_row1 * LDK + 8 * (b_c ^ sw(b_row1))) = sl.h1;
         if (NTERM == 2) {
-            *(u32x4 *)(buf + A_H + B_H + b_row0 * QMM_LDK + b_c * 8) = sl.l0;
-            *(u32x4 *)(buf + A_H + B_H + b_row1 * QMM_LDK + b_c * 8) = sl.l1;
+            *(u32x4 *)(buf + A_H + B_H + b_row0 * LDK + 8 * (b_c ^ sw(b_row0))) = sl.l0;
+            *(u32x4 *)(buf + A_H + B_H + b_row1 * LDK + 8 * (b_c ^ sw(b_row1))) = sl.l1;
         }
         if (sb == 1) {
             const uint32_t m03 = sl.h.z & 0x3F3F3F3Fu, m47 = ((sl.h.w >> 4) & 0x0F0F0F0Fu) | ((sl.h.z >> 2) & 0x30303030u);
@@ -1255,14 +1259,14 @@ __global__ __launch_bounds__(512) void k_qmm_tile2k(QView q, const _Float16 *__r
         half8 wc[2][FN], xhv[2][FM], xlv[2][FM];
 #pragma unroll
         for (int kk = 0; kk < 2; kk++) {
-            const int ko = kk * 16 + 8 * (lane >> 5);
+            const int ko = 8 * ((2 * kk + (lane >> 5)) ^ sw(li)); // (tile bases are multiples of 32 rows)
 #pragma unroll
-            for (int a = 0; a < FN; a++) wc[kk][a] = *(const half8 *)(buf + ((wn * FN + a) * 32 + li) * QMM_LDK + ko);
+            for (int a = 0; a < FN; a++) wc[kk][a] = *(const half8 *)(buf + ((wn * FN + a) * 32 + li) * LDK + ko);
 #pragma unroll
             for (int b = 0; b < FM; b++) {
                 const int row = (wm * FM + b) * 32 + li;
-                xhv[kk][b] = *(const half8 *)(buf + A_H + row * QMM_LDK + ko);
-                if (NTERM == 2) xlv[kk][b] = *(const half8 *)(buf + A_H + B_H + row * QMM_LDK + ko);
+                xhv[kk][b] = *(const half8 *)(buf + A_H + row * LDK + ko);
+                if (NTERM == 2) xlv[kk][b] = *(const half8 *)(buf + A_H + B_H + row * LDK + ko);
             }
         }
 #pragma unroll
@@ -1554,7 +1558,7 @@ static fh_status qmm_launch_tile2q(const fh_qmatrix *q, const _Float16 *xh, cons
 template <int NTERM>
 static fh_status qmm_launch_tile2k(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const _Float16 *xs,
                                    const float *rs, int m, float *y, int ksplit) {
-    constexpr size_t lds = 2 * (size_t)(128 * QMM_LDK + NTERM * 256 * QMM_LDK) * 2 + 128 * 8 * 2 + 2 * 256 * 8 * 2 + 128 * 2 * 4;
+    constexpr size_t lds = 2 * (size_t)(128 * 32 + NTERM * 256 * 32) * 2 + 128 * 8 * 2 + 2 * 256 * 8 * 2 + 128 * 2 * 4;
     static bool attr_done = false;
     if (!attr_done) {
         FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2k<NTERM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
