@@ -26,6 +26,10 @@ static int qmm_tail_tiles(const fh_device *dev, int tiles) {
 }
 
 #define QMM_LDK 40 // halfs per LDS row: 32 + 8 padding (80 B stride: 16-byte reads of 16 rows hit 16 distinct chunks)
+// The pipelined kernels use unpadded rows of 32 halfs (four 16-byte pieces) instead, piece c of row r at position
+// c ^ ((r >> 2) & 3): the 16-byte reads of 16 consecutive rows at one c and the writes of four consecutive rows cover the
+// 64 banks once.  QMM_AT(row, pos): half offset of position pos (0 .. 31) of row `row` inside a plane.
+#define QMM_AT(row, pos) ((row) * 32 + 8 * ((((pos) >> 3)) ^ (((row) >> 2) & 3)) + ((pos) & 7))
 
 // ------------------------------------------------------------------------------ activation planes
 // One workgroup per row.  xh / xl are [m, kp] f16 (zero from k to kp), rs[m] = 2^-e undoes the normalisation at the
@@ -496,7 +500,7 @@ __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__re
     constexpr int WM = 8 / WN, TN = WN * FN * 32, TM = WM * FM * 32;
     static_assert(TN == 128, "512 threads decode 128 weight rows x 4 pieces per step");
     constexpr int NB = (TM * 4 + 511) / 512; // 16-byte activation pieces per thread, plane and step
-    constexpr int A_H = TN * QMM_LDK, B_H = TM * QMM_LDK;         // halfs per plane
+    constexpr int A_H = TN * 32, B_H = TM * 32;         // halfs per plane
     constexpr int BUF = 2 * A_H + NTERM * B_H;                    // halfs per buffer: A hi, A lo, B hi (, B lo)
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -552,15 +556,15 @@ __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__re
         __builtin_memcpy(&a1, hi + 4, 8);
         __builtin_memcpy(&l0, lo, 8);
         __builtin_memcpy(&l1, lo + 4, 8);
-        *(uint2 *)(buf + a_row * QMM_LDK + p0) = a0;
-        *(uint2 *)(buf + a_row * QMM_LDK + p1) = a1;
-        *(uint2 *)(buf + A_H + a_row * QMM_LDK + p0) = l0;
-        *(uint2 *)(buf + A_H + a_row * QMM_LDK + p1) = l1;
-        *(uint4 *)(buf + 2 * A_H + b_row0 * QMM_LDK + b_c * 8) = sl.h0;
-        if (NB == 2) *(uint4 *)(buf + 2 * A_H + b_row1 * QMM_LDK + b_c * 8) = sl.h1;
+        *(uint2 *)(buf + QMM_AT(a_row, p0)) = a0;
+        *(uint2 *)(buf + QMM_AT(a_row, p1)) = a1;
+        *(uint2 *)(buf + A_H + QMM_AT(a_row, p0)) = l0;
+        *(uint2 *)(buf + A_H + QMM_AT(a_row, p1)) = l1;
+        *(uint4 *)(buf + 2 * A_H + QMM_AT(b_row0, b_c * 8)) = sl.h0;
+        if (NB == 2) *(uint4 *)(buf + 2 * A_H + QMM_AT(b_row1, b_c * 8)) = sl.h1;
         if (NTERM == 2) {
-            *(uint4 *)(buf + 2 * A_H + B_H + b_row0 * QMM_LDK + b_c * 8) = sl.l0;
-            if (NB == 2) *(uint4 *)(buf + 2 * A_H + B_H + b_row1 * QMM_LDK + b_c * 8) = sl.l1;
+            *(uint4 *)(buf + 2 * A_H + B_H + QMM_AT(b_row0, b_c * 8)) = sl.l0;
+            if (NB == 2) *(uint4 *)(buf + 2 * A_H + B_H + QMM_AT(b_row1, b_c * 8)) = sl.l1;
         }
     };
     floatx16 acc[FN][FM];
@@ -587,14 +591,14 @@ __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__re
 #pragma unroll
                     for (int a = 0; a < FN; a++) {
                         const int row = (wn * FN + a) * 32 + li;
-                        ah[a] = *(const half8 *)(buf + row * QMM_LDK + ko);
-                        al[a] = *(const half8 *)(buf + A_H + row * QMM_LDK + ko);
+                        ah[a] = *(const half8 *)(buf + QMM_AT(row, ko));
+                        al[a] = *(const half8 *)(buf + A_H + QMM_AT(row, ko));
                     }
 #pragma unroll
                     for (int b = 0; b < FM; b++) {
                         const int row = (wm * FM + b) * 32 + li;
-                        bhv[b] = *(const half8 *)(buf + 2 * A_H + row * QMM_LDK + ko);
-                        if (NTERM == 2) blv[b] = *(const half8 *)(buf + 2 * A_H + B_H + row * QMM_LDK + ko);
+                        bhv[b] = *(const half8 *)(buf + 2 * A_H + QMM_AT(row, ko));
+                        if (NTERM == 2) blv[b] = *(const half8 *)(buf + 2 * A_H + B_H + QMM_AT(row, ko));
                     }
 #pragma unroll
                     for (int a = 0; a < FN; a++)
@@ -664,7 +668,7 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2i(QView q, const _Float16
     // WM = 4: eight wavefronts, 256 activation rows; WM = 2: four wavefronts, 128 activation rows - two such workgroups
     // share a compute unit and are at different points of their steps (one's MFMAs under the other's scaling and staging)
     constexpr int WN = 2, FN = 2, FM = 2, TN = WN * FN * 32, TM = WM * FM * 32, NT = 128 * WM, NA = 512 / NT;
-    constexpr int A_H = TN * QMM_LDK, B_H = TM * QMM_LDK;       // halfs per plane
+    constexpr int A_H = TN * 32, B_H = TM * 32;       // halfs per plane
     constexpr int BUF = A_H + NTERM * B_H + 2 * TN;            // halfs per buffer: codes, x hi (, x lo), TN f32 scales
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31;
@@ -724,7 +728,7 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2i(QView q, const _Float16
             c.y = codes2(ua, 0x04030402u, 1152.f);
             c.z = codes2(ub, 0x04010400u, 1152.f);
             c.w = codes2(ub, 0x04030402u, 1152.f);
-            *(uint4 *)(buf + a_row[u] * QMM_LDK + 8 * a_g) = c;
+            *(uint4 *)(buf + QMM_AT(a_row[u], 8 * a_g)) = c;
         } else { // low nibbles: positions 4 g .. 4 g + 3, high nibbles: 16 + 4 g .. 16 + 4 g + 3
             const uint32_t lo = sl.raw[u].a & 0x0F0F0F0Fu, hi = (sl.raw[u].a >> 4) & 0x0F0F0F0Fu;
             uint2 c0, c1;
@@ -732,16 +736,16 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2i(QView q, const _Float16
             c0.y = codes2(lo, 0x04030402u, 1032.f);
             c1.x = codes2(hi, 0x04010400u, 1032.f);
             c1.y = codes2(hi, 0x04030402u, 1032.f);
-            *(uint2 *)(buf + a_row[u] * QMM_LDK + 4 * a_g) = c0;
-            *(uint2 *)(buf + a_row[u] * QMM_LDK + 16 + 4 * a_g) = c1;
+            *(uint2 *)(buf + QMM_AT(a_row[u], 4 * a_g)) = c0;
+            *(uint2 *)(buf + QMM_AT(a_row[u], 16 + 4 * a_g)) = c1;
         }
         ((float *)(buf + A_H + NTERM * B_H))[a_row[u]] = fh_h2f((uint16_t)sl.raw[u].h.x); // the four threads of a row: same value
         }
-        *(uint4 *)(buf + A_H + b_row0 * QMM_LDK + b_c * 8) = sl.h0;
-        *(uint4 *)(buf + A_H + b_row1 * QMM_LDK + b_c * 8) = sl.h1;
+        *(uint4 *)(buf + A_H + QMM_AT(b_row0, b_c * 8)) = sl.h0;
+        *(uint4 *)(buf + A_H + QMM_AT(b_row1, b_c * 8)) = sl.h1;
         if (NTERM == 2) {
-            *(uint4 *)(buf + A_H + B_H + b_row0 * QMM_LDK + b_c * 8) = sl.l0;
-            *(uint4 *)(buf + A_H + B_H + b_row1 * QMM_LDK + b_c * 8) = sl.l1;
+            *(uint4 *)(buf + A_H + B_H + QMM_AT(b_row0, b_c * 8)) = sl.l0;
+            *(uint4 *)(buf + A_H + B_H + QMM_AT(b_row1, b_c * 8)) = sl.l1;
         }
     };
     floatx16 acc[FN][FM];
@@ -775,12 +779,12 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2i(QView q, const _Float16
             for (int kk = 0; kk < 2; kk++) {
                 const int ko = kk * 16 + 8 * (lane >> 5);
 #pragma unroll
-                for (int a = 0; a < FN; a++) wc[kk][a] = *(const half8 *)(buf + ((wn * FN + a) * 32 + li) * QMM_LDK + ko);
+                for (int a = 0; a < FN; a++) wc[kk][a] = *(const half8 *)(buf + QMM_AT(((wn * FN + a) * 32 + li), ko));
 #pragma unroll
                 for (int b = 0; b < FM; b++) {
                     const int row = (wm * FM + b) * 32 + li;
-                    xhv[kk][b] = *(const half8 *)(buf + A_H + row * QMM_LDK + ko);
-                    if (NTERM == 2) xlv[kk][b] = *(const half8 *)(buf + A_H + B_H + row * QMM_LDK + ko);
+                    xhv[kk][b] = *(const half8 *)(buf + A_H + QMM_AT(row, ko));
+                    if (NTERM == 2) xlv[kk][b] = *(const half8 *)(buf + A_H + B_H + QMM_AT(row, ko));
                 }
             }
             const float *sd = (const float *)(buf + A_H + NTERM * B_H);
@@ -1099,7 +1103,7 @@ template <int T, int NTERM, int WM>
 static fh_status qmm_launch_tile2i(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const float *rs, int m,
                                    float *y) {
     constexpr int TM = WM * 64;
-    constexpr size_t lds = 2 * (size_t)(128 * QMM_LDK + NTERM * TM * QMM_LDK + 2 * 128) * 2;
+    constexpr size_t lds = 2 * (size_t)(128 * 32 + NTERM * TM * 32 + 2 * 128) * 2;
     static bool attr_done = false;
     if (!attr_done) {
         FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2i<T, NTERM, WM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -1600,7 +1604,7 @@ template <int T, int NTERM, int WN, int FN, int FM>
 static fh_status qmm_launch_tile2(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const float *rs, int m,
                                   float *y, int ksplit = 1) {
     constexpr int TM = (8 / WN) * FM * 32;
-    constexpr size_t lds = 2 * (size_t)(2 * 128 * QMM_LDK + NTERM * TM * QMM_LDK) * 2;
+    constexpr size_t lds = 2 * (size_t)(2 * 128 * 32 + NTERM * TM * 32) * 2;
     static bool attr_done = false;
     if (!attr_done) {
         FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2<T, NTERM, WN, FN, FM>,
