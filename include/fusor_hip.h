@@ -100,6 +100,17 @@ fh_status fh_timer_stop(fh_device *dev, float *elapsed_ms); /* blocks until the 
 fh_status fh_probe_empty(fh_device *dev, int32_t workgroups, int32_t threads);
 fh_status fh_probe_read(fh_device *dev, const void *src_dev, size_t bytes);
 
+/* debug_check_nan_f32, models/kalosm-llama/src/raw/mod.rs:9-58: what that probe logs about an f32 tensor - the
+ * counts of NaN, +inf and -inf, the largest finite magnitude and the indices of the first NaNs (up to four, in
+ * ascending order).  Blocking. */
+typedef struct {
+    uint64_t nan, pos_inf, neg_inf;
+    float max_abs;
+    uint32_t first_nan_count;
+    uint64_t first_nan[4];
+} fh_finite_stats;
+fh_status fh_check_finite(fh_device *dev, const float *x_dev, int64_t count, fh_finite_stats *out_host);
+
 /* Record-and-replay of a sequence of operator calls (the reference records a lazy graph and submits one
  * command buffer per resolve, fusor-ml/core/src/compute_graph/resolve/run.rs).  Between begin and end the
  * operator calls on `dev` are captured into a hipGraph instead of running; fh_graph_launch replays them.
@@ -426,6 +437,18 @@ fh_status fh_llama_reset(fh_llama *m);
  * hidden_host (optional, [d_model], the final-norm hidden state) are of the LAST token. */
 fh_status fh_llama_forward(fh_llama *m, const uint32_t *tokens_host, int32_t count,
                            float *logits_host, float *hidden_host);
+/* Trace of the last fh_llama_forward, as text lines.  Off by default; fh_set_option keys (or the reference's
+ * environment variables, looked up when the device is created, which also send the lines to stderr):
+ *   "trace_nan" = 1 (KALOSM_TRACE_LAYER_NAN, models/kalosm-llama/src/raw/mod.rs:955-1041): the embedding and, for
+ *     every layer, the normed input, the attention output and the layer output are probed with fh_check_finite; a
+ *     tensor with a NaN or an infinity gives one "trace_nan layer=.. label=.. .." line (debug_check_nan_f32, :9-58).
+ *   "trace_timing" = 1 (KALOSM_TRACE_FORWARD_TIMING, raw/mod.rs:943-1043): "[timing] text layer loop: .. ms";
+ *     = 2 (FUSOR_TRACE_GPU_KERNELS, fusor-ml/core/src/compute_graph/resolve/run.rs:141, :483-497): also one
+ *     "[timing] layer L <stage>: .. us" line per stage of every layer, from events on the stream.
+ *   "trace_stderr" = 1: the lines go to stderr as well.
+ * The device-side decode loops (captured steps) are never traced.  buf receives at most capacity - 1 bytes and a
+ * terminating NUL; *length (optional) the full length. */
+fh_status fh_llama_trace_text(const fh_llama *m, char *buf, size_t capacity, size_t *length);
 /* Greedy decode: feeds `first_token`, then each argmax, for `steps` steps entirely on the device
  * (the sampled id stays resident, as the reference's run-ahead path, model/inference.rs:38-173);
  * out_tokens_host receives the `steps` sampled ids.  elapsed_ms (optional) is the device time. */

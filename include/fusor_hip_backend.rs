@@ -434,6 +434,17 @@ impl HipLlama {
         check(unsafe { sys::fh_llama_forward(self.raw, tokens.as_ptr(), tokens.len() as i32, logits.as_mut_ptr(), ptr::null_mut()) })?;
         Ok(logits)
     }
+    /// The lines the last `forward` traced (`KALOSM_TRACE_LAYER_NAN`, `KALOSM_TRACE_FORWARD_TIMING`,
+    /// `FUSOR_TRACE_GPU_KERNELS` in the environment, or the `trace_*` options of the device); the reference hands
+    /// the same lines to `tracing::warn!` / `tracing::info!` (raw/mod.rs:46-52, :946-950, :1041-1043).
+    pub fn trace_text(&self) -> Result<String> {
+        let mut len = 0usize;
+        check(unsafe { sys::fh_llama_trace_text(self.raw, ptr::null_mut(), 0, &mut len) })?;
+        let mut buf = vec![0u8; len + 1];
+        check(unsafe { sys::fh_llama_trace_text(self.raw, buf.as_mut_ptr().cast(), len + 1, ptr::null_mut()) })?;
+        buf.truncate(len);
+        Ok(String::from_utf8_lossy(&buf).into_owned())
+    }
     /// Greedy decoding of `steps` tokens after `first_token`, entirely on the device.
     pub fn decode_greedy(&mut self, first_token: u32, steps: usize) -> Result<Vec<u32>> {
         let mut out = vec![0u32; steps];

@@ -90,6 +90,18 @@ pub struct FhLlamaConfig {
     pub use_graph: i32,
 }
 
+/// `fh_finite_stats` (what `debug_check_nan_f32` logs, models/kalosm-llama/src/raw/mod.rs:9-58)
+#[repr(C)]
+#[derive(Clone, Copy, Debug, Default)]
+pub struct FhFiniteStats {
+    pub nan: u64,
+    pub pos_inf: u64,
+    pub neg_inf: u64,
+    pub max_abs: f32,
+    pub first_nan_count: u32,
+    pub first_nan: [u64; 4],
+}
+
 /// `fh_rope_scaling` (`RopeScalingConfig`, models/kalosm-llama/src/raw/mod.rs:163-169)
 #[repr(C)]
 #[derive(Clone, Copy, Debug)]
@@ -144,6 +156,7 @@ extern "C" {
     pub fn fh_timer_stop(dev: *mut FhDevice, elapsed_ms: *mut f32) -> FhStatus;
     pub fn fh_probe_empty(dev: *mut FhDevice, workgroups: i32, threads: i32) -> FhStatus;
     pub fn fh_probe_read(dev: *mut FhDevice, src_dev: *const c_void, bytes: usize) -> FhStatus;
+    pub fn fh_check_finite(dev: *mut FhDevice, x_dev: *const f32, count: i64, out_host: *mut FhFiniteStats) -> FhStatus;
     pub fn fh_graph_begin(dev: *mut FhDevice) -> FhStatus;
     pub fn fh_graph_end(dev: *mut FhDevice, out: *mut *mut FhGraph) -> FhStatus;
     pub fn fh_graph_launch(g: *mut FhGraph) -> FhStatus;
@@ -210,6 +223,7 @@ extern "C" {
     pub fn fh_llama_finalize(m: *mut FhLlama) -> FhStatus;
     pub fn fh_llama_reset(m: *mut FhLlama) -> FhStatus;
     pub fn fh_llama_forward(m: *mut FhLlama, tokens_host: *const u32, count: i32, logits_host: *mut f32, hidden_host: *mut f32) -> FhStatus;
+    pub fn fh_llama_trace_text(m: *const FhLlama, buf: *mut c_char, capacity: usize, length: *mut usize) -> FhStatus;
     pub fn fh_llama_decode_greedy(m: *mut FhLlama, first_token: u32, steps: i32, out_tokens_host: *mut u32, elapsed_ms: *mut f32) -> FhStatus;
     pub fn fh_llama_decode_sampled(m: *mut FhLlama, first_token: u32, steps: i32, params: *const FhSamplerParams, randoms_host: *const f32, previous_host: *const u32, n_previous: u32, repetition_range: u32, mu: *mut f32, out_tokens_host: *mut u32, elapsed_ms: *mut f32) -> FhStatus;
     pub fn fh_llama_weight_bytes(m: *const FhLlama, bytes: *mut u64) -> FhStatus;

@@ -29,6 +29,11 @@ class LlamaConfig(C.Structure):
                [(n, C.c_int32) for n in ("kv_dtype", "fuse_qkv", "fuse_gate_up", "use_graph")]
 
 
+class FiniteStats(C.Structure):
+    _fields_ = [("nan", C.c_uint64), ("pos_inf", C.c_uint64), ("neg_inf", C.c_uint64), ("max_abs", C.c_float),
+                ("first_nan_count", C.c_uint32), ("first_nan", C.c_uint64 * 4)]
+
+
 class RopeScaling(C.Structure):
     _fields_ = [("factor", C.c_float), ("high_freq_factor", C.c_float), ("low_freq_factor", C.c_float),
                 ("original_max_position_embeddings", C.c_int32)]
@@ -65,6 +70,7 @@ SIGNATURES = {
     "fh_timer_stop": [_p, C.POINTER(_f32)],
     "fh_probe_empty": [_p, _i32, _i32],
     "fh_probe_read": [_p, _p, C.c_size_t],
+    "fh_check_finite": [_p, _p, _i64, C.POINTER(FiniteStats)],
     "fh_graph_begin": [_p],
     "fh_graph_end": [_p, _pp],
     "fh_graph_launch": [_p],
@@ -118,6 +124,7 @@ SIGNATURES = {
     "fh_llama_forward": [_p, _p, _i32, _p, _p],
     "fh_llama_decode_greedy": [_p, _u32, _i32, _p, C.POINTER(_f32)],
     "fh_llama_weight_bytes": [_p, C.POINTER(_u64)],
+    "fh_llama_trace_text": [_p, C.c_char_p, _sz, C.POINTER(C.c_size_t)],
     "fh_llama_config_from_gguf": [_p, C.POINTER(LlamaConfig)],
     "fh_llama_load_gguf": [_p, _p],
     "fh_rope_tables_weighted": [_p, _i32, _i32, _f32, _p, _p, _p],

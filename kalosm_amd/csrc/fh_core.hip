@@ -3,6 +3,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 static thread_local char g_err[512] = "";
@@ -50,6 +51,11 @@ extern "C" fh_status fh_device_create(int32_t ordinal, fh_device **out) {
     FH_HIP(hipEventCreate(&d->ev_start));
     FH_HIP(hipEventCreate(&d->ev_stop));
     FH_HIP(hipMalloc(&d->small_buf, 64 * 1024));
+    // the reference's trace switches (models/kalosm-llama/src/raw/mod.rs:943-955, fusor-ml/core/src/compute_graph/
+    // resolve/run.rs:141): present in the environment = on, lines on stderr
+    if (getenv("KALOSM_TRACE_LAYER_NAN")) d->opt_trace_nan = d->opt_trace_stderr = 1;
+    if (getenv("KALOSM_TRACE_FORWARD_TIMING")) d->opt_trace_timing = d->opt_trace_stderr = 1;
+    if (getenv("FUSOR_TRACE_GPU_KERNELS")) d->opt_trace_timing = 2, d->opt_trace_stderr = 1;
     fh_status st = fh_static_scratch_init(d);
     if (st != FH_OK) {
         (void)fh_device_destroy(d);
@@ -235,6 +241,9 @@ extern "C" fh_status fh_set_option(fh_device *dev, const char *key, int64_t valu
     else if (!strcmp(key, "attn_heads")) dev->opt_attn_heads = value;
     else if (!strcmp(key, "down_tiles")) dev->opt_down_tiles = value;
     else if (!strcmp(key, "deterministic")) dev->opt_deterministic = value;
+    else if (!strcmp(key, "trace_nan")) dev->opt_trace_nan = value;
+    else if (!strcmp(key, "trace_timing")) dev->opt_trace_timing = value;
+    else if (!strcmp(key, "trace_stderr")) dev->opt_trace_stderr = value;
     else FH_FAIL(FH_ERR_INVALID, "unknown option '%s'", key);
     dev->opt_gen++;
     return FH_OK;

@@ -2,7 +2,9 @@
 // head transposes, casts, greedy argmax, KV-cache append.
 #include "fh_internal.h"
 
+#include <algorithm>
 #include <cmath>
+#include <cstring>
 #include <vector>
 
 typedef _Float16 fh_half;
@@ -960,5 +962,92 @@ extern "C" fh_status fh_kvcache_view(const fh_kvcache *c, int32_t layer, int32_t
     if (capacity) *capacity = c->capacity;
     if (k_dev) *k_dev = c->k ? (const uint8_t *)c->k + layer * plane : nullptr;
     if (v_dev) *v_dev = c->v ? (const uint8_t *)c->v + layer * plane : nullptr;
+    return FH_OK;
+}
+
+// ------------------------------------------------------------------------------ non-finite probe
+// debug_check_nan_f32, models/kalosm-llama/src/raw/mod.rs:9-58: counts of NaN / +inf / -inf, the largest finite
+// magnitude and the indices of the first four NaNs of an f32 tensor.  Workgroup g scans the g-th contiguous segment
+// (threads strided inside it, so a thread meets its indices in ascending order and its first four are its smallest);
+// the four smallest of a workgroup come out of four rounds of a 64-bit LDS minimum; the host merges the workgroups.
+struct FiniteRec {
+    uint32_t nan, pos_inf, neg_inf, max_bits;
+    uint64_t first[4];
+};
+__global__ __launch_bounds__(1024) void k_check_finite(const float *x, int64_t n, int64_t seg, FiniteRec *out) {
+    __shared__ uint32_t s_cnt[4];
+    __shared__ unsigned long long s_min;
+    const int64_t lo = (int64_t)blockIdx.x * seg, hi = min(n, lo + seg);
+    if (threadIdx.x < 4) s_cnt[threadIdx.x] = 0;
+    uint32_t c_nan = 0, c_pi = 0, c_ni = 0, mx = 0;
+    uint64_t mine[4] = {~0ull, ~0ull, ~0ull, ~0ull};
+    for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+        const uint32_t b = __float_as_uint(x[i]), a = b & 0x7FFFFFFFu;
+        if (a > 0x7F800000u) {
+            if (c_nan < 4) mine[c_nan] = (uint64_t)i;
+            c_nan++;
+        } else if (a == 0x7F800000u) {
+            if (b >> 31) c_ni++;
+            else c_pi++;
+        } else if (a > mx) {
+            mx = a; // the bit patterns of non-negative floats order like the floats
+        }
+    }
+    __syncthreads();
+    if (c_nan) atomicAdd(&s_cnt[0], c_nan);
+    if (c_pi) atomicAdd(&s_cnt[1], c_pi);
+    if (c_ni) atomicAdd(&s_cnt[2], c_ni);
+    if (mx) atomicMax(&s_cnt[3], mx);
+    uint64_t last = 0;
+    bool have_last = false;
+    for (int r = 0; r < 4; r++) {
+        if (threadIdx.x == 0) s_min = ~0ull;
+        __syncthreads();
+        uint64_t cand = ~0ull;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (mine[j] != ~0ull && (!have_last || mine[j] > last) && mine[j] < cand) cand = mine[j];
+        if (cand != ~0ull) atomicMin(&s_min, (unsigned long long)cand);
+        __syncthreads();
+        last = s_min;
+        have_last = true;
+        if (threadIdx.x == 0) out[blockIdx.x].first[r] = last;
+        __syncthreads();
+        if (last == ~0ull) {
+            if (threadIdx.x == 0)
+                for (int q = r + 1; q < 4; q++) out[blockIdx.x].first[q] = ~0ull;
+            break;
+        }
+    }
+    if (threadIdx.x == 0) {
+        out[blockIdx.x].nan = s_cnt[0];
+        out[blockIdx.x].pos_inf = s_cnt[1];
+        out[blockIdx.x].neg_inf = s_cnt[2];
+        out[blockIdx.x].max_bits = s_cnt[3];
+    }
+}
+
+extern "C" fh_status fh_check_finite(fh_device *dev, const float *x_dev, int64_t count, fh_finite_stats *out_host) {
+    FH_REQUIRE(dev && x_dev && out_host, "NULL argument");
+    FH_REQUIRE(count > 0, "count %lld out of range", (long long)count);
+    const int groups = (int)std::min<int64_t>(256, (count + 1023) / 1024);
+    const int64_t seg = (count + groups - 1) / groups;
+    FH_REQUIRE(seg < (1ll << 32), "count %lld too large", (long long)count);
+    FiniteRec *rec = (FiniteRec *)dev->small_buf; // 256 records of 48 bytes
+    k_check_finite<<<dim3(groups), dim3(1024), 0, dev->stream>>>(x_dev, count, seg, rec);
+    FH_HIP(hipGetLastError());
+    std::vector<FiniteRec> h(groups);
+    FH_TRY(fh_download(dev, h.data(), rec, sizeof(FiniteRec) * groups));
+    fh_finite_stats s = {};
+    uint32_t mx = 0;
+    for (const FiniteRec &r : h) { // segments ascend with the workgroup index, so do the indices
+        s.nan += r.nan;
+        s.pos_inf += r.pos_inf;
+        s.neg_inf += r.neg_inf;
+        mx = std::max(mx, r.max_bits);
+        for (int j = 0; j < 4 && r.first[j] != ~0ull && s.first_nan_count < 4; j++) s.first_nan[s.first_nan_count++] = r.first[j];
+    }
+    memcpy(&s.max_abs, &mx, 4);
+    *out_host = s;
     return FH_OK;
 }

@@ -76,6 +76,9 @@ struct fh_device {
     int64_t opt_wo_acc = 0;          // 0: decode steps accumulate the output projection into the residual stream, 1: never
     int64_t opt_fuse_norm = 0;       // 0: decode steps fold rms_norm into the consuming matvec, 1: separate launches
     int64_t opt_deterministic = 0;   // 1: decode steps never accumulate k-split partial sums with float atomics (run-to-run bit-equal)
+    int64_t opt_trace_nan = 0;       // 1: fh_llama_forward probes the residual stream of every layer for NaN / inf
+    int64_t opt_trace_timing = 0;    // 1: fh_llama_forward times its layer loop, 2: and every stage of every layer
+    int64_t opt_trace_stderr = 0;    // 1: trace lines go to stderr as well as into the decoder's trace text
     uint64_t opt_gen = 0;            // bumped by every fh_set_option: captured decode steps are recorded again after a change
     int64_t opt_matmul_kernel = 0;   // 0 auto, 1 generic for every m, 2 MFMA tile kernels for every m, 3 / 4 and never / always the 128 x 256 one
 };

@@ -5,6 +5,8 @@
 // (decode loop, here greedy).
 #include "fh_internal.h"
 
+#include <algorithm>
+#include <cstdarg>
 #include <cstdio>
 #include <cstring>
 #include <map>
@@ -52,7 +54,77 @@ struct fh_llama {
     int samp_capacity = -1;
     uint32_t samp_range = 0;
     fh_sampler_params samp_params = {};
+    // trace of the last fh_llama_forward (options trace_nan / trace_timing): the lines, and the stage marks
+    std::string trace_text;
+    std::vector<hipEvent_t> trace_ev;      // pool, reused from call to call
+    std::vector<std::string> trace_label;  // label of the stage that ends at mark i (marks used: trace_label.size())
+    int trace_first = -1, trace_last = -1; // the marks before the first and after the last layer
 };
+
+// Tracing of the eager forward pass, off unless an option (or the reference's environment variable, read when the
+// device is created) switches it on.  Non-finite probes: KALOSM_TRACE_LAYER_NAN, raw/mod.rs:955-1041 - the reference
+// looks at the embedding and layer 0 only (raw/mod.rs:20-22), this looks at every layer.  Timing:
+// KALOSM_TRACE_FORWARD_TIMING ("[timing] text layer loop", raw/mod.rs:943-1043) and, per stage of a layer, the
+// timestamp queries of FUSOR_TRACE_GPU_KERNELS (fusor-ml/core/src/compute_graph/resolve/run.rs:141, :483-497).
+static void trace_line(fh_llama *m, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    m->trace_text += buf;
+    m->trace_text += '\n';
+    if (m->dev->opt_trace_stderr) fprintf(stderr, "%s\n", buf);
+}
+static fh_status trace_probe(fh_llama *m, const float *t, int rows, int cols, int layer, const char *label) {
+    if (!m->dev->opt_trace_nan) return FH_OK;
+    fh_finite_stats st;
+    FH_TRY(fh_check_finite(m->dev, t, (int64_t)rows * cols, &st));
+    if (!st.nan && !st.pos_inf && !st.neg_inf) return FH_OK;
+    char idx[128];
+    int o = 0;
+    idx[0] = 0;
+    for (uint32_t i = 0; i < st.first_nan_count; i++)
+        o += snprintf(idx + o, sizeof idx - o, "%s%llu", i ? ", " : "", (unsigned long long)st.first_nan[i]);
+    trace_line(m, "trace_nan layer=%d label=%s index_pos=%d shape=[1, %d, %d] nan=%llu (first_nan_indices=[%s]) +inf=%llu "
+                  "-inf=%llu max_abs=%g",
+               layer, label, m->pos, rows, cols, (unsigned long long)st.nan, idx, (unsigned long long)st.pos_inf,
+               (unsigned long long)st.neg_inf, (double)st.max_abs);
+    return FH_OK;
+}
+// Ends a stage: an event on the stream, labelled with what ran since the previous mark.  level: 1 marks belong to the
+// layer-loop total, 2 to the per-stage trace.
+static fh_status trace_mark(fh_llama *m, int level, int layer, const char *label) {
+    if (m->dev->opt_trace_timing < level) return FH_OK;
+    const size_t i = m->trace_label.size();
+    if (i == m->trace_ev.size()) {
+        hipEvent_t e;
+        FH_HIP(hipEventCreate(&e));
+        m->trace_ev.push_back(e);
+    }
+    FH_HIP(hipEventRecord(m->trace_ev[i], m->dev->stream));
+    char buf[96];
+    if (layer >= 0) snprintf(buf, sizeof buf, "layer %d %s", layer, label);
+    else snprintf(buf, sizeof buf, "%s", label);
+    m->trace_label.push_back(buf);
+    return FH_OK;
+}
+// After the stream has been synchronised: one line per stage, then the total of the layer loop.
+static fh_status trace_report(fh_llama *m, int s) {
+    const int n = (int)m->trace_label.size();
+    if (m->dev->opt_trace_timing >= 2)
+        for (int i = 1; i < n; i++) {
+            float ms = 0;
+            FH_HIP(hipEventElapsedTime(&ms, m->trace_ev[i - 1], m->trace_ev[i]));
+            trace_line(m, "[timing] %s: %.1f us", m->trace_label[i].c_str(), ms * 1e3);
+        }
+    if (m->trace_first >= 0 && m->trace_last > m->trace_first) {
+        float ms = 0;
+        FH_HIP(hipEventElapsedTime(&ms, m->trace_ev[m->trace_first], m->trace_ev[m->trace_last]));
+        trace_line(m, "[timing] text layer loop: %.2f ms seq_len=%d", ms, s);
+    }
+    return FH_OK;
+}
 
 static void free_dev(void *p) {
     if (p) (void)hipFree(p);
@@ -118,6 +190,7 @@ extern "C" fh_status fh_llama_destroy(fh_llama *m) {
     if (m->samp_graph) (void)hipGraphDestroy(m->samp_graph);
     free_steps(m);
     fh_kvcache_destroy(m->cache);
+    for (hipEvent_t e : m->trace_ev) (void)hipEventDestroy(e);
     delete m;
     return FH_OK;
 }
@@ -276,6 +349,12 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
     const int pos = m->pos;
     const float scale = (float)(1.0 / sqrt((double)hd)); // attention_layer.rs:674
     FH_TRY(fh_embed_rows(m->embd, m->ids, nullptr, s, m->x));
+    const bool trace = !dev_pos && (dev->opt_trace_nan || dev->opt_trace_timing); // never inside a captured step
+    if (trace) {
+        FH_TRY(trace_probe(m, m->x, s, D, -1, "embed"));
+        FH_TRY(trace_mark(m, 1, -1, "embed"));
+        m->trace_first = (int)m->trace_label.size() - 1;
+    }
     for (int li = 0; li < c.n_layers; li++) {
         fh_llama_layer &l = m->layers[li];
         // Decode steps fold each rms_norm into the matvec that consumes it (one launch instead of two).
@@ -310,6 +389,10 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
             qp = qb; kp = kb2; vp = vb;
         }
         const int64_t q_st = row ? row : QD, k_st = row ? row : KD;
+        if (trace) {
+            FH_TRY(trace_probe(m, m->xn, s, D, li, "post_attn_norm"));
+            FH_TRY(trace_mark(m, 2, li, "attn_norm+qkv"));
+        }
         if (dev_pos) {
             if (!rope_done) FH_TRY(fh_rope_kv_decode(m->cache, li, qp, kp, vp, H, m->cos_t, m->sin_t, c.ctx, m->qrot));
             size_t plane = (size_t)HK * m->cache->capacity * hd * fh_dtype_size(c.kv_dtype);
@@ -350,12 +433,17 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
                                          (int64_t)m->cache->capacity * hd, hd, 1, H, HK, s, pos + s, hd, scale,
                                          s > 1 ? FH_MASK_CAUSAL : FH_MASK_NONE, nullptr, m->att));
         }
+        if (trace) FH_TRY(trace_mark(m, 2, li, "rope+cache+attention"));
         const float *att_in = m->att; // [H, s, hd]; for s == 1 this already is [s, H*hd]
         if (s > 1) {
             FH_TRY(fh_transpose_shd(dev, m->att, H, s, hd, m->att_t));
             att_in = m->att_t;
         }
         if (!wo_done) FH_TRY(fh_qmatmul(l.wo, att_in, s, m->attn_out));
+        if (trace) {
+            FH_TRY(trace_probe(m, m->attn_out, s, D, li, "attn_out"));
+            FH_TRY(trace_mark(m, 2, li, "wo"));
+        }
         // input of the FFN norm: attn + residual, or the residual stream alone when it already holds the sum
         const float *hin = xacc ? m->x : m->attn_out, *hres = xacc ? nullptr : m->x, *hadd = xacc ? nullptr : m->attn_out;
         bool ffn_done = false, late_swiglu = false;
@@ -386,6 +474,7 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
             FH_TRY(fh_qmatmul(l.up, m->xn, s, m->gu + (size_t)s * F));
             FH_TRY(fh_swiglu(dev, m->gu, m->gu + (size_t)s * F, m->act, (int64_t)s * F));
         }
+        if (trace) FH_TRY(trace_mark(m, 2, li, "ffn_norm+gate_up+swiglu"));
         if (s == 1) { // forward_add_residuals, attention_layer.rs:147-174: (down(act) + attn) + residual
             fh_status st = FH_ERR_UNSUPPORTED;
             if (late_swiglu) { // x += down(silu(gate) * up) + attn
@@ -405,9 +494,18 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
             FH_TRY(fh_qmatmul(l.down, m->act, s, m->ff));
             FH_TRY(fh_add3(dev, m->ff, m->attn_out, m->x, m->x, (int64_t)s * D));
         }
+        if (trace) {
+            FH_TRY(trace_probe(m, m->x, s, D, li, s == 1 ? "ffn_fused" : "ffn_unfused"));
+            FH_TRY(trace_mark(m, 2, li, "down+residuals"));
+        }
+    }
+    if (trace) {
+        if (dev->opt_trace_timing == 1) FH_TRY(trace_mark(m, 1, -1, "layers"));
+        m->trace_last = (int)m->trace_label.size() - 1;
     }
     FH_TRY(fh_rms_norm(dev, m->x + (size_t)(s - 1) * D, nullptr, m->out_norm, nullptr, c.eps, 1, D, m->xn));
     FH_TRY(fh_qmatmul(m->output, m->xn, 1, m->logits));
+    if (trace) FH_TRY(trace_mark(m, 2, -1, "out_norm+lm_head"));
     return FH_OK;
 }
 
@@ -421,6 +519,9 @@ extern "C" fh_status fh_llama_forward(fh_llama *m, const uint32_t *tokens_host, 
                    m->c.vocab);
     FH_TRY(ensure_steps(m, count));
     FH_TRY(fh_upload(m->dev, m->ids, tokens_host, (size_t)count * 4));
+    m->trace_text.clear();
+    m->trace_label.clear();
+    m->trace_first = m->trace_last = -1;
     FH_TRY(run_layers(m, count, false));
     // all layers appended: advance the cache
     m->pos += count;
@@ -429,6 +530,18 @@ extern "C" fh_status fh_llama_forward(fh_llama *m, const uint32_t *tokens_host, 
     if (hidden_host) FH_TRY(fh_download(m->dev, hidden_host, m->xn, (size_t)m->c.d_model * 4));
     if (logits_host) FH_TRY(fh_download(m->dev, logits_host, m->logits, (size_t)m->c.vocab * 4));
     FH_TRY(fh_device_sync(m->dev));
+    if (m->dev->opt_trace_timing) FH_TRY(trace_report(m, count));
+    return FH_OK;
+}
+
+extern "C" fh_status fh_llama_trace_text(const fh_llama *m, char *buf, size_t capacity, size_t *length) {
+    FH_REQUIRE(m && (buf || capacity == 0), "NULL argument");
+    if (length) *length = m->trace_text.size();
+    if (capacity) {
+        const size_t n = std::min(capacity - 1, m->trace_text.size());
+        memcpy(buf, m->trace_text.data(), n);
+        buf[n] = 0;
+    }
     return FH_OK;
 }
 

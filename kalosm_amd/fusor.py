@@ -413,6 +413,16 @@ class Tensor:
         """Tensor::sample_mirostat2_token (fusor-ml/core/src/sampling/pipeline.rs); updates `sampler`'s mu."""
         return self._sample(params, previous_tokens, sampler.state.ptr, previous_gpu_token, want_candidates)
 
+    def check_finite(self) -> dict:
+        """debug_check_nan_f32 (models/kalosm-llama/src/raw/mod.rs:9-58): counts of NaN / +inf / -inf, the largest
+        finite magnitude and the flat indices of the first (up to four) NaNs of an f32 tensor."""
+        assert self.dtype == "f32"
+        st = _lib.FiniteStats()
+        check(self.device._lib.fh_check_finite(self.device._h, C.c_void_p(self.ptr), int(np.prod(self.shape)),
+                                               C.byref(st)))
+        return dict(nan=st.nan, pos_inf=st.pos_inf, neg_inf=st.neg_inf, max_abs=st.max_abs,
+                    first_nan_indices=list(st.first_nan[:st.first_nan_count]))
+
     def top_k_pairs_1(self) -> int:
         """Tensor::top_k_pairs(1) (fusor-ml/fusor/src/lib.rs:416-447): the greedy token id, or -1."""
         out = Tensor(self.device, (1,), "u32")

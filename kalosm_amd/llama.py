@@ -118,6 +118,15 @@ class Model:
             C.byref(mu_c), out.ctypes.data_as(C.c_void_p), C.byref(ms)))
         return out, ms.value, mu_c.value
 
+    def trace_text(self) -> str:
+        """Lines traced by the last `forward` (device options trace_nan / trace_timing, or the reference's
+        KALOSM_TRACE_LAYER_NAN / KALOSM_TRACE_FORWARD_TIMING / FUSOR_TRACE_GPU_KERNELS in the environment)."""
+        n = C.c_size_t()
+        check(self.device._lib.fh_llama_trace_text(self._h, None, 0, C.byref(n)))
+        buf = C.create_string_buffer(n.value + 1)
+        check(self.device._lib.fh_llama_trace_text(self._h, buf, n.value + 1, None))
+        return buf.value.decode()
+
     def weight_bytes(self) -> int:
         b = C.c_uint64()
         check(self.device._lib.fh_llama_weight_bytes(self._h, C.byref(b)))

@@ -89,7 +89,7 @@ C_TO_RUST = {"int32_t": "i32", "int64_t": "i64", "uint8_t": "u8", "uint16_t": "u
              "fh_status": "FhStatus", "fh_device": "FhDevice", "fh_qmatrix": "FhQMatrix", "fh_kvcache": "FhKvCache",
              "fh_llama": "FhLlama", "fh_graph": "FhGraph", "fh_gguf": "FhGguf", "fh_llama_config": "FhLlamaConfig",
              "fh_rope_scaling": "FhRopeScaling", "fh_sampler_params": "FhSamplerParams",
-             "fh_gguf_tensor": "FhGgufTensor"}
+             "fh_gguf_tensor": "FhGgufTensor", "fh_finite_stats": "FhFiniteStats"}
 
 
 def c_param_to_rust(param: str) -> str:

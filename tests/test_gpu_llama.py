@@ -386,3 +386,99 @@ def test_deterministic_option_gives_identical_bits(dev, oracle):
     toks, lg = run()                       # default kernels again: same tokens, logits within tolerance
     assert toks == want
     assert_close(lg, runs[0][1], what="default step against the deterministic one")
+
+
+def test_forward_trace_reports_timing_and_non_finite_layers(dev):
+    """The trace switches of the reference's forward (KALOSM_TRACE_FORWARD_TIMING / FUSOR_TRACE_GPU_KERNELS /
+    KALOSM_TRACE_LAYER_NAN, models/kalosm-llama/src/raw/mod.rs:943-1043) as device options: per-stage and layer-loop
+    timing lines, no NaN line for a healthy model, and - with one NaN planted in layer 1's attention norm weight -
+    NaN lines from layer 1 on, with the counts and first indices that weight implies."""
+    cfg = SMALL
+    D, L = cfg["d_model"], cfg["n_layers"]
+    prompt = np.random.default_rng(5).integers(0, cfg["vocab"], 9)
+
+    def build(poison):
+        m = Model(dev, cfg, use_graph=False)
+        for name, ty, n, k in synth.llama_tensor_specs(cfg):
+            data = synth.llama_random_tensor(name, ty, n, k, 0, 2e-4)
+            if poison and name == "blk.1.attn_norm.weight":
+                data = data.copy()
+                data.view(np.float32)[3] = np.nan
+            m.load_tensor(name, ty, n, k, data)
+        m.finalize()
+        return m
+
+    try:
+        m = build(False)
+        m.forward(prompt)
+        assert m.trace_text() == ""  # everything off: nothing recorded
+        dev.set_option("trace_nan", 1)
+        dev.set_option("trace_timing", 2)
+        lg = m.forward([1, 2, 3])
+        lines = m.trace_text().splitlines()
+        assert not [l for l in lines if l.startswith("trace_nan")]
+        stage = [l for l in lines if l.startswith("[timing] layer ")]
+        assert len(stage) == 5 * L and stage[0].startswith("[timing] layer 0 attn_norm+qkv: ")
+        assert sum(l.startswith("[timing] out_norm+lm_head: ") for l in lines) == 1
+        total = [l for l in lines if l.startswith("[timing] text layer loop: ")]
+        assert len(total) == 1 and total[0].endswith("seq_len=3")
+        loop_ms = float(total[0].split(": ")[1].split(" ms")[0])
+        stage_us = sum(float(l.rsplit(": ", 1)[1].split(" us")[0]) for l in stage)
+        assert loop_ms > 0 and abs(stage_us / 1e3 - loop_ms) < 1e-3 * max(1.0, loop_ms) + 0.01  # stages tile the loop
+        # tracing does not change the result
+        dev.set_option("trace_nan", 0)
+        dev.set_option("trace_timing", 0)
+        m.reset()
+        m.forward(prompt)
+        assert np.array_equal(m.forward([1, 2, 3]), lg)
+        # layer-loop total only
+        dev.set_option("trace_timing", 1)
+        m.forward([4])
+        assert [l.split(":")[0] for l in m.trace_text().splitlines()] == ["[timing] text layer loop"]
+        dev.set_option("trace_timing", 0)
+
+        bad = build(True)
+        dev.set_option("trace_nan", 1)
+        out = bad.forward(prompt)
+        assert np.isnan(out).all()
+        lines = [l for l in bad.trace_text().splitlines() if l.startswith("trace_nan")]
+        assert lines and all(" layer=1 " in l for l in lines)  # the embedding and layer 0 are clean
+        s = prompt.size
+        first = lines[0]
+        assert first.startswith(f"trace_nan layer=1 label=post_attn_norm index_pos=0 shape=[1, {s}, {D}] nan={s} ")
+        assert f"first_nan_indices=[3, {3 + D}, {3 + 2 * D}, {3 + 3 * D}]" in first and "+inf=0 -inf=0" in first
+        labels = [l.split("label=")[1].split(" ")[0] for l in lines]
+        assert labels == ["post_attn_norm", "attn_out", "ffn_unfused"]
+        assert f"nan={s * D} " in lines[1] and f"nan={s * D} " in lines[2]  # a NaN input poisons every output
+        # single-token steps take the fused residual form
+        bad.forward([7])
+        assert [l.split("label=")[1].split(" ")[0] for l in bad.trace_text().splitlines()][-1] == "ffn_fused"
+    finally:
+        for key in ("trace_nan", "trace_timing", "trace_stderr"):
+            dev.set_option(key, 0)
+
+
+def test_trace_switches_from_the_environment():
+    """The reference's variables, present in the environment when the device is created, switch the trace on and send
+    its lines to stderr (raw/mod.rs:943-955; fusor-ml/core/src/compute_graph/resolve/run.rs:141)."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import numpy as np\n"
+        "from kalosm_amd.fusor import Device\n"
+        "from kalosm_amd.llama import Model\n"
+        f"cfg = {SMALL!r}\n"
+        "m = Model.random_init(Device.gpu(0), cfg, seed=0, sigma=2e-4, use_graph=False)\n"
+        "m.forward([1, 2, 3, 4])\n"
+        "print('TEXT', len(m.trace_text().splitlines()))\n")
+    env = dict(os.environ, PYTHONPATH=root, FUSOR_TRACE_GPU_KERNELS="1", KALOSM_TRACE_LAYER_NAN="1")
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stderr[-2000:]
+    err = [l for l in r.stderr.splitlines() if l.startswith("[timing]") or l.startswith("trace_nan")]
+    assert len(err) == 5 * SMALL["n_layers"] + 2 and err[-1].startswith("[timing] text layer loop: ")
+    assert f"TEXT {len(err)}" in r.stdout
+    env = {k: v for k, v in env.items() if k not in ("FUSOR_TRACE_GPU_KERNELS", "KALOSM_TRACE_LAYER_NAN")}
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0 and "TEXT 0" in r.stdout and "[timing]" not in r.stderr

@@ -508,3 +508,29 @@ def test_sample_token_previous_gpu_token(dev, oracle):
     seen = dict(zip(ids.tolist(), vals.tolist()))
     assert seen[int(order[1])] == x[order[1]]                       # outside the window: not penalised
     assert seen.get(int(order[0]), None) != x[order[0]]             # the device-side id is penalised
+
+
+@pytest.mark.parametrize("n", [1, 1000, 70001, 3_000_000])
+def test_check_finite_counts_and_first_indices(dev, n):
+    """debug_check_nan_f32 (models/kalosm-llama/src/raw/mod.rs:9-58): counts, largest finite magnitude and the first
+    four NaN indices, against numpy; clean tensors, NaNs in several scan segments, fewer than four NaNs."""
+    from kalosm_amd.fusor import Tensor
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(np.float32)
+    for variant in range(4):
+        a = x.copy()
+        if variant >= 1:
+            a[rng.integers(0, n, min(n, 3))] = np.inf
+            a[rng.integers(0, n, min(n, 2))] = -np.inf
+        if variant == 2:
+            a[rng.integers(0, n, min(n, 2))] = np.nan  # at most two NaNs
+        if variant == 3:
+            a[rng.integers(0, n, min(n, 50))] = np.nan
+            a[n - 1] = np.float32(np.nan)
+        got = Tensor.from_slice(dev, a).check_finite()
+        nan_idx = np.flatnonzero(np.isnan(a))
+        fin = a[np.isfinite(a)]
+        assert got["nan"] == nan_idx.size
+        assert got["pos_inf"] == int(np.sum(a == np.inf)) and got["neg_inf"] == int(np.sum(a == -np.inf))
+        assert got["max_abs"] == (np.abs(fin).max() if fin.size else 0.0)
+        assert got["first_nan_indices"] == nan_idx[:4].tolist()
