@@ -19,6 +19,8 @@
 // order and the epilogue is applied at the store.
 #include "fh_blocks.h"
 
+#include <type_traits>
+
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
@@ -541,24 +543,24 @@ __global__ __launch_bounds__(1024) void k_qmv_direct(QView q, const uint8_t *__r
             w[tp].load(q, to + (int64_t)(tp / TOUT) * (nout / 16), c, lane);
         }
         __builtin_amdgcn_sched_barrier(0);
-        float tot[TPW][4], off[TPW][4];
+        // each half of the chunk goes into the tile's output as soon as it is multiplied: the scaled sums and
+        // offsets live for one half of one tile only
+        const float4 fv = *(const float4 *)((const float *)(img + QdImg<T>::F_OFF) + 4 * g);
+        auto half = [&](auto H) {
 #pragma unroll
-        for (int tp = 0; tp < TPW; tp++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) tot[tp][i] = off[tp][i] = 0.f;
-#pragma unroll
-        for (int tp = 0; tp < TPW; tp++) qb_steps<T, 16, 0, 4>(w[tp], a, tot[tp], off[tp]);
+            for (int tp = 0; tp < TPW; tp++) {
+                float tot[4] = {0.f, 0.f, 0.f, 0.f}, off[4] = {0.f, 0.f, 0.f, 0.f};
+                qb_steps<T, 16, 4 * decltype(H)::value, 4 * decltype(H)::value + 4>(w[tp], a, tot, off);
+                yacc[tp][0] += fv.x * tot[0] - off[0];
+                yacc[tp][1] += fv.y * tot[1] - off[1];
+                yacc[tp][2] += fv.z * tot[2] - off[2];
+                yacc[tp][3] += fv.w * tot[3] - off[3];
+            }
+        };
+        half(std::integral_constant<int, 0>{});
         __builtin_amdgcn_sched_barrier(0);
         a.template load<1>(img, lane);
-        const float4 fv = *(const float4 *)((const float *)(img + QdImg<T>::F_OFF) + 4 * g);
-#pragma unroll
-        for (int tp = 0; tp < TPW; tp++) {
-            qb_steps<T, 16, 4, 8>(w[tp], a, tot[tp], off[tp]);
-            yacc[tp][0] = fv.x * tot[tp][0] - off[tp][0];
-            yacc[tp][1] = fv.y * tot[tp][1] - off[tp][1];
-            yacc[tp][2] = fv.z * tot[tp][2] - off[tp][2];
-            yacc[tp][3] = fv.w * tot[tp][3] - off[tp][3];
-        }
+        half(std::integral_constant<int, 1>{});
     }
 #pragma unroll
     for (int tp = 0; tp < TPW; tp++)
@@ -620,8 +622,11 @@ static fh_status qd_launch(const fh_qmatrix *q, const float *x, int m, float *y,
     const int64_t nout = EPI == FH_EPI_SWIGLU ? q->n / 2 : q->n, tiles = (nout + 15) / 16;
     // two tiles per wavefront share the activation operands once the device is covered more than twice
     const int64_t force = dev->opt_matvec_tiles;
-    const bool two = EPI == FH_EPI_SWIGLU || force == 2 || (force == 0 && tiles * parts > 2 * (int64_t)dev->compute_units);
-    const int64_t groups = EPI == FH_EPI_SWIGLU ? tiles : (two ? (tiles + 1) / 2 : tiles);
+    // and four once that still leaves a workgroup for most compute units (every workgroup fetches the image of its
+    // chunks), for the formats whose four tiles fit the 128 registers of a 16-wavefront workgroup
+    const bool four = EPI != FH_EPI_SWIGLU && (T == FH_Q4_K || T == FH_Q4_0) && (force == 4 || (force == 0 && 2 * tiles * parts >= 7 * (int64_t)dev->compute_units));
+    const bool two = !four && (EPI == FH_EPI_SWIGLU || force == 2 || (force == 0 && tiles * parts > 2 * (int64_t)dev->compute_units));
+    const int64_t groups = EPI == FH_EPI_SWIGLU ? tiles : (four ? (tiles + 3) / 4 : two ? (tiles + 1) / 2 : tiles);
     FH_REQUIRE(groups <= 0x7FFFFFFF, "matrix too large for one launch");
     FH_TRY(fh_dev_scratch(dev, &dev->act_buf, &dev->act_cap, (size_t)C * IMG));
     float *part = nullptr;
@@ -632,8 +637,16 @@ static fh_status qd_launch(const fh_qmatrix *q, const float *x, int m, float *y,
     k_qb_prep<T, 16, true><<<dim3((unsigned)C, (unsigned)((m + 3) / 4)), dim3(256), 0, dev->stream>>>(
         x, m, q->k, (uint8_t *)dev->act_buf);
     const dim3 grid((unsigned)groups, (unsigned)parts), block(64 * cps);
-    const size_t lds = (size_t)cps * (two ? 2 : 1) * 16 * 17 * 4;
-    if (two)
+    const size_t lds = (size_t)cps * (four ? 4 : two ? 2 : 1) * 16 * 17 * 4;
+    if (four) {
+        if constexpr (EPI != FH_EPI_SWIGLU && (T == FH_Q4_K || T == FH_Q4_0)) {
+            if (lds > 64 * 1024)
+                FH_HIP(hipFuncSetAttribute((const void *)k_qmv_direct<T, 4, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)lds));
+            k_qmv_direct<T, 4, EPI><<<grid, block, lds, dev->stream>>>(fh_view(q), (const uint8_t *)dev->act_buf, m, cps, y,
+                                                                      part, a, b);
+        }
+    } else if (two)
         k_qmv_direct<T, 2, EPI><<<grid, block, lds, dev->stream>>>(fh_view(q), (const uint8_t *)dev->act_buf, m, cps, y,
                                                                   part, a, b);
     else if constexpr (EPI != FH_EPI_SWIGLU)

@@ -336,6 +336,33 @@ def test_batch_matvec_vs_checker(dev, oracle, ty, m, n, k):
 
 
 @pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("m", [3, 5, 16])
+@pytest.mark.parametrize("n,k", [(272, 2048), (37, 256), (300, 3328), (64, 14336)])
+def test_unstaged_batch_matvec_tiles_per_wavefront(dev, oracle, ty, m, n, k):
+    """The kernel that reads prepared activation images straight from memory, with one, two and four row tiles per
+    wavefront forced (four: Q4_K and Q4_0; the other formats then take one): tile groups that end inside the matrix
+    (17, 3, 19 and 4 tiles), k in one part and in four, the two-residual epilogue on the four-tile form."""
+    raw = synth.random_weight(ty, n, k, seed=160 + ty)
+    x = synth.random_activation(m, k, seed=170 + m)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    want = oracle.q_mat_mul(ty, x, raw, n)
+    a, b = synth.random_activation(m, n, seed=171), synth.random_activation(m, n, seed=172)
+    xt = Tensor.from_slice(dev, x)
+    dev.set_option("matvec_kernel", 4)
+    dev.set_option("matvec_direct", 2)  # also for fewer than five rows
+    try:
+        for tiles in (1, 2, 4):
+            dev.set_option("matvec_tiles", tiles)
+            got = xt.q_mat_mul(q, out=Tensor.filled_bytes(dev, (m, n), 0xFF)).as_slice()
+            assert_close(got, want, what=f"{NAMES[ty]} {n}x{k} m={m} tiles={tiles}")
+        got = xt.q_mat_mul_add2(q, Tensor.from_slice(dev, a), Tensor.from_slice(dev, b)).as_slice()
+        assert_close(got, oracle.add3(want, a, b), what=f"add2 {NAMES[ty]} {n}x{k} m={m} tiles=4")
+    finally:
+        for key in ("matvec_kernel", "matvec_direct", "matvec_tiles"):
+            dev.set_option(key, 0)
+
+
+@pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
 def test_batch_matvec_invariants(dev, oracle, ty):
     """One-hot rows pick single weights (tests.rs:951-995), zero rows give exact zeros (:450-476), chunks of very
     different magnitude in one row keep their own scale, ragged n (37 rows: three tiles, the last with 5 rows)."""
