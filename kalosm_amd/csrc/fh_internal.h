@@ -185,6 +185,8 @@ fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf
 // power of two for fh_qmatrix::wscale from the largest |w| of `count` f32 values on the device (blocking)
 fh_status fh_dense_wscale(fh_device *dev, const float *w_dev, int64_t count, float *wscale);
 enum { FH_EPI_NONE = 0, FH_EPI_ADD2 = 1, FH_EPI_SWIGLU = 2, FH_EPI_ROPEKV = 3, FH_EPI_ACC = 4 };
+fh_status fh_launch_kparts_reduce(fh_device *dev, const float *part, int parts, int m, int64_t n, float *y, int epi,
+                                  const float *a, const float *b);
 fh_status fh_launch_q4k_rows(const fh_qmatrix *q, const float *x, int m, float *y, int epi, const float *a, const float *b);
 fh_status fh_launch_q4k_m1(const fh_qmatrix *q, const float *x, float *y, int epi, const float *a, const float *b);
 fh_status fh_launch_q4k_m1_norm(const fh_qmatrix *q, const float *x, const float *xres, const float *nw, float eps,

@@ -613,6 +613,18 @@ __global__ __launch_bounds__(256) void k_qd_reduce(const float *__restrict__ par
     y[at] = rr;
 }
 
+// The same sum for the k parts of another kernel: planes [parts][16][n], epilogue none / add2.
+fh_status fh_launch_kparts_reduce(fh_device *dev, const float *part, int parts, int m, int64_t n, float *y, int epi,
+                                  const float *a, const float *b) {
+    const int64_t total = (int64_t)m * n;
+    const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    if (epi == FH_EPI_ADD2) k_qd_reduce<FH_EPI_ADD2><<<grid, block, 0, dev->stream>>>(part, parts, m, n, n, y, a, b);
+    else if (epi == FH_EPI_NONE) k_qd_reduce<FH_EPI_NONE><<<grid, block, 0, dev->stream>>>(part, parts, m, n, n, y, a, b);
+    else FH_FAIL(FH_ERR_UNSUPPORTED, "epilogue %d of a k-part sum", epi);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
 template <int T, int EPI>
 static fh_status qd_launch(const fh_qmatrix *q, const float *x, int m, float *y, const float *a, const float *b) {
     fh_device *dev = q->dev;

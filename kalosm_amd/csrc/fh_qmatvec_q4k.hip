@@ -444,7 +444,8 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
             }
         } else if (MR > 1) {
             if (row < nout && mr < nsplit) {
-                const int64_t at = (int64_t)mr * nout + row;
+                // k split over gridDim.y workgroups: part p writes its own plane of 16 rows, a second launch adds them
+                const int64_t at = (int64_t)mr * nout + row + (int64_t)blockIdx.y * 16 * nout;
                 y[at] = EPI == FH_EPI_ADD2 ? (v0 + ea[at]) + eb[at] : v0;
             }
         } else if (row < nout) {
@@ -551,8 +552,36 @@ static fh_status q4k_m1_shape(int tpw, int per, const fh_qmatrix *q, const float
     return FH_ERR_UNSUPPORTED;
 }
 
+// Long k (the staged images of all rows of all of k do not fit the LDS, or more than 16 wavefronts): k in `parts`
+// workgroups of at most 16 blocks each, one block per wavefront and two row tiles per workgroup, so that two
+// workgroups fit a compute unit; every part writes its own plane and a second launch adds the planes in order and
+// applies the epilogue.
+template <int FMT, int EPI, int MR>
+static fh_status q4k_mr_parts(const fh_qmatrix *q, const float *x, int m, float *y, const float *a, const float *b) {
+    fh_device *dev = q->dev;
+    const int kb = (int)(q->k / 256);
+    int parts = 2;
+    while (parts <= 16 && (kb % parts != 0 || kb / parts > 16)) parts++;
+    if (parts > 16) return FH_ERR_UNSUPPORTED;
+    const int SW = kb / parts;
+    const size_t lds = (size_t)SW * MR * Q4K_IMG * 16 + (size_t)SW * MR * 64 + (size_t)MR * 2 * 16 * 64 + 64;
+    if (lds > 160 * 1024) return FH_ERR_UNSUPPORTED;
+    const int64_t tiles = (q->n + 15) / 16;
+    int tpw = (int)dev->opt_matvec_tiles;
+    if (tpw != 1 && tpw != 2) tpw = tiles * parts > 2 * (int64_t)dev->compute_units ? 2 : 1;
+    FH_TRY(fh_dev_scratch(dev, (void **)&dev->ksplit_buf, &dev->ksplit_cap, (size_t)parts * 16 * q->n * 4));
+    typedef void (*kern_t)(QView, const float *, float *, const float *, const float *, int, const float *, const float *,
+                           float, int, FhRopeArgs);
+    const kern_t kern = tpw == 2 ? (kern_t)k_qmv_q4k_mr<FMT, 2, 1, FH_EPI_NONE, MR> : (kern_t)k_qmv_q4k_mr<FMT, 1, 1, FH_EPI_NONE, MR>;
+    FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    kern<<<dim3((unsigned)((tiles + tpw - 1) / tpw), (unsigned)parts), dim3(64 * SW), lds, dev->stream>>>(
+        fh_view(q), x, (float *)dev->ksplit_buf, nullptr, nullptr, SW, nullptr, nullptr, 0.f, m, FhRopeArgs{});
+    FH_HIP(hipGetLastError());
+    return fh_launch_kparts_reduce(dev, (const float *)dev->ksplit_buf, parts, m, q->n, y, EPI, a, b);
+}
+
 // y[m, n] for m = 2 .. 4 activation rows of a Q4_K matrix (epilogues none / add2): the weights are unpacked once
-// for all rows.  FH_ERR_UNSUPPORTED when the staged images of all rows do not fit the LDS (the caller falls back).
+// for all rows.  Long k goes through q4k_mr_parts.
 template <int FMT, int EPI, int MR>
 static fh_status q4k_mr_go(const fh_qmatrix *q, const float *x, int m, float *y, const float *a, const float *b) {
     fh_device *dev = q->dev;
@@ -560,9 +589,9 @@ static fh_status q4k_mr_go(const fh_qmatrix *q, const float *x, int m, float *y,
     int per = 1;
     while (kb / per > 16 && per < 2 && kb % (per * 2) == 0) per *= 2;
     const int SW = kb / per;
-    if (SW > 16 || kb % per) return FH_ERR_UNSUPPORTED;
+    if (kb % per) return FH_ERR_UNSUPPORTED;
     const size_t lds = (size_t)kb * MR * Q4K_IMG * 16 + (size_t)kb * MR * 64 + (size_t)MR * 2 * 16 * 64 + 64;
-    if (lds > 160 * 1024) return FH_ERR_UNSUPPORTED;
+    if (SW > 16 || lds > 160 * 1024) return q4k_mr_parts<FMT, EPI, MR>(q, x, m, y, a, b);
     const int64_t tiles = (q->n + 15) / 16;
     // two row tiles per wavefront (one staging for both) once there are more tiles than compute units
     int tpw = (int)dev->opt_matvec_tiles;

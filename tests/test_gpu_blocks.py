@@ -111,6 +111,31 @@ def test_qmatmul_small_m_vs_checker(dev, oracle, ty, m, kernel):
 
 
 @pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("m", [2, 3, 4])
+@pytest.mark.parametrize("n,k", [(100, 14336), (272, 5120), (48, 8704)])
+def test_qmatmul_few_rows_long_k(dev, oracle, ty, m, n, k):
+    """2 .. 4 rows with k longer than one workgroup of the row kernel takes: 56 blocks in four parts of 14, 20 blocks in two
+    parts of 10 (their planes are added by a second launch), 34 blocks (no even split into parts of at most 16: another
+    kernel); ragged last tile; plain and two-residual epilogue; one and two row tiles per wavefront."""
+    raw = synth.random_weight(ty, n, k, seed=180 + ty)
+    x = synth.random_activation(m, k, seed=190 + m)
+    a, b = synth.random_activation(m, n, seed=191), synth.random_activation(m, n, seed=192)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    want = oracle.q_mat_mul(ty, x, raw, n)
+    xt = Tensor.from_slice(dev, x)
+    try:
+        for tiles in (0, 1, 2):
+            dev.set_option("matvec_tiles", tiles)
+            got = xt.q_mat_mul(q, out=Tensor.filled_bytes(dev, (m, n), 0xFF)).as_slice()
+            assert_close(got, want, what=f"{NAMES[ty]} {n}x{k} m={m} tiles={tiles}")
+            got = xt.q_mat_mul_add2(q, Tensor.from_slice(dev, a), Tensor.from_slice(dev, b),
+                                    out=Tensor.filled_bytes(dev, (m, n), 0xFF)).as_slice()
+            assert_close(got, oracle.add3(want, a, b), what=f"add2 {NAMES[ty]} {n}x{k} m={m} tiles={tiles}")
+    finally:
+        dev.set_option("matvec_tiles", 0)
+
+
+@pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
 def test_qmatmul_invariants(dev, oracle, ty):
     """one-hot (tests.rs:951-995), zero input / zero weight -> exact zero (:450-476, :997-1020), batched == unbatched."""
     n, k = 96, 1024
