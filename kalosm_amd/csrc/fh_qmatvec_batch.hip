@@ -19,6 +19,7 @@
 // order and the epilogue is applied at the store.
 #include "fh_blocks.h"
 
+#include <algorithm>
 #include <type_traits>
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -505,6 +506,19 @@ struct QdRegs {
             for (int i = 0; i < 4; i++) s[i] = *(const float4 *)(S + 16 * (4 * H + i));
         }
     }
+    // the second half from the wavefront's LDS copy: operands 8 .. 15 as 1 KB each, then the half's 64 group sums
+    __device__ __forceinline__ void load_second_half_lds(const uint8_t *limg, int lane) {
+        static_assert(T != FH_Q6_K, "layout of the two-plane formats");
+        const uint8_t *A = limg + lane * 16;
+        const float *S = (const float *)(limg + 8192) + 4 * (lane >> 4);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            a[i] = *(const half8 *)(A + (2 * i) * 1024);
+            a[4 + i] = *(const half8 *)(A + (2 * i + 1) * 1024);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) s[i] = *(const float4 *)(S + 16 * i);
+    }
     // the offsets qb_steps asks for, folded to register indices (its loops are unrolled: `off` is a constant)
     __device__ __forceinline__ half8 opnd(int off) const {
         if constexpr (T == FH_Q6_K) return a[(off / 32) & 7];
@@ -513,13 +527,16 @@ struct QdRegs {
     __device__ __forceinline__ float4 sum(int off) const { return s[(off / 16) & (NS - 1)]; }
 };
 
+#define QD_LDS_IMG 8448 // bytes of LDS per wavefront for the second half of a chunk's image: 8 operands + 64 sums
+
 template <int T, int TPW, int EPI>
 __global__ __launch_bounds__(1024) void k_qmv_direct(QView q, const uint8_t *__restrict__ ximg, int M, int cps,
                                                      float *__restrict__ y, float *__restrict__ part,
                                                      const float *__restrict__ ea, const float *__restrict__ eb) {
     constexpr int IMG = QdImg<T>::BYTES;
     constexpr int NT = EPI == FH_EPI_SWIGLU ? 2 : 1, TOUT = TPW / NT;
-    extern __shared__ float qd_o[]; // [wavefront][TPW][16 rows][17]
+    constexpr bool LDS_HALF = TPW == 4;
+    extern __shared__ float qd_o[]; // [wavefront][TPW][16 rows][17]; with LDS_HALF first [wavefront][QD_LDS_IMG bytes]
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int j = lane & 15, g = lane >> 4, SW = blockDim.x >> 6;
     const int C = (int)(q.k >> 8);
@@ -534,6 +551,7 @@ __global__ __launch_bounds__(1024) void k_qmv_direct(QView q, const uint8_t *__r
         const uint8_t *img = ximg + (size_t)c * IMG;
         QdRegs<T> a;
         a.template load<0>(img, lane);
+        const float4 fv = *(const float4 *)((const float *)(img + QdImg<T>::F_OFF) + 4 * g);
         __builtin_amdgcn_sched_barrier(0); // activations (L2) are requested ahead of the weights (HBM)
         QbW<T> w[TPW];
 #pragma unroll
@@ -543,9 +561,21 @@ __global__ __launch_bounds__(1024) void k_qmv_direct(QView q, const uint8_t *__r
             w[tp].load(q, to + (int64_t)(tp / TOUT) * (nout / 16), c, lane);
         }
         __builtin_amdgcn_sched_barrier(0);
+        // Four tiles per wavefront leave no registers for the second half of the image: it is requested now as well,
+        // into the wavefront's 8448 bytes of LDS (LDS-direct loads: lane l's 16 bytes land at base + 16 l, which is
+        // the operand layout), so that it is there when the first half has been multiplied.
+        uint8_t *limg = (uint8_t *)qd_o + wave * QD_LDS_IMG;
+        if constexpr (LDS_HALF) {
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                __builtin_amdgcn_global_load_lds((const uint32_t *)(img + (8 + i) * 1024 + lane * 16),
+                                                 (__attribute__((address_space(3))) uint32_t *)(limg + i * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const uint32_t *)(img + QdImg<T>::S_OFF) + 64 + lane,
+                                             (__attribute__((address_space(3))) uint32_t *)(limg + 8192), 4, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         // each half of the chunk goes into the tile's output as soon as it is multiplied: the scaled sums and
         // offsets live for one half of one tile only
-        const float4 fv = *(const float4 *)((const float *)(img + QdImg<T>::F_OFF) + 4 * g);
         auto half = [&](auto H) {
 #pragma unroll
             for (int tp = 0; tp < TPW; tp++) {
@@ -559,9 +589,15 @@ __global__ __launch_bounds__(1024) void k_qmv_direct(QView q, const uint8_t *__r
         };
         half(std::integral_constant<int, 0>{});
         __builtin_amdgcn_sched_barrier(0);
-        a.template load<1>(img, lane);
+        if constexpr (LDS_HALF) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            a.load_second_half_lds(limg, lane);
+        } else {
+            a.template load<1>(img, lane);
+        }
         half(std::integral_constant<int, 1>{});
     }
+    if constexpr (LDS_HALF) __syncthreads(); // the sums below reuse the image bytes of every wavefront
 #pragma unroll
     for (int tp = 0; tp < TPW; tp++)
 #pragma unroll
@@ -649,7 +685,7 @@ static fh_status qd_launch(const fh_qmatrix *q, const float *x, int m, float *y,
     k_qb_prep<T, 16, true><<<dim3((unsigned)C, (unsigned)((m + 3) / 4)), dim3(256), 0, dev->stream>>>(
         x, m, q->k, (uint8_t *)dev->act_buf);
     const dim3 grid((unsigned)groups, (unsigned)parts), block(64 * cps);
-    const size_t lds = (size_t)cps * (four ? 4 : two ? 2 : 1) * 16 * 17 * 4;
+    const size_t lds = four ? std::max((size_t)cps * 4 * 16 * 17 * 4, (size_t)cps * QD_LDS_IMG) : (size_t)cps * (two ? 2 : 1) * 16 * 17 * 4;
     if (four) {
         if constexpr (EPI != FH_EPI_SWIGLU && (T == FH_Q4_K || T == FH_Q4_0)) {
             if (lds > 64 * 1024)
