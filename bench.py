@@ -271,6 +271,45 @@ def calibration(dev, trains: int, use_graph: bool) -> dict:
         ms, _ = timed_trains(dev, train, trains, use_graph)
         us = ms * 1e3 / L
         out["read"].append({"bytes": used, "us": round(us, 3), "GBps": round(used / us / 1e3, 1)})
+    del buf
+    out["device"] = device_probes(dev)
+    return out
+
+
+def device_probes(dev) -> dict:
+    """fh_probe_device: the dense MFMA rate, LDS read throughput by wavefront count and address pattern, and L2 hits
+    next to an HBM stream inside one compute unit."""
+    from kalosm_amd.fusor import Tensor
+    from kalosm_amd._lib import check
+    import ctypes as C
+
+    res = (C.c_double * 4)()
+
+    def probe(kind, a, b, ptr=None, nbytes=0):
+        check(dev._lib.fh_probe_device(dev._h, kind, a, b, C.c_void_p(ptr) if ptr else None, nbytes, res))
+        return [res[i] for i in range(4)]
+
+    out = {"mfma_32x32x16_f16": [], "lds_read_b128": [], "l2_next_to_hbm": []}
+    for waves in (1, 2):
+        for iters in (2000, 20000, 100000):
+            r = probe(0, waves, iters)
+            out["mfma_32x32x16_f16"].append({"wavefronts_per_simd": waves, "iterations": iters, "TFLOPs": round(r[0], 1),
+                                              "us": round(r[1], 1)})
+    names = ["linear", "operand rows, no swizzle", "operand rows, row & 7", "operand rows, tile kernels' swizzle"]
+    for pattern in range(4):
+        for waves in (4, 8, 16):
+            r = probe(1, waves, pattern)
+            out["lds_read_b128"].append({"pattern": names[pattern], "wavefronts": waves,
+                                         "bytes_per_clock_per_cu": round(r[1], 1)})
+    cus = dev.info()["compute_units"] if hasattr(dev, "info") else 256
+    need = (256 << 10) + cus * 16 * (512 << 10)
+    buf = Tensor(dev, (need,), "u8")
+    dev._lib.fh_memset(dev._h, C.c_void_p(buf.ptr), 1, need)
+    modes = ["all wavefronts on the shared 256 KB", "all wavefronts streaming", "even on the shared region, odd streaming"]
+    for mode in range(3):
+        r = probe(2, mode, 0, buf.ptr, need)
+        out["l2_next_to_hbm"].append({"mode": modes[mode], "l2_bytes_per_ns_per_cu": round(r[0], 1),
+                                      "hbm_bytes_per_ns_per_cu": round(r[1], 1)})
     return out
 
 

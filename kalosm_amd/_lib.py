@@ -70,6 +70,7 @@ SIGNATURES = {
     "fh_timer_stop": [_p, C.POINTER(_f32)],
     "fh_probe_empty": [_p, _i32, _i32],
     "fh_probe_read": [_p, _p, C.c_size_t],
+    "fh_probe_device": [_p, _i32, _i32, _i32, _p, _sz, C.POINTER(C.c_double)],
     "fh_check_finite": [_p, _p, _i64, C.POINTER(FiniteStats)],
     "fh_graph_begin": [_p],
     "fh_graph_end": [_p, _pp],
