@@ -1386,11 +1386,14 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
         const int row = m0 + (tid >> 3) + i * 64;
         b_off[i] = (int64_t)(row < m ? row : m - 1) * K + b_c * 8;
     }
-    struct Slab {
+    // The weight bytes of a step (HBM or the memory-side cache) are requested two steps before they are decoded, into one
+    // of two register sets (even / odd steps); the activation pieces (L2) one step before.
+    struct WSlab {
         uint32_t a0, a1, b, sc0, sc1, d;
-        u32x4 h[4];
-    } sl;
-    auto fetch = [&](int ks) { // ks: step of this workgroup's range
+    };
+    u32x4 xh4[4];
+    auto fetch_w = [&](int ks_, WSlab &sl) { // ks: step of this workgroup's range (past the end: a repeat of the last)
+        const int ks = ks_ < ksteps ? ks_ : ksteps - 1;
         const int g = kbase + ks, t = 2 * (g & 3); // the even sub-block step; t + 1 shares its word of two-bit parts
         const uint8_t *rec = a_rec + (int64_t)(g >> 2) * 3360;
         const uint2 a = *(const uint2 *)(rec + q6k_lword_off(a_j, t, a_g));
@@ -1399,10 +1402,14 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
         sl.sc0 = rec[q6k_sc_off(a_j, 2 * t + (a_g >> 1))];
         sl.sc1 = rec[q6k_sc_off(a_j, 2 * t + 2 + (a_g >> 1))];
         sl.d = fh_ld16(rec + q6k_d_off(a_j));
-#pragma unroll
-        for (int i = 0; i < 4; i++) sl.h[i] = *(const u32x4 *)(xh + b_off[i] + g * 64);
     };
-    auto stage = [&](int ks) {
+    auto fetch_x = [&](int ks_) {
+        const int ks = ks_ < ksteps ? ks_ : ksteps - 1;
+        const int g = kbase + ks;
+#pragma unroll
+        for (int i = 0; i < 4; i++) xh4[i] = *(const u32x4 *)(xh + b_off[i] + g * 64);
+    };
+    auto stage = [&](int ks, const WSlab &sl) {
         _Float16 *buf = smem + (ks & 1) * BUF;
         const qmm_half2 k1056 = {(_Float16)1056.f, (_Float16)1056.f};
 #pragma unroll
@@ -1434,7 +1441,7 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int row = (tid >> 3) + i * 64;
-            *(u32x4 *)(buf + 2 * A_H + row * LDK + 8 * (b_c ^ sw(row))) = sl.h[i];
+            *(u32x4 *)(buf + 2 * A_H + row * LDK + 8 * (b_c ^ sw(row))) = xh4[i];
         }
         // the block's d, staged with its second step: nobody reads the previous block's any more
         if (((kbase + ks) & 3) == 1) s_d[a_row] = fh_h2f((uint16_t)sl.d); // (the four threads of a row: the same value)
@@ -1447,11 +1454,15 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f, part[a][b][r] = 0.f;
 
-    fetch(0);
-    stage(0);
-    for (int ks = 0; ks < ksteps; ks++) {
+    WSlab w0, w1;
+    fetch_w(0, w0);
+    fetch_x(0);
+    fetch_w(1, w1);
+    stage(0, w0);
+    fetch_w(2, w0);
+    auto step = [&](int ks, WSlab &wn1) { // wn1: the weights of step ks + 1
         __syncthreads(); // buffer ks & 1 is complete; the other one is no longer read
-        fetch(ks + 1 < ksteps ? ks + 1 : ks); // (no branch around the requests: past the end, a repeat)
+        fetch_x(ks + 1);
         const _Float16 *buf = smem + (ks & 1) * BUF;
 #pragma unroll
         for (int blk = 0; blk < 2; blk++) {
@@ -1490,7 +1501,12 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
                 }
             }
         }
-        if (ks + 1 < ksteps) stage(ks + 1); // (the last step has nothing to stage)
+        if (ks + 1 < ksteps) stage(ks + 1, wn1); // (the last step has nothing to stage)
+        fetch_w(ks + 3, wn1);
+    };
+    for (int ks = 0; ks < ksteps; ks += 2) { // (four steps per 256-block: an even count)
+        step(ks, w1);
+        step(ks + 1, w0);
     }
     // lane = weight row n (column of the MFMA result), register r = activation row 8 (r / 4) + 4 (lane / 32) + r % 4
 #pragma unroll
