@@ -1364,7 +1364,7 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers, then d per weight row
     float *s_d = (float *)(smem + 2 * BUF);
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, li = lane & 31;
     const int wn = wave / WM, wm = wave % WM;
     const int lin = (int)blockIdx.x, split = tiles_n > 0 && lin >= full, tile = split ? full + ((lin - full) >> 1) : lin;
     const int64_t n0 = (int64_t)(tiles_n > 0 ? tile % tiles_n : (int)blockIdx.x) * TN;
@@ -1378,20 +1378,21 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
     int64_t a_tile = (n0 >> 4) + (a_row >> 4);
     if (a_tile >= tiles16) a_tile = tiles16 - 1; // rows past the end decode a valid tile and are never stored
     const uint8_t *a_rec = q.data + a_tile * q.recs * 3360;
-    // activation duty: four 16-byte pieces per step, the eight threads of a row cover its 128 bytes
-    const int b_c = tid & 7;
+    // Activation duty: four 16-byte pieces per step, the eight threads of a row cover its 128 bytes.  The pieces go from
+    // memory straight into the LDS buffer (LDS-direct loads: lane l's 16 bytes land at base + 16 l, eight rows of 128
+    // bytes per wavefront and request), no registers and no LDS write instruction; the swizzle is applied on the memory
+    // side: the lane at position p of a row fetches piece p ^ sw(row).
     int64_t b_off[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const int row = m0 + (tid >> 3) + i * 64;
-        b_off[i] = (int64_t)(row < m ? row : m - 1) * K + b_c * 8;
+        const int rl = (tid >> 3) + i * 64, row = m0 + rl;
+        b_off[i] = (int64_t)(row < m ? row : m - 1) * K + ((tid & 7) ^ sw(rl)) * 8;
     }
     // The weight bytes of a step (HBM or the memory-side cache) are requested two steps before they are decoded, into one
     // of two register sets (even / odd steps); the activation pieces (L2) one step before.
     struct WSlab {
         uint32_t a0, a1, b, sc0, sc1, d;
     };
-    u32x4 xh4[4];
     auto fetch_w = [&](int ks_, WSlab &sl) { // ks: step of this workgroup's range (past the end: a repeat of the last)
         const int ks = ks_ < ksteps ? ks_ : ksteps - 1;
         const int g = kbase + ks, t = 2 * (g & 3); // the even sub-block step; t + 1 shares its word of two-bit parts
@@ -1403,11 +1404,14 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
         sl.sc1 = rec[q6k_sc_off(a_j, 2 * t + 2 + (a_g >> 1))];
         sl.d = fh_ld16(rec + q6k_d_off(a_j));
     };
-    auto fetch_x = [&](int ks_) {
+    auto fetch_x = [&](int ks_) { // into buffer ks & 1, which nobody reads any more
         const int ks = ks_ < ksteps ? ks_ : ksteps - 1;
         const int g = kbase + ks;
+        _Float16 *dst = smem + (ks_ & 1) * BUF + 2 * A_H + (8 * wave) * LDK;
 #pragma unroll
-        for (int i = 0; i < 4; i++) xh4[i] = *(const u32x4 *)(xh + b_off[i] + g * 64);
+        for (int i = 0; i < 4; i++)
+            __builtin_amdgcn_global_load_lds((const uint32_t *)(xh + b_off[i] + g * 64),
+                                             (__attribute__((address_space(3))) uint32_t *)(dst + i * 64 * LDK), 16, 0, 0);
     };
     auto stage = [&](int ks, const WSlab &sl) {
         _Float16 *buf = smem + (ks & 1) * BUF;
@@ -1438,11 +1442,6 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
             *(u32x4 *)(buf + a_row * LDK + 8 * ((4 * blk + a_g) ^ a_sw)) = chi;
             *(u32x4 *)(buf + A_H + a_row * LDK + 8 * ((4 * blk + a_g) ^ a_sw)) = clo;
         }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int row = (tid >> 3) + i * 64;
-            *(u32x4 *)(buf + 2 * A_H + row * LDK + 8 * (b_c ^ sw(row))) = xh4[i];
-        }
         // the block's d, staged with its second step: nobody reads the previous block's any more
         if (((kbase + ks) & 3) == 1) s_d[a_row] = fh_h2f((uint16_t)sl.d); // (the four threads of a row: the same value)
     };
@@ -1455,13 +1454,16 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f, part[a][b][r] = 0.f;
 
     WSlab w0, w1;
-    fetch_w(0, w0);
     fetch_x(0);
+    fetch_w(0, w0);
     fetch_w(1, w1);
     stage(0, w0);
     fetch_w(2, w0);
     auto step = [&](int ks, WSlab &wn1) { // wn1: the weights of step ks + 1
-        __syncthreads(); // buffer ks & 1 is complete; the other one is no longer read
+        // The activation pieces of buffer ks & 1 were requested a step ago, before the last five weight loads: all but
+        // those have to be back.  Then the barrier: buffer ks & 1 is complete; the other one is no longer read.
+        asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+        __syncthreads();
         fetch_x(ks + 1);
         const _Float16 *buf = smem + (ks & 1) * BUF;
 #pragma unroll
