@@ -867,7 +867,7 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2j(QView q, const _Float16
     constexpr int A_H = TN * LDK, B_H = TM * LDK; // halfs per plane
     constexpr int BUF = A_H + B_H + 4 * TN;       // halfs per buffer: codes, activations, 2 TN f32 scales
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // two buffers
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, li = lane & 31;
     const int wn = wave / WM, wm = wave % WM;
     const int lin = (int)blockIdx.x, split = lin >= full, tile = split ? full + ((lin - full) >> 1) : lin;
     const int64_t n0 = (int64_t)(tile % tiles_n) * TN;
@@ -885,19 +885,27 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2j(QView q, const _Float16
         if (t >= tiles16) t = tiles16 - 1; // rows past the end decode a valid tile and are never stored
         a_rec[u] = q.data + t * q.recs * (T == FH_Q8_0 ? 1088 : 1152);
     }
-    // activation duty: four 16-byte pieces per step, the eight threads of a row cover its 128 bytes
-    const int b_c = tid & 7;
+    // Activation duty: four 16-byte pieces per step, the eight threads of a row cover its 128 bytes.  The pieces go from
+    // memory straight into the LDS buffer (LDS-direct loads: lane l's 16 bytes land at base + 16 l, eight rows of 128
+    // bytes per wavefront and request), no registers and no LDS write instruction; the swizzle is applied on the memory
+    // side: the lane at position p of a row fetches piece p ^ sw(row).
     int64_t b_off[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const int row = m0 + (tid >> 3) + i * (NT / 8);
-        b_off[i] = (int64_t)(row < m ? row : m - 1) * K + b_c * 8;
+        const int rl = (tid >> 3) + i * (NT / 8), row = m0 + rl;
+        b_off[i] = (int64_t)(row < m ? row : m - 1) * K + ((tid & 7) ^ sw(rl)) * 8;
     }
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     struct Slab {
         uint32_t c0[NA], c1[NA], c2[NA], c3[NA], d[NA];
-        u32x4 h[4];
     } sl;
+    auto fetch_x = [&](int ks, int into) { // the pieces of step ks into the buffer of step `into` (nobody reads it any more)
+        _Float16 *dst = smem + (into & 1) * BUF + A_H + (8 * wave) * LDK;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            __builtin_amdgcn_global_load_lds((const uint32_t *)(xh + b_off[i] + ks * 64),
+                                             (__attribute__((address_space(3))) uint32_t *)(dst + i * (NT / 8) * LDK), 16, 0, 0);
+    };
     auto fetch = [&](int ks) {
 #pragma unroll
         for (int u = 0; u < NA; u++) {
@@ -913,8 +921,6 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2j(QView q, const _Float16
                 sl.d[u] = *(const uint32_t *)(rec + 1024 + 8 * a_j + 4 * (ks & 1));
             }
         }
-#pragma unroll
-        for (int i = 0; i < 4; i++) sl.h[i] = *(const u32x4 *)(xh + b_off[i] + ks * 64);
     };
     // two code bytes (already 0 .. 255 resp. 0 .. 15) under the high byte 0x64 are the halfs 1024 + u; minus the bias
     auto codes2 = [&](uint32_t bytes, uint32_t sel, float bias) -> uint32_t {
@@ -957,11 +963,6 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2j(QView q, const _Float16
                 }
                 sd[blk * TN + a_row[u]] = fh_h2f((uint16_t)(sl.d[u] >> (16 * blk))); // the four threads of a row: same value
             }
-        }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int row = (tid >> 3) + i * (NT / 8);
-            *(u32x4 *)(buf + A_H + row * LDK + 8 * (b_c ^ sw(row))) = sl.h[i];
         }
     };
     floatx16 acc[FN][FM];
@@ -1029,16 +1030,20 @@ __global__ __launch_bounds__(128 * WM) void k_qmm_tile2j(QView q, const _Float16
             }
         }
     };
+    fetch_x(kfirst, kfirst);
     fetch(kfirst);
     stage(kfirst);
     // (A schedule in which the second wavefront of every SIMD runs half a step behind the first - one multiplies while
     // the other decodes and stages, two barriers per step - was measured slower: 422 against 378 us at 2048 x 14336 x 4096.)
     for (int ks = kfirst; ks < ksteps; ks++) { // steps [kfirst, ksteps)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the activation pieces of buffer ks & 1 have landed
         __syncthreads(); // buffer ks & 1 is complete; the other one is no longer read
+        fetch_x(ks + 1 < ksteps ? ks + 1 : ks, ks + 1);
         fetch(ks + 1 < ksteps ? ks + 1 : ks); // (no branch in the step: past the end, a repeat)
         compute(ks);
         stage(ks + 1); // (no branch: the last step stages a repeat nobody reads)
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // no LDS-direct load outlives the workgroup's LDS
     // lane = weight row n (column of the MFMA result), register r = activation row 8 (r / 4) + 4 (lane / 32) + r % 4
 #pragma unroll
     for (int a = 0; a < FN; a++) {
@@ -1510,6 +1515,7 @@ __global__ __launch_bounds__(512) void k_qmm_tile2q(QView q, const _Float16 *__r
         step(ks, w1);
         step(ks + 1, w0);
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // no LDS-direct load outlives the workgroup's LDS
     // lane = weight row n (column of the MFMA result), register r = activation row 8 (r / 4) + 4 (lane / 32) + r % 4
 #pragma unroll
     for (int a = 0; a < FN; a++) {
