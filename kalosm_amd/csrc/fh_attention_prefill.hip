@@ -13,6 +13,8 @@
 // KS = 2 (short prompts: fewer workgroups than the device holds, and the launch lasts as long as the workgroup of the
 // last query block): eight wavefronts per query block, the second four take every other key tile with running
 // statistics of their own, and the two halves are merged through LDS at the end - half the tile steps per workgroup.
+// QW = 2 (shorter still: every workgroup of 64 query rows finds a compute unit of its own): two wavefronts per key
+// group, so a SIMD runs one wavefront's chain of a step instead of two.
 // What bounds the loop (measured per stage): the first product is matrix-core bound, the softmax vector-ALU bound
 // (both wavefronts of a SIMD are in it together) and the second product bound by the transposing LDS loads, which
 // run at half the rate of plain 16-byte loads.
@@ -83,23 +85,25 @@ __device__ __forceinline__ half8 ap_vt8(const fh_half *p, int row_stride) {
     return r;
 }
 
-template <typename TQ, typename TKV, int D, bool SPLIT = false, int HW = 1, int KS = 1>
-__global__ __launch_bounds__(256 * HW * KS) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_attn_prefill(const TQ *__restrict__ q, int64_t q_sb, int64_t q_sh, int64_t q_st,
+template <typename TQ, typename TKV, int D, bool SPLIT = false, int HW = 1, int KS = 1, int QW = 4>
+__global__ __launch_bounds__(64 * QW * HW * KS) __attribute__((amdgpu_waves_per_eu(QW == 4 ? 2 : 1, 2))) void k_attn_prefill(const TQ *__restrict__ q, int64_t q_sb, int64_t q_sh, int64_t q_st,
                                                        const TKV *__restrict__ k, const TKV *__restrict__ v,
                                                        int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int hq, int hkv,
                                                        int sq, int skv, float scale, int causal, TQ *__restrict__ out) {
     constexpr int BN = 64, KS_ = D + 8, VS = D + 16, DT = D / 32, KSTEPS = D / 16, CH = D / 8; // CH: 8-element chunks per row
     constexpr int NP = SPLIT ? 2 : 1; // operand planes: hi (, lo)
     static_assert(HW * KS <= 2 && !(SPLIT && KS == 2), "eight wavefronts at most; split operands leave no room for two tiles");
-    constexpr int NTH = 256 * HW * KS, KBUF = NP * BN * KS_, VBUF = NP * BN * VS, TILE = KBUF + VBUF; // halfs per staged tile
+    static_assert(QW == 4 || (QW == 2 && HW == 1 && KS == 2), "query blocks of 128 rows, or of 64 with two key groups");
+    constexpr int QB = 32 * QW; // query rows of a workgroup: QW wavefronts of 32
+    constexpr int NTH = 64 * QW * HW * KS, KBUF = NP * BN * KS_, VBUF = NP * BN * VS, TILE = KBUF + VBUF; // halfs per staged tile
     extern __shared__ __attribute__((aligned(16))) fh_half ap_lds[]; // [2 buffers][K planes | V planes]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
-    const int kset = KS == 2 ? wave >> 2 : 0; // which key tiles of a step this wavefront multiplies
+    const int kset = KS == 2 ? wave / QW : 0; // which key tiles of a step this wavefront multiplies
     const int h = (int)blockIdx.x * HW + (HW == 2 ? wave >> 2 : 0), bi = blockIdx.z, kh = h / (hq / hkv);
     // causal: the last query blocks see the most keys; with the block index on the slow grid axis ALL heads of the
     // longest block are dispatched first and the short blocks fill the tail
-    const int qb0 = (causal ? (int)(gridDim.y - 1 - blockIdx.y) : (int)blockIdx.y) * 128;
-    const int qi = qb0 + (wave & 3) * 32 + li; // this lane's query row (KS = 2: both groups have the same rows)
+    const int qb0 = (causal ? (int)(gridDim.y - 1 - blockIdx.y) : (int)blockIdx.y) * QB;
+    const int qi = qb0 + (wave % QW) * 32 + li; // this lane's query row (KS = 2: both groups have the same rows)
     const int off = skv - sq;                  // causal: query i sees keys 0 .. i + off
     const TKV *kb = k + bi * kv_sb + kh * kv_sh, *vb = v + bi * kv_sb + kh * kv_sh;
 
@@ -133,7 +137,7 @@ __global__ __launch_bounds__(256 * HW * KS) __attribute__((amdgpu_waves_per_eu(2
 
     int kend = skv;
     if (causal) {
-        const int last = (qb0 + 127 < sq ? qb0 + 127 : sq - 1) + off + 1;
+        const int last = (qb0 + QB - 1 < sq ? qb0 + QB - 1 : sq - 1) + off + 1;
         kend = last < skv ? last : skv;
     }
     // A KV tile waits in registers (as f16; SPLIT: as the f32 values) from one tile before it is written to LDS.
@@ -355,25 +359,26 @@ __global__ __launch_bounds__(256 * HW * KS) __attribute__((amdgpu_waves_per_eu(2
         // ---- the second group hands its statistics and output over: [value][query wavefront][lane] floats in the
         // tile buffers (the barrier that ended the last step has passed: nobody reads them any more)
         float *sm = (float *)ap_lds;
-        const int slot = (wave & 3) * 64 + lane;
+        constexpr int NQ = 64 * QW;
+        const int slot = (wave % QW) * 64 + lane;
         if (kset == 1) {
             sm[slot] = m_run;
-            sm[256 + slot] = l_run;
+            sm[NQ + slot] = l_run;
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) sm[(2 + dt * 16 + r) * 256 + slot] = acc[dt][r];
+                for (int r = 0; r < 16; r++) sm[(2 + dt * 16 + r) * NQ + slot] = acc[dt][r];
         }
         __syncthreads();
         if (kset == 1) return;
-        const float m1 = sm[slot], l1 = sm[256 + slot];
+        const float m1 = sm[slot], l1 = sm[NQ + slot];
         const float mm = fmaxf(m_run, m1), ref = mm == -INFINITY ? 0.f : mm;
         const float f0 = __builtin_amdgcn_exp2f(m_run - ref), f1 = __builtin_amdgcn_exp2f(m1 - ref);
         l_run = l_run * f0 + l1 * f1;
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[dt][r] = acc[dt][r] * f0 + sm[(2 + dt * 16 + r) * 256 + slot] * f1;
+            for (int r = 0; r < 16; r++) acc[dt][r] = acc[dt][r] * f0 + sm[(2 + dt * 16 + r) * NQ + slot] * f1;
     }
     // ---- store: lane = query, register r of d-tile dt is d = 32 dt + 8 (r / 4) + 4 g + r % 4
     if (qi < sq) {
@@ -388,22 +393,22 @@ __global__ __launch_bounds__(256 * HW * KS) __attribute__((amdgpu_waves_per_eu(2
     }
 }
 
-template <typename TQ, typename TKV, int D, bool SPLIT, int HW, int KS = 1>
+template <typename TQ, typename TKV, int D, bool SPLIT, int HW, int KS = 1, int QW = 4>
 static fh_status ap_launch_k(fh_device *dev, const void *q, int64_t q_sb, int64_t q_sh, int64_t q_st, const void *k,
                              const void *v, int64_t kv_sb, int64_t kv_sh, int64_t kv_st, int b, int hq, int hkv, int sq,
                              int skv, float scale, int causal, void *out) {
     constexpr int LDS = 2 * KS * (SPLIT ? 2 : 1) * 64 * (D + 8 + D + 16) * 2; // two buffers of KS tiles (K and V planes), bytes
     static_assert(KS == 1 || LDS >= (2 + (D / 32) * 16) * 256 * 4, "the merge of the key groups reuses the tile buffers");
     static_assert(LDS <= 160 * 1024, "KV tiles exceed the LDS of a compute unit");
-    auto kern = k_attn_prefill<TQ, TKV, D, SPLIT, HW, KS>;
+    auto kern = k_attn_prefill<TQ, TKV, D, SPLIT, HW, KS, QW>;
     static bool raised[64] = {}; // per kernel instance and device: allow more than 64 KB of dynamic LDS
     const bool known = dev->ordinal >= 0 && dev->ordinal < 64;
     if (!known || !raised[dev->ordinal]) {
         FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
         if (known) raised[dev->ordinal] = true;
     }
-    dim3 grid((unsigned)(hq / HW), (unsigned)((sq + 127) / 128), (unsigned)b);
-    kern<<<grid, 256 * HW * KS, LDS, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k, (const TKV *)v, kv_sb,
+    dim3 grid((unsigned)(hq / HW), (unsigned)((sq + 32 * QW - 1) / (32 * QW)), (unsigned)b);
+    kern<<<grid, 64 * QW * HW * KS, LDS, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k, (const TKV *)v, kv_sb,
                                                kv_sh, kv_st, hq, hkv, sq, skv, scale, causal, (TQ *)out);
     FH_HIP(hipGetLastError());
     return FH_OK;
@@ -416,14 +421,21 @@ static fh_status ap_launch(fh_device *dev, const void *q, int64_t q_sb, int64_t 
     // Two heads of one KV group share the staged tiles when the launch still has enough workgroups without the
     // split: short prompts are bound by the longest workgroup and by how many compute units have one at all.
     const long wgs = (long)hq * ((sq + 127) / 128) * b;
-    // attn_kernel = 6 / 7 / 8 force the workgroup shape (two heads / two key groups / plain) whatever the size: tests
+    // attn_kernel = 6 / 7 / 8 / 9 force the workgroup shape (two heads / two key groups / plain / 64-row query blocks
+    // with two key groups) whatever the size: tests
     const int64_t force = dev->opt_attn_kernel;
     const bool pair = (hq / hkv) % 2 == 0 && (force == 6 || (force != 7 && force != 8 && wgs >= 1024));
 #define FH_AP(D, HW, KS) ap_launch_k<TQ, TKV, D, SPLIT, HW, KS>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, scale, causal, out)
     if constexpr (!SPLIT) {
         // short prompts: every workgroup is resident at once (two of four wavefronts per compute unit) and the launch
         // lasts as long as the last query block's - its key tiles are shared out over two groups of wavefronts
-        const bool halves = force == 7 || (force != 6 && force != 8 && wgs <= 2L * dev->compute_units && skv > 128);
+        const bool halves = force == 7 || force == 9 || (force != 6 && force != 8 && wgs <= 2L * dev->compute_units && skv > 128);
+        // shorter still: query blocks of 64 rows, four wavefronts, while one workgroup per compute unit holds (nearly) all
+        // of them - a SIMD then runs one wavefront's chain of a step instead of two (512 tokens: 15.0 against 16.8 us)
+        const long wgs64 = (long)hq * ((sq + 63) / 64) * b;
+        const bool rows64 = force == 9 || (force == 0 && halves && 4 * wgs64 <= 5L * dev->compute_units);
+        if (rows64) return d == 128 ? ap_launch_k<TQ, TKV, 128, SPLIT, 1, 2, 2>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, scale, causal, out)
+                                    : ap_launch_k<TQ, TKV, 64, SPLIT, 1, 2, 2>(dev, q, q_sb, q_sh, q_st, k, v, kv_sb, kv_sh, kv_st, b, hq, hkv, sq, skv, scale, causal, out);
         if (halves) return d == 128 ? FH_AP(128, 1, 2) : FH_AP(64, 1, 2);
     }
     if (d == 128) return pair ? FH_AP(128, 2, 1) : FH_AP(128, 1, 1);

@@ -319,13 +319,14 @@ def test_attention_prefill_f32_split(dev, oracle, sq, skv, causal, d):
     assert_close(got, rows, abs_tol=1e-3, rel_tol=1e-4, what="vs the exact row kernel")
 
 
-@pytest.mark.parametrize("force", [6, 7, 8])
+@pytest.mark.parametrize("force", [6, 7, 8, 9])
 @pytest.mark.parametrize("sq,skv,causal,d", [(300, 300, True, 128), (129, 700, True, 128), (257, 190, False, 128),
                                              (64, 65, True, 64), (384, 384, True, 64), (33, 200, True, 128)])
 def test_attention_prefill_workgroup_shapes(dev, oracle, force, sq, skv, causal, d):
-    """The three workgroup shapes of the matrix-core kernel on the same ragged inputs, whatever the dispatch would
+    """The four workgroup shapes of the matrix-core kernel on the same ragged inputs, whatever the dispatch would
     pick for the size (attn_kernel = 6: two heads of a KV group share the staged tiles; 7: the key tiles of a query
-    block shared out over two groups of wavefronts and merged; 8: four wavefronts, one head): f16 and f32 queries on an
+    block shared out over two groups of wavefronts and merged; 8: four wavefronts, one head; 9: query blocks of 64 rows,
+    two key groups of two wavefronts): f16 and f32 queries on an
     f16 cache, causal with the queries at the end of a longer cache, odd tile counts (a group without a tile in the last
     step), a single query block."""
     h, hkv = 8, 2
