@@ -58,7 +58,13 @@ struct Q4kExtra {
 // MR > 1: MR activation rows (nsplit then carries the number of valid ones; plain input, epilogues none / add2):
 // the weights are unpacked once per step and multiplied with the operand of every row; a wavefront stages its
 // blocks of all rows, images interleaved [block][row] so that every operand address is the base plus a constant.
-template <int FMT, int TPW, int PER, int EPI, int IN, int MR = 1>
+// RS > 1 (Q4_K, one row, plain input, epilogues none / add2): a workgroup owns 16 / RS rows of a tile and
+// a wavefront multiplies them over RS consecutive blocks at once: MFMA column c is row c % (16 / RS) of block
+// c / (16 / RS), A row i carries the (hi | lo) halves of sub-blocks (i >> 1) % (8 / RS) + a * (8 / RS) of block
+// i / (16 / RS) in the steps of accumulator a = 0 .. RS - 1.  The accumulator entries whose row and column name the
+// same block are the dots; the rest is discarded.  As many MFMAs per weight byte as with whole tiles, RS times the
+// workgroups: matrices with fewer row tiles than compute units fill the device in one launch.
+template <int FMT, int TPW, int PER, int EPI, int IN, int MR = 1, int RS = 1>
 __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict__ x, float *__restrict__ y,
                                                       const float *__restrict__ ea, const float *__restrict__ eb,
                                                       int SW, const float *__restrict__ xres,
@@ -66,6 +72,10 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
                                                       FhRopeArgs rk) {
     static_assert(MR == 1 || (IN == 0 && (EPI == FH_EPI_NONE || EPI == FH_EPI_ADD2)), "rows: plain input, none / add2");
     static_assert(MR == 1 || MR == 2 || MR == 4, "rows per launch");
+    static_assert(RS == 1 || (FMT == FH_Q4_K && TPW == 1 && MR == 1 && IN == 0 && (EPI == FH_EPI_NONE || EPI == FH_EPI_ADD2)),
+                  "row split: Q4_K, one tile part, one row, plain input, epilogues none / add2");
+    static_assert(RS == 1 || RS == 2 || RS == 4, "row split");
+    constexpr int NB = PER * RS; // blocks a wavefront stages and multiplies
     // SwiGLU with one tile per wavefront: the "tile" is rows 8h .. 8h+7 of a gate tile (columns 0-7 of the MFMA) and
     // the same rows of the matching up tile (columns 8-15), h = workgroup parity: workgroups half as heavy as with a
     // whole gate and a whole up tile, which divides the Llama FFN evenly over the compute units
@@ -78,7 +88,7 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     constexpr int TOUT = TPW / NT; // output tiles of the workgroup
     extern __shared__ uint4 lds[];
     // gridDim.y > 1: k is split over workgroups (blocks [boff, boff + kb) here) that add into y with atomics
-    const int kb = SW * PER, boff = (int)blockIdx.y * kb; // the host launches with SW * PER * gridDim.y == q.kb
+    const int kb = SW * NB, boff = (int)blockIdx.y * kb; // the host launches with SW * NB * gridDim.y == q.kb
     uint4 *img = lds;
     float *sf = (float *)(lds + kb * MR * Q4K_IMG); // per block and row: [0..7] group sums, [8..15] factors
     float *l_red = sf + kb * MR * 16;               // [MR][TPW][SW][16]
@@ -88,7 +98,7 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t nout = EPI == FH_EPI_SWIGLU ? q.n / 2 : q.n;
     const int64_t tiles_out = (nout + 15) / 16;
-    const int b0 = wave * PER;
+    const int b0 = wave * NB;
     constexpr int REC = FMT == FH_Q4_0 ? 1152 : (FMT == FH_Q8_0 ? 1088 : 2304); // bytes of a tiled record
     constexpr int CHUNK = FMT == FH_Q8_0 ? 4352 : 2304;                          // bytes per 256 activations and tile
     const uint8_t *ph[TPW], *pq[TPW];
@@ -108,8 +118,16 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
             pq[0] = rec + 256 + (16 * g + rr) * 16;
         }
     }
+    if constexpr (RS > 1) { // column j: row (16 / RS) * part + j % (16 / RS) of the tile, block j / (16 / RS) of the group
+        constexpr int RW = 16 / RS;
+        const int64_t tile = (int64_t)(blockIdx.x / RS);
+        const int rr = RW * (int)(blockIdx.x % RS) + j % RW;
+        const uint8_t *rec = q.data + tile * q.recs * REC + (int64_t)(boff + b0 + j / RW) * CHUNK;
+        ph[0] = rec + 16 * rr;
+        pq[0] = rec + 256 + (16 * g + rr) * 16;
+    }
 #pragma unroll
-    for (int tp = 0; tp < (HP ? 0 : TPW); tp++) {
+    for (int tp = 0; tp < ((HP || RS > 1) ? 0 : TPW); tp++) {
         const int64_t to = (int64_t)blockIdx.x * TOUT + (tp % TOUT);
         const int64_t tile = to + (int64_t)(tp / TOUT) * (nout / 16); // up tiles follow the gate tiles
         // a tile past the end re-reads the last tile (its rows are never stored)
@@ -130,15 +148,15 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     // ---- 0. the activations of this wavefront's blocks are requested first: they are needed first and are short
     // With nw the input is rms_norm(x [+ xres]) * nw (composite/normalization.rs:287-401): the weight nw is
     // folded into the staged values and the common factor 1 / rms is applied to the finished dot product.
-    float4 xv[PER * MR], rv[PER], wv[PER], pacc[IN == 2 ? PER : 1][8];
+    float4 xv[NB * MR], rv[NB], wv[NB], pacc[IN == 2 ? PER : 1][8];
     float2 pm[IN == 2 ? PER : 1][8];
 #pragma unroll
-    for (int i = 0; i < PER; i++) {
+    for (int i = 0; i < NB; i++) {
         const int64_t at = (int64_t)(boff + b0 + i) * 256 + lane * 4;
         if (IN != 2) xv[i] = *(const float4 *)(x + at);
 #pragma unroll
         for (int mr = 1; mr < MR; mr++) // rows past the valid ones repeat the last (never stored)
-            xv[mr * PER + i] = *(const float4 *)(x + (int64_t)(mr < nsplit ? mr : nsplit - 1) * q.k + at);
+            xv[mr * NB + i] = *(const float4 *)(x + (int64_t)(mr < nsplit ? mr : nsplit - 1) * q.k + at);
         if (IN == 1 && xres) rv[i] = *(const float4 *)(xres + at);
         if (IN == 1) wv[i] = *(const float4 *)(nw + at);
         if (IN == 2) { // x holds attention partials [head][nsplit][128 + 4]: unnormalised output, max, sum
@@ -172,9 +190,9 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
                 w[tp][r].qc = *(const uint4 *)(pq[tp] + r * 4352 + 2176);
                 w[tp][r].qd = *(const uint4 *)(pq[tp] + r * 4352 + 3264);
             } else {
-                w[tp][r].h = *(const uint4 *)(ph[tp] + r * 2304);
-                w[tp][r].qa = *(const uint4 *)(pq[tp] + r * 2304);
-                w[tp][r].qb = *(const uint4 *)(pq[tp] + r * 2304 + 1024);
+                w[tp][r].h = *(const uint4 *)(ph[tp] + r * RS * 2304);
+                w[tp][r].qa = *(const uint4 *)(pq[tp] + r * RS * 2304);
+                w[tp][r].qb = *(const uint4 *)(pq[tp] + r * RS * 2304 + 1024);
             }
         }
     // ---- 2. stage x (lane owns k = 256*b + 4*lane .. +3).  A wavefront stages exactly the blocks it multiplies:
@@ -182,9 +200,9 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     // around it either: the compiler would sink the activation loads into it, behind the weight loads.)
     float ss = 0.f;
 #pragma unroll
-    for (int ii = 0; ii < PER * MR; ii++) {
-        const int i = ii % PER;
-        const int b = (b0 + i) * MR + ii / PER; // image index: [block][row]
+    for (int ii = 0; ii < NB * MR; ii++) {
+        const int i = ii % NB;
+        const int b = (b0 + i) * MR + ii / NB; // image index: [block][row]
         float4 v = xv[ii];
         if (IN == 2) { // merge the splits: softmax weights exp(m_s - max), then num / den
             float mx = -INFINITY;
@@ -265,141 +283,219 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         if (lane == 0) l_ss[wave] = ss;
     }
     // ---- 3. eight chained MFMA steps per block and tile; the TPW tiles share every operand read
-    const int mysb = j >> 1, part = j & 1;
-    // per-lane operand address of each step: its own sub-block's (hi|lo) in step mysb, the zero slot otherwise.
-    // Lanes with (lane >> 1) % 8 == st are bits 2 st, 2 st + 1 of every 16.
-    uint32_t pa[8];
-    const uint32_t own = lds_addr(img + b0 * MR * Q4K_IMG + (mysb * 4 + g) * 2 + part);
-    {
-        const uint32_t zero = lds_addr(img + b0 * MR * Q4K_IMG + 64);
+    if constexpr (RS > 1) {
+        constexpr int SL = 8 / RS, RW = 16 / RS;
+        const int blk = j / RW, sloc = (j >> 1) % SL, part = j & 1;
+        // A row j: block blk of the group, local sub-block sloc; in step st it carries sub-block st when
+        // st % SL == sloc and is zero otherwise
+        const uint32_t base = lds_addr(img + (b0 + blk) * Q4K_IMG + g * 2 + part);
+        const uint32_t zero = lds_addr(img + b0 * Q4K_IMG + 64);
+        uint32_t pa[8];
 #pragma unroll
-        for (int st = 0; st < 8; st++) pa[st] = sel_lanes(0x0003000300030003ull << (2 * st), own, zero);
-    }
-    // the operands do not depend on the weights: RING of them are always on their way from the LDS
-    constexpr int RING = 4;
-    uint4 ring[RING];
-    // operand number t = (block r, step st, row mr) in the order of use; its image is (r * MR + mr) after the base
-    auto operand = [&](int t) {
-        const int mr = t % MR, st = (t / MR) % 8, r = t / (8 * MR);
-        return lds_read16(pa[st] + (r * MR + mr) * Q4K_IMG * 16);
-    };
+        for (int st = 0; st < 8; st++) {
+            const uint64_t m16 = RS == 2 ? (0x0303ull << (2 * (st & 3))) : (0x3333ull << (2 * (st & 1)));
+            pa[st] = sel_lanes(m16 * 0x0001000100010001ull, base + st * 8 * 16, zero);
+        }
+        constexpr int RING = 4;
+        uint4 ring[RING];
+        auto operand = [&](int t) { return lds_read16(pa[t % 8] + (t / 8) * RS * Q4K_IMG * 16); };
 #pragma unroll
-    for (int t = 0; t < RING; t++) ring[t] = operand(t);
-    const float *psf = sf + b0 * MR * 16 + 2 * g;
-    const uint32_t LO = 0x000F000Fu, HI = 0x00F000F0u;
-    // lane group g applies sub-blocks 2g, 2g+1: bytes (g&1)*2, +1 of the low (g < 2) or high (g >= 2) scale word
-    const uint32_t selhi = (g & 2) ? 0xFFFFFFFFu : 0u;
-    const int sh = (g & 1) * 16;
-    float acc[TPW][MR], mins[TPW][MR];
+        for (int t = 0; t < RING; t++) ring[t] = operand(t);
+        const uint32_t LO = 0x000F000Fu, HI = 0x00F000F0u;
+        // accumulator entries (rows 4 g .. 4 g + 3, column j) belong together when both name the same block
+        const bool valid = g / (4 / RS) == blk;
+        const float *psf = sf + (b0 + blk) * 16;
+        float acc = 0.f, mins = 0.f;
 #pragma unroll
-    for (int tp = 0; tp < TPW; tp++)
-#pragma unroll
-        for (int mr = 0; mr < MR; mr++) acc[tp][mr] = mins[tp][mr] = 0.f;
-#pragma unroll
-    for (int r = 0; r < PER; r++) {
-        floatx4 dd[TPW][MR];
-#pragma unroll
-        for (int tp = 0; tp < TPW; tp++)
-#pragma unroll
-            for (int mr = 0; mr < MR; mr++) dd[tp][mr] = floatx4{0.f, 0.f, 0.f, 0.f};
-        // rows 2s, 2s + 1 of dsum: the sum of the staged hi / lo values of sub-block s (the same in every
-        // column, so one product serves all tiles)
-        floatx4 dsum[ONES ? MR : 1];
-        if constexpr (ONES) {
+        for (int r = 0; r < PER; r++) {
+            floatx4 dd[RS], dsum[RS];
             const uint4 one = make_uint4(0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u); // f16 1.0
             half8 ov;
             __builtin_memcpy(&ov, &one, 16);
 #pragma unroll
-            for (int mr = 0; mr < MR; mr++) {
-                const uint4 ao = lds_read16(own + (r * MR + mr) * Q4K_IMG * 16);
+            for (int a = 0; a < RS; a++) {
+                dd[a] = floatx4{0.f, 0.f, 0.f, 0.f};
+                const uint4 ao = lds_read16(base + ((a * SL + sloc) * 8 + r * RS * Q4K_IMG) * 16);
                 half8 av;
                 __builtin_memcpy(&av, &ao, 16);
-                dsum[mr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, ov, floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-            }
-        }
-#pragma unroll
-        for (int st = 0; st < 8; st++) {
-            const int t = (r * 8 + st) * MR;
-            half8 av[MR];
-#pragma unroll
-            for (int mr = 0; mr < MR; mr++) {
-                const uint4 ao = ring[(t + mr) % RING];
-                __builtin_memcpy(&av[mr], &ao, 16);
+                dsum[a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, ov, floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
             }
 #pragma unroll
-            for (int tp = 0; tp < TPW; tp++) {
-                const uint4 wq = FMT == FH_Q8_0 ? ((st >> 1) == 0 ? w[tp][r].qa : ((st >> 1) == 1 ? w[tp][r].qb : ((st >> 1) == 2 ? w[tp][r].qc : w[tp][r].qd)))
-                                                 : ((st & 4) ? w[tp][r].qb : w[tp][r].qa);
-                uint4 bo;
-                if (FMT == FH_Q8_0) { // eight code bytes of block st -> f16 1152 + q, pairs in the order of the staging
-                    const uint32_t c0 = ((st & 1) ? wq.z : wq.x) ^ 0x80808080u, c1 = ((st & 1) ? wq.w : wq.y) ^ 0x80808080u;
-                    const uint32_t k64 = 0x64646464u;
-                    bo = make_uint4(__builtin_amdgcn_perm(k64, c0, 0x04020400u), __builtin_amdgcn_perm(k64, c0, 0x04030401u),
-                                    __builtin_amdgcn_perm(k64, c1, 0x04020400u), __builtin_amdgcn_perm(k64, c1, 0x04030401u));
-                } else if (FMT == FH_Q4_0) { // one word per block: low nibbles, then high nibbles
-                    const uint32_t w0 = (st & 3) == 0 ? wq.x : ((st & 3) == 1 ? wq.y : ((st & 3) == 2 ? wq.z : wq.w));
-                    bo = make_uint4(w0 & LO, (w0 >> 8) & LO, w0 & HI, (w0 >> 8) & HI);
-                } else {
-                    const uint32_t w0 = (st & 2) ? wq.z : wq.x, w1 = (st & 2) ? wq.w : wq.y;
-                    const uint32_t msk = (st & 1) ? HI : LO;
-                    bo = make_uint4(w0 & msk, (w0 >> 8) & msk, w1 & msk, (w1 >> 8) & msk);
-                }
-                half8 bv;
+            for (int st = 0; st < 8; st++) {
+                const int t = r * 8 + st;
+                half8 av, bv;
+                const uint4 ao = ring[t % RING];
+                __builtin_memcpy(&av, &ao, 16);
+                const uint4 wq = (st & 4) ? w[0][r].qb : w[0][r].qa;
+                const uint32_t w0 = (st & 2) ? wq.z : wq.x, w1 = (st & 2) ? wq.w : wq.y;
+                const uint32_t msk = (st & 1) ? HI : LO;
+                const uint4 bo = make_uint4(w0 & msk, (w0 >> 8) & msk, w1 & msk, (w1 >> 8) & msk);
                 __builtin_memcpy(&bv, &bo, 16);
-#pragma unroll
-                for (int mr = 0; mr < MR; mr++)
-                    dd[tp][mr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[mr], bv, dd[tp][mr], 0, 0, 0);
+                dd[st / SL] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, dd[st / SL], 0, 0, 0);
+                if (t + RING < PER * 8) ring[t % RING] = operand(t + RING);
             }
+            const uint4 h = w[0][r].h;
+            const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
+            const uint32_t sc_l = h.y & 0x3F3F3F3Fu, sc_h = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
+            const uint32_t mn_l = h.z & 0x3F3F3F3Fu, mn_h = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
 #pragma unroll
-            for (int mr = 0; mr < MR; mr++)
-                if (t + mr + RING < PER * 8 * MR) ring[(t + mr) % RING] = operand(t + mr + RING);
-        }
-#pragma unroll
-        for (int mr = 0; mr < MR; mr++) {
-            const float2 fc = *(const float2 *)(psf + (r * MR + mr) * 16 + 8);
-            float2 sx;
-            if constexpr (ONES) { // odd sub-blocks are staged 16 times lower (their codes are 16 times higher)
-                sx.x = (dsum[mr][0] + dsum[mr][1]) * (fc.x * 0x1p-24f);
-                sx.y = (dsum[mr][2] + dsum[mr][3]) * (fc.y * 0x1p-20f);
-            } else {
-                sx = *(const float2 *)(psf + (r * MR + mr) * 16);
-            }
-#pragma unroll
-            for (int tp = 0; tp < TPW; tp++) {
-                const uint4 h = w[tp][r].h;
-                if (FMT == FH_Q4_0 || FMT == FH_Q8_0) {
-                    const float off = FMT == FH_Q8_0 ? 1152.0f : 8.0f;
-                    const float da = fh_h2f((uint16_t)(h.x & 0xFFFF)), db = fh_h2f((uint16_t)(h.x >> 16));
-                    acc[tp][mr] = fmaf(dd[tp][mr][0] + dd[tp][mr][1], da * fc.x, acc[tp][mr]);
-                    acc[tp][mr] = fmaf(dd[tp][mr][2] + dd[tp][mr][3], db * fc.y, acc[tp][mr]);
-                    mins[tp][mr] = fmaf(off * da, sx.x, mins[tp][mr]);
-                    mins[tp][mr] = fmaf(off * db, sx.y, mins[tp][mr]);
-                    continue;
-                }
-                const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
-                const uint32_t sc_l = h.y & 0x3F3F3F3Fu, sc_h = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
-                const uint32_t mn_l = h.z & 0x3F3F3F3Fu, mn_h = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
-                const uint32_t scw = ((sc_l & ~selhi) | (sc_h & selhi)) >> sh;
-                const uint32_t mnw = ((mn_l & ~selhi) | (mn_h & selhi)) >> sh;
+            for (int a = 0; a < RS; a++) {
+                // rows 4 g .. 4 g + 3 of accumulator a: sub-blocks s0, s0 + 1 (hi, lo each)
+                const int s0 = a * SL + (2 * g) % SL;
+                const float2 fc = *(const float2 *)(psf + r * RS * 16 + 8 + s0);
+                const float sxa = (dsum[a][0] + dsum[a][1]) * (fc.x * 0x1p-24f);
+                const float sxb = (dsum[a][2] + dsum[a][3]) * (fc.y * 0x1p-20f);
+                const uint32_t scw = ((s0 & 4) ? sc_h : sc_l) >> ((s0 & 2) * 8);
+                const uint32_t mnw = ((s0 & 4) ? mn_h : mn_l) >> ((s0 & 2) * 8);
                 const float sca = (float)(scw & 0xFFu), scb = (float)((scw >> 8) & 0xFFu);
                 const float mna = (float)(mnw & 0xFFu), mnb = (float)((mnw >> 8) & 0xFFu);
-                const float sa = (sca * d) * fc.x, sb = (scb * d) * fc.y;
-                acc[tp][mr] = fmaf(dd[tp][mr][0] + dd[tp][mr][1], sa, acc[tp][mr]);
-                acc[tp][mr] = fmaf(dd[tp][mr][2] + dd[tp][mr][3], sb, acc[tp][mr]);
-                mins[tp][mr] = fmaf(mna * dmin, sx.x, mins[tp][mr]);
-                mins[tp][mr] = fmaf(mnb * dmin, sx.y, mins[tp][mr]);
+                acc = fmaf(dd[a][0] + dd[a][1], (sca * d) * fc.x, acc);
+                acc = fmaf(dd[a][2] + dd[a][3], (scb * d) * fc.y, acc);
+                mins = fmaf(mna * dmin, sxa, mins);
+                mins = fmaf(mnb * dmin, sxb, mins);
             }
         }
-    }
-#pragma unroll
-    for (int mr = 0; mr < MR; mr++)
-#pragma unroll
-        for (int tp = 0; tp < TPW; tp++) {
-            const float v = rows_sum(acc[tp][mr] - mins[tp][mr]);
-            if (lane < 16) l_red[((mr * TPW + tp) * SW + wave) * 16 + lane] = v;
+        float v = rows_sum(valid ? acc - mins : 0.f);
+        v += __shfl_xor(v, 8, 64); // the blocks of a row sit RW columns apart
+        if (RS == 4) v += __shfl_xor(v, 4, 64);
+        if (lane < RW) l_red[wave * 16 + lane] = v;
+    } else {
+        const int mysb = j >> 1, part = j & 1;
+        // per-lane operand address of each step: its own sub-block's (hi|lo) in step mysb, the zero slot otherwise.
+        // Lanes with (lane >> 1) % 8 == st are bits 2 st, 2 st + 1 of every 16.
+        uint32_t pa[8];
+        const uint32_t own = lds_addr(img + b0 * MR * Q4K_IMG + (mysb * 4 + g) * 2 + part);
+        {
+            const uint32_t zero = lds_addr(img + b0 * MR * Q4K_IMG + 64);
+    #pragma unroll
+            for (int st = 0; st < 8; st++) pa[st] = sel_lanes(0x0003000300030003ull << (2 * st), own, zero);
         }
+        // the operands do not depend on the weights: RING of them are always on their way from the LDS
+        constexpr int RING = 4;
+        uint4 ring[RING];
+        // operand number t = (block r, step st, row mr) in the order of use; its image is (r * MR + mr) after the base
+        auto operand = [&](int t) {
+            const int mr = t % MR, st = (t / MR) % 8, r = t / (8 * MR);
+            return lds_read16(pa[st] + (r * MR + mr) * Q4K_IMG * 16);
+        };
+    #pragma unroll
+        for (int t = 0; t < RING; t++) ring[t] = operand(t);
+        const float *psf = sf + b0 * MR * 16 + 2 * g;
+        const uint32_t LO = 0x000F000Fu, HI = 0x00F000F0u;
+        // lane group g applies sub-blocks 2g, 2g+1: bytes (g&1)*2, +1 of the low (g < 2) or high (g >= 2) scale word
+        const uint32_t selhi = (g & 2) ? 0xFFFFFFFFu : 0u;
+        const int sh = (g & 1) * 16;
+        float acc[TPW][MR], mins[TPW][MR];
+    #pragma unroll
+        for (int tp = 0; tp < TPW; tp++)
+    #pragma unroll
+            for (int mr = 0; mr < MR; mr++) acc[tp][mr] = mins[tp][mr] = 0.f;
+    #pragma unroll
+        for (int r = 0; r < PER; r++) {
+            floatx4 dd[TPW][MR];
+    #pragma unroll
+            for (int tp = 0; tp < TPW; tp++)
+    #pragma unroll
+                for (int mr = 0; mr < MR; mr++) dd[tp][mr] = floatx4{0.f, 0.f, 0.f, 0.f};
+            // rows 2s, 2s + 1 of dsum: the sum of the staged hi / lo values of sub-block s (the same in every
+            // column, so one product serves all tiles)
+            floatx4 dsum[ONES ? MR : 1];
+            if constexpr (ONES) {
+                const uint4 one = make_uint4(0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u); // f16 1.0
+                half8 ov;
+                __builtin_memcpy(&ov, &one, 16);
+    #pragma unroll
+                for (int mr = 0; mr < MR; mr++) {
+                    const uint4 ao = lds_read16(own + (r * MR + mr) * Q4K_IMG * 16);
+                    half8 av;
+                    __builtin_memcpy(&av, &ao, 16);
+                    dsum[mr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, ov, floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                }
+            }
+    #pragma unroll
+            for (int st = 0; st < 8; st++) {
+                const int t = (r * 8 + st) * MR;
+                half8 av[MR];
+    #pragma unroll
+                for (int mr = 0; mr < MR; mr++) {
+                    const uint4 ao = ring[(t + mr) % RING];
+                    __builtin_memcpy(&av[mr], &ao, 16);
+                }
+    #pragma unroll
+                for (int tp = 0; tp < TPW; tp++) {
+                    const uint4 wq = FMT == FH_Q8_0 ? ((st >> 1) == 0 ? w[tp][r].qa : ((st >> 1) == 1 ? w[tp][r].qb : ((st >> 1) == 2 ? w[tp][r].qc : w[tp][r].qd)))
+                                                     : ((st & 4) ? w[tp][r].qb : w[tp][r].qa);
+                    uint4 bo;
+                    if (FMT == FH_Q8_0) { // eight code bytes of block st -> f16 1152 + q, pairs in the order of the staging
+                        const uint32_t c0 = ((st & 1) ? wq.z : wq.x) ^ 0x80808080u, c1 = ((st & 1) ? wq.w : wq.y) ^ 0x80808080u;
+                        const uint32_t k64 = 0x64646464u;
+                        bo = make_uint4(__builtin_amdgcn_perm(k64, c0, 0x04020400u), __builtin_amdgcn_perm(k64, c0, 0x04030401u),
+                                        __builtin_amdgcn_perm(k64, c1, 0x04020400u), __builtin_amdgcn_perm(k64, c1, 0x04030401u));
+                    } else if (FMT == FH_Q4_0) { // one word per block: low nibbles, then high nibbles
+                        const uint32_t w0 = (st & 3) == 0 ? wq.x : ((st & 3) == 1 ? wq.y : ((st & 3) == 2 ? wq.z : wq.w));
+                        bo = make_uint4(w0 & LO, (w0 >> 8) & LO, w0 & HI, (w0 >> 8) & HI);
+                    } else {
+                        const uint32_t w0 = (st & 2) ? wq.z : wq.x, w1 = (st & 2) ? wq.w : wq.y;
+                        const uint32_t msk = (st & 1) ? HI : LO;
+                        bo = make_uint4(w0 & msk, (w0 >> 8) & msk, w1 & msk, (w1 >> 8) & msk);
+                    }
+                    half8 bv;
+                    __builtin_memcpy(&bv, &bo, 16);
+    #pragma unroll
+                    for (int mr = 0; mr < MR; mr++)
+                        dd[tp][mr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[mr], bv, dd[tp][mr], 0, 0, 0);
+                }
+    #pragma unroll
+                for (int mr = 0; mr < MR; mr++)
+                    if (t + mr + RING < PER * 8 * MR) ring[(t + mr) % RING] = operand(t + mr + RING);
+            }
+    #pragma unroll
+            for (int mr = 0; mr < MR; mr++) {
+                const float2 fc = *(const float2 *)(psf + (r * MR + mr) * 16 + 8);
+                float2 sx;
+                if constexpr (ONES) { // odd sub-blocks are staged 16 times lower (their codes are 16 times higher)
+                    sx.x = (dsum[mr][0] + dsum[mr][1]) * (fc.x * 0x1p-24f);
+                    sx.y = (dsum[mr][2] + dsum[mr][3]) * (fc.y * 0x1p-20f);
+                } else {
+                    sx = *(const float2 *)(psf + (r * MR + mr) * 16);
+                }
+    #pragma unroll
+                for (int tp = 0; tp < TPW; tp++) {
+                    const uint4 h = w[tp][r].h;
+                    if (FMT == FH_Q4_0 || FMT == FH_Q8_0) {
+                        const float off = FMT == FH_Q8_0 ? 1152.0f : 8.0f;
+                        const float da = fh_h2f((uint16_t)(h.x & 0xFFFF)), db = fh_h2f((uint16_t)(h.x >> 16));
+                        acc[tp][mr] = fmaf(dd[tp][mr][0] + dd[tp][mr][1], da * fc.x, acc[tp][mr]);
+                        acc[tp][mr] = fmaf(dd[tp][mr][2] + dd[tp][mr][3], db * fc.y, acc[tp][mr]);
+                        mins[tp][mr] = fmaf(off * da, sx.x, mins[tp][mr]);
+                        mins[tp][mr] = fmaf(off * db, sx.y, mins[tp][mr]);
+                        continue;
+                    }
+                    const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
+                    const uint32_t sc_l = h.y & 0x3F3F3F3Fu, sc_h = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
+                    const uint32_t mn_l = h.z & 0x3F3F3F3Fu, mn_h = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
+                    const uint32_t scw = ((sc_l & ~selhi) | (sc_h & selhi)) >> sh;
+                    const uint32_t mnw = ((mn_l & ~selhi) | (mn_h & selhi)) >> sh;
+                    const float sca = (float)(scw & 0xFFu), scb = (float)((scw >> 8) & 0xFFu);
+                    const float mna = (float)(mnw & 0xFFu), mnb = (float)((mnw >> 8) & 0xFFu);
+                    const float sa = (sca * d) * fc.x, sb = (scb * d) * fc.y;
+                    acc[tp][mr] = fmaf(dd[tp][mr][0] + dd[tp][mr][1], sa, acc[tp][mr]);
+                    acc[tp][mr] = fmaf(dd[tp][mr][2] + dd[tp][mr][3], sb, acc[tp][mr]);
+                    mins[tp][mr] = fmaf(mna * dmin, sx.x, mins[tp][mr]);
+                    mins[tp][mr] = fmaf(mnb * dmin, sx.y, mins[tp][mr]);
+                }
+            }
+        }
+    #pragma unroll
+        for (int mr = 0; mr < MR; mr++)
+    #pragma unroll
+            for (int tp = 0; tp < TPW; tp++) {
+                const float v = rows_sum(acc[tp][mr] - mins[tp][mr]);
+                if (lane < 16) l_red[((mr * TPW + tp) * SW + wave) * 16 + lane] = v;
+            }
+    }
     __syncthreads();
-    if (tid < TOUT * 16 * MR) {
+    if (tid < (RS > 1 ? 16 / RS : TOUT * 16 * MR)) {
         const int t = (tid >> 4) % TOUT, mr = (tid >> 4) / TOUT, jr = tid & 15;
         float v0 = 0.f, v1 = 0.f;
         for (int s = 0; s < SW; s++) {
@@ -413,7 +509,8 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
             v0 = v0 / rms;
             v1 = v1 / rms;
         }
-        const int64_t row = ((int64_t)blockIdx.x * TOUT + t) * 16 + jr;
+        const int64_t row = RS > 1 ? (int64_t)(blockIdx.x / RS) * 16 + (int)(blockIdx.x % RS) * (16 / RS) + jr
+                                   : ((int64_t)blockIdx.x * TOUT + t) * 16 + jr;
         if constexpr (HP) {
             const float up = __shfl_xor(v0, 8, 64); // column j + 8 is the up row of gate row j
             if (jr < 8) y[(int64_t)blockIdx.x * 8 + jr] = (v0 / (__expf(-v0) + 1.0f)) * up;
@@ -471,6 +568,11 @@ template <int TPW, int PER, int EPI, int IN>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_qmv_q4k_m1_w8(Q4K_M1_PARAMS) {
     qmv_q4k_m1_body<FH_Q4_K, TPW, PER, EPI, IN>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
 }
+// 16 / RS rows of a tile per workgroup, RS blocks at once per wavefront (matrices with few row tiles)
+template <int RS, int PER, int EPI, int IN>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_qmv_q4k_m1_rs(Q4K_M1_PARAMS) {
+    qmv_q4k_m1_body<FH_Q4_K, 1, PER, EPI, IN, 1, RS>(q, x, y, ea, eb, SW, xres, nw, eps, nsplit, rk);
+}
 // 2 .. 4 activation rows (plain input; epilogues none / add2); nsplit = number of valid rows
 template <int FMT, int TPW, int PER, int EPI, int MR>
 __global__ __launch_bounds__(1024) void k_qmv_q4k_mr(Q4K_M1_PARAMS) {
@@ -503,11 +605,7 @@ static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, co
             } else {
                 kern = q8 ? k_qmv_q40_m1<FH_Q8_0, TPW, PER, EPI> : k_qmv_q40_m1<FH_Q4_0, TPW, PER, EPI>;
             }
-            static bool attr40[2] = {false, false};
-            if (!attr40[q8]) {
-                FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-                attr40[q8] = true;
-            }
+            FH_TRY(fh_kernel_lds(q->dev, (const void *)kern, 160 * 1024));
             kern<<<dim3(grid, 1), dim3(64 * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, nullptr, nullptr, 0.f, 0,
                                                                         ex.rk);
             FH_HIP(hipGetLastError());
@@ -526,15 +624,32 @@ static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, co
         if (in == 2) return FH_ERR_UNSUPPORTED; // the merge of the attention partials needs the registers
         kern = in == 1 ? k_qmv_q4k_m1<TPW, PER, EPI, 1> : k_qmv_q4k_m1<TPW, PER, EPI, 0>;
     }
-    static bool attr_done[3] = {false, false, false};
-    if (!attr_done[in]) {
-        FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_done[in] = true;
-    }
+    FH_TRY(fh_kernel_lds(q->dev, (const void *)kern, 160 * 1024));
     kern<<<dim3(grid, (unsigned)ex.ksplit), dim3(64 * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, ex.xres,
                                                                                   ex.nw, ex.eps, ex.nsplit, ex.rk);
     FH_HIP(hipGetLastError());
     return FH_OK;
+}
+
+template <int EPI>
+static fh_status q4k_m1_launch_rs(int rs, int per, const fh_qmatrix *q, const float *x, float *y, const float *a,
+                                  const float *b, int SW, unsigned grid, size_t lds, const Q4kExtra &ex) {
+    if constexpr (EPI == FH_EPI_NONE || EPI == FH_EPI_ADD2) {
+        typedef void (*kern_t)(QView, const float *, float *, const float *, const float *, int, const float *,
+                               const float *, float, int, FhRopeArgs);
+        kern_t kern = nullptr;
+        if (rs == 2 && per == 1) kern = k_qmv_q4k_m1_rs<2, 1, EPI, 0>;
+        else if (rs == 2 && per == 2) kern = k_qmv_q4k_m1_rs<2, 2, EPI, 0>;
+        else if (rs == 4 && per == 1) kern = k_qmv_q4k_m1_rs<4, 1, EPI, 0>;
+        else return FH_ERR_UNSUPPORTED;
+        FH_TRY(fh_kernel_lds(q->dev, (const void *)kern, 160 * 1024));
+        kern<<<dim3(grid, 1), dim3(64 * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, ex.xres, ex.nw, ex.eps, 0,
+                                                                    ex.rk);
+        FH_HIP(hipGetLastError());
+        return FH_OK;
+    } else {
+        return FH_ERR_UNSUPPORTED;
+    }
 }
 
 // (tiles per wavefront, blocks per wavefront) with at most four block tiles (48 registers of weights) per wavefront
@@ -573,7 +688,7 @@ static fh_status q4k_mr_parts(const fh_qmatrix *q, const float *x, int m, float 
     typedef void (*kern_t)(QView, const float *, float *, const float *, const float *, int, const float *, const float *,
                            float, int, FhRopeArgs);
     const kern_t kern = tpw == 2 ? (kern_t)k_qmv_q4k_mr<FMT, 2, 1, FH_EPI_NONE, MR> : (kern_t)k_qmv_q4k_mr<FMT, 1, 1, FH_EPI_NONE, MR>;
-    FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    FH_TRY(fh_kernel_lds(q->dev, (const void *)kern, 160 * 1024));
     kern<<<dim3((unsigned)((tiles + tpw - 1) / tpw), (unsigned)parts), dim3(64 * SW), lds, dev->stream>>>(
         fh_view(q), x, (float *)dev->ksplit_buf, nullptr, nullptr, SW, nullptr, nullptr, 0.f, m, FhRopeArgs{});
     FH_HIP(hipGetLastError());
@@ -602,12 +717,7 @@ static fh_status q4k_mr_go(const fh_qmatrix *q, const float *x, int m, float *y,
                            float, int, FhRopeArgs);
     const kern_t kern = per == 2 ? (kern_t)k_qmv_q4k_mr<FMT, 1, 2, EPI, MR>
                                  : (tpw == 2 ? (kern_t)k_qmv_q4k_mr<FMT, 2, 1, EPI, MR> : (kern_t)k_qmv_q4k_mr<FMT, 1, 1, EPI, MR>);
-    static bool attr_done[3] = {false, false, false};
-    const int ki = per == 2 ? 2 : tpw - 1;
-    if (!attr_done[ki]) {
-        FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_done[ki] = true;
-    }
+    FH_TRY(fh_kernel_lds(q->dev, (const void *)kern, 160 * 1024));
     kern<<<dim3(grid, 1), dim3(64 * SW), lds, dev->stream>>>(fh_view(q), x, y, a, b, SW, nullptr, nullptr, 0.f, m, FhRopeArgs{});
     FH_HIP(hipGetLastError());
     return FH_OK;
@@ -696,6 +806,24 @@ static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra 
     const int nt = epi == FH_EPI_SWIGLU ? 2 : 1;
     const int64_t nout = epi == FH_EPI_SWIGLU ? q->n / 2 : q->n;
     const int64_t tiles = (nout + 15) / 16;
+    // Few row tiles (k / v projections): 16 / rs rows per workgroup, rs blocks at once per wavefront, so that the
+    // launch has rs times the workgroups
+    if (q->type == FH_Q4_K && (epi == FH_EPI_NONE || epi == FH_EPI_ADD2) && ex.nsplit == 0 && ex.ksplit == 1 && !ex.nw) {
+        int rs = (int)dev->opt_matvec_rowsplit;
+        if (rs != 1 && rs != 2 && rs != 4) rs = tiles * 2 <= dev->compute_units ? 2 : 1; // measured: 4 parts gain nothing over 2
+        int per = (int)dev->opt_matvec_per == 2 && rs == 2 ? 2 : 1;
+        while (rs > 1 && kb % (rs * per)) rs /= 2;
+        while (kb / (rs * per) > 16 && rs == 2 && per == 1 && kb % 4 == 0) per = 2;
+        if (rs > 1 && kb / (rs * per) <= 16) {
+            const size_t lds = (size_t)kb * Q4K_IMG * 16 + (size_t)kb * 64 + 16 * 64 + 64;
+            if (lds <= 160 * 1024) {
+                const int SW = kb / (rs * per);
+                const unsigned grid = (unsigned)(tiles * rs);
+                if (epi == FH_EPI_ADD2) return q4k_m1_launch_rs<FH_EPI_ADD2>(rs, per, q, x, y, a, b, SW, grid, lds, ex);
+                return q4k_m1_launch_rs<FH_EPI_NONE>(rs, per, q, x, y, a, b, SW, grid, lds, ex);
+            }
+        }
+    }
     // tiles per wavefront (they share the staged activations and every operand read): two once there are more
     // tiles than compute units; the SwiGLU epilogue needs the gate and the up tile in one wavefront
     int tpw = (int)dev->opt_matvec_tiles;

@@ -135,6 +135,31 @@ def test_qmatmul_few_rows_long_k(dev, oracle, ty, m, n, k):
         dev.set_option("matvec_tiles", 0)
 
 
+@pytest.mark.parametrize("n,k", [(1024, 4096), (1000, 4096), (40, 256), (264, 2048), (512, 14336), (2048, 8192)])
+def test_q4k_single_row_rows_of_a_tile_split_over_workgroups(dev, oracle, n, k):
+    """The single-row Q4_K kernel with the 16 rows of a tile shared out over 2 or 4 workgroups (2 or 4 blocks per
+    wavefront and MFMA): few row tiles for the device (the default for up to 128 tiles on 256 compute units), a ragged
+    last tile, 1 .. 56 blocks of k, one and two block groups per wavefront; plain and two-residual epilogue."""
+    raw = synth.random_weight(Q4_K, n, k, seed=210)
+    x = synth.random_activation(1, k, seed=211)
+    a, b = synth.random_activation(1, n, seed=212), synth.random_activation(1, n, seed=213)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, Q4_K)
+    want = oracle.q_mat_mul(Q4_K, x, raw, n)
+    xt = Tensor.from_slice(dev, x)
+    try:
+        for rs, per in ((0, 0), (1, 0), (2, 0), (2, 2), (4, 0)):
+            dev.set_option("matvec_rowsplit", rs)
+            dev.set_option("matvec_per", per)
+            got = xt.q_mat_mul(q, out=Tensor.filled_bytes(dev, (1, n), 0xFF)).as_slice()
+            assert_close(got, want, what=f"Q4_K {n}x{k} row split {rs} per {per}")
+            got = xt.q_mat_mul_add2(q, Tensor.from_slice(dev, a), Tensor.from_slice(dev, b),
+                                    out=Tensor.filled_bytes(dev, (1, n), 0xFF)).as_slice()
+            assert_close(got, oracle.add3(want, a, b), what=f"add2 Q4_K {n}x{k} row split {rs} per {per}")
+    finally:
+        dev.set_option("matvec_rowsplit", 0)
+        dev.set_option("matvec_per", 0)
+
+
 @pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
 def test_qmatmul_invariants(dev, oracle, ty):
     """one-hot (tests.rs:951-995), zero input / zero weight -> exact zero (:450-476, :997-1020), batched == unbatched."""
