@@ -94,23 +94,6 @@ fh_status fh_copy(fh_device *dev, void *dst_dev, const void *src_dev, size_t byt
 fh_status fh_timer_start(fh_device *dev);
 fh_status fh_timer_stop(fh_device *dev, float *elapsed_ms); /* blocks until the stream reaches it */
 
-/* Measurement probes (same purpose as the timestamp queries above): an empty kernel of `workgroups` x `threads`,
- * and a plain streaming read of `bytes` (a multiple of 16384) from src_dev.  A benchmark prices the matvec kernels
- * against what these cost on the same device in the same launch pattern. */
-fh_status fh_probe_empty(fh_device *dev, int32_t workgroups, int32_t threads);
-fh_status fh_probe_read(fh_device *dev, const void *src_dev, size_t bytes);
-/* What the device sustains under three patterns the kernels are built from; blocking, every call measures itself.
- *   kind 0: dense v_mfma_f32_32x32x16_f16, a = wavefronts per SIMD (1, 2), b = iterations of four MFMAs:
- *           out4[0] = TFLOP/s, out4[1] = microseconds.
- *   kind 1: ds_read_b128, eight reads in flight per wavefront, a = wavefronts per compute unit (4, 8, 16),
- *           b = address pattern (0 linear; MFMA operand addressing with 1 no swizzle, 2 row & 7, 3 the tile kernels'):
- *           out4[0] = bytes per ns and compute unit, out4[1] = bytes per shader clock and compute unit.
- *   kind 2: 16 wavefronts per compute unit, a = 0 all read a shared 256 KB region (L2 hits), 1 all stream 512 KB each,
- *           2 even ones the first and odd ones the second; src_dev = 256 KB + compute units x 16 x 512 KB:
- *           out4[0] / out4[1] = bytes per ns and compute unit from the L2 / from memory. */
-fh_status fh_probe_device(fh_device *dev, int32_t kind, int32_t a, int32_t b, const void *src_dev, size_t src_bytes,
-                          double *out4);
-
 /* debug_check_nan_f32, models/kalosm-llama/src/raw/mod.rs:9-58: what that probe logs about an f32 tensor - the
  * counts of NaN, +inf and -inf, the largest finite magnitude and the indices of the first NaNs (up to four, in
  * ascending order).  Blocking. */

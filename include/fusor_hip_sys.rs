@@ -154,9 +154,6 @@ extern "C" {
     pub fn fh_copy(dev: *mut FhDevice, dst_dev: *mut c_void, src_dev: *const c_void, bytes: usize) -> FhStatus;
     pub fn fh_timer_start(dev: *mut FhDevice) -> FhStatus;
     pub fn fh_timer_stop(dev: *mut FhDevice, elapsed_ms: *mut f32) -> FhStatus;
-    pub fn fh_probe_empty(dev: *mut FhDevice, workgroups: i32, threads: i32) -> FhStatus;
-    pub fn fh_probe_read(dev: *mut FhDevice, src_dev: *const c_void, bytes: usize) -> FhStatus;
-    pub fn fh_probe_device(dev: *mut FhDevice, kind: i32, a: i32, b: i32, src_dev: *const c_void, src_bytes: usize, out4: *mut f64) -> FhStatus;
     pub fn fh_check_finite(dev: *mut FhDevice, x_dev: *const f32, count: i64, out_host: *mut FhFiniteStats) -> FhStatus;
     pub fn fh_graph_begin(dev: *mut FhDevice) -> FhStatus;
     pub fn fh_graph_end(dev: *mut FhDevice, out: *mut *mut FhGraph) -> FhStatus;

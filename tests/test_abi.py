@@ -1,4 +1,5 @@
-"""The C-ABI library loads and exports every symbol include/fusor_hip.h declares (no device work)."""
+"""The C-ABI library loads and exports every symbol include/fusor_hip.h and include/fusor_hip_probe.h declare (no
+device work)."""
 import os
 import re
 
@@ -7,10 +8,14 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "fusor_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(fh_[a-z0-9_]+)\s*\(", text)))
+def declared_symbols(headers=("fusor_hip.h", "fusor_hip_probe.h")):
+    """Function names declared by the boundary header and by the header of the measurement probes."""
+    names = set()
+    for h in headers:
+        text = open(os.path.join(ROOT, "include", h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(fh_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_header_symbols_are_exported():
@@ -75,7 +80,8 @@ def test_rust_declarations_cover_the_header():
     r = {}
     for name, args in re.findall(r"pub fn (fh_[a-z0-9_]+)\(([^)]*)\)", rs):
         r[name] = 0 if not args.strip() else args.count(",") + 1
-    assert set(c) == set(declared_symbols())
+    assert set(c) == set(declared_symbols(("fusor_hip.h",)))
+    assert not any(n.startswith("fh_probe") for n in c), "measurement probes belong in fusor_hip_probe.h"
     assert c == r, {k: (c.get(k), r.get(k)) for k in set(c) | set(r) if c.get(k) != r.get(k)}
     # the two structs passed by pointer have the header's field order
     cfg = re.search(r"typedef struct \{([^{}]*)\} fh_llama_config;", text).group(1)
