@@ -88,6 +88,24 @@ def assert_close(got, want, abs_tol=1e-2, rel_tol=1e-3, what=""):
     return ma, mr
 
 
+def assert_greedy_follows(ref, first_token, got, margin=2e-2, what="greedy decode"):
+    """The device's greedy tokens against the checker's decoder fed with the SAME tokens: token i must be the checker's
+    pick after [first_token, got[0], .., got[i-1]] or have a checker logit within `margin` of its best one.  A greedy
+    pick is only defined up to the logit tolerance, and the k-split sums of a decode step are accumulated with float
+    atomics whose order varies from run to run, so a near tie may fall either way; feeding the device's own tokens
+    keeps every later step checked all the same.  Leaves the checker's cache where the device's is and returns the
+    number of steps whose pick was the checker's own."""
+    t, same = int(first_token), 0
+    for i, g in enumerate(np.asarray(got).tolist()):
+        wl = ref.forward([t])
+        best = float(np.max(wl))
+        assert float(wl[g]) >= best - margin, (f"{what}: step {i} picked {g} (checker logit {float(wl[g]):.5f}) but the "
+                                               f"checker's best is {int(np.argmax(wl))} ({best:.5f})")
+        same += int(float(wl[g]) == best)
+        t = int(g)
+    return same
+
+
 # ----------------------------------------------------------------------------------------------
 # The reference's deterministic byte generators (conformance/src/common/quantized.rs:175-272 and
 # core/src/quantized/matmul/tests.rs:306-345, :478-489).  Scales are computed in f32, rounded with

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 import refgen
-from refgen import Q4_0, Q4_K, Q6_K, Q8_0, assert_close
+from refgen import Q4_0, Q4_K, Q6_K, Q8_0, assert_close, assert_greedy_follows
 from kalosm_amd import synth
 from kalosm_amd.fusor import MaskKind, QMatrix, Tensor
 from kalosm_amd.llama import Model
@@ -104,12 +104,34 @@ def test_config4_decoder_full_width(dev, oracle):
     assert_close(lg, wl, what="prefill logits, full width")
     tok = int(np.argmax(wl))
     got, _ = m.decode_greedy(tok, 12)
-    want, t = [], tok
-    for _ in range(12):
-        t = oracle.argmax(ref.forward([t]))
-        want.append(t)
-    assert got.tolist() == want
-    assert_close(m.forward([want[-1]]), ref.forward([want[-1]]), what="logits after 12 device-side steps")
+    assert_greedy_follows(ref, tok, got)
+    last = int(got[-1])
+    assert_close(m.forward([last]), ref.forward([last]), what="logits after 12 device-side steps")
+
+
+def test_config4_prompt_and_step_counts_of_the_benchmark(dev, oracle):
+    """configs[4] at the lengths the benchmark times - a 512-token prompt in ONE forward pass (256-row tiles, k split
+    over workgroups, plane sums, split-operand f32 attention) and 256 greedy steps on the device (cache positions
+    512 .. 767: every boundary of the attention's key splits in that range) - on 2 layers at the real widths and a
+    vocabulary of 16384 (the 128256-row output matrix is covered by the tests above), so that the checker's decoder
+    finishes in a minute: prefill logits, every one of the 256 picks against the checker fed with the same tokens,
+    and the logits after them."""
+    cfg = dict(synth.LLAMA3_8B, n_layers=2, ctx=1024, vocab=16384)
+    weights = {}
+    m = Model.random_init(dev, cfg, seed=11, sigma=2e-4, keep=lambda n, a: weights.__setitem__(n, a))
+    ocfg = dict(cfg, type_attn=synth.Q4_K, type_ffn_gate_up=synth.Q4_K, type_ffn_down=synth.Q6_K, type_embd=synth.Q4_K,
+                type_output=synth.Q6_K)
+    ref = oracle.Llama(ocfg, weights)
+    prompt = np.random.default_rng(12).integers(0, cfg["vocab"], 512)
+    lg = m.forward(prompt)
+    wl = ref.forward(prompt)
+    assert_close(lg, wl, what="logits of the 512-token prompt")
+    tok = oracle.argmax(wl)
+    got, _ = m.decode_greedy(tok, 256)
+    same = assert_greedy_follows(ref, tok, got, what="256 steps after a 512-token prompt")
+    assert same >= 200, f"only {same} of 256 picks were the checker's own"
+    last = int(got[-1])
+    assert_close(m.forward([last]), ref.forward([last]), what="logits at position 768")
 
 
 def test_decoder_from_gguf_file_full_width(dev, oracle, tmp_path):
@@ -137,11 +159,7 @@ def test_decoder_from_gguf_file_full_width(dev, oracle, tmp_path):
     assert_close(lg, wl, what="prefill logits from the model file")
     tok = oracle.argmax(wl)
     got, _ = m.decode_greedy(tok, 8)
-    want, t = [], tok
-    for _ in range(8):
-        t = oracle.argmax(ref.forward([t]))
-        want.append(t)
-    assert got.tolist() == want
+    assert_greedy_follows(ref, tok, got, what="decoder from the model file")
 
 
 def test_config4_decoder_all_32_layers(dev, oracle):

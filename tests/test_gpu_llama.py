@@ -3,7 +3,7 @@ weights (the reference stores no logits for any model, so this is pinned by the 
 import numpy as np
 import pytest
 
-from refgen import assert_close
+from refgen import assert_close, assert_greedy_follows
 from kalosm_amd import synth
 from kalosm_amd.llama import Model
 
@@ -50,32 +50,21 @@ def test_decoder_matches_checker(dev, oracle, variant, cfg):
     # greedy decode on the device (graph replay when enabled) against the checker's greedy loop
     steps = 6
     got, ms = m.decode_greedy(tok, steps)
-    want = []
-    t = tok
-    for _ in range(steps):
-        wl = ref.forward([t])
-        t = oracle.argmax(wl)
-        want.append(t)
-    assert got.tolist() == want, f"greedy tokens differ: {got.tolist()} vs {want}"
+    assert_greedy_follows(ref, tok, got)
     # a second greedy run after a reset replays the captured step from position 0
     m.reset(); ref.reset()
     lg = m.forward(prompt); wl = ref.forward(prompt)
     assert_close(lg, wl, what="prefill logits after reset", **tol)
     got2, _ = m.decode_greedy(int(np.argmax(wl)), 4)
-    t = int(np.argmax(wl)); want2 = []
-    for _ in range(4):
-        t = oracle.argmax(ref.forward([t])); want2.append(t)
-    assert got2.tolist() == want2
+    assert_greedy_follows(ref, int(np.argmax(wl)), got2, what="after reset")
     # a longer run crosses the key ranges of the attention splits; afterwards the cache the device-side steps wrote
     # must give the checker's logits through the eager path
-    got3, _ = m.decode_greedy(want2[-1], 40)
-    t = want2[-1]; want3 = []
-    for _ in range(40):
-        t = oracle.argmax(ref.forward([t])); want3.append(t)
-    assert got3.tolist() == want3
+    got3, _ = m.decode_greedy(int(got2[-1]), 40)
+    assert_greedy_follows(ref, int(got2[-1]), got3, what="40 more steps")
+    last = int(got3[-1])
     if variant.get("kv_dtype") == "f16":  # 60 cached positions rounded to f16 (the checker's cache is f32)
         tol = dict(abs_tol=5e-2, rel_tol=5e-3)
-    assert_close(m.forward([want3[-1]]), ref.forward([want3[-1]]), what="logits after 40 device-side steps", **tol)
+    assert_close(m.forward([last]), ref.forward([last]), what="logits after 40 device-side steps", **tol)
 
 
 @pytest.mark.parametrize("heads,kv_heads", [(4, 1), (4, 2), (8, 1), (2, 2), (6, 2)], ids=["g4", "g2", "g8", "g1", "g3"])
@@ -99,12 +88,9 @@ def test_decode_step_kernel_variants(dev, oracle, heads, kv_heads, opts):
         assert_close(lg, wl, what="prefill logits")
         t = int(np.argmax(wl))
         got, _ = m.decode_greedy(t, 70)
-        want = []
-        for _ in range(70):
-            t = oracle.argmax(ref.forward([t]))
-            want.append(t)
-        assert got.tolist() == want
-        assert_close(m.forward([want[-1]]), ref.forward([want[-1]]), what="logits after 70 device-side steps")
+        assert_greedy_follows(ref, t, got)
+        last = int(got[-1])
+        assert_close(m.forward([last]), ref.forward([last]), what="logits after 70 device-side steps")
     finally:
         for k in opts:
             dev.set_option(k, 0)
@@ -146,12 +132,9 @@ def test_decoder_from_gguf_file(dev, oracle, variant, tmp_path):
     assert_close(lg, wl, what="prefill logits")
     tok = oracle.argmax(wl)
     got, _ = m.decode_greedy(tok, 30)
-    want, t = [], tok
-    for _ in range(30):
-        t = oracle.argmax(ref.forward([t]))
-        want.append(t)
-    assert got.tolist() == want
-    assert_close(m.forward([want[-1]]), ref.forward([want[-1]]), what="logits after 30 device-side steps")
+    assert_greedy_follows(ref, tok, got)
+    last = int(got[-1])
+    assert_close(m.forward([last]), ref.forward([last]), what="logits after 30 device-side steps")
     # the rope_freqs factors matter: the same file without them gives other logits
     cos, sin = oracle.rope_tables_weighted(64, 4, 500000.0, weights["rope_freqs.weight"])
     c0, s0 = oracle.rope_tables(64, 4, 500000.0)
@@ -277,11 +260,7 @@ def test_decoder_with_rope_scaling(dev, oracle, tmp_path, rope_freqs):
     assert np.abs(plain.forward(prompt) - wl).max() > 50 * np.abs(lg - wl).max()    # the scaling is not a no-op
     tok = oracle.argmax(wl)
     got, _ = m.decode_greedy(tok, 12)
-    want, t = [], tok
-    for _ in range(12):
-        t = oracle.argmax(ref.forward([t]))
-        want.append(t)
-    assert got.tolist() == want
+    assert_greedy_follows(ref, tok, got, what="scaled RoPE")
     with pytest.raises(Exception):
         m.set_rope_scaling(*scaling)            # the tables are built: too late
 
@@ -304,12 +283,6 @@ def test_graph_decode_survives_scratch_reallocation(oracle):
     m, ref = build_pair(d, oracle, cfg, seed=9)
     rng = np.random.default_rng(3)
 
-    def greedy_ref(t, steps):
-        out = []
-        for _ in range(steps):
-            t = oracle.argmax(ref.forward([t]))
-            out.append(t)
-        return out
 
     # a user graph over a small matvec, captured while the scratch is small
     w = QMatrix.from_raw_bytes(d, (64, 512), synth.random_weight(synth.Q8_0, 64, 512, 1), synth.Q8_0)
@@ -328,10 +301,10 @@ def test_graph_decode_survives_scratch_reallocation(oracle):
     first = oracle.argmax(wl)
     p = GpuStandardSamplerParams(1, 1.0, 1.0, 1.0, 0.0, 0.0)      # top_k 1: the sampled step picks the argmax
     got, _, _ = m.decode_sampled(first, 5, p, np.full(5, 0.5, np.float32), repetition_range=0)
-    assert got.tolist() == greedy_ref(first, 5)
+    assert_greedy_follows(ref, first, got, what="sampled steps with top_k 1")
     last = int(got[-1])
     got, _ = m.decode_greedy(last, 5)
-    assert got.tolist() == greedy_ref(last, 5)
+    assert_greedy_follows(ref, last, got)
     # larger calls on the same device: every scratch buffer is outgrown
     m.reset(); ref.reset()
     long_prompt = rng.integers(0, cfg["vocab"], 100)
@@ -343,10 +316,9 @@ def test_graph_decode_survives_scratch_reallocation(oracle):
     # same parameters, same cache capacity: only the reallocation can trigger the new capture
     first = oracle.argmax(wl)
     got, _, _ = m.decode_sampled(first, 6, p, np.full(6, 0.5, np.float32), repetition_range=0)
-    want = greedy_ref(first, 6)
-    assert got.tolist() == want
-    got2, _ = m.decode_greedy(want[-1], 6)
-    assert got2.tolist() == greedy_ref(want[-1], 6)
+    assert_greedy_follows(ref, first, got, what="sampled steps after the reallocation")
+    got2, _ = m.decode_greedy(int(got[-1]), 6)
+    assert_greedy_follows(ref, int(got[-1]), got2, what="greedy steps after the reallocation")
     # the user graph is refused with an error that says why
     with pytest.raises(FusorHipError, match="captured"):
         g.launch()
