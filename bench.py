@@ -5,8 +5,9 @@ A step is one pass of the Q4_K decode matvec (batch 1) over the four Llama-3-8B 
 (4096x4096 q/o, 1024x4096 k/v, 14336x4096 gate/up, 4096x14336 down), activations f32 N(0,1), weights
 random Q4_K super-blocks (f16 d/dmin ~ N(0, 0.02), 6-bit scales/mins, uniform nibbles), all resident in
 HBM before the timed region.  Each shape rotates over enough distinct weight buffers to exceed the
-256 MB last-level cache, so the bytes really come from HBM.  The K launches of a shape are one recorded train;
-the train is replayed `--trains` times and the median replay is the shape's time (K steps are timed, the
+256 MB last-level cache and every timed train walks on through that pool from where the train before it stopped
+(each train is a recording of its own), so the bytes come from HBM whatever K is.  The K launches of a shape are one
+recorded train; `--trains` trains are timed and the median train is the shape's time (K steps are timed, the
 repetitions only steady the number).
 
 Prints ONE JSON line: whole-path GB/s (algorithmic bytes / device time), the roofline of the dominant
@@ -53,11 +54,29 @@ def measured_traffic():
     return (int(m.group(1)) if m else None), (c.group(1) if c else None)
 
 
-def timed_trains(dev, enqueue, trains: int, use_graph: bool = True):
-    """Median device milliseconds of `trains` runs of the launch sequence `enqueue()` (recorded once and replayed
-    unless use_graph is off)."""
+def timed_trains(dev, enqueue, trains: int, use_graph: bool = True, rotate: bool = False):
+    """Median device milliseconds of `trains` runs of a launch sequence (recorded and replayed unless use_graph is
+    off).  rotate: `enqueue(t)` enqueues train number t (0 is run untimed first) and every train is a recording of
+    its own, so that consecutive trains walk on through a pool of buffers instead of reading the first train's
+    again - a train of few launches would otherwise find its few buffers in the 256 MB memory-side cache.
+    Otherwise `enqueue()` is recorded once and replayed."""
     ms = []
-    if use_graph:
+    if rotate:
+        runs = []
+        for t in range(trains + 1):
+            if use_graph:
+                dev.graph_begin()
+                enqueue(t)
+                runs.append(dev.graph_end().launch)
+            else:
+                runs.append(lambda t=t: enqueue(t))
+        runs[0]()
+        dev.sync()
+        for run in runs[1:]:
+            dev.timer_start()
+            run()
+            ms.append(dev.timer_stop())
+    elif use_graph:
         dev.graph_begin()
         enqueue()
         g = dev.graph_end()
@@ -113,7 +132,7 @@ def batch_leg(dev, sets_m1, steps: int, warmup: int, trains: int) -> list:
                      bytes=synth.matvec_bytes(synth.Q4_K, n, k, m))
             run_shape(t, warmup)
             dev.sync()
-            ms, _ = timed_trains(dev, lambda: run_shape(t, steps, offset=warmup), trains)
+            ms, _ = timed_trains(dev, lambda i: run_shape(t, steps, offset=warmup + i * steps), trains, rotate=True)
             tot_ms += ms
             tot_bytes += t["bytes"]
             per.append({"n": n, "k": k, "us_per_launch": round(ms * 1e3 / steps, 3)})
@@ -140,7 +159,7 @@ def decoder_shapes_leg(dev, steps: int, warmup: int, trains: int) -> list:
         nbytes = synth.matvec_bytes(synth.Q4_K, n, k, 1)
         run_shape(s, warmup)
         dev.sync()
-        ms, _ = timed_trains(dev, lambda: run_shape(s, steps, offset=warmup), trains)
+        ms, _ = timed_trains(dev, lambda i: run_shape(s, steps, offset=warmup + i * steps), trains, rotate=True)
         us = ms * 1e3 / steps
         out.append({"n": n, "k": k, "us_per_launch": round(us, 3), "GBps": round(nbytes / us / 1e3, 1),
                     "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
@@ -148,7 +167,19 @@ def decoder_shapes_leg(dev, steps: int, warmup: int, trains: int) -> list:
     return out
 
 
-def prefill_legs(dev, trains: int, use_graph: bool = True) -> dict:
+def _errs(got, want):
+    """Largest absolute and largest relative difference (relative to max(|got|, |want|), over the elements whose
+    absolute difference exceeds 1e-2: the ones the relative bound has to cover) and the tolerance verdict."""
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    d = np.abs(got - want)
+    scale = np.maximum(np.abs(got), np.abs(want))
+    rel = np.where(scale > 0, d / np.where(scale > 0, scale, 1.0), 0.0)
+    ok = bool(((d <= 1e-2) | (d <= 1e-3 * scale)).all())
+    return {"max_abs_err": float(d.max()), "max_rel_err": float(rel.max()),
+            "max_rel_err_where_abs_above_1e-2": float(rel[d > 1e-2].max()) if (d > 1e-2).any() else 0.0, "ok": ok}
+
+
+def prefill_legs(dev, trains: int, use_graph: bool = True, check: bool = False) -> dict:
     """configs[2]: Y = X . W^T with bf16 X [m, 4096] and Q6_K / Q8_0 W [14336, 4096]; configs[3]: causal attention,
     f16, 32 query heads on 8 KV heads, head_dim 128, and its decode variant.  Device time per call: the median over
     `trains` replays of a recorded train of CALLS back-to-back calls (as the headline and the decode variant are timed:
@@ -175,22 +206,39 @@ def prefill_legs(dev, trains: int, use_graph: bool = True) -> dict:
         return {"bound": "mfma", "achieved": round(tf, 1), "peak": peak, "unit": unit, "frac": round(tf / peak, 4)}
 
     res = {"calls_per_train": CALLS, "matmul": [], "attention": [], "attention_decode": []}
+    if check:
+        from oracle import oracle
+        res["parity"] = "one checked call per configuration, outside the timed trains: CPU checker on 48 sampled weight " \
+                        "rows (matmul), float64 softmax attention on sampled query rows (causal), the checker's " \
+                        "attention (single query); tolerance 1e-2 absolute or 1e-3 relative"
     n, k = 14336, 4096
     for ty, name in ((synth.Q6_K, "Q6_K"), (synth.Q8_0, "Q8_0")):
-        q = QMatrix.from_raw_bytes(dev, (n, k), synth.random_weight(ty, n, k, seed=7), ty)
+        raw = synth.random_weight(ty, n, k, seed=7)
+        q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+        rows = (np.arange(48) * 293 + 5) % n
+        bpr = len(raw) // n
+        sub = np.concatenate([raw[r * bpr:(r + 1) * bpr] for r in rows]) if check else None
         for m in (512, 2048):
-            x = Tensor.from_slice(dev, synth.to_bf16_bits(synth.random_activation(m, k, seed=8)), dtype="bf16")
+            xa = synth.random_activation(m, k, seed=8)
+            bits = synth.to_bf16_bits(xa)
+            x = Tensor.from_slice(dev, bits, dtype="bf16")
             y = Tensor(dev, (m, n), "f32")
             ms = med(lambda: x.q_mat_mul(q, out=y))
             tf = 2.0 * m * n * k / ms / 1e9
-            res["matmul"].append({"weights": name, "activations": "bf16", "m": m, "n": n, "k": k,
-                                  "us": round(ms * 1e3, 1), "roofline": mfma(tf)})
+            e = {"weights": name, "activations": "bf16", "m": m, "n": n, "k": k, "us": round(ms * 1e3, 1), "roofline": mfma(tf)}
+            if check:
+                xb = (bits.astype(np.uint32) << 16).view(np.float32).reshape(m, k)
+                e["parity"] = _errs(y.as_slice()[:, rows], oracle.q_mat_mul(ty, xb, sub, len(rows), fast=True))
+            res["matmul"].append(e)
             if ty == synth.Q8_0:  # the integer variant: f32 activations quantised per 32 inside the call, int8 MFMA
-                xf = Tensor.from_slice(dev, synth.random_activation(m, k, seed=8))
+                xf = Tensor.from_slice(dev, xa)
                 ms = med(lambda: xf.q_mat_mul_q8(q, out=y))
                 tf = 2.0 * m * n * k / ms / 1e9
-                res["matmul"].append({"weights": name, "activations": "Q8_0 per 32 (int8 MFMA)", "m": m, "n": n, "k": k,
-                                      "us": round(ms * 1e3, 1), "roofline": mfma(tf, MFMA_I8_PEAK_TOPS, "TOP/s")})
+                e = {"weights": name, "activations": "Q8_0 per 32 (int8 MFMA)", "m": m, "n": n, "k": k,
+                     "us": round(ms * 1e3, 1), "roofline": mfma(tf, MFMA_I8_PEAK_TOPS, "TOP/s")}
+                if check:
+                    e["parity"] = _errs(y.as_slice()[:, rows], oracle.q8_0_matmul_q8(xa, sub, len(rows)))
+                res["matmul"].append(e)
     # the decoder's own prefill projections with few output tiles (k split over workgroups): f32 activations
     for ty, name, n2, k2 in ((synth.Q4_K, "Q4_K", 4096, 4096), (synth.Q6_K, "Q6_K", 4096, 14336)):
         q = QMatrix.from_raw_bytes(dev, (n2, k2), synth.random_weight(ty, n2, k2, seed=9), ty)
@@ -204,12 +252,25 @@ def prefill_legs(dev, trains: int, use_graph: bool = True) -> dict:
     h, hkv, d = 32, 8, 128
     for s in (512, 2048, 8192):
         rng = np.random.default_rng(s)
-        qt, kt, vt = (Tensor.from_slice(dev, rng.standard_normal((1, hh, s, d)).astype(np.float16), "f16")
-                      for hh in (h, hkv, hkv))
+        qa, ka, va = (rng.standard_normal((1, hh, s, d)).astype(np.float16) for hh in (h, hkv, hkv))
+        qt, kt, vt = (Tensor.from_slice(dev, a, "f16") for a in (qa, ka, va))
         ot = Tensor(dev, (1, h, s, d), "f16")
         ms = med(lambda: qt.flash_attention(kt, vt, 1 / np.sqrt(d), MaskKind.Causal, out=ot))
         tf = 4.0 * s * s * d * h / 2 / ms / 1e9
-        res["attention"].append({"seq": s, "us": round(ms * 1e3, 1), "roofline": mfma(tf)})
+        e = {"seq": s, "us": round(ms * 1e3, 1), "roofline": mfma(tf)}
+        if check:  # float64 softmax attention on 24 sampled query rows of three heads
+            got = ot.as_slice().astype(np.float32)
+            rows = sorted(set([0, 1, 63, 64, 127, 128, s // 2, s - 129, s - 64, s - 1] + rng.integers(0, s, 14).tolist()))
+            g, w = [], []
+            for hh in (0, 5, 31):
+                kf, vf = ka[0, hh // (h // hkv)].astype(np.float64), va[0, hh // (h // hkv)].astype(np.float64)
+                for i in rows:
+                    sc = (qa[0, hh, i].astype(np.float64) @ kf[:i + 1].T) / np.sqrt(d)
+                    pr = np.exp(sc - sc.max())
+                    w.append((pr / pr.sum()) @ vf[:i + 1])
+                    g.append(got[0, hh, i])
+            e["parity"] = _errs(np.array(g), np.array(w))
+        res["attention"].append(e)
     # configs[3], decode variant: one query per head against a cache of L keys (f16 K / V), HBM bound:
     # bytes = K and V once (2 * hkv * L * d * 2) + the query and the output (2 * h * d * 2); caches rotate over
     # more than the Infinity Cache
@@ -232,26 +293,34 @@ def prefill_legs(dev, trains: int, use_graph: bool = True) -> dict:
 
         train()
         dev.sync()
-        ms, _ = timed_trains(dev, lambda: train(7), trains)
+        ms, _ = timed_trains(dev, lambda i: train(7 + i * reps), trains, rotate=True)
         ms /= reps
         nbytes = kv_bytes + 2 * h * d * 2
         gbs = nbytes / ms / 1e6
-        res["attention_decode"].append({"kv_len": L, "us": round(ms * 1e3, 2), "bytes": nbytes,
-                                        "cache_copies_rotated": len(kvs),
-                                        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                                                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4)}})
+        e = {"kv_len": L, "us": round(ms * 1e3, 2), "bytes": nbytes, "cache_copies_rotated": len(kvs),
+             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(gbs / HBM_PEAK_GBS, 4)}}
+        if check:
+            qa = qt.as_slice().astype(np.float32)
+            qt.flash_attention(*kvs[0], 1 / np.sqrt(d), None, out=ot)
+            e["parity"] = _errs(ot.as_slice().astype(np.float32),
+                                oracle.flash_attention(qa, base_k.astype(np.float32), base_v.astype(np.float32), 1 / np.sqrt(d)))
+        res["attention_decode"].append(e)
         del kvs
     return res
 
 
-def calibration(dev, trains: int, use_graph: bool) -> dict:
+def calibration(dev, trains: int, use_graph: bool, probes: bool = True) -> dict:
     """What one dependent launch costs on this device whatever the kernel does: an empty kernel, and a plain
     streaming read of the byte counts of the benchmark's matrices (rotating like the weights do)."""
     from kalosm_amd.fusor import Tensor
     import ctypes as C
 
     L = 100
-    out = {"launches_per_train": L, "empty_us": {}, "read": []}
+    out = {"launches_per_train": L, "empty_us": {}, "read": [],
+           "what": "an empty kernel and a plain streaming read (k_probe_read: 16 bytes per lane and request, 4 KB per "
+                   "wavefront) launched like the matvec: trains of dependent launches in a replayed graph, buffers of "
+                   "the matrices' sizes rotated over 768 MB"}
     for wg, th in ((1, 64), (256, 1024)):
         ms, _ = timed_trains(dev, lambda: [dev._lib.fh_probe_empty(dev._h, wg, th) for _ in range(L)], trains, use_graph)
         out["empty_us"]["%dx%d" % (wg, th)] = round(ms * 1e3 / L, 3)
@@ -262,17 +331,18 @@ def calibration(dev, trains: int, use_graph: bool) -> dict:
         used = nbytes // 16384 * 16384
         copies = max(1, total // used)
 
-        def train():
+        def train(t=0):
             for i in range(L):
-                dev._lib.fh_probe_read(dev._h, C.c_void_p(buf.ptr + (i % copies) * used), used)
+                dev._lib.fh_probe_read(dev._h, C.c_void_p(buf.ptr + ((t * L + i) % copies) * used), used)
 
         train()
         dev.sync()
-        ms, _ = timed_trains(dev, train, trains, use_graph)
+        ms, _ = timed_trains(dev, train, trains, use_graph, rotate=True)
         us = ms * 1e3 / L
         out["read"].append({"bytes": used, "us": round(us, 3), "GBps": round(used / us / 1e3, 1)})
     del buf
-    out["device"] = device_probes(dev)
+    if probes:
+        out["device"] = device_probes(dev)
     return out
 
 
@@ -360,7 +430,9 @@ def main() -> int:
                     help="run 32 decode steps of the decoder with stream launches instead (for a kernel tracer)")
     ap.add_argument("--prefill", action="store_true", help="(default) kept for older command lines")
     ap.add_argument("--no-graph", action="store_true", help="launch on the stream instead of replaying a recorded graph")
-    ap.add_argument("--calib", action="store_true", help="also time an empty kernel and plain streaming reads")
+    ap.add_argument("--calib", action="store_true", help="(default) kept for older command lines")
+    ap.add_argument("--no-calib", action="store_true",
+                    help="skip the launch-floor calibration (an empty kernel and plain streaming reads of the matrices' sizes)")
     ap.add_argument("--calib-copy", action="store_true", help="append 4 device copies of 256 MiB (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -385,7 +457,8 @@ def main() -> int:
     per_shape_ms, all_ms = [], []
     t_wall0 = time.perf_counter()
     for s in sets:
-        ms, every = timed_trains(dev, lambda: run_shape(s, args.steps, offset=args.warmup), args.trains, not args.no_graph)
+        ms, every = timed_trains(dev, lambda i: run_shape(s, args.steps, offset=args.warmup + i * args.steps), args.trains,
+                                 not args.no_graph, rotate=True)
         per_shape_ms.append(ms)
         all_ms.append(every)
     if args.calib_copy:  # a device-to-device copy of known size, to scale the FETCH_SIZE / WRITE_SIZE counters
@@ -461,20 +534,33 @@ def main() -> int:
                                          "%d threads with the reference's static column split" % (reps_done, threads)}
         # parity of the timed configuration against the checker
         worst = 0.0
-        for s, x in zip(sets, xs):
+        for s, x, sh in zip(sets, xs, shapes_out):
             s["x"].q_mat_mul(s["qs"][0], out=s["y"])
-            got = s["y"].as_slice()
-            want = oracle.q_mat_mul(ty, x, s["raw"], s["n"], threads=threads)
-            diff = np.abs(got - want)
-            ok = (diff <= 1e-2) | (diff <= 1e-3 * np.maximum(np.abs(got), np.abs(want)))
-            if not ok.all():
-                print("bench.py: PARITY FAILURE at shape", s["n"], s["k"], "max abs", diff.max(), file=sys.stderr)
+            e = _errs(s["y"].as_slice(), oracle.q_mat_mul(ty, x, s["raw"], s["n"], threads=threads))
+            sh["parity"] = e
+            if not e["ok"]:
+                print("bench.py: PARITY FAILURE at shape", s["n"], s["k"], e, file=sys.stderr)
                 return 1
-            worst = max(worst, float(diff.max()))
+            worst = max(worst, e["max_abs_err"])
         out["parity_max_abs_err"] = worst
 
-    if args.calib:
-        out["calibration"] = calibration(dev, args.trains, not args.no_graph)
+    if not args.no_calib:
+        # what one dependent launch costs on this device whatever the kernel does, in the same run and launch pattern
+        cal = calibration(dev, args.trains, not args.no_graph, probes=not args.no_legs)
+        out["calibration"] = cal
+        floor = {r["bytes"]: r["us"] for r in cal["read"]}
+        tot = 0.0
+        for sh in shapes_out:
+            wbytes = sh["n"] * (sh["k"] // 256) * 144 // 16384 * 16384
+            sh["read_floor_us"] = floor.get(wbytes)
+            if sh["read_floor_us"]:
+                sh["vs_read_floor"] = round(sh["us_per_launch"] / sh["read_floor_us"], 3)
+                tot += sh["read_floor_us"]
+        if tot:
+            cal["step_read_floor_us"] = round(tot, 3)
+            cal["step_read_floor_GBps"] = round(step_bytes / tot / 1e3, 1)
+            cal["step_read_floor_frac_hbm_peak"] = round(step_bytes / tot / 1e3 / HBM_PEAK_GBS, 4)
+            out["roofline"]["frac_of_same_run_read_floor"] = round(value / (step_bytes / tot / 1e3), 4)
     if not args.no_legs:
         out["batch"] = batch_leg(dev, sets, args.steps, args.warmup, args.trains)
     for s in sets:
@@ -482,7 +568,11 @@ def main() -> int:
     del sets
     if not args.no_legs:
         out["decoder_shapes"] = decoder_shapes_leg(dev, args.steps, args.warmup, args.trains)
-        out["prefill"] = prefill_legs(dev, max(3, min(args.trains, 5)), not args.no_graph)
+        out["prefill"] = prefill_legs(dev, max(3, min(args.trains, 5)), not args.no_graph, check=not args.no_cpu)
+        if not all(e["parity"]["ok"] for grp in ("matmul", "attention", "attention_decode") for e in out["prefill"][grp]
+                   if "parity" in e):
+            print("bench.py: a prefill / attention leg differs from the CPU checker beyond the tolerance", file=sys.stderr)
+            rc = 1
 
     if args.e2e_eager:
         from kalosm_amd import e2e
