@@ -543,12 +543,7 @@ static fh_status ad_launch(fh_device *dev, const float *q, const void *k, const 
     const size_t lds = ((size_t)G * chunk_max + (size_t)NWV * G * D) * 4;
     FH_REQUIRE(lds <= 150 * 1024, "KV capacity %d too large for the decode attention kernel", max_len);
     FH_TRY(fh_dev_scratch(dev, (void **)&dev->part_buf, &dev->part_cap, (size_t)hq * S * (D + 4) * 4));
-    static bool attr_done = false;
-    if (!attr_done) {
-        FH_HIP(hipFuncSetAttribute((const void *)k_attn_decode_dl<TKV, D, G, NWV>,
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024));
-        attr_done = true;
-    }
+    FH_TRY(fh_kernel_lds(dev, (const void *)k_attn_decode_dl<TKV, D, G, NWV>, 152 * 1024));
     k_attn_decode_dl<TKV, D, G, NWV><<<dim3((unsigned)S, (unsigned)hkv, (unsigned)(gtot / G)), dim3(64 * NWV), lds, dev->stream>>>(
         q, (const TKV *)k, (const TKV *)v, kv_sh, kv_st, len_dev, len_host, scale, chunk_max, max_len, gtot, dev->part_buf);
     FH_HIP(hipGetLastError());

@@ -401,12 +401,7 @@ static fh_status ap_launch_k(fh_device *dev, const void *q, int64_t q_sb, int64_
     static_assert(KS == 1 || LDS >= (2 + (D / 32) * 16) * 256 * 4, "the merge of the key groups reuses the tile buffers");
     static_assert(LDS <= 160 * 1024, "KV tiles exceed the LDS of a compute unit");
     auto kern = k_attn_prefill<TQ, TKV, D, SPLIT, HW, KS, QW>;
-    static bool raised[64] = {}; // per kernel instance and device: allow more than 64 KB of dynamic LDS
-    const bool known = dev->ordinal >= 0 && dev->ordinal < 64;
-    if (!known || !raised[dev->ordinal]) {
-        FH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-        if (known) raised[dev->ordinal] = true;
-    }
+    FH_TRY(fh_kernel_lds(dev, (const void *)kern, LDS)); // allow more than 64 KB of dynamic LDS
     dim3 grid((unsigned)(hq / HW), (unsigned)((sq + 32 * QW - 1) / (32 * QW)), (unsigned)b);
     kern<<<grid, 64 * QW * HW * KS, LDS, dev->stream>>>((const TQ *)q, q_sb, q_sh, q_st, (const TKV *)k, (const TKV *)v, kv_sb,
                                                kv_sh, kv_st, hq, hkv, sq, skv, scale, causal, (TQ *)out);

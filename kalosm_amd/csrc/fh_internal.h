@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <stddef.h>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "../../include/fusor_hip.h"
@@ -58,12 +59,15 @@ struct fh_device {
     // must not allocate
     void *static_scratch = nullptr;
     size_t static_scratch_bytes = 0;
+    // kernels whose dynamic LDS limit was raised on this device, with the limit (fh_kernel_lds)
+    std::vector<std::pair<const void *, size_t>> lds_raised;
     // options (fh_set_option)
     int64_t opt_matvec_kernel = 0;   // 0 auto, 1 generic VALU, 2 MFMA, 3 first-generation Q4_K MFMA, 4 batch MFMA
     int64_t opt_matvec_splitk = 0;   // 0 auto, else forced split count
     int64_t opt_matvec_waves = 0;    // 0 auto
     int64_t opt_matvec_tiles = 0;    // 0 auto, else 1 / 2 / 4 row tiles per workgroup
     int64_t opt_matvec_per = 0;      // 0 auto, else 1 / 2 / 4 blocks per wavefront
+    int64_t opt_matvec_rowsplit = 0; // 0 auto, else 1 / 2 / 4 workgroups per row tile of the single-row Q4_K kernel
     int64_t opt_attn_splits = 0;     // 0 auto
     int64_t opt_attn_kernel = 0;     // 0 auto, 1 first-generation kernels only, 2 matrix-core prefill for f32 too
     int64_t opt_down_splitk = 0;     // 0: decode steps split k of a Q6_K down projection (atomic adds), 1: never, 3: and SwiGLU in its staging
@@ -84,6 +88,8 @@ struct fh_device {
 };
 
 fh_status fh_dev_scratch(fh_device *dev, void **buf, size_t *cap, size_t need);
+// Allows the kernel `bytes` of dynamic LDS on this device (hipFuncSetAttribute, once per kernel and device).
+fh_status fh_kernel_lds(fh_device *dev, const void *kernel, size_t bytes);
 fh_status fh_static_scratch_init(fh_device *dev); // with dev->ordinal current
 
 // ---------------------------------------------------------------- weights

@@ -303,12 +303,7 @@ static fh_status launch_q4k_t(const fh_qmatrix *q, const float *x, float *y, int
     QView v = fh_view(q);
 #define FH_Q4K_LAUNCH(EPI_)                                                                                     \
     do {                                                                                                        \
-        static bool attr_done = false;                                                                          \
-        if (!attr_done) {                                                                                       \
-            FH_HIP(hipFuncSetAttribute((const void *)k_qmv_q4k_mfma<M, T, EPI_>,                                \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));                \
-            attr_done = true;                                                                                   \
-        }                                                                                                       \
+        FH_TRY(fh_kernel_lds(q->dev, (const void *)k_qmv_q4k_mfma<M, T, EPI_>, 160 * 1024));                    \
         k_qmv_q4k_mfma<M, T, EPI_><<<dim3(grid), dim3(64 * S), lds, st>>>(v, x, y, a, b, S, per);                \
     } while (0)
     if (epi == FH_EPI_NONE) FH_Q4K_LAUNCH(FH_EPI_NONE);

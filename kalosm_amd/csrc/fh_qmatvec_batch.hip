@@ -688,9 +688,7 @@ static fh_status qd_launch(const fh_qmatrix *q, const float *x, int m, float *y,
     const size_t lds = four ? std::max((size_t)cps * 4 * 16 * 17 * 4, (size_t)cps * QD_LDS_IMG) : (size_t)cps * (two ? 2 : 1) * 16 * 17 * 4;
     if (four) {
         if constexpr (EPI != FH_EPI_SWIGLU && (T == FH_Q4_K || T == FH_Q4_0)) {
-            if (lds > 64 * 1024)
-                FH_HIP(hipFuncSetAttribute((const void *)k_qmv_direct<T, 4, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)lds));
+            if (lds > 64 * 1024) FH_TRY(fh_kernel_lds(dev, (const void *)k_qmv_direct<T, 4, EPI>, lds));
             k_qmv_direct<T, 4, EPI><<<grid, block, lds, dev->stream>>>(fh_view(q), (const uint8_t *)dev->act_buf, m, cps, y,
                                                                       part, a, b);
         }

@@ -233,12 +233,7 @@ __global__ __launch_bounds__(1024) void k_qmv_q6k_m1(QView q, const float *__res
 template <int TPW, int PER, int EPI>
 static fh_status q6k_m1_launch(const fh_qmatrix *q, const float *x, float *y, const float *a, const float *b, int SW,
                                unsigned grid, size_t lds, unsigned ksplit = 1, const float *xup = nullptr) {
-    static bool attr_done = false;
-    if (!attr_done) {
-        FH_HIP(hipFuncSetAttribute((const void *)k_qmv_q6k_m1<TPW, PER, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   160 * 1024));
-        attr_done = true;
-    }
+    FH_TRY(fh_kernel_lds(q->dev, (const void *)k_qmv_q6k_m1<TPW, PER, EPI>, 160 * 1024));
     k_qmv_q6k_m1<TPW, PER, EPI><<<dim3(grid, ksplit), dim3(64 * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, xup);
     FH_HIP(hipGetLastError());
     return FH_OK;

@@ -1080,11 +1080,7 @@ template <int T, int WM>
 static fh_status qmm_launch_tile2j(const fh_qmatrix *q, const _Float16 *xh, const float *rs, int m, float *y) {
     constexpr int TM = WM * 64;
     constexpr size_t lds = 2 * (size_t)(128 * 64 + TM * 64 + 4 * 128) * 2;
-    static bool attr_done = false;
-    if (!attr_done) {
-        FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2j<T, WM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_done = true;
-    }
+    FH_TRY(fh_kernel_lds(q->dev, (const void *)k_qmm_tile2j<T, WM>, (int)lds));
     fh_device *dev = q->dev;
     const int tiles_n = (int)((q->n + 127) / 128), tiles = tiles_n * ((m + TM - 1) / TM);
     // the last round of workgroups: split its tiles along k when they fill at most half the device
@@ -1109,11 +1105,7 @@ static fh_status qmm_launch_tile2i(const fh_qmatrix *q, const _Float16 *xh, cons
                                    float *y) {
     constexpr int TM = WM * 64;
     constexpr size_t lds = 2 * (size_t)(128 * 32 + NTERM * TM * 32 + 2 * 128) * 2;
-    static bool attr_done = false;
-    if (!attr_done) {
-        FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2i<T, NTERM, WM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_done = true;
-    }
+    FH_TRY(fh_kernel_lds(q->dev, (const void *)k_qmm_tile2i<T, NTERM, WM>, (int)lds));
     dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + TM - 1) / TM));
     if (WM == 4 && q->k % 128 == 0) { // split the tiles of a short last round along k
         fh_device *dev = q->dev;
@@ -1548,11 +1540,7 @@ __global__ void k_qmm_sum_planes(const float4 *__restrict__ part, int planes, in
 
 static fh_status qmm_launch_tile2q(const fh_qmatrix *q, const _Float16 *xh, const float *rs, int m, float *y, int ksplit) {
     constexpr size_t lds = 2 * (size_t)(2 * 128 * 64 + 256 * 64) * 2 + 128 * 4;
-    static bool attr_done = false;
-    if (!attr_done) {
-        FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2q, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_done = true;
-    }
+    FH_TRY(fh_kernel_lds(q->dev, (const void *)k_qmm_tile2q, (int)lds));
     fh_device *dev = q->dev;
     dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + 255) / 256), (unsigned)ksplit);
     if (ksplit == 1 && q->k % 512 == 0) { // split the tiles of a short last round along k
@@ -1587,11 +1575,7 @@ template <int NTERM>
 static fh_status qmm_launch_tile2k(const fh_qmatrix *q, const _Float16 *xh, const _Float16 *xl, const _Float16 *xs,
                                    const float *rs, int m, float *y, int ksplit) {
     constexpr size_t lds = 2 * (size_t)(128 * 32 + NTERM * 256 * 32) * 2 + 128 * 8 * 2 + 2 * 256 * 8 * 2 + 128 * 2 * 4;
-    static bool attr_done = false;
-    if (!attr_done) {
-        FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2k<NTERM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_done = true;
-    }
+    FH_TRY(fh_kernel_lds(q->dev, (const void *)k_qmm_tile2k<NTERM>, (int)lds));
     dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + 255) / 256), (unsigned)ksplit);
     if (ksplit == 1 && q->k % 512 == 0) { // split the tiles of a short last round along k
         fh_device *dev = q->dev;
@@ -1629,12 +1613,7 @@ static fh_status qmm_launch_tile2(const fh_qmatrix *q, const _Float16 *xh, const
                                   float *y, int ksplit = 1) {
     constexpr int TM = (8 / WN) * FM * 32;
     constexpr size_t lds = 2 * (size_t)(2 * 128 * 32 + NTERM * TM * 32) * 2;
-    static bool attr_done = false;
-    if (!attr_done) {
-        FH_HIP(hipFuncSetAttribute((const void *)k_qmm_tile2<T, NTERM, WN, FN, FM>,
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_done = true;
-    }
+    FH_TRY(fh_kernel_lds(q->dev, (const void *)k_qmm_tile2<T, NTERM, WN, FN, FM>, (int)lds));
     dim3 grid((unsigned)((q->n + 127) / 128), (unsigned)((m + TM - 1) / TM), (unsigned)ksplit);
     if (TM == 256 && ksplit == 1 && q->k % 128 == 0) { // split the tiles of a short last round along k
         fh_device *dev = q->dev;
