@@ -279,7 +279,10 @@ fh_status fh_flash_attention_ex(fh_device *dev, int32_t q_dtype, int32_t kv_dtyp
  * heads x 16 key parts x 132 floats) that every GPU the library runs on holds until the process ends, and calls
  * no hipMalloc, hipFree or other allocating routine.  q and out are [hq, 128] contiguous, of q_dtype; k and v are
  * [hkv, skv, 128] views of kv_dtype with head stride kv_sh and position stride kv_st (elements, multiples of 8).
- * Same kernels and the same cut of the key range as fh_flash_attention, so the same bits.  hq x parts beyond the
+ * For f32 caches, and for f16 caches of fewer than 4096 keys, it runs the same kernels with the same cut of the key
+ * range as fh_flash_attention and returns the same bits; for f16 caches from 4096 keys on fh_flash_attention takes
+ * its matrix-core kernel while this entry point keeps the vector-ALU one with its 16 parts, and the two agree within
+ * the attention tolerance (1e-2 absolute or 1e-3 relative).  hq x parts beyond the
  * array (more than 64 heads at 16 parts) is FH_ERR_INVALID with a message; shapes outside the list above are
  * FH_ERR_UNSUPPORTED.  All calls on one GPU share the array: calls that overlap on one GPU (two streams, two
  * device handles, two threads) race; calls on one handle's stream are ordered and safe.  Nothing needs clearing
@@ -428,7 +431,10 @@ fh_status fh_llama_set_rope_scaling(fh_llama *m, const fh_rope_scaling *scaling)
 fh_status fh_llama_finalize(fh_llama *m);
 fh_status fh_llama_reset(fh_llama *m);
 /* Run `count` new tokens at the current position; logits_host (optional, [vocab]) and
- * hidden_host (optional, [d_model], the final-norm hidden state) are of the LAST token. */
+ * hidden_host (optional, [d_model], the final-norm hidden state) are of the LAST token.  When the new tokens do not
+ * fit the context, the cache is cleared and the last context_length - 32 (at least 8) of all tokens, cached and
+ * new, are run again from position 0, as Model::forward does (raw/mod.rs:769-801).  The device-side decode loops
+ * below stop at the context length with FH_ERR_INVALID instead. */
 fh_status fh_llama_forward(fh_llama *m, const uint32_t *tokens_host, int32_t count,
                            float *logits_host, float *hidden_host);
 /* Trace of the last fh_llama_forward, as text lines.  Off by default; fh_set_option keys (or the reference's

@@ -33,6 +33,9 @@ struct fh_llama {
     fh_kvcache *cache = nullptr;
     bool finalized = false;
     int pos = 0;
+    // the token ids whose keys and values the cache holds (KvCache::tokens of the reference, raw/cache.rs): what a
+    // forward pass re-runs the tail of when the context is full
+    std::vector<uint32_t> history;
     // step buffers (sized for `cap_s` tokens)
     int cap_s = 0;
     uint32_t *ids = nullptr;
@@ -322,6 +325,7 @@ extern "C" fh_status fh_llama_finalize(fh_llama *m) {
 extern "C" fh_status fh_llama_reset(fh_llama *m) {
     FH_REQUIRE(m && m->finalized, "decoder not finalized");
     m->pos = 0;
+    m->history.clear();
     return fh_kvcache_reset(m->cache);
 }
 
@@ -406,10 +410,11 @@ static fh_status run_layers(fh_llama *m, int s, bool dev_pos) {
                                 : fh_attention_decode_devlen(dev, c.kv_dtype, m->qrot, kc, vc, (int64_t)m->cache->capacity * hd,
                                                              hd, H, HK, hd, scale, m->cache->len_dev, m->cache->capacity,
                                                              merge_in_wo ? nullptr : m->att, &nsplit);
-            if (ast == FH_ERR_UNSUPPORTED)
+            const bool parts = ast != FH_ERR_UNSUPPORTED; // the attention left partial results per key split
+            if (!parts)
                 ast = fh_attention_decode_devlen_v1(dev, c.kv_dtype, m->qrot, kc, vc, (int64_t)m->cache->capacity * hd, hd, H,
                                                     HK, hd, scale, m->cache->len_dev, m->cache->capacity, m->att);
-            else if (ast == FH_OK && merge_in_wo) {
+            if (parts && ast == FH_OK && merge_in_wo) {
                 // first choice: x += Wo . att with k split over small workgroups; the residual stream then already
                 // holds x + attn for the FFN norm and the final sum ((ffn + attn) + residual, raw/mod.rs:1036)
                 fh_status st = (dev->opt_wo_acc == 1 || dev->opt_deterministic) ? FH_ERR_UNSUPPORTED
@@ -513,10 +518,24 @@ extern "C" fh_status fh_llama_forward(fh_llama *m, const uint32_t *tokens_host, 
                                       float *hidden_host) {
     FH_REQUIRE(m && m->finalized && tokens_host, "decoder not finalized or NULL tokens");
     FH_REQUIRE(count > 0 && count <= 65535, "count %d out of range", count);
-    FH_REQUIRE(m->pos + count <= m->c.ctx, "context overflow: %d + %d > %d", m->pos, count, m->c.ctx);
     for (int i = 0; i < count; i++)
         FH_REQUIRE(tokens_host[i] < (uint32_t)m->c.vocab, "token id %u at %d outside the vocabulary of %d", tokens_host[i], i,
                    m->c.vocab);
+    // Model::forward, raw/mod.rs:769-801: when the new tokens do not fit the context, the cache is cleared and the last
+    // context_length - 32 (at least 8) of all tokens, cached and new, are run again from position 0.
+    std::vector<uint32_t> trimmed;
+    if (m->pos + count > m->c.ctx) {
+        const int cutoff = std::max(m->c.ctx - 32, 8);
+        FH_REQUIRE(cutoff <= m->c.ctx && cutoff <= 65535, "context of %d positions is too short to trim to %d", m->c.ctx, cutoff);
+        FH_REQUIRE((int)m->history.size() == m->pos, "the cache holds %d positions but %zu token ids are on record", m->pos,
+                   m->history.size());
+        trimmed = m->history;
+        trimmed.insert(trimmed.end(), tokens_host, tokens_host + count);
+        trimmed.erase(trimmed.begin(), trimmed.end() - cutoff);
+        FH_TRY(fh_llama_reset(m));
+        tokens_host = trimmed.data();
+        count = cutoff;
+    }
     FH_TRY(ensure_steps(m, count));
     FH_TRY(fh_upload(m->dev, m->ids, tokens_host, (size_t)count * 4));
     m->trace_text.clear();
@@ -524,6 +543,7 @@ extern "C" fh_status fh_llama_forward(fh_llama *m, const uint32_t *tokens_host, 
     m->trace_first = m->trace_last = -1;
     FH_TRY(run_layers(m, count, false));
     // all layers appended: advance the cache
+    m->history.insert(m->history.end(), tokens_host, tokens_host + count);
     m->pos += count;
     m->cache->len = m->pos;
     FH_TRY(fh_kvcache_set_len_dev(m->cache, m->pos));
@@ -557,7 +577,9 @@ static fh_status decode_step_enqueue(fh_llama *m) {
 extern "C" fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, int32_t steps, uint32_t *out_tokens_host,
                                             float *elapsed_ms) {
     FH_REQUIRE(m && m->finalized && out_tokens_host, "decoder not finalized or NULL output");
-    FH_REQUIRE(steps > 0 && m->pos + steps <= m->c.ctx, "context overflow: %d + %d > %d", m->pos, steps, m->c.ctx);
+    FH_REQUIRE(steps > 0 && m->pos + steps <= m->c.ctx,
+               "context overflow: %d + %d > %d (the device-side loops stop at the context length; fh_llama_forward trims)", m->pos,
+               steps, m->c.ctx);
     FH_REQUIRE(first_token < (uint32_t)m->c.vocab, "token id %u outside the vocabulary", first_token);
     fh_device *dev = m->dev;
     hipStream_t s = dev->stream;
@@ -602,6 +624,8 @@ extern "C" fh_status fh_llama_decode_greedy(fh_llama *m, uint32_t first_token, i
     m->pos += steps;
     m->cache->len = m->pos;
     FH_TRY(fh_download(dev, out_tokens_host, m->out_tok_dev, (size_t)steps * 4));
+    m->history.push_back(first_token); // the cache now holds the step inputs: the first token and all outputs but the last
+    m->history.insert(m->history.end(), out_tokens_host, out_tokens_host + steps - 1);
     return FH_OK;
 }
 
@@ -640,7 +664,9 @@ extern "C" fh_status fh_llama_decode_sampled(fh_llama *m, uint32_t first_token, 
                                              const uint32_t *previous_host, uint32_t n_previous, uint32_t repetition_range,
                                              float *mu, uint32_t *out_tokens_host, float *elapsed_ms) {
     FH_REQUIRE(m && m->finalized && out_tokens_host && params && randoms_host, "decoder not finalized or NULL argument");
-    FH_REQUIRE(steps > 0 && m->pos + steps <= m->c.ctx, "context overflow: %d + %d > %d", m->pos, steps, m->c.ctx);
+    FH_REQUIRE(steps > 0 && m->pos + steps <= m->c.ctx,
+               "context overflow: %d + %d > %d (the device-side loops stop at the context length; fh_llama_forward trims)", m->pos,
+               steps, m->c.ctx);
     FH_REQUIRE(first_token < (uint32_t)m->c.vocab, "token id %u outside the vocabulary", first_token);
     FH_REQUIRE(n_previous == 0 || previous_host, "previous tokens missing");
     FH_REQUIRE(params->kind != FH_SAMPLER_MIROSTAT2 || mu, "Mirostat 2 needs its state");
@@ -709,5 +735,7 @@ extern "C" fh_status fh_llama_decode_sampled(fh_llama *m, uint32_t first_token, 
     m->cache->len = m->pos;
     FH_TRY(fh_download(dev, out_tokens_host, m->out_tok_dev, (size_t)steps * 4));
     if (mu) FH_TRY(fh_download(dev, mu, m->samp_dev + 66, 4));
+    m->history.push_back(first_token);
+    m->history.insert(m->history.end(), out_tokens_host, out_tokens_host + steps - 1);
     return FH_OK;
 }

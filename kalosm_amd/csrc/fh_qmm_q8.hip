@@ -4,11 +4,14 @@
 // over the blocks of a row in k order in f32 (the Q8-activation matmul of fusor-ml/cpu/src/quantized.rs).
 //
 // One v_mfma_i32_32x32x32_i8 is exactly one 32-element block of 32 weight rows against 32 activation rows: the
-// integer block sums are exact, and the scaling  acc = acc + f32(isum) * (d_w * d_a)  is done per block in the same
-// operation order as the reference, so results agree with the CPU path bit for bit.
+// integer block sums are exact (the reference fixes nothing else: the order in which the f32 block terms are scaled
+// and added is the caller's).  A block term is added as  acc = fma(f32(isum) * d_a, d_w, acc):  three vector
+// operations per accumulator element and block (convert, multiply, fused multiply-add) with the MFMA result in
+// vector registers, where  acc + f32(isum) * (d_w * d_a)  with separate roundings took five (accumulator-register
+// read, convert, two multiplies, add).
 // Workgroup: 128 weight rows x 128 activation rows, 4 wavefronts of 64 x 64 (2 x 2 MFMA tiles), two blocks (one
-// device record) per barrier round through LDS.  The kernel is bound by the per-block scaling (4 VALU operations per
-// accumulator element and block against one MFMA per 1024 of them), not by the matrix cores.
+// device record) per barrier round through LDS.  The kernel is bound by the per-block scaling (48 vector
+// instructions per MFMA, i.e. 192 cycles against the 32 of the MFMA), not by the matrix cores.
 #include "fh_blocks.h"
 
 typedef int intx4 __attribute__((ext_vector_type(4)));
@@ -45,7 +48,8 @@ __global__ void k_q8_split_quantize(const float *__restrict__ x, int64_t nblocks
 
 #define Q8M_ROW 80 // LDS bytes per row and round: 2 blocks x 32 codes + 16 padding
 
-__global__ __launch_bounds__(256) void k_qmm_q8_mfma(QView q, const int8_t *__restrict__ xc, const float *__restrict__ xs,
+// (at least two wavefronts per SIMD: with at most 256 registers per lane the MFMA results stay in vector registers)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k_qmm_q8_mfma(QView q, const int8_t *__restrict__ xc, const float *__restrict__ xs,
                                                       int m, float *__restrict__ y) {
     __shared__ __attribute__((aligned(16))) uint8_t sA[128 * Q8M_ROW], sB[128 * Q8M_ROW];
     __shared__ __attribute__((aligned(16))) float sAs[2][128], sBs[2][128];
@@ -114,11 +118,7 @@ __global__ __launch_bounds__(256) void k_qmm_q8_mfma(QView q, const int8_t *__re
                     for (int r = 0; r < 16; r++) d[r] = 0;
                     d = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[fn], bv[fm], d, 0, 0, 0);
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const float scale = dw[r] * dx[fm];
-                        const float term = (float)d[r] * scale;
-                        acc[fn][fm][r] = acc[fn][fm][r] + term;
-                    }
+                    for (int r = 0; r < 16; r++) acc[fn][fm][r] = fmaf((float)d[r] * dx[fm], dw[r], acc[fn][fm][r]);
                 }
             }
         }

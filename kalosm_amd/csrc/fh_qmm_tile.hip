@@ -14,6 +14,14 @@
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+// lo half of the two-term f16 split of w whose hi half is h.  A non-finite w (inf, NaN) keeps its kind in h alone:
+// inf - inf would put a NaN into the lo plane and turn every product of the row into NaN, where the reference's
+// f32 arithmetic gives +-inf.
+__device__ __forceinline__ _Float16 fh_split_lo(float w, _Float16 h) {
+    const float d = w - (float)h;
+    return (_Float16)(d == d ? d : 0.f);
+}
+
 // adds the two k halves of the tiles of a split last round (see k_qmm_tile2j) into y
 __global__ void k_qmm_tail_sum(const float *__restrict__ planes, int tail, int full, int tiles_n, int m, int64_t n,
                                float *__restrict__ y);
@@ -55,11 +63,17 @@ __global__ __launch_bounds__(256) void k_act_split(const void *__restrict__ xin,
     int e = 141 - (int)((__float_as_uint(amax) >> 23) & 0xFFu); // 14 - floor(log2 amax); zero / inf / nan clamp
     e = e > 100 ? 100 : (e < -100 ? -100 : e);
     const float sc = __uint_as_float((uint32_t)(e + 127) << 23);
+    // A row with an infinity: its finite values vanish next to it (sc flushes them to zero), the infinity itself is
+    // carried as +-32768 and the row's output scale is infinite, so that the product comes out as +-inf with the
+    // sign of the reference's f32 sum (NaN where the other operand is zero or NaN) instead of inf * 0 = NaN from the
+    // lo plane of the other operand.
+    const bool infrow = amax == INFINITY;
     for (int c = threadIdx.x; c < kp; c += 256) {
-        const float v = c < k ? ld(c) * sc : 0.f;
+        float v = c < k ? ld(c) * sc : 0.f;
+        if (infrow && fabsf(v) == INFINITY) v = copysignf(32768.f, v);
         const _Float16 h = (_Float16)v;
         xh[oo + c] = h;
-        if (IN != 1) xl[oo + c] = (_Float16)(v - (float)h);
+        if (IN != 1) xl[oo + c] = fh_split_lo(v, h);
         if (xs) { // (kp is a multiple of 256 then) sums of the 32-groups of the normalised row, / 64, as hi + lo planes
             float t = v;
 #pragma unroll
@@ -73,7 +87,7 @@ __global__ __launch_bounds__(256) void k_act_split(const void *__restrict__ xin,
             }
         }
     }
-    if (threadIdx.x == 0) rs[blockIdx.x] = __uint_as_float((uint32_t)(127 - e) << 23);
+    if (threadIdx.x == 0) rs[blockIdx.x] = infrow ? INFINITY : __uint_as_float((uint32_t)(127 - e) << 23);
 }
 
 // The same for contiguous rows with k a multiple of 8 and at most 16384: a thread holds its (up to 64) elements of
@@ -121,6 +135,7 @@ __global__ __launch_bounds__(256) void k_act_split_rows(const void *__restrict__
     int e2 = 141 - (int)((__float_as_uint(amax) >> 23) & 0xFFu); // 14 - floor(log2 amax); zero / inf / nan clamp
     e2 = e2 > 100 ? 100 : (e2 < -100 ? -100 : e2);
     const float sc = __uint_as_float((uint32_t)(e2 + 127) << 23);
+    const bool infrow = amax == INFINITY;
 #pragma unroll
     for (int it = 0; it < NCH; it++) {
         const int c = (it * 256 + (int)threadIdx.x) * 8;
@@ -129,9 +144,10 @@ __global__ __launch_bounds__(256) void k_act_split_rows(const void *__restrict__
         float t = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const float w = v[it][e] * sc;
+            float w = v[it][e] * sc;
+            if (infrow && fabsf(w) == INFINITY) w = copysignf(32768.f, w); // as in k_act_split
             h[e] = (_Float16)w;
-            l[e] = (_Float16)(w - (float)h[e]);
+            l[e] = fh_split_lo(w, h[e]);
             t += w;
         }
         if (live) {
@@ -155,7 +171,7 @@ __global__ __launch_bounds__(256) void k_act_split_rows(const void *__restrict__
             }
         }
     }
-    if (threadIdx.x == 0) rs[blockIdx.x] = __uint_as_float((uint32_t)(127 - e2) << 23);
+    if (threadIdx.x == 0) rs[blockIdx.x] = infrow ? INFINITY : __uint_as_float((uint32_t)(127 - e2) << 23);
 }
 
 // Rows of a dense right-hand side as the tile kernel's "weights": row r (one output column of the product) scaled by
@@ -305,7 +321,7 @@ __global__ __launch_bounds__(64 * WGN * WGM) void k_qmm_tile(QView q, const _Flo
 #pragma unroll
                 for (int c = 0; c < 8; c++) {
                     hi[c] = (_Float16)w[c];
-                    lo[c] = (_Float16)(w[c] - (float)hi[c]);
+                    lo[c] = (T == FH_W_F32 || T == FH_W_F16) ? fh_split_lo(w[c], hi[c]) : (_Float16)(w[c] - (float)hi[c]);
                 }
                 const int row = t16 * 16 + j;
                 uint2 a0, a1, b0, b1;
@@ -549,7 +565,7 @@ __global__ __launch_bounds__(512) void k_qmm_tile2(QView q, const _Float16 *__re
 #pragma unroll
         for (int c = 0; c < 8; c++) {
             hi[c] = (_Float16)w[c];
-            lo[c] = (_Float16)(w[c] - (float)hi[c]);
+            lo[c] = (T == FH_W_F32 || T == FH_W_F16) ? fh_split_lo(w[c], hi[c]) : (_Float16)(w[c] - (float)hi[c]);
         }
         uint2 a0, a1, l0, l1;
         __builtin_memcpy(&a0, hi, 8);

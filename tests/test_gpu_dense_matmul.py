@@ -48,6 +48,26 @@ def test_matmul_keeps_f32_accuracy_over_magnitudes(dev):
     assert (np.abs(got - want) <= 2e-6 * scale).all()
 
 
+def test_matmul_non_finite_operands_keep_their_kind(dev):
+    """An infinity in A and a NaN in B: the outputs they reach are +-inf / NaN exactly where the f32 product of the
+    reference has them (an infinity must not become a NaN on its way through the operand split), and every other
+    output keeps its accuracy."""
+    rng = np.random.default_rng(11)
+    m, k, n = 70, 96, 50
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    b = rng.standard_normal((k, n)).astype(np.float32)
+    a[5, 17] = np.inf
+    a[40, 3] = -np.inf
+    b[60, 9] = np.nan
+    with np.errstate(invalid="ignore"):
+        want = a.astype(np.float64) @ b.astype(np.float64)
+    got = Tensor.from_slice(dev, a).matmul(Tensor.from_slice(dev, b)).as_slice().astype(np.float64)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(np.isposinf(got), np.isposinf(want)) and np.array_equal(np.isneginf(got), np.isneginf(want))
+    fin = np.isfinite(want)
+    assert fin.sum() == (m - 2) * (n - 1) and np.abs(got[fin] - want[fin]).max() < 3e-5
+
+
 def test_batched_and_attention_shaped(dev):
     """matmul_batched_3d / matmul_attention_4d ([1, 2, 16, 16], data ((i + seed) % 31 - 15) * 0.05, tolerance 1e-3)."""
     def data(seed, shape):

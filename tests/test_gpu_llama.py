@@ -265,6 +265,30 @@ def test_decoder_with_rope_scaling(dev, oracle, tmp_path, rope_freqs):
         m.set_rope_scaling(*scaling)            # the tables are built: too late
 
 
+def test_forward_trims_the_context_when_it_is_full(dev, oracle):
+    """Model::forward with a full context (raw/mod.rs:769-801): the cache is cleared and the last context_length - 32
+    tokens of everything seen so far, the new ones included, are run again from position 0.  48 + 12 device-side steps
+    fill a context of 64; the next 7 tokens overflow it; the logits must be the checker's for the 32 most recent ids
+    alone, and decoding goes on from position 32."""
+    cfg = dict(HD128, ctx=64)
+    m, ref = build_pair(dev, oracle, cfg, seed=13)
+    rng = np.random.default_rng(14)
+    prompt = rng.integers(0, cfg["vocab"], 48)
+    first = int(np.argmax(m.forward(prompt)))
+    got, _ = m.decode_greedy(first, 12)                      # cache: prompt, first, got[:-1] = 60 positions
+    seen = prompt.tolist() + [first] + got.tolist()[:-1]
+    more = rng.integers(0, cfg["vocab"], 7).tolist()         # 60 + 7 > 64
+    lg = m.forward(more)
+    tail = (seen + more)[-32:]
+    want = ref.forward(tail)
+    assert_close(lg, want, what="logits after the context was trimmed")
+    t = int(np.argmax(want))
+    got2, _ = m.decode_greedy(t, 5)
+    assert_greedy_follows(ref, t, got2, what="steps after the trim")
+    with pytest.raises(Exception, match="context overflow"):
+        m.decode_greedy(int(got2[-1]), 64)                   # the device-side loop does not trim
+
+
 def _bytes_source(data, tmp_path):
     p = tmp_path / f"m{len(list(tmp_path.iterdir()))}.gguf"
     p.write_bytes(data)
