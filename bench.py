@@ -179,6 +179,38 @@ def _errs(got, want):
             "max_rel_err_where_abs_above_1e-2": float(rel[d > 1e-2].max()) if (d > 1e-2).any() else 0.0, "ok": ok}
 
 
+def five_bit_leg(dev, steps: int, warmup: int, trains: int) -> list:
+    """Q5_K and Q5_0 (the 5-bit formats of Q5_K_M / Q5_0 model files) through the single-row matrix-core kernel, beside
+    Q4_K on the same two shapes in the same run: batch 1, weights rotated over 640 MB, HBM bound."""
+    from kalosm_amd import synth
+    from kalosm_amd.fusor import QMatrix, Tensor
+
+    out = []
+    for n, k in ((4096, 4096), (14336, 4096)):
+        base = None
+        for ty in (synth.Q4_K, synth.Q5_K, synth.Q5_0):
+            wbytes = n * (k // synth.BLOCK_ELEMS[ty]) * synth.BLOCK_BYTES[ty]
+            copies = max(2, -(-ROTATE_BYTES // wbytes))
+            raw = synth.random_weight(ty, n, k, seed=1200 + ty)
+            s = dict(qs=[QMatrix.from_raw_bytes(dev, (n, k), raw, ty) for _ in range(copies)],
+                     x=Tensor.from_slice(dev, synth.random_activation(1, k, seed=2300)), y=Tensor(dev, (1, n), "f32"))
+            nbytes = synth.matvec_bytes(ty, n, k, 1)
+            run_shape(s, warmup)
+            dev.sync()
+            ms, _ = timed_trains(dev, lambda i: run_shape(s, steps, offset=warmup + i * steps), trains, rotate=True)
+            us = ms * 1e3 / steps
+            e = {"weights": synth.TYPE_NAMES[ty], "n": n, "k": k, "us_per_launch": round(us, 3), "ns_per_KB": round(us * 1e6 / nbytes, 3),
+                 "roofline": {"bound": "hbm", "achieved": round(nbytes / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                              "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}}
+            if ty == synth.Q4_K:
+                base = us / nbytes
+            else:
+                e["time_per_byte_vs_Q4_K"] = round(us / nbytes / base, 3)
+            out.append(e)
+            del s
+    return out
+
+
 def prefill_legs(dev, trains: int, use_graph: bool = True, check: bool = False) -> dict:
     """configs[2]: Y = X . W^T with bf16 X [m, 4096] and Q6_K / Q8_0 W [14336, 4096]; configs[3]: causal attention,
     f16, 32 query heads on 8 KV heads, head_dim 128, and its decode variant.  Device time per call: the median over
@@ -568,6 +600,7 @@ def main() -> int:
     del sets
     if not args.no_legs:
         out["decoder_shapes"] = decoder_shapes_leg(dev, args.steps, args.warmup, args.trains)
+        out["five_bit"] = five_bit_leg(dev, args.steps, args.warmup, args.trains)
         out["prefill"] = prefill_legs(dev, max(3, min(args.trains, 5)), not args.no_graph, check=not args.no_cpu)
         if not all(e["parity"]["ok"] for grp in ("matmul", "attention", "attention_decode") for e in out["prefill"][grp]
                    if "parity" in e):

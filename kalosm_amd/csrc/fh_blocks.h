@@ -125,35 +125,44 @@ __device__ __forceinline__ float deq_elem_q6_k(const QView &q, int64_t row, int6
     return ds * (float)v;
 }
 
-// ---- formats kept in the file's block order: block b of row `row` starts at (row * kb + b) * block bytes
+// ---- the 5-bit formats: the Q4_0 / Q4_K record followed by a plane of fifth bits
+// Q5_K: record 2816 B; byte l (0..31) of the block's qh
+__device__ __host__ __forceinline__ int q5k_qh_off(int j, int l) { return 2304 + ((l >> 3) * 16 + j) * 8 + (l & 7); }
+// Q5_0: record 1408 B; the byte of block u that holds the fifth bits of the lane group g = (e % 16) / 4 of row j
+__device__ __host__ __forceinline__ int q50_qh_off(int j, int u, int g) { return 1152 + (g * 16 + j) * 4 + u; }
+
 // BlockQ5_0::dequantize, gguf/src/lib.rs:1046-1073: f16 d | 32 high bits | 16 bytes of nibbles;
 // element i < 16: low nibble of byte i with bit i, element i + 16: high nibble with bit i + 16; (code - 16) * d
 __device__ __forceinline__ float deq_elem_q5_0(const QView &q, int64_t row, int64_t k) {
-    const uint8_t *blk = q.data + (row * q.kb + (k >> 5)) * 22;
-    const int e = (int)(k & 31);
-    const float d = fh_h2f(fh_ld16(blk));
-    const uint32_t qh = (uint32_t)fh_ld16(blk + 2) | ((uint32_t)fh_ld16(blk + 4) << 16);
-    const uint8_t byte = blk[6 + (e & 15)];
+    const int64_t b = k >> 5;
+    const int e = (int)(k & 31), j = (int)(row & 15), u = (int)(b & 3);
+    const uint8_t *rec = q.data + ((row >> 4) * q.recs + (b >> 2)) * (int64_t)q.rec_bytes;
+    const float d = fh_h2f(fh_ld16(rec + q40_d_off(j, u)));
+    const uint8_t byte = rec[q40_q_off(j, u, e & 15)];
+    const uint8_t hb = rec[q50_qh_off(j, u, (e & 15) >> 2)];
     const int nib = e < 16 ? (byte & 0x0F) : (byte >> 4);
-    const int v = (nib | (int)(((qh >> e) & 1u) << 4)) - 16;
+    const int bit = (hb >> ((e & 3) + (e < 16 ? 0 : 4))) & 1;
+    const int v = (nib | (bit << 4)) - 16;
     return (float)v * d;
 }
 // BlockQ5K::dequantize, gguf/src/lib.rs:1819-1861: f16 d | f16 dmin | 12 scale bytes | qh[32] | qs[128];
 // sub-block s (32 elements): nibble of qs[32 (s / 2) + l] (low for even s) + 16 * bit s of qh[l];
 // (sc * d) * code - mn * dmin
 __device__ __forceinline__ float deq_elem_q5_k(const QView &q, int64_t row, int64_t k) {
-    const uint8_t *blk = q.data + (row * q.kb + (k >> 8)) * 176;
-    const int e = (int)(k & 255), s = e >> 5, l = e & 31;
-    const float d = fh_h2f(fh_ld16(blk)), dmin = fh_h2f(fh_ld16(blk + 2));
+    const uint8_t *rec = q.data + ((row >> 4) * q.recs + (k >> 8)) * (int64_t)q.rec_bytes;
+    const int e = (int)(k & 255), s = e >> 5, l = e & 31, j = (int)(row & 15);
+    const uint8_t *h = rec + q4k_hdr_off(j);
+    const float d = fh_h2f(fh_ld16(h)), dmin = fh_h2f(fh_ld16(h + 2));
     int sc, mn;
-    q4k_scale_min(blk + 4, s, sc, mn);
-    const uint8_t ql = blk[48 + 32 * (s >> 1) + l], qh = blk[16 + l];
+    q4k_scale_min(h + 4, s, sc, mn);
+    const uint8_t ql = rec[q4k_qs_off(j, 32 * (s >> 1) + l)], qh = rec[q5k_qh_off(j, l)];
     const int v = ((s & 1) ? (ql >> 4) : (ql & 0x0F)) + (((qh >> s) & 1) ? 16 : 0);
     const float scale = (float)sc * d;
     const float off = (float)mn * dmin;
     const float prod = scale * (float)v;
     return prod - off;
 }
+// ---- dense rows in the file's order
 __device__ __forceinline__ float deq_elem_f16(const QView &q, int64_t row, int64_t k) {
     return fh_h2f(((const uint16_t *)q.data)[row * q.k + k]);
 }

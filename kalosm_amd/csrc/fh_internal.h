@@ -119,6 +119,11 @@ fh_status fh_static_scratch_init(fh_device *dev); // with dev->ordinal current
 // FH_Q4_0 (record = four 32-blocks of 16 rows, 1152 B; kb padded to a multiple of 4)
 //   [0,1024)     quants: lane l = g*16 + j: 16 B at l*16 = for u in 0..3: qs_j[blk 4r+u][4g .. +4]
 //   [1024,1152)  d: row j at 1024 + 8*j: d[blk 4r .. 4r+3] (f16 x4)
+// FH_Q5_K (record = one 256-block of 16 rows, 2816 B): the FH_Q4_K record followed by
+//   [2304,2816)  fifth bits: lane l = g*16 + j: 8 B at 2304 + l*8 = qh_j[8g .. +8] (bit s of byte e: element 8g+e of sub-block s)
+// FH_Q5_0 (record = four 32-blocks of 16 rows, 1408 B): the FH_Q4_0 record followed by
+//   [1152,1408)  fifth bits: lane l = g*16 + j: 4 B at 1152 + l*4, byte u for block 4r+u: bits 0-3 = qh bits 4g .. 4g+3
+//                (elements of the low nibbles of the lane's four bytes), bits 4-7 = qh bits 16+4g .. 16+4g+3 (high nibbles)
 struct fh_qmatrix {
     fh_device *dev = nullptr;
     uint32_t type = 0;
@@ -134,10 +139,12 @@ struct fh_qmatrix {
     float wscale = 1.f;
 };
 
-// Weight types kept in the file's own row-major block order (no tiled re-layout): dense f32 / f16 rows and the
-// 5-bit formats.  They run through the per-element kernels only.
+// Weight types kept in the file's own row-major order (no tiled re-layout): dense f32 / f16 rows.
 enum { FH_W_F32 = 0, FH_W_F16 = 1 };
-static inline bool fh_is_plain(uint32_t t) { return t == FH_W_F32 || t == FH_W_F16 || t == FH_Q5_0 || t == FH_Q5_K; }
+static inline bool fh_is_plain(uint32_t t) { return t == FH_W_F32 || t == FH_W_F16; }
+// Types without kernels for several activation rows (batch, row and tile kernels): those go row by row or element by
+// element.  The 5-bit formats have the single-row matrix-core kernel only.
+static inline bool fh_single_row_only(uint32_t t) { return fh_is_plain(t) || t == FH_Q5_0 || t == FH_Q5_K; }
 static inline int fh_block_elems(uint32_t t) {
     switch (t) {
     case FH_W_F32: case FH_W_F16: return 1;
@@ -161,7 +168,7 @@ static inline int fh_block_bytes(uint32_t t) { // gguf/src/lib.rs:109-121
 }
 static inline int fh_rec_blocks(uint32_t t) {   // blocks per record (per row)
     switch (t) {
-    case FH_Q4_0: return 4;
+    case FH_Q4_0: case FH_Q5_0: return 4;
     case FH_Q8_0: return 2;
     default: return 1;
     }

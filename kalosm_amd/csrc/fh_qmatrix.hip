@@ -74,6 +74,34 @@ __global__ void k_repack_q4_0(const uint8_t *__restrict__ src, uint8_t *__restri
     for (int i = 0; i < 16; i++) rec[q40_q_off(j, u, i)] = s[2 + i];
 }
 
+__global__ void k_repack_q5_k(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int64_t n, int64_t kb,
+                              int64_t recs) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n * kb) return;
+    int64_t row = idx / kb, b = idx % kb;
+    const uint8_t *s = src + idx * 176; // d, dmin, 12 scale bytes | qh[32] | qs[128]
+    uint8_t *rec = dst + ((row >> 4) * recs + b) * 2816;
+    int j = (int)(row & 15);
+    for (int i = 0; i < 16; i++) rec[q4k_hdr_off(j) + i] = s[i];
+    for (int i = 0; i < 32; i++) rec[q5k_qh_off(j, i)] = s[16 + i];
+    for (int i = 0; i < 128; i++) rec[q4k_qs_off(j, i)] = s[48 + i];
+}
+__global__ void k_repack_q5_0(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int64_t n, int64_t kb,
+                              int64_t recs) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n * kb) return;
+    int64_t row = idx / kb, b = idx % kb;
+    const uint8_t *s = src + idx * 22; // f16 d | 32 high bits | qs[16]
+    uint8_t *rec = dst + ((row >> 4) * recs + (b >> 2)) * 1408;
+    int j = (int)(row & 15), u = (int)(b & 3);
+    rec[q40_d_off(j, u)] = s[0];
+    rec[q40_d_off(j, u) + 1] = s[1];
+    const uint32_t qh = (uint32_t)s[2] | ((uint32_t)s[3] << 8) | ((uint32_t)s[4] << 16) | ((uint32_t)s[5] << 24);
+    for (int g = 0; g < 4; g++)
+        rec[q50_qh_off(j, u, g)] = (uint8_t)(((qh >> (4 * g)) & 0xFu) | (((qh >> (16 + 4 * g)) & 0xFu) << 4));
+    for (int i = 0; i < 16; i++) rec[q40_q_off(j, u, i)] = s[6 + i];
+}
+
 static fh_status qm_alloc(fh_device *dev, uint32_t type, int64_t n, int64_t k, fh_qmatrix **out) {
     int e = fh_block_elems(type);
     if (!e)
@@ -156,6 +184,8 @@ extern "C" fh_status fh_qmatrix_from_gguf_bytes(fh_device *dev, uint32_t ggml_ty
         case FH_Q6_K: k_repack_q6_k<<<grid, block, 0, dev->stream>>>(staging, q->data, n, q->kb, q->recs); break;
         case FH_Q8_0: k_repack_q8_0<<<grid, block, 0, dev->stream>>>(staging, q->data, n, q->kb, q->recs); break;
         case FH_Q4_0: k_repack_q4_0<<<grid, block, 0, dev->stream>>>(staging, q->data, n, q->kb, q->recs); break;
+        case FH_Q5_K: k_repack_q5_k<<<grid, block, 0, dev->stream>>>(staging, q->data, n, q->kb, q->recs); break;
+        case FH_Q5_0: k_repack_q5_0<<<grid, block, 0, dev->stream>>>(staging, q->data, n, q->kb, q->recs); break;
         }
         if (hipGetLastError() != hipSuccess) { st = FH_ERR_HIP; break; }
         if (hipStreamSynchronize(dev->stream) != hipSuccess) { st = FH_ERR_HIP; break; }

@@ -351,11 +351,11 @@ fh_status fh_launch_qmatvec(const fh_qmatrix *q, const float *x, int m, float *y
     if (epi == FH_EPI_SWIGLU) FH_REQUIRE(q->n % 32 == 0, "SwiGLU epilogue needs n %% 32 == 0 (n = %lld)", (long long)q->n);
     int kernel = (int)dev->opt_matvec_kernel;
     if (kernel == 4 && fh_qmatvec_batch_supports(q, m, epi)) return fh_launch_qmatvec_batch(q, x, m, y, epi, a, b);
-    if (kernel != 1 && kernel != 3 && (q->type == FH_Q4_K || ((q->type == FH_Q4_0 || q->type == FH_Q8_0) && q->k % 256 == 0)) && m == 1) {
+    if (kernel != 1 && kernel != 3 && (q->type == FH_Q4_K || q->type == FH_Q5_K || ((q->type == FH_Q4_0 || q->type == FH_Q8_0 || q->type == FH_Q5_0) && q->k % 256 == 0)) && m == 1) {
         fh_status st = fh_launch_q4k_m1(q, x, y, epi, a, b);
         if (st != FH_ERR_UNSUPPORTED) return st;
     }
-    if (kernel == 0 && q->type != FH_Q6_K && !fh_is_plain(q->type) && m >= 2 && m <= 4 && dev->opt_matvec_rows != 1) {
+    if (kernel == 0 && q->type != FH_Q6_K && !fh_single_row_only(q->type) && m >= 2 && m <= 4 && dev->opt_matvec_rows != 1) {
         fh_status st = fh_launch_q4k_rows(q, x, m, y, epi, a, b);
         if (st != FH_ERR_UNSUPPORTED) return st;
     }
@@ -393,7 +393,7 @@ extern "C" fh_status fh_qmatmul(const fh_qmatrix *q, const float *x_dev, int32_t
     // dense f16 / f32 weight rows (core/src/quantized/matmul/kernel.rs:132-193 routes them to the dense matmul) take
     // the matrix-core tiles as well once there are rows to fill them
     const bool dense = (q->type == FH_W_F16 || q->type == FH_W_F32) && q->k % 32 == 0;
-    if (((m > 16 && mk != 1) || mk >= 2) && (!fh_is_plain(q->type) || dense)) return fh_launch_qmatmul_tile(q, x_dev, 0, m, y_dev);
+    if (((m > 16 && mk != 1) || mk >= 2) && (!fh_single_row_only(q->type) || dense)) return fh_launch_qmatmul_tile(q, x_dev, 0, m, y_dev);
     return fh_launch_qmatvec(q, x_dev, m, y_dev, FH_EPI_NONE, nullptr, nullptr);
 }
 

@@ -733,7 +733,7 @@ static fh_status qb_epi(const fh_qmatrix *q, const float *x, int m, float *y, in
 }
 
 bool fh_qmatvec_batch_supports(const fh_qmatrix *q, int m, int epi) {
-    if (m < 1 || m > 16 || q->k % 256 != 0 || fh_is_plain(q->type)) return false;
+    if (m < 1 || m > 16 || q->k % 256 != 0 || fh_single_row_only(q->type)) return false;
     if (epi == FH_EPI_SWIGLU && (q->n % 32) != 0) return false;
     return true;
 }

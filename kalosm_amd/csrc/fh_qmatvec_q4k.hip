@@ -55,6 +55,12 @@ struct Q4kExtra {
 // FMT = FH_Q8_0: eight 32-blocks = four records of 1088 bytes; a code byte q becomes the f16 1152 + q (xor 0x80,
 // then v_perm_b32 sets it under the high byte 0x64: 1024 + (q + 128) exactly), so the offset is 1152 d and the
 // activation factor carries no 2^24.
+// FMT = FH_Q5_K: Q4_K plus one high bit per code (gguf/src/lib.rs:1819-1861).  The tiled record is the Q4_K record
+// followed by the lanes' qh bytes: lane (row j, group g) holds the bytes 8 g .. 8 g + 7 of its row's qh, whose bit s is
+// the fifth bit of the lane's element in sub-block s: one rotate and one and-or per operand word put it on bit 4 (low
+// nibbles) or 8 (high nibbles) of the 16-bit code, still an exact f16 subnormal.
+// FMT = FH_Q5_0: Q4_0 plus one high bit per code (gguf/src/lib.rs:1046-1073), d * (code - 16): the Q4_0 record followed
+// by one byte per lane and block with the fifth bits of the lane's eight elements.
 // MR > 1: MR activation rows (nsplit then carries the number of valid ones; plain input, epilogues none / add2):
 // the weights are unpacked once per step and multiplied with the operand of every row; a wavefront stages its
 // blocks of all rows, images interleaved [block][row] so that every operand address is the base plus a constant.
@@ -82,8 +88,11 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     // Q4_K: the sums of the activations per sub-block (they multiply the block minimums) come from one more MFMA per
     // block, whose B operand is the constant code 1 and whose A operand is the whole image (every row at once),
     // instead of from adds and lane exchanges in the staging
-    constexpr bool ONES = FMT == FH_Q4_K;
+    constexpr bool ONES = FMT == FH_Q4_K || FMT == FH_Q5_K;
+    constexpr bool Q5 = FMT == FH_Q5_K || FMT == FH_Q5_0;
+    constexpr bool Q40 = FMT == FH_Q4_0 || FMT == FH_Q5_0; // eight 32-blocks per 256 activations, a byte = elements i, i + 16
     constexpr bool HP = EPI == FH_EPI_SWIGLU && TPW == 1;
+    static_assert(!(HP && Q5) && (!Q5 || (MR == 1 && RS == 1)), "5-bit formats: whole tiles, one row");
     constexpr int NT = (EPI == FH_EPI_SWIGLU && !HP) ? 2 : 1;
     constexpr int TOUT = TPW / NT; // output tiles of the workgroup
     extern __shared__ uint4 lds[];
@@ -99,8 +108,9 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     const int64_t nout = EPI == FH_EPI_SWIGLU ? q.n / 2 : q.n;
     const int64_t tiles_out = (nout + 15) / 16;
     const int b0 = wave * NB;
-    constexpr int REC = FMT == FH_Q4_0 ? 1152 : (FMT == FH_Q8_0 ? 1088 : 2304); // bytes of a tiled record
-    constexpr int CHUNK = FMT == FH_Q8_0 ? 4352 : 2304;                          // bytes per 256 activations and tile
+    // bytes of a tiled record, and per 256 activations and tile
+    constexpr int REC = FMT == FH_Q4_0 ? 1152 : (FMT == FH_Q8_0 ? 1088 : (FMT == FH_Q5_0 ? 1408 : (FMT == FH_Q5_K ? 2816 : 2304)));
+    constexpr int CHUNK = FMT == FH_Q8_0 ? 4352 : ((FMT == FH_Q5_0 || FMT == FH_Q5_K) ? 2816 : 2304);
     const uint8_t *ph[TPW], *pq[TPW];
     if constexpr (HP) {
         const int64_t tile = (int64_t)(blockIdx.x >> 1) + (j < 8 ? 0 : nout / 16);
@@ -133,8 +143,8 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         // a tile past the end re-reads the last tile (its rows are never stored)
         const int64_t tl = to < tiles_out ? tile : tile - (to - (tiles_out - 1));
         const uint8_t *rec = q.data + tl * q.recs * REC + (int64_t)(boff + b0) * CHUNK;
-        if (FMT == FH_Q4_0) { // d of the blocks 2g, 2g+1 of this lane's row; quants of the two records
-            ph[tp] = rec + (g >> 1) * 1152 + 1024 + 8 * j + 4 * (g & 1);
+        if (Q40) { // d of the blocks 2g, 2g+1 of this lane's row; quants of the two records
+            ph[tp] = rec + (g >> 1) * REC + 1024 + 8 * j + 4 * (g & 1);
             pq[tp] = rec + lane * 16;
         } else if (FMT == FH_Q8_0) { // record g holds the blocks 2g, 2g+1
             ph[tp] = rec + g * 1088 + 1024 + 4 * j;
@@ -179,7 +189,20 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     for (int r = 0; r < PER; r++)
 #pragma unroll
         for (int tp = 0; tp < TPW; tp++) {
-            if (FMT == FH_Q4_0) {
+            if constexpr (FMT == FH_Q5_0) { // the Q4_0 records, each followed by the lane's fifth bits (one byte per block)
+                w[tp][r].h.x = *(const uint32_t *)(ph[tp] + r * CHUNK);
+                w[tp][r].qa = *(const uint4 *)(pq[tp] + r * CHUNK);
+                w[tp][r].qb = *(const uint4 *)(pq[tp] + r * CHUNK + REC);
+                w[tp][r].qc.x = *(const uint32_t *)(pq[tp] + 1152 - 12 * lane + r * CHUNK);
+                w[tp][r].qc.y = *(const uint32_t *)(pq[tp] + 1152 - 12 * lane + r * CHUNK + REC);
+            } else if constexpr (FMT == FH_Q5_K) { // the Q4_K record followed by the lane's eight qh bytes
+                w[tp][r].h = *(const uint4 *)(ph[tp] + r * CHUNK);
+                w[tp][r].qa = *(const uint4 *)(pq[tp] + r * CHUNK);
+                w[tp][r].qb = *(const uint4 *)(pq[tp] + r * CHUNK + 1024);
+                const uint2 hb = *(const uint2 *)(pq[tp] + 2048 - 8 * lane + r * CHUNK);
+                w[tp][r].qc.x = hb.x;
+                w[tp][r].qc.y = hb.y;
+            } else if (FMT == FH_Q4_0) {
                 w[tp][r].h.x = *(const uint32_t *)(ph[tp] + r * 2304);
                 w[tp][r].qa = *(const uint4 *)(pq[tp] + r * 2304);
                 w[tp][r].qb = *(const uint4 *)(pq[tp] + r * 2304 + 1152);
@@ -238,12 +261,12 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
         am = max(am, dpp_u32<DPP_HALF_MIRROR>(am)); // quads are uniform now: lane 7-i is in the other quad
         // Q4_K: lanes 2 gg, 2 gg + 1 of a sub-block fill the two halves of operand slot gg; odd sub-blocks are the
         // high nibbles.  Q4_0: lanes gg and gg + 4 do, the second with the high nibbles' elements.
-        const int s = lane >> 3, gg = FMT == FH_Q4_0 ? lane & 3 : (lane >> 1) & 3;
-        const int half = FMT == FH_Q4_0 ? (lane >> 2) & 1 : lane & 1;
+        const int s = lane >> 3, gg = Q40 ? lane & 3 : (lane >> 1) & 3;
+        const int half = Q40 ? (lane >> 2) & 1 : lane & 1;
         // e = 14 - floor(log2(amax)) from the exponent field (zero / subnormal / inf / nan just clamp)
         int e = 141 - (int)((am >> 23) & 0xFFu);
         e = e > 100 ? 100 : (e < -100 ? -100 : e);
-        const int eo = e - (FMT == FH_Q8_0 ? 0 : 4 * (FMT == FH_Q4_0 ? half : s & 1)); // high nibbles: codes x 16
+        const int eo = e - (FMT == FH_Q8_0 ? 0 : 4 * (Q40 ? half : s & 1)); // high nibbles: codes x 16
         const float sc = __uint_as_float((uint32_t)(eo + 127) << 23);
         // hi = f16(x * sc), lo = f16(x * sc - hi) (x * sc is exact, a power of two, so the fused form rounds once),
         // written straight into the halves of the packed words in operand order (elements 0, 2 | 1, 3)
@@ -431,13 +454,33 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
                         const uint32_t k64 = 0x64646464u;
                         bo = make_uint4(__builtin_amdgcn_perm(k64, c0, 0x04020400u), __builtin_amdgcn_perm(k64, c0, 0x04030401u),
                                         __builtin_amdgcn_perm(k64, c1, 0x04020400u), __builtin_amdgcn_perm(k64, c1, 0x04030401u));
-                    } else if (FMT == FH_Q4_0) { // one word per block: low nibbles, then high nibbles
+                    } else if (Q40) { // one word per block: low nibbles, then high nibbles
                         const uint32_t w0 = (st & 3) == 0 ? wq.x : ((st & 3) == 1 ? wq.y : ((st & 3) == 2 ? wq.z : wq.w));
                         bo = make_uint4(w0 & LO, (w0 >> 8) & LO, w0 & HI, (w0 >> 8) & HI);
+                        if constexpr (FMT == FH_Q5_0) {
+                            // the block's byte of fifth bits: bits 0-3 for the low-nibble elements of the lane's four
+                            // bytes, bits 4-7 for the high-nibble ones; a multiplication copies four bits to the two
+                            // halves of a word, the mask keeps the one of each half (on bit 4 / 8 of the 16-bit code)
+                            const uint32_t hw = ((st & 4) ? w[tp][r].qc.y : w[tp][r].qc.x) >> (8 * (st & 3));
+                            const uint32_t l4 = hw & 0xFu, h4 = (hw >> 4) & 0xFu;
+                            bo.x |= (l4 * 0x40010u) & 0x00100010u;
+                            bo.y |= (l4 * 0x20008u) & 0x00100010u;
+                            bo.z |= (h4 * 0x400100u) & 0x01000100u;
+                            bo.w |= (h4 * 0x200080u) & 0x01000100u;
+                        }
                     } else {
                         const uint32_t w0 = (st & 2) ? wq.z : wq.x, w1 = (st & 2) ? wq.w : wq.y;
                         const uint32_t msk = (st & 1) ? HI : LO;
                         bo = make_uint4(w0 & msk, (w0 >> 8) & msk, w1 & msk, (w1 >> 8) & msk);
+                        if constexpr (FMT == FH_Q5_K) { // bit st of qh byte e is the fifth bit of element e in this step
+                            const int pos = (st & 1) ? 8 : 4;
+                            const uint32_t m5 = 0x00010001u << pos, hx = w[tp][r].qc.x, hy = w[tp][r].qc.y;
+                            const int r0 = (st - pos) & 31, r1 = (8 + st - pos) & 31;
+                            bo.x |= __builtin_amdgcn_alignbit(hx, hx, r0) & m5;
+                            bo.y |= __builtin_amdgcn_alignbit(hx, hx, r1) & m5;
+                            bo.z |= __builtin_amdgcn_alignbit(hy, hy, r0) & m5;
+                            bo.w |= __builtin_amdgcn_alignbit(hy, hy, r1) & m5;
+                        }
                     }
                     half8 bv;
                     __builtin_memcpy(&bv, &bo, 16);
@@ -462,8 +505,8 @@ __device__ __forceinline__ void qmv_q4k_m1_body(QView q, const float *__restrict
     #pragma unroll
                 for (int tp = 0; tp < TPW; tp++) {
                     const uint4 h = w[tp][r].h;
-                    if (FMT == FH_Q4_0 || FMT == FH_Q8_0) {
-                        const float off = FMT == FH_Q8_0 ? 1152.0f : 8.0f;
+                    if (Q40 || FMT == FH_Q8_0) {
+                        const float off = FMT == FH_Q8_0 ? 1152.0f : (FMT == FH_Q5_0 ? 16.0f : 8.0f);
                         const float da = fh_h2f((uint16_t)(h.x & 0xFFFF)), db = fh_h2f((uint16_t)(h.x >> 16));
                         acc[tp][mr] = fmaf(dd[tp][mr][0] + dd[tp][mr][1], da * fc.x, acc[tp][mr]);
                         acc[tp][mr] = fmaf(dd[tp][mr][2] + dd[tp][mr][3], db * fc.y, acc[tp][mr]);
@@ -595,6 +638,34 @@ static fh_status q4k_m1_launch(const fh_qmatrix *q, const float *x, float *y, co
                            float, int, FhRopeArgs);
     kern_t kern;
     const int in = ex.nsplit > 0 ? 2 : (ex.nw ? 1 : 0); // input: plain, rms_norm, attention partials
+    if (q->type == FH_Q5_0) { // (17 registers of weights per block tile, as Q8_0)
+        if constexpr ((EPI == FH_EPI_NONE || EPI == FH_EPI_ADD2 || EPI == FH_EPI_SWIGLU) && !(EPI == FH_EPI_SWIGLU && TPW == 1)) {
+            if (in != 0) return FH_ERR_UNSUPPORTED;
+            if constexpr (TPW * PER == 1) kern = k_qmv_q40_m1_w8<FH_Q5_0, TPW, PER, EPI>;
+            else kern = k_qmv_q40_m1<FH_Q5_0, TPW, PER, EPI>;
+            FH_TRY(fh_kernel_lds(q->dev, (const void *)kern, 160 * 1024));
+            kern<<<dim3(grid, 1), dim3(64 * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, nullptr, nullptr, 0.f, 0,
+                                                                        ex.rk);
+            FH_HIP(hipGetLastError());
+            return FH_OK;
+        } else {
+            return FH_ERR_UNSUPPORTED;
+        }
+    }
+    if (q->type == FH_Q5_K) { // (14 registers of weights per block tile: budgeted like Q8_0)
+        if constexpr ((EPI == FH_EPI_NONE || EPI == FH_EPI_ADD2 || EPI == FH_EPI_SWIGLU) && !(EPI == FH_EPI_SWIGLU && TPW == 1)) {
+            if (in != 0) return FH_ERR_UNSUPPORTED;
+            if constexpr (TPW * PER == 1) kern = k_qmv_q40_m1_w8<FH_Q5_K, TPW, PER, EPI>;
+            else kern = k_qmv_q40_m1<FH_Q5_K, TPW, PER, EPI>;
+            FH_TRY(fh_kernel_lds(q->dev, (const void *)kern, 160 * 1024));
+            kern<<<dim3(grid, 1), dim3(64 * SW), lds, q->dev->stream>>>(fh_view(q), x, y, a, b, SW, nullptr, nullptr, 0.f, 0,
+                                                                        ex.rk);
+            FH_HIP(hipGetLastError());
+            return FH_OK;
+        } else {
+            return FH_ERR_UNSUPPORTED;
+        }
+    }
     if (q->type == FH_Q4_0 || q->type == FH_Q8_0) {
         if constexpr (EPI == FH_EPI_NONE || EPI == FH_EPI_ADD2 || EPI == FH_EPI_SWIGLU) {
             if (in != 0) return FH_ERR_UNSUPPORTED;
@@ -798,7 +869,8 @@ fh_status fh_launch_q4k_m1_ropekv(const fh_qmatrix *q, const float *x, const flo
 static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra &ex, float *y, int epi, const float *a,
                             const float *b) {
     fh_device *dev = q->dev;
-    if (q->type != FH_Q4_K && !((q->type == FH_Q4_0 || q->type == FH_Q8_0) && q->k % 256 == 0 && ex.ksplit == 1))
+    if (q->type != FH_Q4_K && !((q->type == FH_Q4_0 || q->type == FH_Q8_0) && q->k % 256 == 0 && ex.ksplit == 1) &&
+        !((q->type == FH_Q5_K || (q->type == FH_Q5_0 && q->k % 256 == 0)) && ex.ksplit == 1 && !ex.nw && ex.nsplit == 0))
         return FH_ERR_UNSUPPORTED;
     const int64_t kb256 = q->k / 256; // 256-element blocks (Q4_0: eight of its 32-blocks, two records)
     if (ex.ksplit < 1 || kb256 % ex.ksplit || (ex.ksplit > 1 && (epi != FH_EPI_ACC || ex.nw))) return FH_ERR_UNSUPPORTED;
@@ -829,7 +901,7 @@ static fh_status q4k_m1_any(const fh_qmatrix *q, const float *x, const Q4kExtra 
     int tpw = (int)dev->opt_matvec_tiles;
     if (tpw != 1 && tpw != 2 && tpw != 4) tpw = tiles > dev->compute_units ? 2 : 1;
     // SwiGLU: half a gate tile and half an up tile per wavefront when the rows allow it (workgroups half as heavy)
-    const bool half_pairs = epi == FH_EPI_SWIGLU && nout % 16 == 0 && dev->opt_matvec_tiles <= 1;
+    const bool half_pairs = epi == FH_EPI_SWIGLU && nout % 16 == 0 && dev->opt_matvec_tiles <= 1 && q->type != FH_Q5_K && q->type != FH_Q5_0;
     if (epi == FH_EPI_SWIGLU) tpw = half_pairs ? 1 : (tpw < 2 ? 2 : tpw);
     if (ex.nsplit > 0) { // merging attention partials: every workgroup merges its slice again, so fewer, fatter ones
         tpw = (int)dev->opt_wo_tiles;

@@ -1754,7 +1754,7 @@ static fh_status qmm_launch_dense(const fh_qmatrix *q, const _Float16 *xh, const
 fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y) {
     fh_device *dev = q->dev;
     const int64_t K = q->k;
-    if (fh_is_plain(q->type) && ((q->type != FH_W_F16 && q->type != FH_W_F32) || K % 32 != 0))
+    if (fh_single_row_only(q->type) && ((q->type != FH_W_F16 && q->type != FH_W_F32) || K % 32 != 0))
         FH_FAIL(FH_ERR_UNSUPPORTED, "type %u with k = %lld has no matrix-core matmul (it runs through fh_qmatmul)", q->type,
                 (long long)K);
     FH_REQUIRE((m + 127) / 128 <= 65535, "m = %d too large for one launch", m);

@@ -337,11 +337,48 @@ def test_plain_types_known_answers(dev):
     assert y[0, 0] == 32896.0
 
 
+@pytest.mark.parametrize("ty", [synth.Q5_K, synth.Q5_0], ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("n,k", [(72, 1024), (1000, 4096), (96, 14336), (4096, 256), (40, 8192)])
+def test_five_bit_formats_single_row_matrix_core_kernel(dev, oracle, ty, n, k):
+    """Q5_K and Q5_0 with one activation row go through the single-row matrix-core kernel, which reads the file's own
+    block order and adds the fifth bit to the 4-bit code of its Q4_K / Q4_0 form: ragged last tile, 1 .. 56 chunks of
+    k, one / two / four row tiles and one / two / four chunks per wavefront, plain, two-residual and SwiGLU epilogues,
+    against the checker and against the per-element kernel."""
+    raw = synth.random_weight(ty, n, k, seed=330 + ty, sigma=2e-3)
+    x = synth.random_activation(1, k, seed=331)
+    a, b = synth.random_activation(1, n, seed=332), synth.random_activation(1, n, seed=333)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    want = oracle.q_mat_mul(ty, x, raw, n)
+    xt = Tensor.from_slice(dev, x)
+    dev.set_option("matvec_kernel", 1)
+    slow = xt.q_mat_mul(q).as_slice()
+    dev.set_option("matvec_kernel", 0)
+    assert_close(slow, want, what="per-element kernel")
+    try:
+        for tiles, per in ((0, 0), (1, 1), (2, 1), (1, 2), (4, 1), (1, 4), (2, 2)):
+            dev.set_option("matvec_tiles", tiles)
+            dev.set_option("matvec_per", per)
+            got = xt.q_mat_mul(q, out=Tensor.filled_bytes(dev, (1, n), 0xFF)).as_slice()
+            assert_close(got, want, what=f"{NAMES[ty]} {n}x{k} tiles={tiles} per={per}")
+            assert_close(got, slow, abs_tol=2e-3, rel_tol=1e-4, what=f"{NAMES[ty]} {n}x{k} against the per-element kernel")
+            got = xt.q_mat_mul_add2(q, Tensor.from_slice(dev, a), Tensor.from_slice(dev, b),
+                                    out=Tensor.filled_bytes(dev, (1, n), 0xFF)).as_slice()
+            assert_close(got, oracle.add3(want, a, b), what=f"add2 {NAMES[ty]} {n}x{k} tiles={tiles} per={per}")
+            if n % 32 == 0:
+                got = xt.q_mat_mul_swiglu(q, out=Tensor.filled_bytes(dev, (1, n // 2), 0xFF)).as_slice()
+                assert_close(got, oracle.swiglu(want[:, :n // 2], want[:, n // 2:]),
+                             what=f"swiglu {NAMES[ty]} {n}x{k} tiles={tiles} per={per}")
+    finally:
+        dev.set_option("matvec_tiles", 0)
+        dev.set_option("matvec_per", 0)
+
+
 @pytest.mark.parametrize("ty", PLAIN, ids=lambda t: NAMES[t])
 @pytest.mark.parametrize("m", [1, 4, 33])
 def test_plain_types_matmul_and_glue(dev, oracle, ty, m):
-    """q_mat_mul, the SwiGLU / add2 epilogues, concat_rows (any row counts) and the embedding gather."""
-    n, k = 72, 1024
+    """q_mat_mul, the SwiGLU / add2 epilogues, concat_rows (any row counts for dense rows, whole 16-row tiles for the
+    5-bit formats, which are tiled like the 4-bit ones) and the embedding gather."""
+    n, k = (72, 1024) if ty in (synth.W_F32, synth.W_F16) else (80, 1024)
     raw_g = synth.random_weight(ty, n, k, seed=310 + ty, sigma=2e-3)
     raw_u = synth.random_weight(ty, n, k, seed=311 + ty, sigma=2e-3)
     x = synth.random_activation(m, k, seed=312 + m)
