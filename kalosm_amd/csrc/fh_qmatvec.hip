@@ -355,6 +355,16 @@ fh_status fh_launch_qmatvec(const fh_qmatrix *q, const float *x, int m, float *y
         fh_status st = fh_launch_q4k_m1(q, x, y, epi, a, b);
         if (st != FH_ERR_UNSUPPORTED) return st;
     }
+    // the 5-bit formats have the single-row kernel only: a few rows are a launch each (10 us a row against 110 - 640 us
+    // for 2 .. 16 rows through the per-element kernel at 14336 x 4096)
+    if (kernel != 1 && kernel != 3 && (q->type == FH_Q5_K || q->type == FH_Q5_0) && q->k % 256 == 0 && m >= 2 && m <= 16) {
+        const int64_t nout = epi == FH_EPI_SWIGLU ? q->n / 2 : q->n;
+        fh_status st = FH_OK;
+        for (int r = 0; r < m && st == FH_OK; r++)
+            st = fh_launch_q4k_m1(q, x + (int64_t)r * q->k, y + (int64_t)r * nout, epi, a ? a + (int64_t)r * nout : nullptr,
+                                  b ? b + (int64_t)r * nout : nullptr);
+        if (st != FH_ERR_UNSUPPORTED) return st;
+    }
     if (kernel == 0 && q->type != FH_Q6_K && !fh_single_row_only(q->type) && m >= 2 && m <= 4 && dev->opt_matvec_rows != 1) {
         fh_status st = fh_launch_q4k_rows(q, x, m, y, epi, a, b);
         if (st != FH_ERR_UNSUPPORTED) return st;
@@ -393,7 +403,9 @@ extern "C" fh_status fh_qmatmul(const fh_qmatrix *q, const float *x_dev, int32_t
     // dense f16 / f32 weight rows (core/src/quantized/matmul/kernel.rs:132-193 routes them to the dense matmul) take
     // the matrix-core tiles as well once there are rows to fill them
     const bool dense = (q->type == FH_W_F16 || q->type == FH_W_F32) && q->k % 32 == 0;
-    if (((m > 16 && mk != 1) || mk >= 2) && (!fh_single_row_only(q->type) || dense)) return fh_launch_qmatmul_tile(q, x_dev, 0, m, y_dev);
+    // (the 5-bit formats have no batch kernel for 2 .. 16 rows: rows are a launch each up to 12, tiles above)
+    const int tile_from = (q->type == FH_Q5_K || q->type == FH_Q5_0) && q->k % 256 == 0 ? 12 : 16;
+    if (((m > tile_from && mk != 1) || mk >= 2) && (!fh_is_plain(q->type) || dense)) return fh_launch_qmatmul_tile(q, x_dev, 0, m, y_dev);
     return fh_launch_qmatvec(q, x_dev, m, y_dev, FH_EPI_NONE, nullptr, nullptr);
 }
 

@@ -243,10 +243,25 @@ __device__ __forceinline__ void decode8(const QView &q, int64_t tile16, int j, i
             w[i] = (float)((int)((c >> (8 * i)) & 15u) - 8) * d;
             w[4 + i] = (float)((int)((c >> (8 * i + 4)) & 15u) - 8) * d;
         }
-    } else if (T == FH_Q4_K) {
-        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 3)) * 2304;
+    } else if (T == FH_Q5_0) { // the Q4_0 record plus one byte of fifth bits per lane and block; d * (code - 16)
+        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 2)) * 1408;
+        const int u = ks & 3;
+        const uint32_t c = *(const uint32_t *)(rec + (g * 16 + j) * 16 + 4 * u);
+        const uint32_t hb = rec[q50_qh_off(j, u, g)];
+        const float d = fh_h2f(fh_ld16(rec + 1024 + 8 * j + 2 * u));
+        p0 = 4 * g;
+        p1 = 16 + 4 * g;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[i] = (float)((int)(((c >> (8 * i)) & 15u) | (((hb >> i) & 1u) << 4)) - 16) * d;
+            w[4 + i] = (float)((int)(((c >> (8 * i + 4)) & 15u) | (((hb >> (4 + i)) & 1u) << 4)) - 16) * d;
+        }
+    } else if (T == FH_Q4_K || T == FH_Q5_K) { // Q5_K: the Q4_K record plus the lane's eight qh bytes
+        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 3)) * (T == FH_Q5_K ? 2816 : 2304);
         const int sb = ks & 7, p = sb >> 2, u = (sb >> 1) & 1, hn = sb & 1;
         const uint2 c = *(const uint2 *)(rec + 256 + p * 1024 + (g * 16 + j) * 16 + 8 * u);
+        uint2 hb = make_uint2(0, 0);
+        if (T == FH_Q5_K) hb = *(const uint2 *)(rec + 2304 + (g * 16 + j) * 8);
         const uint4 h = *(const uint4 *)(rec + 16 * j);
         const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
         const uint32_t scw = sb < 4 ? (h.y & 0x3F3F3F3Fu) : ((h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u));
@@ -256,8 +271,8 @@ __device__ __forceinline__ void decode8(const QView &q, int64_t tile16, int j, i
         const int sh = 4 * hn;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float a = scale * (float)((c.x >> (8 * i + sh)) & 15u);
-            const float b = scale * (float)((c.y >> (8 * i + sh)) & 15u);
+            const float a = scale * (float)(((c.x >> (8 * i + sh)) & 15u) + (((hb.x >> (8 * i + sb)) & 1u) << 4));
+            const float b = scale * (float)(((c.y >> (8 * i + sh)) & 15u) + (((hb.y >> (8 * i + sb)) & 1u) << 4));
             w[i] = a - off;
             w[4 + i] = b - off;
         }
@@ -422,11 +437,12 @@ __global__ __launch_bounds__(64 * WGN * WGM) void k_qmm_tile(QView q, const _Flo
 struct QmmRaw {
     uint32_t a, b; // code words
     uint4 h;       // scale material (format dependent)
+    uint32_t e0, e1; // fifth bits (Q5_0: one byte; Q5_K: the lane's eight qh bytes)
 };
 
 template <int T>
 __device__ __forceinline__ void qmm_load_raw(const QView &q, int64_t tile16, int j, int g, int ks, QmmRaw &r) {
-    r.a = r.b = 0;
+    r.a = r.b = r.e0 = r.e1 = 0;
     r.h = make_uint4(0, 0, 0, 0);
     if (T == FH_Q8_0) {
         const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 1)) * 1088;
@@ -435,18 +451,24 @@ __device__ __forceinline__ void qmm_load_raw(const QView &q, int64_t tile16, int
         r.a = c.x;
         r.b = c.y;
         r.h.x = fh_ld16(rec + 1024 + 4 * j + 2 * u);
-    } else if (T == FH_Q4_0) {
-        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 2)) * 1152;
+    } else if (T == FH_Q4_0 || T == FH_Q5_0) {
+        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 2)) * (T == FH_Q5_0 ? 1408 : 1152);
         const int u = ks & 3;
         r.a = *(const uint32_t *)(rec + (g * 16 + j) * 16 + 4 * u);
         r.h.x = fh_ld16(rec + 1024 + 8 * j + 2 * u);
-    } else if (T == FH_Q4_K) {
-        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 3)) * 2304;
+        if (T == FH_Q5_0) r.e0 = rec[q50_qh_off(j, u, g)];
+    } else if (T == FH_Q4_K || T == FH_Q5_K) {
+        const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 3)) * (T == FH_Q5_K ? 2816 : 2304);
         const int sb = ks & 7, p = sb >> 2, u = (sb >> 1) & 1;
         const uint2 c = *(const uint2 *)(rec + 256 + p * 1024 + (g * 16 + j) * 16 + 8 * u);
         r.a = c.x;
         r.b = c.y;
         r.h = *(const uint4 *)(rec + 16 * j);
+        if (T == FH_Q5_K) {
+            const uint2 hb = *(const uint2 *)(rec + 2304 + (g * 16 + j) * 8);
+            r.e0 = hb.x;
+            r.e1 = hb.y;
+        }
     } else {
         const uint8_t *rec = q.data + (tile16 * q.recs + (ks >> 3)) * 3360;
         const int t = ks & 7;
@@ -478,7 +500,16 @@ __device__ __forceinline__ void qmm_decode_raw(const QmmRaw &r, int g, int ks, f
             w[i] = (float)((int)((r.a >> (8 * i)) & 15u) - 8) * d;
             w[4 + i] = (float)((int)((r.a >> (8 * i + 4)) & 15u) - 8) * d;
         }
-    } else if (T == FH_Q4_K) {
+    } else if (T == FH_Q5_0) {
+        const float d = fh_h2f((uint16_t)r.h.x);
+        p0 = 4 * g;
+        p1 = 16 + 4 * g;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[i] = (float)((int)(((r.a >> (8 * i)) & 15u) | (((r.e0 >> i) & 1u) << 4)) - 16) * d;
+            w[4 + i] = (float)((int)(((r.a >> (8 * i + 4)) & 15u) | (((r.e0 >> (4 + i)) & 1u) << 4)) - 16) * d;
+        }
+    } else if (T == FH_Q4_K || T == FH_Q5_K) {
         const int sb = ks & 7, hn = sb & 1;
         const uint4 h = r.h;
         const float d = fh_h2f((uint16_t)(h.x & 0xFFFF)), dmin = fh_h2f((uint16_t)(h.x >> 16));
@@ -489,8 +520,8 @@ __device__ __forceinline__ void qmm_decode_raw(const QmmRaw &r, int g, int ks, f
         const int sh = 4 * hn;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float a = scale * (float)((r.a >> (8 * i + sh)) & 15u);
-            const float b = scale * (float)((r.b >> (8 * i + sh)) & 15u);
+            const float a = scale * (float)(((r.a >> (8 * i + sh)) & 15u) + (T == FH_Q5_K ? ((r.e0 >> (8 * i + sb)) & 1u) << 4 : 0u));
+            const float b = scale * (float)(((r.b >> (8 * i + sh)) & 15u) + (T == FH_Q5_K ? ((r.e1 >> (8 * i + sb)) & 1u) << 4 : 0u));
             w[i] = a - off;
             w[4 + i] = b - off;
         }
@@ -1754,7 +1785,7 @@ static fh_status qmm_launch_dense(const fh_qmatrix *q, const _Float16 *xh, const
 fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf16, int m, float *y) {
     fh_device *dev = q->dev;
     const int64_t K = q->k;
-    if (fh_single_row_only(q->type) && ((q->type != FH_W_F16 && q->type != FH_W_F32) || K % 32 != 0))
+    if (fh_is_plain(q->type) && K % 32 != 0)
         FH_FAIL(FH_ERR_UNSUPPORTED, "type %u with k = %lld has no matrix-core matmul (it runs through fh_qmatmul)", q->type,
                 (long long)K);
     FH_REQUIRE((m + 127) / 128 <= 65535, "m = %d too large for one launch", m);
@@ -1781,6 +1812,8 @@ fh_status fh_launch_qmatmul_tile(const fh_qmatrix *q, const void *x, int x_is_bf
     case FH_Q8_0: QMM_GO(FH_Q8_0);
     case FH_Q4_K: QMM_GO(FH_Q4_K);
     case FH_Q6_K: QMM_GO(FH_Q6_K);
+    case FH_Q5_0: QMM_GO(FH_Q5_0);
+    case FH_Q5_K: QMM_GO(FH_Q5_K);
     case FH_W_F16: return x_is_bf16 ? qmm_launch_dense<FH_W_F16, 1>(q, xh, xl, rs, m, y) : qmm_launch_dense<FH_W_F16, 2>(q, xh, xl, rs, m, y);
     case FH_W_F32: return x_is_bf16 ? qmm_launch_dense<FH_W_F32, 1>(q, xh, xl, rs, m, y) : qmm_launch_dense<FH_W_F32, 2>(q, xh, xl, rs, m, y);
     }

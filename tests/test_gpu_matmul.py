@@ -46,6 +46,26 @@ def test_tile_matmul_f32_vs_checker(dev, oracle, ty, m, n, k):
         assert_close(got, want, what=f"{NAMES[ty]} {n}x{k} m={m} kernel option {force}")
 
 
+@pytest.mark.parametrize("ty", [synth.Q5_0, synth.Q5_K], ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("m,n,k", [(17, 272, 2048), (33, 130, 1024), (65, 100, 768), (130, 300, 1024), (300, 1024, 4096),
+                                   (3, 37, 512)])
+def test_tile_matmul_five_bit_formats(dev, oracle, ty, m, n, k):
+    """Q5_0 and Q5_K through the matrix-core tile kernels (decoded with the exact f32 block arithmetic, then split
+    into f16 pairs like the other formats): ragged m and n, the 128 x 128 and the pipelined 128 x 256 kernel, the
+    default dispatch (per-element kernel up to 16 rows, tiles above), f32 and bf16 activations."""
+    raw = synth.random_weight(ty, n, k, seed=250 + ty, sigma=2e-3)
+    x = synth.random_activation(m, k, seed=260 + m)
+    q = QMatrix.from_raw_bytes(dev, (n, k), raw, ty)
+    want = oracle.q_mat_mul(ty, x, raw, n, fast=True)
+    for force in (0, 2, 4):
+        got = tile_matmul(dev, x, q, force)
+        assert_close(got, want, what=f"{NAMES[ty]} {n}x{k} m={m} kernel option {force}")
+    if m > 16:
+        bits, xb = bf16_round(x)
+        got = Tensor.from_slice(dev, bits, dtype="bf16").q_mat_mul(q, out=Tensor.filled_bytes(dev, (m, n), 0xFF)).as_slice()
+        assert_close(got, oracle.q_mat_mul(ty, xb, raw, n, fast=True), what=f"{NAMES[ty]} {n}x{k} m={m} bf16")
+
+
 @pytest.mark.parametrize("ty", ALL, ids=lambda t: NAMES[t])
 @pytest.mark.parametrize("m,n,k", [(200, 384, 4096), (70, 132, 8192), (512, 4096, 2048), (512, 4096, 4096)])
 def test_tile_matmul_split_k(dev, oracle, ty, m, n, k):
