@@ -5,10 +5,10 @@ A step is one pass of the Q4_K decode matvec (batch 1) over the four Llama-3-8B 
 (4096x4096 q/o, 1024x4096 k/v, 14336x4096 gate/up, 4096x14336 down), activations f32 N(0,1), weights
 random Q4_K super-blocks (f16 d/dmin ~ N(0, 0.02), 6-bit scales/mins, uniform nibbles), all resident in
 HBM before the timed region.  Each shape rotates over enough distinct weight buffers to exceed the
-256 MB last-level cache and every timed train walks on through that pool from where the train before it stopped
-(each train is a recording of its own), so the bytes come from HBM whatever K is.  The K launches of a shape are one
-recorded train; `--trains` trains are timed and the median train is the shape's time (K steps are timed, the
-repetitions only steady the number).
+256 MB last-level cache, and a recorded train of a shape has max(K, copies, 100) launches, one after the other through
+the whole pool, so a buffer is read again only after 640 MB of others: the bytes come from HBM whatever K is.  The
+train is replayed `--trains` times and the median replay gives the shape's time per launch; the reported step time is
+K steps at that rate (the repetitions only steady the number).
 
 Prints ONE JSON line: whole-path GB/s (algorithmic bytes / device time), the roofline of the dominant
 kernel and the CPU checker timed on the host cores beside it.  The same line carries the other benchmark
@@ -54,29 +54,11 @@ def measured_traffic():
     return (int(m.group(1)) if m else None), (c.group(1) if c else None)
 
 
-def timed_trains(dev, enqueue, trains: int, use_graph: bool = True, rotate: bool = False):
-    """Median device milliseconds of `trains` runs of a launch sequence (recorded and replayed unless use_graph is
-    off).  rotate: `enqueue(t)` enqueues train number t (0 is run untimed first) and every train is a recording of
-    its own, so that consecutive trains walk on through a pool of buffers instead of reading the first train's
-    again - a train of few launches would otherwise find its few buffers in the 256 MB memory-side cache.
-    Otherwise `enqueue()` is recorded once and replayed."""
+def timed_trains(dev, enqueue, trains: int, use_graph: bool = True):
+    """Median device milliseconds of `trains` runs of the launch sequence `enqueue()` (recorded once and replayed
+    unless use_graph is off; one untimed run first)."""
     ms = []
-    if rotate:
-        runs = []
-        for t in range(trains + 1):
-            if use_graph:
-                dev.graph_begin()
-                enqueue(t)
-                runs.append(dev.graph_end().launch)
-            else:
-                runs.append(lambda t=t: enqueue(t))
-        runs[0]()
-        dev.sync()
-        for run in runs[1:]:
-            dev.timer_start()
-            run()
-            ms.append(dev.timer_stop())
-    elif use_graph:
+    if use_graph:
         dev.graph_begin()
         enqueue()
         g = dev.graph_end()
@@ -88,11 +70,21 @@ def timed_trains(dev, enqueue, trains: int, use_graph: bool = True, rotate: bool
             ms.append(dev.timer_stop())
         del g
     else:
+        enqueue()
+        dev.sync()
         for _ in range(trains):
             dev.timer_start()
             enqueue()
             ms.append(dev.timer_stop())
     return statistics.median(ms), ms
+
+
+def train_length(steps: int, copies: int) -> int:
+    """Launches of one timed train over a pool of `copies` buffers that together exceed the memory-side cache twice
+    over: at least `steps`, at least once through the whole pool, so that a buffer is read again only after 640 MB of
+    others - every replay of the train then reads from HBM whatever `steps` is - and at least 100, so that what
+    starting a replay costs (some 17 us between the two events) does not weigh on the figure per launch."""
+    return max(steps, copies, 100)
 
 
 def matvec_sets(dev, ty, m: int):
@@ -132,11 +124,12 @@ def batch_leg(dev, sets_m1, steps: int, warmup: int, trains: int) -> list:
                      bytes=synth.matvec_bytes(synth.Q4_K, n, k, m))
             run_shape(t, warmup)
             dev.sync()
-            ms, _ = timed_trains(dev, lambda i: run_shape(t, steps, offset=warmup + i * steps), trains, rotate=True)
-            tot_ms += ms
+            L = train_length(steps, len(t["qs"]))
+            ms, _ = timed_trains(dev, lambda: run_shape(t, L, offset=warmup), trains)
+            tot_ms += ms / L
             tot_bytes += t["bytes"]
-            per.append({"n": n, "k": k, "us_per_launch": round(ms * 1e3 / steps, 3)})
-        gbs = tot_bytes * steps / (tot_ms * 1e-3) / 1e9
+            per.append({"n": n, "k": k, "us_per_launch": round(ms * 1e3 / L, 3), "launches_per_train": L})
+        gbs = tot_bytes / (tot_ms * 1e-3) / 1e9
         out.append({"rows": m, "GBps": round(gbs, 1), "shapes": per,
                     "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                  "frac": round(gbs / HBM_PEAK_GBS, 4)}})
@@ -159,8 +152,9 @@ def decoder_shapes_leg(dev, steps: int, warmup: int, trains: int) -> list:
         nbytes = synth.matvec_bytes(synth.Q4_K, n, k, 1)
         run_shape(s, warmup)
         dev.sync()
-        ms, _ = timed_trains(dev, lambda i: run_shape(s, steps, offset=warmup + i * steps), trains, rotate=True)
-        us = ms * 1e3 / steps
+        L = train_length(steps, copies)
+        ms, _ = timed_trains(dev, lambda: run_shape(s, L, offset=warmup), trains)
+        us = ms * 1e3 / L
         out.append({"n": n, "k": k, "us_per_launch": round(us, 3), "GBps": round(nbytes / us / 1e3, 1),
                     "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
         del s
@@ -197,8 +191,9 @@ def five_bit_leg(dev, steps: int, warmup: int, trains: int) -> list:
             nbytes = synth.matvec_bytes(ty, n, k, 1)
             run_shape(s, warmup)
             dev.sync()
-            ms, _ = timed_trains(dev, lambda i: run_shape(s, steps, offset=warmup + i * steps), trains, rotate=True)
-            us = ms * 1e3 / steps
+            L = train_length(steps, copies)
+            ms, _ = timed_trains(dev, lambda: run_shape(s, L, offset=warmup), trains)
+            us = ms * 1e3 / L
             e = {"weights": synth.TYPE_NAMES[ty], "n": n, "k": k, "us_per_launch": round(us, 3), "ns_per_KB": round(us * 1e6 / nbytes, 3),
                  "roofline": {"bound": "hbm", "achieved": round(nbytes / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                               "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}}
@@ -325,7 +320,8 @@ def prefill_legs(dev, trains: int, use_graph: bool = True, check: bool = False) 
 
         train()
         dev.sync()
-        ms, _ = timed_trains(dev, lambda i: train(7 + i * reps), trains, rotate=True)
+        reps = train_length(reps, len(kvs))
+        ms, _ = timed_trains(dev, lambda: train(7), trains)
         ms /= reps
         nbytes = kv_bytes + 2 * h * d * 2
         gbs = nbytes / ms / 1e6
@@ -363,14 +359,16 @@ def calibration(dev, trains: int, use_graph: bool, probes: bool = True) -> dict:
         used = nbytes // 16384 * 16384
         copies = max(1, total // used)
 
-        def train(t=0):
-            for i in range(L):
-                dev._lib.fh_probe_read(dev._h, C.c_void_p(buf.ptr + ((t * L + i) % copies) * used), used)
+        Lr = train_length(L, min(copies, -(-ROTATE_BYTES // used)))
+
+        def train():
+            for i in range(Lr):
+                dev._lib.fh_probe_read(dev._h, C.c_void_p(buf.ptr + (i % copies) * used), used)
 
         train()
         dev.sync()
-        ms, _ = timed_trains(dev, train, trains, use_graph, rotate=True)
-        us = ms * 1e3 / L
+        ms, _ = timed_trains(dev, train, trains, use_graph)
+        us = ms * 1e3 / Lr
         out["read"].append({"bytes": used, "us": round(us, 3), "GBps": round(used / us / 1e3, 1)})
     del buf
     if probes:
@@ -462,7 +460,8 @@ def main() -> int:
                     help="run 32 decode steps of the decoder with stream launches instead (for a kernel tracer)")
     ap.add_argument("--prefill", action="store_true", help="(default) kept for older command lines")
     ap.add_argument("--no-graph", action="store_true", help="launch on the stream instead of replaying a recorded graph")
-    ap.add_argument("--calib", action="store_true", help="(default) kept for older command lines")
+    ap.add_argument("--calib", action="store_true",
+                    help="add the device probes (dense MFMA rate, LDS read throughput, L2 next to an HBM stream) to the calibration")
     ap.add_argument("--no-calib", action="store_true",
                     help="skip the launch-floor calibration (an empty kernel and plain streaming reads of the matrices' sizes)")
     ap.add_argument("--calib-copy", action="store_true", help="append 4 device copies of 256 MiB (counter calibration)")
@@ -486,13 +485,14 @@ def main() -> int:
     for s in sets:
         run_shape(s, args.warmup)
     dev.sync()
-    per_shape_ms, all_ms = [], []
+    per_shape_ms, all_ms, lens = [], [], []
     t_wall0 = time.perf_counter()
     for s in sets:
-        ms, every = timed_trains(dev, lambda i: run_shape(s, args.steps, offset=args.warmup + i * args.steps), args.trains,
-                                 not args.no_graph, rotate=True)
-        per_shape_ms.append(ms)
-        all_ms.append(every)
+        L = train_length(args.steps, len(s["qs"]))
+        ms, every = timed_trains(dev, lambda: run_shape(s, L, offset=args.warmup), args.trains, not args.no_graph)
+        per_shape_ms.append(ms * args.steps / L)   # device time of `steps` launches at the train's rate
+        all_ms.append([e * args.steps / L for e in every])
+        lens.append(L)
     if args.calib_copy:  # a device-to-device copy of known size, to scale the FETCH_SIZE / WRITE_SIZE counters
         nbytes = 256 << 20
         a, b = Tensor(dev, (nbytes,), "u8"), Tensor(dev, (nbytes,), "u8")
@@ -529,7 +529,8 @@ def main() -> int:
                                "(4096x4096, 1024x4096, 14336x4096, 4096x14336), batch %d, one launch each per step" % m,
                    "batch": m, "weights_rotated_bytes_per_shape": ROTATE_BYTES, "device": info["name"],
                    "compute_units": info["compute_units"],
-                   "timing": "median of %d replays of each shape's %d-launch train" % (args.trains, args.steps)},
+                   "timing": "median of %d replays of each shape's recorded train of max(steps, weight copies, 100) = %s launches; "
+                             "the figures are per launch, scaled to %d steps" % (args.trains, lens, args.steps)},
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "shapes": shapes_out,
         "wall_ms_timed_region": round(wall_ms, 2),
@@ -578,7 +579,7 @@ def main() -> int:
 
     if not args.no_calib:
         # what one dependent launch costs on this device whatever the kernel does, in the same run and launch pattern
-        cal = calibration(dev, args.trains, not args.no_graph, probes=not args.no_legs)
+        cal = calibration(dev, args.trains, not args.no_graph, probes=args.calib)
         out["calibration"] = cal
         floor = {r["bytes"]: r["us"] for r in cal["read"]}
         tot = 0.0
