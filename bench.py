@@ -5,7 +5,7 @@ A step is one pass of the Q4_K decode matvec (batch 1) over the four Llama-3-8B 
 (4096x4096 q/o, 1024x4096 k/v, 14336x4096 gate/up, 4096x14336 down), activations f32 N(0,1), weights
 random Q4_K super-blocks (f16 d/dmin ~ N(0, 0.02), 6-bit scales/mins, uniform nibbles), all resident in
 HBM before the timed region.  Each shape rotates over enough distinct weight buffers to exceed the
-256 MB last-level cache, and a recorded train of a shape has max(K, copies, 100) launches, one after the other through
+256 MB last-level cache, and a recorded train of a shape has max(K, copies, 200) launches, one after the other through
 the whole pool, so a buffer is read again only after 640 MB of others: the bytes come from HBM whatever K is.  The
 train is replayed `--trains` times and the median replay gives the shape's time per launch; the reported step time is
 K steps at that rate (the repetitions only steady the number).
@@ -82,9 +82,9 @@ def timed_trains(dev, enqueue, trains: int, use_graph: bool = True):
 def train_length(steps: int, copies: int) -> int:
     """Launches of one timed train over a pool of `copies` buffers that together exceed the memory-side cache twice
     over: at least `steps`, at least once through the whole pool, so that a buffer is read again only after 640 MB of
-    others - every replay of the train then reads from HBM whatever `steps` is - and at least 100, so that what
+    others - every replay of the train then reads from HBM whatever `steps` is - and at least 200, so that what
     starting a replay costs (some 17 us between the two events) does not weigh on the figure per launch."""
-    return max(steps, copies, 100)
+    return max(steps, copies, 200)
 
 
 def matvec_sets(dev, ty, m: int):
@@ -529,7 +529,7 @@ def main() -> int:
                                "(4096x4096, 1024x4096, 14336x4096, 4096x14336), batch %d, one launch each per step" % m,
                    "batch": m, "weights_rotated_bytes_per_shape": ROTATE_BYTES, "device": info["name"],
                    "compute_units": info["compute_units"],
-                   "timing": "median of %d replays of each shape's recorded train of max(steps, weight copies, 100) = %s launches; "
+                   "timing": "median of %d replays of each shape's recorded train of max(steps, weight copies, 200) = %s launches; "
                              "the figures are per launch, scaled to %d steps" % (args.trains, lens, args.steps)},
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "shapes": shapes_out,
